@@ -1,0 +1,87 @@
+"""ctypes binding of libhyclora.so (the C ABI declared in include/hyclora.h).
+
+The library is the only implementation: if it is missing, or a call returns an error
+code, an exception is raised — there is no CPU or torch fallback.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_char_p, c_int, c_int64, c_void_p
+from pathlib import Path
+
+import torch
+
+_HERE = Path(__file__).resolve().parent
+LIB_PATH = _HERE / "libhyclora.so"
+
+_lib = None
+
+
+class HycError(RuntimeError):
+    """A C-ABI entry point returned a negative code."""
+
+    def __init__(self, fn: str, code: int, text: str):
+        super().__init__(f"{fn} failed: {text} (code {code})")
+        self.code = code
+
+
+# name -> (restype, argtypes)
+_P, _I, _L = c_void_p, c_int, c_int64
+_SIGNATURES = {
+    "hyc_error_string": (c_char_p, [_I]),
+    "hyc_abi_version": (_I, []),
+    "hyc_set_tuning": (_I, [c_char_p, _I]),
+    "hyc_quant_pack": (_I, [_P, _P, _P, _P, _P, _L, _P, _I, _L, _L, _L, _L, _L, _L, _L, _I, _P]),
+    "hyc_unpack_dequant": (_I, [_P, _P, _P, _P, _P, _L, _P, _L, _L, _L, _L, _L, _L, _L, _I, _P]),
+}
+
+
+def declared_symbols():
+    return sorted(_SIGNATURES)
+
+
+def lib() -> ctypes.CDLL:
+    """Load the kernel library once; fail loudly when it has not been built."""
+    global _lib
+    if _lib is None:
+        if not LIB_PATH.exists():
+            raise RuntimeError(
+                f"{LIB_PATH} not found: build it with `python {(_HERE / 'build.py')}` "
+                "(hipcc, gfx950). There is no fallback implementation.")
+        handle = ctypes.CDLL(str(LIB_PATH))
+        for name, (res, args) in _SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def error_string(code: int) -> str:
+    return lib().hyc_error_string(code).decode()
+
+
+def call(name: str, *args) -> None:
+    rc = getattr(lib(), name)(*args)
+    if rc != 0:
+        raise HycError(name, rc, error_string(rc))
+
+
+def ptr(t):
+    """Device address of a tensor (None -> NULL)."""
+    return None if t is None else t.data_ptr()
+
+
+def stream_of(t: torch.Tensor):
+    """The HIP stream torch is currently enqueuing on for t's device."""
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def require_gpu(*tensors) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError("hyclora kernels run on the GPU only; got a tensor on " + str(t.device))
+
+
+def set_tuning(key: str, value: int) -> None:
+    call("hyc_set_tuning", key.encode(), int(value))

@@ -1,0 +1,443 @@
+// Per-channel quantise + sub-byte pack and its inverse for gfx950.
+//
+// Work decomposition (both directions): a lane owns one 16-byte chunk of a row, i.e. 8
+// consecutive channels, and walks down a strip of rows, so the per-channel constants
+// (step, its reciprocal, zero point) live in registers for the whole strip.  A wave64
+// therefore reads 1 KiB of contiguous bf16 per row with one 128-bit load per lane; a
+// workgroup is 4 waves that take neighbouring row strips of the same 512 channels.
+//
+// Packed layout (fixed by the reference's 32-column tiles,
+// operators/compress_function_kernel.py:77-112): in every block of 32 columns, with
+// epp = 8/q codes per byte and w = 32/epp, byte j collects columns j + i*w, code i at bit
+// q*i.  In chunk terms (4 chunks a = 0..3 per block):
+//   q=8  chunk a  -> bytes 8a..8a+7, no sharing;
+//   q=4  chunks a and a^2 share bytes 8(a&1)..8(a&1)+7, chunk a in nibble a>>1;
+//   q=2  all four chunks share bytes 0..7, chunk a in bit pair a.
+// Each lane spreads its 8 codes over a 64-bit word (one code per byte, pre-shifted into
+// its sub-byte slot); the sharing lanes then OR their words together with DPP quad
+// permutes — no LDS, no bpermute — and each stores a different dword of the result, so
+// the wave writes one contiguous run per row.
+#include "hyc_common.hpp"
+
+namespace hyc {
+
+constexpr int kQuantWaves = 4;      // waves per workgroup
+constexpr int kQuantThreads = kQuantWaves * kWave;
+constexpr int kRowUnroll = 4;       // independent 128-bit loads in flight per lane
+
+static int g_rows_per_wave = 16;    // strip height; see hyc_set_tuning
+
+struct QuantArgs {
+    uint16_t* x;            // bf16 activations (input of quantise / output of dequantise)
+    const uint16_t* scale;  // bf16 [N]
+    const uint16_t* zp;     // bf16 [N] or null
+    uint8_t* q;             // packed codes, contiguous [T, N*q/8]
+    const int64_t* oidx;    // outlier channels or null
+    uint16_t* xo;           // bf16 [T, k]
+    int64_t T;              // B*M rows
+    int64_t stride_b, stride_m, stride_h;
+    int M, N, C;            // C = N/8 chunks per row
+    int head_dim;
+    int k;
+    int zero_input;
+    int rows_per_wave;
+    int col_tiles;
+};
+
+// Which of this lane's 8 columns are outlier channels, and at which position of the list.
+// The wave scans the list 64 entries at a time; only entries that fall into the wave's
+// 512-column window are broadcast and examined.
+struct OutlierLane {
+    uint32_t mask = 0;        // bit j: column col0 + j is an outlier
+    uint32_t pos[4] = {0, 0, 0, 0};  // 16-bit list positions, two per dword
+};
+
+__device__ __forceinline__ OutlierLane find_outliers(const int64_t* oidx, int k, int wave_col0, int col0, int lane) {
+    OutlierLane o;
+    for (int base = 0; base < k; base += kWave) {
+        const int e = base + lane;
+        const int ch = (e < k) ? (int)oidx[e] : -1;
+        const bool hit = (unsigned)(ch - wave_col0) < (unsigned)(kWave * 8);
+        unsigned long long hits = __ballot(hit);
+        while (hits) {
+            const int src = __ffsll((long long)hits) - 1;
+            hits &= hits - 1;
+            const int c = __builtin_amdgcn_readlane(ch, src);
+            const int d = c - col0;
+            if ((unsigned)d < 8u) {
+                o.mask |= 1u << d;
+                const uint32_t p = (uint32_t)(base + src) << (16 * (d & 1));
+                const uint32_t keep = 0xffff0000u >> (16 * (d & 1));
+#pragma unroll
+                for (int w = 0; w < 4; ++w)
+                    if ((d >> 1) == w) o.pos[w] = (o.pos[w] & keep) | p;
+            }
+        }
+    }
+    return o;
+}
+
+__device__ __forceinline__ uint32_t outlier_pos(const OutlierLane& o, int j) {
+    return (o.pos[j >> 1] >> (16 * (j & 1))) & 0xffffu;
+}
+
+// Walks the rows t = b*M + m of a [B, M, .] tensor with independent batch and row strides
+// without a division per row.
+struct RowCursor {
+    int64_t off;   // b*stride_b + m*stride_m
+    int m;
+    __device__ __forceinline__ RowCursor(int64_t t, int M, int64_t stride_b, int64_t stride_m) {
+        const int64_t b = t / M;
+        m = (int)(t - b * M);
+        off = b * stride_b + m * stride_m;
+    }
+    __device__ __forceinline__ void next(int M, int64_t stride_b, int64_t stride_m) {
+        ++m;
+        off += stride_m;
+        if (m == M) {
+            m = 0;
+            off += stride_b - (int64_t)M * stride_m;
+        }
+    }
+};
+
+// Element offset of the chunk that starts at column col0 (see hyclora.h: head layout).
+__device__ __forceinline__ int64_t chunk_offset(int col0, int head_dim, int64_t stride_h) {
+    const int h = col0 / head_dim;
+    return (int64_t)h * stride_h + (col0 - h * head_dim);
+}
+
+// ------------------------------------------------------------------------------------
+// quantise + pack
+// ------------------------------------------------------------------------------------
+template <int QBIT, bool ZP, bool FAST>
+__device__ __forceinline__ void codes_to_words(const float (&f)[8], const float (&s)[8], const float (&r)[8],
+                                               const float (&z)[8], uint32_t& lo, uint32_t& hi) {
+    int c[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        if constexpr (ZP) {
+            // zero-point form: IEEE quotient, then + z, then exact roundf
+            c[j] = hyc_code_from_t_exact(f[j] / s[j] + z[j], QBIT);
+        } else if constexpr (FAST) {
+            c[j] = hyc_code_from_t(hyc_quot_fast(f[j], s[j], r[j]), QBIT);
+        } else {
+            c[j] = hyc_code_from_t(f[j] / s[j], QBIT);
+        }
+    }
+    lo = (uint32_t)c[0] | ((uint32_t)c[1] << 8) | ((uint32_t)c[2] << 16) | ((uint32_t)c[3] << 24);
+    hi = (uint32_t)c[4] | ((uint32_t)c[5] << 8) | ((uint32_t)c[6] << 16) | ((uint32_t)c[7] << 24);
+}
+
+template <int QBIT, bool ZP, bool OUTL, bool FAST>
+__device__ __forceinline__ void quant_rows(const QuantArgs& a, int64_t row0, int64_t row1, bool active, int chunk,
+                                           int64_t coff, const float (&s)[8], const float (&r)[8],
+                                           const float (&z)[8], const OutlierLane& ol) {
+    const int quad = chunk & 3;            // chunk position inside its 32-column block
+    const int blk = chunk >> 2;
+    const int row_bytes = a.N * QBIT / 8;
+
+    if (row0 >= row1) return;
+    RowCursor cur(row0, a.M, a.stride_b, a.stride_m);
+    for (int64_t t0 = row0; t0 < row1; t0 += kRowUnroll) {
+        u32x4 v[kRowUnroll];
+        uint16_t* xrow[kRowUnroll];
+#pragma unroll
+        for (int u = 0; u < kRowUnroll; ++u) {
+            const int64_t t = t0 + u;
+            xrow[u] = a.x + cur.off + coff;
+            v[u] = u32x4{0, 0, 0, 0};
+            if (active && t < row1) v[u] = ld16(xrow[u]);
+            cur.next(a.M, a.stride_b, a.stride_m);
+        }
+#pragma unroll
+        for (int u = 0; u < kRowUnroll; ++u) {
+            const int64_t t = t0 + u;
+            if (t >= row1) break;          // uniform across the wave
+            if constexpr (OUTL) {
+                if (ol.mask) {
+                    uint32_t d[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        if (ol.mask & (1u << j)) {
+                            const uint32_t sh = 16 * (j & 1);
+                            a.xo[t * a.k + outlier_pos(ol, j)] = (uint16_t)(d[j >> 1] >> sh);
+                            d[j >> 1] &= ~(0xffffu << sh);
+                            if (a.zero_input) xrow[u][j] = 0;
+                        }
+                    }
+                    v[u] = u32x4{d[0], d[1], d[2], d[3]};
+                }
+            }
+            float f[8];
+            unpack8(v[u], f);
+            uint32_t lo, hi;
+            codes_to_words<QBIT, ZP, FAST>(f, s, r, z, lo, hi);
+            uint8_t* qrow = a.q + t * row_bytes;
+            if constexpr (QBIT == 8) {
+                if (active) st8(qrow + (int64_t)chunk * 8, u32x2{lo, hi});
+            } else if constexpr (QBIT == 4) {
+                const int sub = quad >> 1;
+                lo <<= 4 * sub;
+                hi <<= 4 * sub;
+                lo |= quad_xor2(lo);
+                hi |= quad_xor2(hi);
+                if (active)
+                    *reinterpret_cast<uint32_t*>(qrow + blk * 16 + 8 * (quad & 1) + 4 * sub) = sub ? hi : lo;
+            } else {
+                lo <<= 2 * quad;
+                hi <<= 2 * quad;
+                lo |= quad_xor1(lo);
+                hi |= quad_xor1(hi);
+                lo |= quad_xor2(lo);
+                hi |= quad_xor2(hi);
+                if (active && quad < 2) *reinterpret_cast<uint32_t*>(qrow + blk * 8 + 4 * quad) = quad ? hi : lo;
+            }
+        }
+    }
+}
+
+template <int QBIT, bool ZP, bool OUTL>
+__global__ __launch_bounds__(kQuantThreads) void quant_pack_kernel(const QuantArgs a) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int col_tile = blockIdx.x % a.col_tiles;
+    const int64_t row_tile = blockIdx.x / a.col_tiles;
+    const int chunk = col_tile * kWave + lane;
+    const bool active = chunk < a.C;
+    const int col0 = chunk * 8;
+
+    float s[8], r[8], z[8];
+    bool fast = true;
+    {
+        u32x4 sv = {0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};  // 1.0 for idle lanes
+        if (active) sv = ld16(a.scale + col0);
+        unpack8(sv, s);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            r[j] = 1.0f / s[j];
+            fast = fast && hyc_scale_is_fast(s[j]);
+            z[j] = 0.0f;
+        }
+        if constexpr (ZP) {
+            if (active) unpack8(ld16(a.zp + col0), z);
+        }
+    }
+    OutlierLane ol;
+    if constexpr (OUTL) ol = find_outliers(a.oidx, a.k, col_tile * kWave * 8, col0, lane);
+
+    const int64_t coff = active ? chunk_offset(col0, a.head_dim, a.stride_h) : 0;
+    const int64_t row0 = (row_tile * kQuantWaves + wave) * (int64_t)a.rows_per_wave;
+    int64_t row1 = row0 + a.rows_per_wave;
+    if (row1 > a.T) row1 = a.T;
+
+    // one slow column anywhere in the wave sends the whole wave down the IEEE-division path
+    if (ZP || __ballot(!fast) != 0ull)
+        quant_rows<QBIT, ZP, OUTL, false>(a, row0, row1, active, chunk, coff, s, r, z, ol);
+    else
+        quant_rows<QBIT, ZP, OUTL, true>(a, row0, row1, active, chunk, coff, s, r, z, ol);
+}
+
+// ------------------------------------------------------------------------------------
+// unpack + dequantise
+// ------------------------------------------------------------------------------------
+template <int QBIT, bool ZP, bool OUTL>
+__global__ __launch_bounds__(kQuantThreads) void unpack_dequant_kernel(const QuantArgs a) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int col_tile = blockIdx.x % a.col_tiles;
+    const int64_t row_tile = blockIdx.x / a.col_tiles;
+    const int chunk = col_tile * kWave + lane;
+    const bool active = chunk < a.C;
+    const int col0 = chunk * 8;
+    const int quad = chunk & 3;
+    const int blk = chunk >> 2;
+    constexpr float kHalf = (float)(1 << (QBIT - 1));
+
+    float s[8], z[8];
+    {
+        u32x4 sv = {0, 0, 0, 0};
+        if (active) sv = ld16(a.scale + col0);
+        unpack8(sv, s);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) z[j] = 0.0f;
+        if constexpr (ZP) {
+            if (active) unpack8(ld16(a.zp + col0), z);
+        }
+    }
+    OutlierLane ol;
+    if constexpr (OUTL) ol = find_outliers(a.oidx, a.k, col_tile * kWave * 8, col0, lane);
+
+    const int64_t coff = active ? chunk_offset(col0, a.head_dim, a.stride_h) : 0;
+    const int64_t row0 = (row_tile * kQuantWaves + wave) * (int64_t)a.rows_per_wave;
+    int64_t row1 = row0 + a.rows_per_wave;
+    if (row1 > a.T) row1 = a.T;
+    const int row_bytes = a.N * QBIT / 8;
+
+    // byte offset of the 8 packed bytes that hold this chunk's codes, and the bit shift
+    int qoff, shift;
+    uint32_t mask;
+    if constexpr (QBIT == 8) { qoff = chunk * 8; shift = 0; mask = 0xffffffffu; }
+    else if constexpr (QBIT == 4) { qoff = blk * 16 + 8 * (quad & 1); shift = 4 * (quad >> 1); mask = 0x0f0f0f0fu; }
+    else { qoff = blk * 8; shift = 2 * quad; mask = 0x03030303u; }
+
+    if (row0 >= row1) return;
+    RowCursor cur(row0, a.M, a.stride_b, a.stride_m);
+    for (int64_t t0 = row0; t0 < row1; t0 += kRowUnroll) {
+        u32x2 w[kRowUnroll];
+#pragma unroll
+        for (int u = 0; u < kRowUnroll; ++u) {
+            const int64_t t = t0 + u;
+            w[u] = u32x2{0, 0};
+            if (active && t < row1) w[u] = ld8(a.q + t * row_bytes + qoff);
+        }
+#pragma unroll
+        for (int u = 0; u < kRowUnroll; ++u) {
+            const int64_t t = t0 + u;
+            if (t >= row1) break;
+            const uint32_t lo = (w[u].x >> shift) & mask;
+            const uint32_t hi = (w[u].y >> shift) & mask;
+            float f[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float c = (float)(((j < 4 ? lo : hi) >> (8 * (j & 3))) & 0xffu);
+                if constexpr (ZP) {
+                    // bf16 arithmetic step by step: (c - 2^(q-1)) is exact, minus z rounds to bf16
+                    f[j] = rbf((c - kHalf) - z[j]) * s[j];
+                } else {
+                    // not fma(c, s, -2^(q-1) s): that loses the sign of zero and turns an
+                    // infinite step into NaN where the reference's product does not
+                    f[j] = (c - kHalf) * s[j];
+                }
+            }
+            u32x4 o = pack8(f);
+            uint16_t* xrow = a.x + cur.off + coff;
+            cur.next(a.M, a.stride_b, a.stride_m);
+            if constexpr (OUTL) {
+                if (ol.mask) {
+                    uint32_t d[4] = {o.x, o.y, o.z, o.w};
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        if (ol.mask & (1u << j)) {
+                            const uint32_t sh = 16 * (j & 1);
+                            const uint32_t val = a.xo[t * a.k + outlier_pos(ol, j)];
+                            d[j >> 1] = (d[j >> 1] & ~(0xffffu << sh)) | (val << sh);
+                        }
+                    }
+                    o = u32x4{d[0], d[1], d[2], d[3]};
+                }
+            }
+            if (active) st16(xrow, o);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------
+// host side
+// ------------------------------------------------------------------------------------
+static int check_common(const void* x, const void* scale, const void* q, const int64_t* oidx, int64_t k,
+                        const void* xo, int64_t B, int64_t M, int64_t N, int64_t stride_b, int64_t stride_m,
+                        int64_t head_dim, int64_t stride_h, int q_bit) {
+    if (q_bit != 2 && q_bit != 4 && q_bit != 8) return HYC_ERR_QBIT;
+    if (B < 0 || M < 0 || N < 0 || k < 0 || k > 65535) return HYC_ERR_SHAPE;
+    if (N % 32 != 0 || N > (1 << 28) || M > INT32_MAX || B * M > (int64_t)1 << 40) return HYC_ERR_SHAPE;
+    if (B * M * N == 0) return HYC_OK;
+    if (!x || !scale || !q) return HYC_ERR_NULL;
+    if (k > 0 && (!oidx || !xo)) return HYC_ERR_NULL;
+    if (head_dim <= 0 || head_dim % 8 != 0 || N % head_dim != 0) return HYC_ERR_SHAPE;
+    if (!aligned16(x) || !aligned16(scale) || !aligned16(q)) return HYC_ERR_ALIGN;
+    if (stride_b % 8 != 0 || stride_m % 8 != 0 || stride_h % 8 != 0) return HYC_ERR_ALIGN;
+    return 1;  // proceed
+}
+
+static QuantArgs make_args(const void* x, const void* scale, const void* zp, const void* q, const int64_t* oidx,
+                           int64_t k, const void* xo, int zero_input, int64_t B, int64_t M, int64_t N,
+                           int64_t stride_b, int64_t stride_m, int64_t head_dim, int64_t stride_h) {
+    QuantArgs a;
+    a.x = (uint16_t*)x;
+    a.scale = (const uint16_t*)scale;
+    a.zp = (const uint16_t*)zp;
+    a.q = (uint8_t*)q;
+    a.oidx = oidx;
+    a.xo = (uint16_t*)xo;
+    a.T = B * M;
+    a.stride_b = stride_b;
+    a.stride_m = stride_m;
+    a.stride_h = stride_h;
+    a.M = (int)M;
+    a.N = (int)N;
+    a.C = (int)(N / 8);
+    a.head_dim = (int)head_dim;
+    a.k = (int)k;
+    a.zero_input = zero_input;
+    a.rows_per_wave = g_rows_per_wave;
+    a.col_tiles = (int)cdiv(a.C, kWave);
+    return a;
+}
+
+#define HYC_LAUNCH_QBIT(KERNEL, QB)                                                                 \
+    do {                                                                                            \
+        if (zp && k)       hipLaunchKernelGGL((KERNEL<QB, true, true>), grid, block, 0, st, a);    \
+        else if (zp)       hipLaunchKernelGGL((KERNEL<QB, true, false>), grid, block, 0, st, a);   \
+        else if (k)        hipLaunchKernelGGL((KERNEL<QB, false, true>), grid, block, 0, st, a);   \
+        else               hipLaunchKernelGGL((KERNEL<QB, false, false>), grid, block, 0, st, a);  \
+    } while (0)
+
+#define HYC_LAUNCH(KERNEL)                                       \
+    do {                                                         \
+        if (q_bit == 8) HYC_LAUNCH_QBIT(KERNEL, 8);              \
+        else if (q_bit == 4) HYC_LAUNCH_QBIT(KERNEL, 4);         \
+        else HYC_LAUNCH_QBIT(KERNEL, 2);                         \
+    } while (0)
+
+}  // namespace hyc
+
+using namespace hyc;
+
+extern "C" int hyc_quant_pack(const void* x, const void* scale, const void* zero_point, void* q,
+                              const int64_t* outlier_idx, int64_t k, void* x_outlier, int zero_input, int64_t B,
+                              int64_t M, int64_t N, int64_t stride_b, int64_t stride_m, int64_t head_dim,
+                              int64_t stride_h, int q_bit, void* stream) {
+    const int rc = check_common(x, scale, q, outlier_idx, k, x_outlier, B, M, N, stride_b, stride_m, head_dim,
+                                stride_h, q_bit);
+    if (rc <= 0) return rc;
+    if (zero_point && !aligned16(zero_point)) return HYC_ERR_ALIGN;
+    const void* zp = zero_point;
+    QuantArgs a = make_args(x, scale, zp, q, outlier_idx, k, x_outlier, zero_input, B, M, N, stride_b, stride_m,
+                            head_dim, stride_h);
+    const int64_t row_tiles = cdiv(a.T, (int64_t)kQuantWaves * a.rows_per_wave);
+    if (row_tiles * a.col_tiles > INT32_MAX) return HYC_ERR_SHAPE;
+    const dim3 grid((unsigned)(row_tiles * a.col_tiles)), block(kQuantThreads);
+    hipStream_t st = (hipStream_t)stream;
+    HYC_LAUNCH(quant_pack_kernel);
+    return check_launch();
+}
+
+extern "C" int hyc_unpack_dequant(const void* q, const void* scale, const void* zero_point, void* x,
+                                  const int64_t* outlier_idx, int64_t k, const void* x_outlier, int64_t B,
+                                  int64_t M, int64_t N, int64_t stride_b, int64_t stride_m, int64_t head_dim,
+                                  int64_t stride_h, int q_bit, void* stream) {
+    const int rc = check_common(x, scale, q, outlier_idx, k, x_outlier, B, M, N, stride_b, stride_m, head_dim,
+                                stride_h, q_bit);
+    if (rc <= 0) return rc;
+    if (zero_point && !aligned16(zero_point)) return HYC_ERR_ALIGN;
+    if (!((reinterpret_cast<uintptr_t>(q) & 7u) == 0)) return HYC_ERR_ALIGN;
+    const void* zp = zero_point;
+    QuantArgs a = make_args(x, scale, zp, q, outlier_idx, k, x_outlier, 0, B, M, N, stride_b, stride_m, head_dim,
+                            stride_h);
+    const int64_t row_tiles = cdiv(a.T, (int64_t)kQuantWaves * a.rows_per_wave);
+    if (row_tiles * a.col_tiles > INT32_MAX) return HYC_ERR_SHAPE;
+    const dim3 grid((unsigned)(row_tiles * a.col_tiles)), block(kQuantThreads);
+    hipStream_t st = (hipStream_t)stream;
+    HYC_LAUNCH(unpack_dequant_kernel);
+    return check_launch();
+}
+
+int hyc::tune_quant(const char* key, int value) {
+    if (strcmp(key, "quant_rows_per_wave") == 0) {
+        if (value < 1 || value > 4096) return HYC_ERR_ARG;
+        g_rows_per_wave = value;
+        return HYC_OK;
+    }
+    return 1;  // not one of this file's keys
+}

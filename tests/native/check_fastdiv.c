@@ -1,0 +1,57 @@
+/* Exhaustive host-side check of the reciprocal-based quotient used by the HIP quantiser.
+ *
+ * For every bf16 step s accepted by hyc_scale_is_fast and every one of the 65536 bf16
+ * inputs x (NaNs and infinities included), the integer code computed from
+ * hyc_quot_fast(x, s, 1/s) must equal the code computed from the IEEE quotient x / s
+ * with libm's roundf, for code widths 2, 4 and 8.  Prints the number of pairs examined
+ * and the number of mismatches; exit status 0 iff there are none.
+ *
+ * Build (done by the test that runs it):
+ *   gcc -O2 -fopenmp -ffp-contract=off -I<package>/csrc check_fastdiv.c -lm
+ */
+#include <stdio.h>
+#include <stdlib.h>
+#include "hyc_quant_math.h"
+
+static int code_ieee(float x, float s, int q_bit) {
+    float t = x / s;
+    float half = (float)(1 << (q_bit - 1));
+    t = roundf(t);
+    if (t < -half) t = -half;
+    if (t > half - 1.0f) t = half - 1.0f;
+    t += half;
+    return isnan(t) ? 0 : (int)lrintf(t);
+}
+
+int main(int argc, char **argv) {
+    /* optional stride over s patterns for a quicker partial run */
+    int stride = argc > 1 ? atoi(argv[1]) : 1;
+    if (stride < 1) stride = 1;
+    unsigned long long pairs = 0, bad = 0, inexact = 0;
+    unsigned first_bad_x = 0, first_bad_s = 0;
+#pragma omp parallel for schedule(dynamic, 64) reduction(+ : pairs, bad, inexact)
+    for (int sb = 1; sb < 0x7f80; sb += stride) {
+        float s = hyc_bf16_to_f32((uint16_t)sb);
+        if (!hyc_scale_is_fast(s)) continue;
+        float r = 1.0f / s;
+        for (unsigned xb = 0; xb < 65536u; ++xb) {
+            float x = hyc_bf16_to_f32((uint16_t)xb);
+            float tf = hyc_quot_fast(x, s, r);
+            float ti = x / s;
+            ++pairs;
+            if (fabsf(ti) <= 512.0f && !(tf == ti)) ++inexact;
+            int ok = 1;
+            for (int q = 2; q <= 8; q *= 2)
+                if (hyc_code_from_t(tf, q) != code_ieee(x, s, q) ||
+                    hyc_code_from_t_exact(ti, q) != code_ieee(x, s, q)) ok = 0;
+            if (!ok) {
+                ++bad;
+#pragma omp critical
+                if (!first_bad_s) { first_bad_s = (unsigned)sb; first_bad_x = xb; }
+            }
+        }
+    }
+    printf("pairs=%llu mismatches=%llu quotient_not_bit_equal_within_512=%llu\n", pairs, bad, inexact);
+    if (bad) printf("first mismatch: x=0x%04x s=0x%04x\n", first_bad_x, first_bad_s);
+    return bad ? 1 : 0;
+}
