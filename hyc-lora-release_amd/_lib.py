@@ -33,6 +33,24 @@ _SIGNATURES = {
     "hyc_set_tuning": (_I, [c_char_p, _I]),
     "hyc_quant_pack": (_I, [_P, _P, _P, _P, _P, _L, _P, _I, _L, _L, _L, _L, _L, _L, _L, _I, _P]),
     "hyc_unpack_dequant": (_I, [_P, _P, _P, _P, _P, _L, _P, _L, _L, _L, _L, _L, _L, _L, _I, _P]),
+    "hyc_channel_stats": (_I, [_P, _L, _L, _L, _L, _L, _P, _P]),
+    "hyc_channel_select": (_I, [_P, _L, _L, _I, _I, _P, _P, _P, _P]),
+    "hyc_hist16": (_I, [_P, _L, _P, _P]),
+    "hyc_hist_select": (_I, [_P, _L, _P, _P]),
+    "hyc_sparse_num_segments": (_L, [_L]),
+    "hyc_sparse_count": (_I, [_P, _L, _P, _P, _P, _P]),
+    "hyc_sparse_write": (_I, [_P, _L, _P, _P, _P, _P, _P]),
+    "hyc_sparse_segment_offsets": (_I, [_P, _L, _L, _P, _P]),
+    "hyc_sparse_restore": (_I, [_P, _P, _P, _L, _P, _P]),
+    "hyc_softmax_bwd": (_I, [_P, _P, _P, _L, _L, _P]),
+    "hyc_rmsnorm_fwd": (_I, [_P, _P, _I, _P, _P, _L, _L, ctypes.c_float, _P]),
+    "hyc_rmsnorm_bwd_workspace": (_L, [_L, _L]),
+    "hyc_rmsnorm_bwd": (_I, [_P, _P, _P, _I, _P, _P, _P, _P, _L, _L, _L, _P]),
+    "hyc_silu_bwd": (_I, [_P, _P, _P, _L, _P]),
+    "hyc_silu_mul": (_I, [_P, _P, _P, _L, _P]),
+    "hyc_gelu_bwd": (_I, [_P, _P, _P, _L, _P]),
+    "hyc_lora_silu_mul_fwd": (_I, [_P] * 11 + [_L, _L, _L, _I, _P]),
+    "hyc_lora_silu_mul_bwd": (_I, [_P] * 12 + [_L, _L, _L, _I, _P]),
 }
 
 

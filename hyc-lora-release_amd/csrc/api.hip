@@ -22,5 +22,7 @@ extern "C" int hyc_set_tuning(const char* key, int value) {
     if (!key) return HYC_ERR_NULL;
     int rc = hyc::tune_quant(key, value);
     if (rc != 1) return rc;
+    rc = hyc::tune_fuse(key, value);
+    if (rc != 1) return rc;
     return HYC_ERR_ARG;
 }

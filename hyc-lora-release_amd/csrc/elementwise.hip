@@ -1,0 +1,95 @@
+// Element-wise backward operators for gfx950: SiLU backward, SiLU*x2 (forward of the gated
+// MLP product) and tanh-GELU backward.  Pure streaming kernels: one 128-bit load per
+// operand per lane, four independent chunks in flight per lane.
+//
+// The SiLU kernels round to bf16 after every arithmetic operation, as the reference's bf16
+// Triton expressions do (operators/silu_kernels.py:42-43, :103-104); the sigmoid itself is
+// evaluated in fp32 and rounded once.
+#include "hyc_common.hpp"
+
+namespace hyc {
+
+constexpr int kEwThreads = 256;
+constexpr int kEwUnroll = 4;
+
+struct SiluBwd {   // o = g * (sig * (1 + x * (1 - sig)))
+    __device__ __forceinline__ float operator()(float x, float g) const {
+        const float sig = rbf(sigmoidf_(x));
+        const float t = rbf(1.0f + rbf(x * rbf(1.0f - sig)));
+        return g * rbf(sig * t);
+    }
+};
+struct SiluMul {   // o = (sig(x1) * x1) * x2
+    __device__ __forceinline__ float operator()(float x1, float x2) const {
+        return rbf(rbf(sigmoidf_(x1)) * x1) * x2;
+    }
+};
+struct GeluBwd {   // d/dx of 0.5 x (1 + tanh(gamma (x + kappa x^3))), times g; fp32 throughout
+    __device__ __forceinline__ float operator()(float x, float g) const {
+        constexpr float gamma = 0.7978845608028654f, kappa = 0.044715f;
+        const float x2 = x * x;
+        const float y = gamma * (x + kappa * x2 * x);
+        const float t = 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + __expf(2.0f * y));   // tanh(y)
+        return 0.5f * ((1.0f + t) + x * ((1.0f - t * t) * gamma * (1.0f + 3.0f * kappa * x2))) * g;
+    }
+};
+
+template <class Op>
+__global__ __launch_bounds__(kEwThreads) void binary_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ b,
+                                                            uint16_t* __restrict__ o, int64_t n) {
+    const Op op;
+    const int64_t chunks = n / 8;
+    const int64_t c0 = (int64_t)blockIdx.x * (kEwThreads * kEwUnroll) + threadIdx.x;
+    u32x4 av[kEwUnroll], bv[kEwUnroll];
+#pragma unroll
+    for (int u = 0; u < kEwUnroll; ++u) {
+        const int64_t c = c0 + u * kEwThreads;
+        if (c < chunks) {
+            av[u] = ld16(a + c * 8);
+            bv[u] = ld16(b + c * 8);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < kEwUnroll; ++u) {
+        const int64_t c = c0 + u * kEwThreads;
+        if (c < chunks) {
+            float af[8], bf[8], of[8];
+            unpack8(av[u], af);
+            unpack8(bv[u], bf);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) of[j] = op(af[j], bf[j]);
+            st16(o + c * 8, pack8(of));
+        }
+    }
+    if (blockIdx.x == 0 && threadIdx.x < (n & 7)) {       // ragged tail
+        const int64_t i = chunks * 8 + threadIdx.x;
+        o[i] = f_to_bf(op(bf_to_f(a[i]), bf_to_f(b[i])));
+    }
+}
+
+template <class Op>
+static int launch_binary(const void* a, const void* b, void* o, int64_t n, void* stream) {
+    if (n < 0) return HYC_ERR_SHAPE;
+    if (n == 0) return HYC_OK;
+    if (!a || !b || !o) return HYC_ERR_NULL;
+    if (!aligned16(a) || !aligned16(b) || !aligned16(o)) return HYC_ERR_ALIGN;
+    const int64_t blocks = cdiv(cdiv(n, 8), kEwThreads * kEwUnroll);
+    if (blocks > INT32_MAX) return HYC_ERR_SHAPE;
+    hipLaunchKernelGGL(binary_kernel<Op>, dim3((unsigned)(blocks < 1 ? 1 : blocks)), dim3(kEwThreads), 0,
+                       (hipStream_t)stream, (const uint16_t*)a, (const uint16_t*)b, (uint16_t*)o, n);
+    return check_launch();
+}
+
+}  // namespace hyc
+
+using namespace hyc;
+
+extern "C" int hyc_silu_bwd(const void* x, const void* g, void* out, int64_t n, void* stream) {
+    return launch_binary<SiluBwd>(x, g, out, n, stream);
+}
+extern "C" int hyc_silu_mul(const void* x1, const void* x2, void* out, int64_t n, void* stream) {
+    return launch_binary<SiluMul>(x1, x2, out, n, stream);
+}
+extern "C" int hyc_gelu_bwd(const void* x, const void* g, void* out, int64_t n, void* stream) {
+    return launch_binary<GeluBwd>(x, g, out, n, stream);
+}

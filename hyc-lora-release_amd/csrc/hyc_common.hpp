@@ -97,11 +97,12 @@ inline int check_launch() {
     return hipGetLastError() == hipSuccess ? HYC_OK : HYC_ERR_LAUNCH;
 }
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
-inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
+__host__ __device__ inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
 
 // Per-file tuning hooks behind hyc_set_tuning: HYC_OK / HYC_ERR_* if the key belongs to the
 // file, 1 if it does not.
 int tune_quant(const char* key, int value);
+int tune_fuse(const char* key, int value);
 
 }  // namespace hyc

@@ -1,0 +1,102 @@
+// Lane-level building blocks of the packed-code format, shared by the standalone
+// quantise / dequantise kernels and the fused LoRA-SiLU kernels.
+//
+// A lane owns chunk `chunk` of a row: the 8 consecutive channels 8*chunk .. 8*chunk+7.
+// Four neighbouring lanes (a DPP quad) own the four chunks of one 32-column block, which is
+// the unit the packed layout is defined on (operators/compress_function_kernel.py:77-112):
+//   q=8  chunk a  -> bytes 8a..8a+7 of the block, no sharing;
+//   q=4  chunks a and a^2 share bytes 8(a&1)..8(a&1)+7, chunk a in nibble a>>1;
+//   q=2  all four chunks share bytes 0..7, chunk a in bit pair a.
+#pragma once
+
+#include "hyc_common.hpp"
+
+namespace hyc {
+
+// 8 values -> 8 codes, one per byte of (lo, hi).
+template <int QBIT, bool ZP, bool FAST>
+__device__ __forceinline__ void codes_to_words(const float (&f)[8], const float (&s)[8], const float (&r)[8],
+                                               const float (&z)[8], uint32_t& lo, uint32_t& hi) {
+    int c[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        if constexpr (ZP) {
+            // zero-point form: IEEE quotient, then + z, then exact roundf
+            c[j] = hyc_code_from_t_exact(f[j] / s[j] + z[j], QBIT);
+        } else if constexpr (FAST) {
+            c[j] = hyc_code_from_t(hyc_quot_fast(f[j], s[j], r[j]), QBIT);
+        } else {
+            c[j] = hyc_code_from_t(f[j] / s[j], QBIT);
+        }
+    }
+    lo = (uint32_t)c[0] | ((uint32_t)c[1] << 8) | ((uint32_t)c[2] << 16) | ((uint32_t)c[3] << 24);
+    hi = (uint32_t)c[4] | ((uint32_t)c[5] << 8) | ((uint32_t)c[6] << 16) | ((uint32_t)c[7] << 24);
+}
+
+// Merge the quad's code words into packed bytes and store this lane's share of them.
+// Every lane of the quad must call this (the exchange is a DPP quad permute); `active`
+// only gates the store.  qrow = first packed byte of the row.
+template <int QBIT>
+__device__ __forceinline__ void store_packed(uint8_t* qrow, int chunk, bool active, uint32_t lo, uint32_t hi) {
+    const int quad = chunk & 3;
+    const int blk = chunk >> 2;
+    if constexpr (QBIT == 8) {
+        if (active) st8(qrow + (int64_t)chunk * 8, u32x2{lo, hi});
+    } else if constexpr (QBIT == 4) {
+        const int sub = quad >> 1;
+        lo <<= 4 * sub;
+        hi <<= 4 * sub;
+        lo |= quad_xor2(lo);
+        hi |= quad_xor2(hi);
+        if (active) *reinterpret_cast<uint32_t*>(qrow + blk * 16 + 8 * (quad & 1) + 4 * sub) = sub ? hi : lo;
+    } else {
+        lo <<= 2 * quad;
+        hi <<= 2 * quad;
+        lo |= quad_xor1(lo);
+        hi |= quad_xor1(hi);
+        lo |= quad_xor2(lo);
+        hi |= quad_xor2(hi);
+        if (active && quad < 2) *reinterpret_cast<uint32_t*>(qrow + blk * 8 + 4 * quad) = quad ? hi : lo;
+    }
+}
+
+// Where a chunk's codes sit inside a packed row: the 8 bytes at `offset`, each shifted
+// right by `shift` and masked with `mask` (replicated per byte).
+template <int QBIT>
+struct PackedSlot {
+    int offset;
+    int shift;
+    static constexpr uint32_t mask = QBIT == 8 ? 0xffffffffu : (QBIT == 4 ? 0x0f0f0f0fu : 0x03030303u);
+    __device__ __forceinline__ explicit PackedSlot(int chunk) {
+        const int quad = chunk & 3, blk = chunk >> 2;
+        if constexpr (QBIT == 8) { offset = chunk * 8; shift = 0; }
+        else if constexpr (QBIT == 4) { offset = blk * 16 + 8 * (quad & 1); shift = 4 * (quad >> 1); }
+        else { offset = blk * 8; shift = 2 * quad; }
+    }
+    // the 8 codes of the chunk as floats
+    __device__ __forceinline__ void decode(u32x2 w, float (&c)[8]) const {
+        const uint32_t lo = (w.x >> shift) & mask, hi = (w.y >> shift) & mask;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) c[j] = (float)(((j < 4 ? lo : hi) >> (8 * (j & 3))) & 0xffu);
+    }
+};
+
+// Per-lane column constants of the quantiser: step, reciprocal, and whether every one of the
+// lane's 8 steps may use the reciprocal path.
+struct QuantCols {
+    float s[8], r[8];
+    bool fast;
+    __device__ __forceinline__ void load(const uint16_t* scale, int col0, bool active) {
+        u32x4 sv = {0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};   // 1.0 for idle lanes
+        if (active) sv = ld16(scale + col0);
+        unpack8(sv, s);
+        fast = true;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            r[j] = 1.0f / s[j];
+            fast = fast && hyc_scale_is_fast(s[j]);
+        }
+    }
+};
+
+}  // namespace hyc

@@ -1,0 +1,334 @@
+// Fused LoRA-SiLU-Hadamard forward and backward for gfx950.
+//
+//   forward :  q1 = Q(x1; s1), q2 = Q(x2; s2)                      (packed codes, saved for backward)
+//              y1 = x1 + bf16(xa1 . b1),  y2 = x2 + bf16(xa2 . b2)   (LoRA up-projection, K = rank)
+//              o  = (y1 * bf16(sigmoid(y1))) * y2
+//   backward:  x1 = DQ(q1; s1), x2 = DQ(q2; s2), y1, y2, sigma as above,
+//              o, grad_gate = (g*y2) * (sigma * (1 + y1*(1 - sigma))), grad_up = g * silu(y1)
+//   (operators/triton_fuse_lora_silu_hadamard_forward_kernels.py:104-146,
+//    operators/triton_fuse_lora_silu_hadamard_backward_kernels.py:106-149; bf16 after every
+//    arithmetic operation, as there.)
+//
+// Both kernels move 7-9 bytes per element pair and do 64 MFMA flops for it: they are HBM-bound
+// and are laid out for the memory system first.  A wave owns a tile of 128 columns and walks
+// down a strip of rows 16 at a time.  The rank-R contraction runs on the matrix cores as
+// v_mfma_f32_16x16x16_bf16 with the *column slots permuted*: MFMA number t (t = 0..7) is fed
+// columns c0 + 8j + t (j = 0..15) of the LoRA-B tile, so that lane l, which receives column
+// slot j = l % 16 of every MFMA result, ends up with the 8 consecutive columns
+// c0 + 8j .. c0 + 8j + 7 of rows 4*(l/16) .. 4*(l/16)+3.  That is exactly the "one lane = one
+// 16-byte chunk" ownership the quantiser and the 128-bit loads/stores want: no LDS, no
+// transposes, and every global access is a full 256-byte run per row.
+// The LoRA-B operand registers are built once per wave and reused for the whole strip.
+#include "hyc_pack.hpp"
+
+namespace hyc {
+
+constexpr int kFuseThreads = 256;                  // 4 waves
+constexpr int kFuseWaves = kFuseThreads / kWave;
+constexpr int kTileCols = 128;                     // 16 lanes x 8 columns
+constexpr int kTileRows = 16;
+
+static int g_fuse_rows_per_wave = 64;
+
+struct FuseArgs {
+    const uint16_t* xa1; const uint16_t* b1; const uint16_t* s1;
+    const uint16_t* xa2; const uint16_t* b2; const uint16_t* s2;
+    const uint16_t* x1; const uint16_t* x2;     // forward inputs
+    uint8_t* q1; uint8_t* q2;                   // packed codes (forward output / backward input)
+    const uint16_t* g;                          // backward: upstream gradient
+    uint16_t* o; uint16_t* gg; uint16_t* gu;    // outputs: hadamard, grad_gate, grad_up
+    int64_t T;                                  // rows
+    int N, C, R;                                // columns, chunks per row, LoRA rank
+    int rows_per_wave, col_tiles;
+};
+
+// LoRA-B operands of one 128-column tile: for each 16-deep K step and each of the 8 MFMAs, the
+// 4 bf16 values b[16*ks + 4g + kk][c0 + 8j + t], kk = 0..3, for lane (g = l/16, j = l%16).
+template <int KSTEPS>
+struct BOperand {
+    s16x4 v[KSTEPS][8];
+    __device__ __forceinline__ void load(const uint16_t* b, int N, int R, int col0, bool active, int g) {
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) {
+            uint32_t rows[4][4];
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) {
+                const int k = 16 * ks + 4 * g + kk;
+                u32x4 r = {0, 0, 0, 0};
+                if (active && k < R) r = ld16(b + (int64_t)k * N + col0);
+                rows[kk][0] = r.x; rows[kk][1] = r.y; rows[kk][2] = r.z; rows[kk][3] = r.w;
+            }
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                uint32_t e[4];
+#pragma unroll
+                for (int kk = 0; kk < 4; ++kk) e[kk] = (t & 1) ? (rows[kk][t >> 1] >> 16) : (rows[kk][t >> 1] & 0xffffu);
+                const u32x2 pk = {e[0] | (e[1] << 16), e[2] | (e[3] << 16)};
+                v[ks][t] = __builtin_bit_cast(s16x4, pk);
+            }
+        }
+    }
+};
+
+// acc[t][v]: column col0 + t, row row0 + 4g + v
+template <int KSTEPS>
+__device__ __forceinline__ void lora_tile(const uint16_t* xa, int R, int64_t row0, int64_t T, int lane,
+                                          const BOperand<KSTEPS>& B, f32x4 (&acc)[8]) {
+    const int i = lane & 15, g = lane >> 4;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) acc[t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+        const int k = 16 * ks + 4 * g;
+        u32x2 av = {0, 0};
+        if (row0 + i < T && k < R) av = ld8(xa + (row0 + i) * R + k);
+        const s16x4 A = __builtin_bit_cast(s16x4, av);
+#pragma unroll
+        for (int t = 0; t < 8; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(A, B.v[ks][t], acc[t], 0, 0, 0);
+    }
+}
+
+__device__ __forceinline__ float acc_elem(const f32x4& a, int v) {
+    return v == 0 ? a.x : (v == 1 ? a.y : (v == 2 ? a.z : a.w));
+}
+
+// ------------------------------------------------------------------------------------
+template <int QBIT, int KSTEPS, bool FAST>
+__device__ __forceinline__ void fuse_fwd_rows(const FuseArgs& a, int64_t row_begin, int64_t row_end, int lane, int chunk,
+                                              bool active, const QuantCols& c1, const QuantCols& c2,
+                                              const BOperand<KSTEPS>& B1, const BOperand<KSTEPS>& B2) {
+    const int g = lane >> 4;
+    const int row_bytes = a.N * QBIT / 8;
+    const float zero8[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int64_t row0 = row_begin; row0 < row_end; row0 += kTileRows) {
+        u32x4 xv1[4], xv2[4];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int64_t t = row0 + 4 * g + v;
+            xv1[v] = u32x4{0, 0, 0, 0};
+            xv2[v] = u32x4{0, 0, 0, 0};
+            if (active && t < row_end) {
+                xv1[v] = ld16(a.x1 + t * a.N + chunk * 8);
+                xv2[v] = ld16(a.x2 + t * a.N + chunk * 8);
+            }
+        }
+        f32x4 acc1[8], acc2[8];
+        lora_tile<KSTEPS>(a.xa1, a.R, row0, row_end, lane, B1, acc1);
+        lora_tile<KSTEPS>(a.xa2, a.R, row0, row_end, lane, B2, acc2);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int64_t t = row0 + 4 * g + v;
+            const bool live = active && t < row_end;
+            float f1[8], f2[8], of[8];
+            unpack8(xv1[v], f1);
+            unpack8(xv2[v], f2);
+            uint32_t lo, hi;
+            // rows past the end still take part in the quad exchange; their stores are masked
+            const int64_t tq = t < row_end ? t : row_end - 1;
+            codes_to_words<QBIT, false, FAST>(f1, c1.s, c1.r, zero8, lo, hi);
+            store_packed<QBIT>(a.q1 + tq * row_bytes, chunk, live, lo, hi);
+            codes_to_words<QBIT, false, FAST>(f2, c2.s, c2.r, zero8, lo, hi);
+            store_packed<QBIT>(a.q2 + tq * row_bytes, chunk, live, lo, hi);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                float y1 = rbf(f1[j] + rbf(acc_elem(acc1[j], v)));
+                y1 = rbf(y1 * rbf(sigmoidf_(y1)));
+                const float y2 = rbf(f2[j] + rbf(acc_elem(acc2[j], v)));
+                of[j] = y1 * y2;
+            }
+            if (live) st16(a.o + t * a.N + chunk * 8, pack8(of));
+        }
+    }
+}
+
+template <int QBIT, int KSTEPS>
+__global__ __launch_bounds__(kFuseThreads) void lora_silu_fwd_kernel(const FuseArgs a) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int col_tile = blockIdx.x % a.col_tiles;
+    const int64_t row_tile = blockIdx.x / a.col_tiles;
+    const int chunk = col_tile * (kTileCols / 8) + (lane & 15);
+    const bool active = chunk < a.C;
+    const int col0 = chunk * 8;
+
+    QuantCols c1, c2;
+    c1.load(a.s1, col0, active);
+    c2.load(a.s2, col0, active);
+    BOperand<KSTEPS> B1, B2;
+    B1.load(a.b1, a.N, a.R, col0, active, lane >> 4);
+    B2.load(a.b2, a.N, a.R, col0, active, lane >> 4);
+
+    const int64_t row_begin = (row_tile * kFuseWaves + wave) * (int64_t)a.rows_per_wave;
+    int64_t row_end = row_begin + a.rows_per_wave;
+    if (row_end > a.T) row_end = a.T;
+    if (row_begin >= row_end) return;
+    if (__ballot(!(c1.fast && c2.fast)) != 0ull)
+        fuse_fwd_rows<QBIT, KSTEPS, false>(a, row_begin, row_end, lane, chunk, active, c1, c2, B1, B2);
+    else
+        fuse_fwd_rows<QBIT, KSTEPS, true>(a, row_begin, row_end, lane, chunk, active, c1, c2, B1, B2);
+}
+
+// ------------------------------------------------------------------------------------
+template <int QBIT, int KSTEPS>
+__global__ __launch_bounds__(kFuseThreads) void lora_silu_bwd_kernel(const FuseArgs a) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int col_tile = blockIdx.x % a.col_tiles;
+    const int64_t row_tile = blockIdx.x / a.col_tiles;
+    const int chunk = col_tile * (kTileCols / 8) + (lane & 15);
+    const bool active = chunk < a.C;
+    const int col0 = chunk * 8;
+    const int g = lane >> 4;
+    constexpr float kHalf = (float)(1 << (QBIT - 1));
+
+    float s1[8], s2[8];
+    {
+        u32x4 v1 = {0, 0, 0, 0}, v2 = {0, 0, 0, 0};
+        if (active) { v1 = ld16(a.s1 + col0); v2 = ld16(a.s2 + col0); }
+        unpack8(v1, s1);
+        unpack8(v2, s2);
+    }
+    BOperand<KSTEPS> B1, B2;
+    B1.load(a.b1, a.N, a.R, col0, active, g);
+    B2.load(a.b2, a.N, a.R, col0, active, g);
+    const PackedSlot<QBIT> slot(chunk);
+    const int row_bytes = a.N * QBIT / 8;
+
+    const int64_t row_begin = (row_tile * kFuseWaves + wave) * (int64_t)a.rows_per_wave;
+    int64_t row_end = row_begin + a.rows_per_wave;
+    if (row_end > a.T) row_end = a.T;
+
+    for (int64_t row0 = row_begin; row0 < row_end; row0 += kTileRows) {
+        u32x2 w1[4], w2[4];
+        u32x4 gv[4];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int64_t t = row0 + 4 * g + v;
+            w1[v] = u32x2{0, 0};
+            w2[v] = u32x2{0, 0};
+            gv[v] = u32x4{0, 0, 0, 0};
+            if (active && t < row_end) {
+                w1[v] = ld8(a.q1 + t * row_bytes + slot.offset);
+                w2[v] = ld8(a.q2 + t * row_bytes + slot.offset);
+                gv[v] = ld16(a.g + t * a.N + col0);
+            }
+        }
+        f32x4 acc1[8], acc2[8];
+        lora_tile<KSTEPS>(a.xa1, a.R, row0, row_end, lane, B1, acc1);
+        lora_tile<KSTEPS>(a.xa2, a.R, row0, row_end, lane, B2, acc2);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int64_t t = row0 + 4 * g + v;
+            if (!(active && t < row_end)) continue;
+            float cd1[8], cd2[8], gf[8], of[8], gg[8], gu[8];
+            slot.decode(w1[v], cd1);
+            slot.decode(w2[v], cd2);
+            unpack8(gv[v], gf);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float x1 = rbf((cd1[j] - kHalf) * s1[j]);
+                const float x2 = rbf((cd2[j] - kHalf) * s2[j]);
+                const float y1 = rbf(x1 + rbf(acc_elem(acc1[j], v)));
+                const float y2 = rbf(x2 + rbf(acc_elem(acc2[j], v)));
+                const float sig = rbf(sigmoidf_(y1));
+                const float sil = rbf(y1 * sig);
+                of[j] = sil * y2;
+                const float gh1 = rbf(gf[j] * y2);
+                gu[j] = gf[j] * sil;
+                const float dsilu = rbf(sig * rbf(1.0f + rbf(y1 * rbf(1.0f - sig))));
+                gg[j] = gh1 * dsilu;
+            }
+            st16(a.o + t * a.N + col0, pack8(of));
+            st16(a.gg + t * a.N + col0, pack8(gg));
+            st16(a.gu + t * a.N + col0, pack8(gu));
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------
+static int fuse_check(const FuseArgs& a, int64_t T, int64_t N, int64_t R, int q_bit, bool fwd) {
+    if (q_bit != 2 && q_bit != 4 && q_bit != 8) return HYC_ERR_QBIT;
+    if (T < 0 || N < 0 || N % 32 != 0 || N > (1 << 28) || T > ((int64_t)1 << 40)) return HYC_ERR_SHAPE;
+    if (R < 4 || R > 64 || R % 4 != 0) return HYC_ERR_RANK;
+    if (T * N == 0) return HYC_OK;
+    const void* need[] = {a.xa1, a.b1, a.s1, a.xa2, a.b2, a.s2, a.q1, a.q2, a.o,
+                          fwd ? (const void*)a.x1 : (const void*)a.g, fwd ? (const void*)a.x2 : (const void*)a.gg,
+                          fwd ? (const void*)a.o : (const void*)a.gu};
+    for (const void* p : need) if (!p) return HYC_ERR_NULL;
+    const void* al16[] = {a.b1, a.s1, a.b2, a.s2, a.o, fwd ? (const void*)a.x1 : (const void*)a.g,
+                          fwd ? (const void*)a.x2 : (const void*)a.gg, fwd ? (const void*)a.o : (const void*)a.gu};
+    for (const void* p : al16) if (!aligned16(p)) return HYC_ERR_ALIGN;
+    const void* al8[] = {a.xa1, a.xa2, a.q1, a.q2};
+    for (const void* p : al8) if (reinterpret_cast<uintptr_t>(p) & 7u) return HYC_ERR_ALIGN;
+    return 1;
+}
+
+#define HYC_FUSE_LAUNCH_K(KERNEL, QB)                                                                     \
+    do {                                                                                                  \
+        if (ksteps == 1) hipLaunchKernelGGL((KERNEL<QB, 1>), grid, block, 0, st, a);                      \
+        else if (ksteps == 2) hipLaunchKernelGGL((KERNEL<QB, 2>), grid, block, 0, st, a);                 \
+        else if (ksteps == 3) hipLaunchKernelGGL((KERNEL<QB, 3>), grid, block, 0, st, a);                 \
+        else hipLaunchKernelGGL((KERNEL<QB, 4>), grid, block, 0, st, a);                                  \
+    } while (0)
+#define HYC_FUSE_LAUNCH(KERNEL)                                  \
+    do {                                                         \
+        if (q_bit == 8) HYC_FUSE_LAUNCH_K(KERNEL, 8);            \
+        else if (q_bit == 4) HYC_FUSE_LAUNCH_K(KERNEL, 4);       \
+        else HYC_FUSE_LAUNCH_K(KERNEL, 2);                       \
+    } while (0)
+
+static int fuse_launch(FuseArgs& a, int64_t T, int64_t N, int64_t R, int q_bit, bool fwd, void* stream) {
+    const int rc = fuse_check(a, T, N, R, q_bit, fwd);
+    if (rc <= 0) return rc;
+    a.T = T;
+    a.N = (int)N;
+    a.C = (int)(N / 8);
+    a.R = (int)R;
+    a.rows_per_wave = g_fuse_rows_per_wave;
+    a.col_tiles = (int)cdiv(N, kTileCols);
+    const int64_t row_tiles = cdiv(T, (int64_t)kFuseWaves * a.rows_per_wave);
+    if (row_tiles * a.col_tiles > INT32_MAX) return HYC_ERR_SHAPE;
+    const dim3 grid((unsigned)(row_tiles * a.col_tiles)), block(kFuseThreads);
+    const int ksteps = (int)cdiv(R, 16);
+    hipStream_t st = (hipStream_t)stream;
+    if (fwd) HYC_FUSE_LAUNCH(lora_silu_fwd_kernel);
+    else HYC_FUSE_LAUNCH(lora_silu_bwd_kernel);
+    return check_launch();
+}
+
+int tune_fuse(const char* key, int value) {
+    if (strcmp(key, "fuse_rows_per_wave") == 0) {
+        if (value < kTileRows || value > 65536 || value % kTileRows != 0) return HYC_ERR_ARG;
+        g_fuse_rows_per_wave = value;
+        return HYC_OK;
+    }
+    return 1;
+}
+
+}  // namespace hyc
+
+using namespace hyc;
+
+extern "C" int hyc_lora_silu_mul_fwd(const void* xa1, const void* b1, const void* x1, const void* s1,
+                                     const void* xa2, const void* b2, const void* x2, const void* s2,
+                                     void* q1, void* q2, void* o, int64_t T, int64_t N, int64_t R, int q_bit,
+                                     void* stream) {
+    FuseArgs a{};
+    a.xa1 = (const uint16_t*)xa1; a.b1 = (const uint16_t*)b1; a.s1 = (const uint16_t*)s1;
+    a.xa2 = (const uint16_t*)xa2; a.b2 = (const uint16_t*)b2; a.s2 = (const uint16_t*)s2;
+    a.x1 = (const uint16_t*)x1; a.x2 = (const uint16_t*)x2;
+    a.q1 = (uint8_t*)q1; a.q2 = (uint8_t*)q2; a.o = (uint16_t*)o;
+    return fuse_launch(a, T, N, R, q_bit, true, stream);
+}
+
+extern "C" int hyc_lora_silu_mul_bwd(const void* xa1, const void* b1, const void* q1, const void* s1,
+                                     const void* xa2, const void* b2, const void* q2, const void* s2,
+                                     const void* grad_o, void* o, void* grad_gate, void* grad_up, int64_t T,
+                                     int64_t N, int64_t R, int q_bit, void* stream) {
+    FuseArgs a{};
+    a.xa1 = (const uint16_t*)xa1; a.b1 = (const uint16_t*)b1; a.s1 = (const uint16_t*)s1;
+    a.xa2 = (const uint16_t*)xa2; a.b2 = (const uint16_t*)b2; a.s2 = (const uint16_t*)s2;
+    a.q1 = (uint8_t*)q1; a.q2 = (uint8_t*)q2;
+    a.g = (const uint16_t*)grad_o; a.o = (uint16_t*)o; a.gg = (uint16_t*)grad_gate; a.gu = (uint16_t*)grad_up;
+    return fuse_launch(a, T, N, R, q_bit, false, stream);
+}

@@ -1,0 +1,285 @@
+// RMSNorm forward / backward for gfx950.
+//
+// One wave owns one row: each lane keeps CH 16-byte chunks of the row in registers, so the
+// row is read once, reduced with a wave-level sum and written once.  Rows longer than
+// 64*8*16 = 8192 channels fall back to a two-pass loop over the row (second pass hits L2).
+//
+// Backward also produces the weight gradient dw = sum_rows dy * x^ without the reference's
+// spin-lock accumulation (operators/rmsnorm_kernels.py:103-113): each wave accumulates its
+// rows in fp32 registers, the workgroup combines its waves in LDS and writes one partial
+// row; a second kernel adds the partial rows in a fixed order.  Deterministic, no atomics.
+#include "hyc_common.hpp"
+
+namespace hyc {
+
+constexpr int kNormThreads = 256;
+constexpr int kNormWaves = kNormThreads / kWave;
+constexpr int kNormMaxBlocks = 512;
+
+template <bool W32>
+__device__ __forceinline__ void load_w8(const void* w, int col, float (&wf)[8]) {
+    if constexpr (W32) {
+        const f32x4 a = *reinterpret_cast<const f32x4*>((const float*)w + col);
+        const f32x4 b = *reinterpret_cast<const f32x4*>((const float*)w + col + 4);
+        wf[0] = a.x; wf[1] = a.y; wf[2] = a.z; wf[3] = a.w;
+        wf[4] = b.x; wf[5] = b.y; wf[6] = b.z; wf[7] = b.w;
+    } else {
+        unpack8(ld16((const uint16_t*)w + col), wf);
+    }
+}
+
+// y = bf16(x * rstd * w), rstd = 1/sqrt(mean(x^2) + eps)   (operators/rmsnorm_kernels.py:34-54)
+template <int CH, bool W32>
+__global__ __launch_bounds__(kNormThreads) void rmsnorm_fwd_kernel(const uint16_t* __restrict__ x, const void* __restrict__ w,
+                                                                   uint16_t* __restrict__ y, float* __restrict__ rstd_out,
+                                                                   int64_t rows, int N, float eps) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t row = (int64_t)blockIdx.x * kNormWaves + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const uint16_t* xr = x + row * N;
+    u32x4 xv[CH];
+    float ss = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int col = (c * kWave + lane) * 8;
+        xv[c] = u32x4{0, 0, 0, 0};
+        if (col < N) xv[c] = ld16(xr + col);
+    }
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        float f[8];
+        unpack8(xv[c], f);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ss = fmaf(f[j], f[j], ss);
+    }
+    ss = wave_sum(ss);
+    const float rstd = 1.0f / sqrtf(ss / (float)N + eps);
+    if (lane == 0) rstd_out[row] = rstd;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int col = (c * kWave + lane) * 8;
+        if (col < N) {
+            float f[8], wf[8], o[8];
+            unpack8(xv[c], f);
+            load_w8<W32>(w, col, wf);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) o[j] = (f[j] * rstd) * wf[j];
+            st16(y + row * N + col, pack8(o));
+        }
+    }
+}
+
+// Long rows: the row does not fit in registers; read it twice.
+template <bool W32>
+__global__ __launch_bounds__(kNormThreads) void rmsnorm_fwd_long_kernel(const uint16_t* __restrict__ x, const void* __restrict__ w,
+                                                                        uint16_t* __restrict__ y, float* __restrict__ rstd_out,
+                                                                        int64_t rows, int N, float eps) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t row = (int64_t)blockIdx.x * kNormWaves + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const uint16_t* xr = x + row * N;
+    float ss = 0.0f;
+    for (int col = lane * 8; col < N; col += kWave * 8) {
+        float f[8];
+        unpack8(ld16(xr + col), f);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ss = fmaf(f[j], f[j], ss);
+    }
+    ss = wave_sum(ss);
+    const float rstd = 1.0f / sqrtf(ss / (float)N + eps);
+    if (lane == 0) rstd_out[row] = rstd;
+    for (int col = lane * 8; col < N; col += kWave * 8) {
+        float f[8], wf[8], o[8];
+        unpack8(ld16(xr + col), f);
+        load_w8<W32>(w, col, wf);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) o[j] = (f[j] * rstd) * wf[j];
+        st16(y + row * N + col, pack8(o));
+    }
+}
+
+// dx = (w*dy - (x^*c1 + c2)) * rstd,  c1 = mean(x^ * w*dy),  c2 = mean(w*dy),  x^ = x*rstd.
+// The c2 term belongs to LayerNorm; the reference keeps it for RMSNorm
+// (operators/rmsnorm_kernels.py:92-100) and so does this kernel.
+template <int CH, bool W32, bool DW>
+__global__ __launch_bounds__(kNormThreads) void rmsnorm_bwd_kernel(const uint16_t* __restrict__ dy, const uint16_t* __restrict__ x,
+                                                                   const void* __restrict__ w, const float* __restrict__ rstd_in,
+                                                                   uint16_t* __restrict__ dx, float* __restrict__ dw_partial,
+                                                                   int64_t rows, int N) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x >> 6;
+    float wf[CH][8];
+    float dwacc[DW ? CH : 1][8];
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int col = (c * kWave + lane) * 8;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) wf[c][j] = 0.0f;
+        if (col < N) load_w8<W32>(w, col, wf[c]);
+        if constexpr (DW) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) dwacc[c][j] = 0.0f;
+        }
+    }
+    const float inv_n = 1.0f / (float)N;
+    for (int64_t row = (int64_t)blockIdx.x * kNormWaves + wave; row < rows; row += (int64_t)gridDim.x * kNormWaves) {
+        const float rstd = rstd_in[row];
+        u32x4 xv[CH], gv[CH];
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int col = (c * kWave + lane) * 8;
+            xv[c] = u32x4{0, 0, 0, 0};
+            gv[c] = u32x4{0, 0, 0, 0};
+            if (col < N) {
+                xv[c] = ld16(x + row * N + col);
+                gv[c] = ld16(dy + row * N + col);
+            }
+        }
+        float s1 = 0.0f, s2 = 0.0f;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            float xf[8], gf[8];
+            unpack8(xv[c], xf);
+            unpack8(gv[c], gf);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float xh = xf[j] * rstd, wdy = wf[c][j] * gf[j];
+                s1 = fmaf(xh, wdy, s1);
+                s2 += wdy;
+                if constexpr (DW) dwacc[c][j] = fmaf(gf[j], xh, dwacc[c][j]);
+            }
+        }
+        const float c1 = wave_sum(s1) * inv_n, c2 = wave_sum(s2) * inv_n;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int col = (c * kWave + lane) * 8;
+            if (col < N) {
+                float xf[8], gf[8], o[8];
+                unpack8(xv[c], xf);
+                unpack8(gv[c], gf);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float xh = xf[j] * rstd, wdy = wf[c][j] * gf[j];
+                    o[j] = (wdy - (xh * c1 + c2)) * rstd;
+                }
+                st16(dx + row * N + col, pack8(o));
+            }
+        }
+    }
+    if constexpr (DW) {
+        // combine the workgroup's waves through LDS, one chunk index at a time, wave order fixed
+        __shared__ float red[kNormWaves][kWave * 8];
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            __syncthreads();
+#pragma unroll
+            for (int j = 0; j < 8; ++j) red[wave][lane * 8 + j] = dwacc[c][j];
+            __syncthreads();
+            for (int i = threadIdx.x; i < kWave * 8; i += kNormThreads) {
+                const int col = c * kWave * 8 + i;
+                if (col < N) {
+                    float s = red[0][i];
+#pragma unroll
+                    for (int v = 1; v < kNormWaves; ++v) s += red[v][i];
+                    dw_partial[(int64_t)blockIdx.x * N + col] = s;
+                }
+            }
+        }
+    }
+}
+
+// dw[c] = sum over partial rows, fixed order; output in the weight's dtype.
+template <bool W32>
+__global__ void rmsnorm_dw_reduce_kernel(const float* __restrict__ partial, int nparts, int N, void* __restrict__ dw) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= N) return;
+    float s = 0.0f;
+    for (int p = 0; p < nparts; ++p) s += partial[(int64_t)p * N + c];
+    if constexpr (W32) ((float*)dw)[c] = s;
+    else ((uint16_t*)dw)[c] = f_to_bf(s);
+}
+
+static int bwd_blocks(int64_t rows) {
+    int64_t b = cdiv(rows, kNormWaves * 4);
+    if (b > kNormMaxBlocks) b = kNormMaxBlocks;
+    if (b < 1) b = 1;
+    return (int)b;
+}
+
+template <bool W32>
+static int launch_fwd(const uint16_t* x, const void* w, uint16_t* y, float* rstd, int64_t rows, int N, float eps,
+                      hipStream_t st) {
+    const dim3 grid((unsigned)cdiv(rows, kNormWaves)), block(kNormThreads);
+#define HYC_FWD(CH) hipLaunchKernelGGL((rmsnorm_fwd_kernel<CH, W32>), grid, block, 0, st, x, w, y, rstd, rows, N, eps)
+    if (N <= 512) HYC_FWD(1);
+    else if (N <= 1024) HYC_FWD(2);
+    else if (N <= 2048) HYC_FWD(4);
+    else if (N <= 4096) HYC_FWD(8);
+    else if (N <= 8192) HYC_FWD(16);
+    else hipLaunchKernelGGL((rmsnorm_fwd_long_kernel<W32>), grid, block, 0, st, x, w, y, rstd, rows, N, eps);
+#undef HYC_FWD
+    return check_launch();
+}
+
+template <bool W32, bool DW>
+static int launch_bwd(const uint16_t* dy, const uint16_t* x, const void* w, const float* rstd, uint16_t* dx,
+                      float* partial, int64_t rows, int N, int blocks, hipStream_t st) {
+    const dim3 grid((unsigned)blocks), block(kNormThreads);
+#define HYC_BWD(CH) hipLaunchKernelGGL((rmsnorm_bwd_kernel<CH, W32, DW>), grid, block, 0, st, dy, x, w, rstd, dx, partial, rows, N)
+    if (N <= 512) HYC_BWD(1);
+    else if (N <= 1024) HYC_BWD(2);
+    else if (N <= 2048) HYC_BWD(4);
+    else if (N <= 4096) HYC_BWD(8);
+    else HYC_BWD(16);
+#undef HYC_BWD
+    return check_launch();
+}
+
+}  // namespace hyc
+
+using namespace hyc;
+
+extern "C" int hyc_rmsnorm_fwd(const void* x, const void* weight, int weight_is_fp32, void* y, float* rstd,
+                               int64_t rows, int64_t N, float eps, void* stream) {
+    if (rows < 0 || N < 0 || N % 8 != 0 || N > 65536) return HYC_ERR_SHAPE;
+    if (rows == 0 || N == 0) return HYC_OK;
+    if (!x || !weight || !y || !rstd) return HYC_ERR_NULL;
+    if (!aligned16(x) || !aligned16(weight) || !aligned16(y)) return HYC_ERR_ALIGN;
+    if (cdiv(rows, kNormWaves) > INT32_MAX) return HYC_ERR_SHAPE;
+    hipStream_t st = (hipStream_t)stream;
+    return weight_is_fp32 ? launch_fwd<true>((const uint16_t*)x, weight, (uint16_t*)y, rstd, rows, (int)N, eps, st)
+                          : launch_fwd<false>((const uint16_t*)x, weight, (uint16_t*)y, rstd, rows, (int)N, eps, st);
+}
+
+extern "C" int64_t hyc_rmsnorm_bwd_workspace(int64_t rows, int64_t N) {
+    if (rows <= 0 || N <= 0) return 0;
+    return (int64_t)bwd_blocks(rows) * N * (int64_t)sizeof(float);
+}
+
+extern "C" int hyc_rmsnorm_bwd(const void* dy, const void* x, const void* weight, int weight_is_fp32,
+                               const float* rstd, void* dx, void* dw, void* workspace, int64_t workspace_bytes,
+                               int64_t rows, int64_t N, void* stream) {
+    if (rows < 0 || N < 0 || N % 8 != 0 || N > 8192) return HYC_ERR_SHAPE;
+    if (rows == 0 || N == 0) return HYC_OK;
+    if (!dy || !x || !weight || !rstd || !dx) return HYC_ERR_NULL;
+    if (!aligned16(dy) || !aligned16(x) || !aligned16(weight) || !aligned16(dx)) return HYC_ERR_ALIGN;
+    hipStream_t st = (hipStream_t)stream;
+    const int blocks = bwd_blocks(rows);
+    int rc;
+    if (dw) {
+        if (!workspace) return HYC_ERR_NULL;
+        if (workspace_bytes < hyc_rmsnorm_bwd_workspace(rows, N)) return HYC_ERR_WORKSPACE;
+        rc = weight_is_fp32
+                 ? launch_bwd<true, true>((const uint16_t*)dy, (const uint16_t*)x, weight, rstd, (uint16_t*)dx, (float*)workspace, rows, (int)N, blocks, st)
+                 : launch_bwd<false, true>((const uint16_t*)dy, (const uint16_t*)x, weight, rstd, (uint16_t*)dx, (float*)workspace, rows, (int)N, blocks, st);
+        if (rc != HYC_OK) return rc;
+        const dim3 grid((unsigned)cdiv(N, 256)), block(256);
+        if (weight_is_fp32) hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel<true>, grid, block, 0, st, (const float*)workspace, blocks, (int)N, dw);
+        else hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel<false>, grid, block, 0, st, (const float*)workspace, blocks, (int)N, dw);
+        return check_launch();
+    }
+    // without dw the grid need not be capped, but the same persistent loop is used
+    return weight_is_fp32
+               ? launch_bwd<true, false>((const uint16_t*)dy, (const uint16_t*)x, weight, rstd, (uint16_t*)dx, nullptr, rows, (int)N, (int)(cdiv(rows, kNormWaves) > 65535 * 16 ? 65535 * 16 : cdiv(rows, kNormWaves)), st)
+               : launch_bwd<false, false>((const uint16_t*)dy, (const uint16_t*)x, weight, rstd, (uint16_t*)dx, nullptr, rows, (int)N, (int)(cdiv(rows, kNormWaves) > 65535 * 16 ? 65535 * 16 : cdiv(rows, kNormWaves)), st);
+}

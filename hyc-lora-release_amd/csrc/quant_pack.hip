@@ -17,7 +17,7 @@
 // its sub-byte slot); the sharing lanes then OR their words together with DPP quad
 // permutes — no LDS, no bpermute — and each stores a different dword of the result, so
 // the wave writes one contiguous run per row.
-#include "hyc_common.hpp"
+#include "hyc_pack.hpp"
 
 namespace hyc {
 
@@ -110,33 +110,11 @@ __device__ __forceinline__ int64_t chunk_offset(int col0, int head_dim, int64_t 
 // ------------------------------------------------------------------------------------
 // quantise + pack
 // ------------------------------------------------------------------------------------
-template <int QBIT, bool ZP, bool FAST>
-__device__ __forceinline__ void codes_to_words(const float (&f)[8], const float (&s)[8], const float (&r)[8],
-                                               const float (&z)[8], uint32_t& lo, uint32_t& hi) {
-    int c[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        if constexpr (ZP) {
-            // zero-point form: IEEE quotient, then + z, then exact roundf
-            c[j] = hyc_code_from_t_exact(f[j] / s[j] + z[j], QBIT);
-        } else if constexpr (FAST) {
-            c[j] = hyc_code_from_t(hyc_quot_fast(f[j], s[j], r[j]), QBIT);
-        } else {
-            c[j] = hyc_code_from_t(f[j] / s[j], QBIT);
-        }
-    }
-    lo = (uint32_t)c[0] | ((uint32_t)c[1] << 8) | ((uint32_t)c[2] << 16) | ((uint32_t)c[3] << 24);
-    hi = (uint32_t)c[4] | ((uint32_t)c[5] << 8) | ((uint32_t)c[6] << 16) | ((uint32_t)c[7] << 24);
-}
-
 template <int QBIT, bool ZP, bool OUTL, bool FAST>
 __device__ __forceinline__ void quant_rows(const QuantArgs& a, int64_t row0, int64_t row1, bool active, int chunk,
                                            int64_t coff, const float (&s)[8], const float (&r)[8],
                                            const float (&z)[8], const OutlierLane& ol) {
-    const int quad = chunk & 3;            // chunk position inside its 32-column block
-    const int blk = chunk >> 2;
     const int row_bytes = a.N * QBIT / 8;
-
     if (row0 >= row1) return;
     RowCursor cur(row0, a.M, a.stride_b, a.stride_m);
     for (int64_t t0 = row0; t0 < row1; t0 += kRowUnroll) {
@@ -173,26 +151,7 @@ __device__ __forceinline__ void quant_rows(const QuantArgs& a, int64_t row0, int
             unpack8(v[u], f);
             uint32_t lo, hi;
             codes_to_words<QBIT, ZP, FAST>(f, s, r, z, lo, hi);
-            uint8_t* qrow = a.q + t * row_bytes;
-            if constexpr (QBIT == 8) {
-                if (active) st8(qrow + (int64_t)chunk * 8, u32x2{lo, hi});
-            } else if constexpr (QBIT == 4) {
-                const int sub = quad >> 1;
-                lo <<= 4 * sub;
-                hi <<= 4 * sub;
-                lo |= quad_xor2(lo);
-                hi |= quad_xor2(hi);
-                if (active)
-                    *reinterpret_cast<uint32_t*>(qrow + blk * 16 + 8 * (quad & 1) + 4 * sub) = sub ? hi : lo;
-            } else {
-                lo <<= 2 * quad;
-                hi <<= 2 * quad;
-                lo |= quad_xor1(lo);
-                hi |= quad_xor1(hi);
-                lo |= quad_xor2(lo);
-                hi |= quad_xor2(hi);
-                if (active && quad < 2) *reinterpret_cast<uint32_t*>(qrow + blk * 8 + 4 * quad) = quad ? hi : lo;
-            }
+            store_packed<QBIT>(a.q + t * row_bytes, chunk, active, lo, hi);
         }
     }
 }
@@ -207,21 +166,13 @@ __global__ __launch_bounds__(kQuantThreads) void quant_pack_kernel(const QuantAr
     const bool active = chunk < a.C;
     const int col0 = chunk * 8;
 
-    float s[8], r[8], z[8];
-    bool fast = true;
-    {
-        u32x4 sv = {0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};  // 1.0 for idle lanes
-        if (active) sv = ld16(a.scale + col0);
-        unpack8(sv, s);
+    QuantCols qc;
+    qc.load(a.scale, col0, active);
+    float z[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            r[j] = 1.0f / s[j];
-            fast = fast && hyc_scale_is_fast(s[j]);
-            z[j] = 0.0f;
-        }
-        if constexpr (ZP) {
-            if (active) unpack8(ld16(a.zp + col0), z);
-        }
+    for (int j = 0; j < 8; ++j) z[j] = 0.0f;
+    if constexpr (ZP) {
+        if (active) unpack8(ld16(a.zp + col0), z);
     }
     OutlierLane ol;
     if constexpr (OUTL) ol = find_outliers(a.oidx, a.k, col_tile * kWave * 8, col0, lane);
@@ -232,10 +183,10 @@ __global__ __launch_bounds__(kQuantThreads) void quant_pack_kernel(const QuantAr
     if (row1 > a.T) row1 = a.T;
 
     // one slow column anywhere in the wave sends the whole wave down the IEEE-division path
-    if (ZP || __ballot(!fast) != 0ull)
-        quant_rows<QBIT, ZP, OUTL, false>(a, row0, row1, active, chunk, coff, s, r, z, ol);
+    if (ZP || __ballot(!qc.fast) != 0ull)
+        quant_rows<QBIT, ZP, OUTL, false>(a, row0, row1, active, chunk, coff, qc.s, qc.r, z, ol);
     else
-        quant_rows<QBIT, ZP, OUTL, true>(a, row0, row1, active, chunk, coff, s, r, z, ol);
+        quant_rows<QBIT, ZP, OUTL, true>(a, row0, row1, active, chunk, coff, qc.s, qc.r, z, ol);
 }
 
 // ------------------------------------------------------------------------------------
@@ -250,8 +201,6 @@ __global__ __launch_bounds__(kQuantThreads) void unpack_dequant_kernel(const Qua
     const int chunk = col_tile * kWave + lane;
     const bool active = chunk < a.C;
     const int col0 = chunk * 8;
-    const int quad = chunk & 3;
-    const int blk = chunk >> 2;
     constexpr float kHalf = (float)(1 << (QBIT - 1));
 
     float s[8], z[8];
@@ -274,12 +223,7 @@ __global__ __launch_bounds__(kQuantThreads) void unpack_dequant_kernel(const Qua
     if (row1 > a.T) row1 = a.T;
     const int row_bytes = a.N * QBIT / 8;
 
-    // byte offset of the 8 packed bytes that hold this chunk's codes, and the bit shift
-    int qoff, shift;
-    uint32_t mask;
-    if constexpr (QBIT == 8) { qoff = chunk * 8; shift = 0; mask = 0xffffffffu; }
-    else if constexpr (QBIT == 4) { qoff = blk * 16 + 8 * (quad & 1); shift = 4 * (quad >> 1); mask = 0x0f0f0f0fu; }
-    else { qoff = blk * 8; shift = 2 * quad; mask = 0x03030303u; }
+    const PackedSlot<QBIT> slot(chunk);
 
     if (row0 >= row1) return;
     RowCursor cur(row0, a.M, a.stride_b, a.stride_m);
@@ -289,25 +233,23 @@ __global__ __launch_bounds__(kQuantThreads) void unpack_dequant_kernel(const Qua
         for (int u = 0; u < kRowUnroll; ++u) {
             const int64_t t = t0 + u;
             w[u] = u32x2{0, 0};
-            if (active && t < row1) w[u] = ld8(a.q + t * row_bytes + qoff);
+            if (active && t < row1) w[u] = ld8(a.q + t * row_bytes + slot.offset);
         }
 #pragma unroll
         for (int u = 0; u < kRowUnroll; ++u) {
             const int64_t t = t0 + u;
             if (t >= row1) break;
-            const uint32_t lo = (w[u].x >> shift) & mask;
-            const uint32_t hi = (w[u].y >> shift) & mask;
-            float f[8];
+            float c[8], f[8];
+            slot.decode(w[u], c);
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                const float c = (float)(((j < 4 ? lo : hi) >> (8 * (j & 3))) & 0xffu);
                 if constexpr (ZP) {
                     // bf16 arithmetic step by step: (c - 2^(q-1)) is exact, minus z rounds to bf16
-                    f[j] = rbf((c - kHalf) - z[j]) * s[j];
+                    f[j] = rbf((c[j] - kHalf) - z[j]) * s[j];
                 } else {
                     // not fma(c, s, -2^(q-1) s): that loses the sign of zero and turns an
                     // infinite step into NaN where the reference's product does not
-                    f[j] = (c - kHalf) * s[j];
+                    f[j] = (c[j] - kHalf) * s[j];
                 }
             }
             u32x4 o = pack8(f);

@@ -1,0 +1,420 @@
+// Attention-map compression for gfx950: exact k-th value of a bf16 tensor (the keep
+// threshold), ordered compaction of the kept entries to (int64 index, bf16 value) pairs,
+// the dense restore, and the softmax backward that consumes the map.
+//
+// The threshold is an exact order statistic.  A bf16 tensor has at most 65536 distinct
+// values, so one pass that histograms the bit patterns followed by a scan of the
+// histogram gives the k-th value without sorting or copying the tensor to fp32.
+//
+// Compaction keeps the ascending index order torch's to_sparse() produces.  The flattened
+// tensor is cut into segments of kSeg elements, one per wave: pass 1 counts the kept
+// entries of each segment, a single workgroup turns the counts into offsets, pass 2
+// writes each segment's entries at its offset (lane-ordered with a wave prefix sum).
+// The same offsets let the restore kernel rebuild every segment independently: stage the
+// segment in LDS (zeros, then its entries), then stream it out with 128-bit stores.
+#include "hyc_common.hpp"
+
+namespace hyc {
+
+constexpr int kHistThreads = 1024;
+constexpr int kHistLdsBins = 16384;   // keys 0x8000..0xBFFF: bf16 values in [+0, 2), 64 KiB of counters
+constexpr int kSeg = 4096;            // elements per compaction segment (one wave)
+constexpr int kSegThreads = 256;      // 4 segments per workgroup
+constexpr int kSegSteps = kSeg / (kWave * 8);
+
+// Monotonic 16-bit key of a bf16 bit pattern: ascending key = ascending value, NaN last
+// (torch.kthvalue orders NaN above everything).
+__device__ __forceinline__ uint32_t bf16_key(uint32_t bits) {
+    if ((bits & 0x7fffu) > 0x7f80u) return 0xffffu;
+    return (bits & 0x8000u) ? (0x7fffu - (bits & 0x7fffu)) : (0x8000u | bits);
+}
+__device__ __forceinline__ uint32_t key_to_bf16(uint32_t key) {
+    if (key == 0xffffu) return 0x7fc0u;
+    return (key & 0x8000u) ? (key & 0x7fffu) : (0x8000u | (0x7fffu - key));
+}
+
+__global__ void fill_u32_kernel(uint32_t* p, int64_t n, uint32_t v) {
+    for (int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = v;
+}
+
+// ---- histogram of bit patterns ------------------------------------------------------
+__device__ __forceinline__ void hist_add(uint32_t bits, uint32_t* lds, uint32_t* hist, uint32_t& zeros) {
+    if (bits == 0) { ++zeros; return; }           // +0 is by far the most common value of a masked softmax
+    const uint32_t key = bf16_key(bits);
+    const uint32_t rel = key - 0x8000u;
+    if (rel < (uint32_t)kHistLdsBins) atomicAdd(&lds[rel], 1u);
+    else atomicAdd(&hist[key], 1u);
+}
+
+__global__ __launch_bounds__(kHistThreads) void hist16_kernel(const uint16_t* __restrict__ a, int64_t n,
+                                                              uint32_t* __restrict__ hist) {
+    __shared__ uint32_t lds[kHistLdsBins];
+    for (int i = threadIdx.x; i < kHistLdsBins; i += kHistThreads) lds[i] = 0;
+    __syncthreads();
+    uint32_t zeros = 0;
+    const int64_t chunks = n / 8;
+    for (int64_t c = blockIdx.x * (int64_t)kHistThreads + threadIdx.x; c < chunks; c += (int64_t)gridDim.x * kHistThreads) {
+        const u32x4 v = ld16(a + c * 8);
+        const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            hist_add(d[j] & 0xffffu, lds, hist, zeros);
+            hist_add(d[j] >> 16, lds, hist, zeros);
+        }
+    }
+    if (blockIdx.x == 0 && threadIdx.x < (n & 7)) hist_add(a[chunks * 8 + threadIdx.x], lds, hist, zeros);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) zeros += (uint32_t)__shfl_xor((int)zeros, o, kWave);
+    if ((threadIdx.x & (kWave - 1)) == 0 && zeros) atomicAdd(&lds[0], zeros);
+    __syncthreads();
+    for (int i = threadIdx.x; i < kHistLdsBins; i += kHistThreads) {
+        const uint32_t v = lds[i];
+        if (v) atomicAdd(&hist[0x8000 + i], v);
+    }
+}
+
+// Single workgroup: the k-th smallest value (1-based) from the histogram.
+__global__ __launch_bounds__(1024) void hist_select_kernel(const uint32_t* __restrict__ hist, int64_t kth,
+                                                           float* __restrict__ thr) {
+    __shared__ unsigned long long incl[1024];
+    const int t = threadIdx.x;
+    unsigned long long sum = 0;
+    for (int i = 0; i < 64; ++i) sum += hist[t * 64 + i];
+    incl[t] = sum;
+    __syncthreads();
+    for (int o = 1; o < 1024; o <<= 1) {
+        const unsigned long long add = t >= o ? incl[t - o] : 0;
+        __syncthreads();
+        incl[t] += add;
+        __syncthreads();
+    }
+    const unsigned long long hi = incl[t], lo = hi - sum, k = (unsigned long long)kth;
+    if (lo < k && k <= hi) {
+        unsigned long long cum = lo;
+        for (int i = 0; i < 64; ++i) {
+            cum += hist[t * 64 + i];
+            if (cum >= k) {
+                *thr = __builtin_bit_cast(float, key_to_bf16((uint32_t)(t * 64 + i)) << 16);
+                break;
+            }
+        }
+    }
+}
+
+// ---- ordered compaction ---------------------------------------------------------------
+// kept: a > thr and a != 0 (to_sparse drops exact zeros); NaN is never kept.  The caller
+// passes thr already rounded to bf16: torch compares a bf16 tensor with a 0-d fp32
+// threshold in bf16.
+__device__ __forceinline__ bool keep(uint32_t bits, float thr) {
+    const float v = bf_to_f((uint16_t)bits);
+    return v > thr && v != 0.0f;
+}
+
+// Loads the 8 elements of chunk `c` of the flattened tensor, zero-filling past n.
+__device__ __forceinline__ void load_chunk(const uint16_t* a, int64_t c, int64_t n, uint32_t (&e)[8]) {
+    const int64_t i0 = c * 8;
+    if (i0 + 8 <= n) {
+        const u32x4 v = ld16(a + i0);
+        e[0] = v.x & 0xffffu; e[1] = v.x >> 16; e[2] = v.y & 0xffffu; e[3] = v.y >> 16;
+        e[4] = v.z & 0xffffu; e[5] = v.z >> 16; e[6] = v.w & 0xffffu; e[7] = v.w >> 16;
+    } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) e[j] = (i0 + j < n) ? a[i0 + j] : 0u;
+    }
+}
+
+__global__ __launch_bounds__(kSegThreads) void sparse_count_kernel(const uint16_t* __restrict__ a, int64_t n,
+                                                                   const float* __restrict__ thr_p, int64_t nseg,
+                                                                   uint32_t* __restrict__ counts) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t seg = blockIdx.x * (int64_t)(kSegThreads / kWave) + (threadIdx.x >> 6);
+    if (seg >= nseg) return;
+    const float thr = rbf(*thr_p);
+    uint32_t cnt = 0;
+#pragma unroll
+    for (int s = 0; s < kSegSteps; ++s) {
+        const int64_t c = seg * (kSeg / 8) + s * kWave + lane;
+        if (c * 8 < n) {
+            uint32_t e[8];
+            load_chunk(a, c, n, e);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) cnt += keep(e[j], thr) ? 1u : 0u;
+        }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) cnt += (uint32_t)__shfl_xor((int)cnt, o, kWave);
+    if (lane == 0) counts[seg] = cnt;
+}
+
+// Single workgroup: offsets[s] = sum of counts[0..s), offsets[nseg] = total.
+__global__ __launch_bounds__(1024) void seg_scan_kernel(const uint32_t* __restrict__ counts, int64_t nseg,
+                                                        int64_t* __restrict__ offsets) {
+    __shared__ long long incl[1024];
+    const int t = threadIdx.x;
+    const int64_t per = cdiv(nseg, 1024);
+    const int64_t b = t * per, e = b + per < nseg ? b + per : nseg;
+    long long sum = 0;
+    for (int64_t i = b; i < e; ++i) sum += counts[i];
+    incl[t] = sum;
+    __syncthreads();
+    for (int o = 1; o < 1024; o <<= 1) {
+        const long long add = t >= o ? incl[t - o] : 0;
+        __syncthreads();
+        incl[t] += add;
+        __syncthreads();
+    }
+    long long run = incl[t] - sum;
+    for (int64_t i = b; i < e; ++i) {
+        offsets[i] = run;
+        run += counts[i];
+    }
+    if (t == 1023) offsets[nseg] = incl[1023];
+}
+
+__global__ __launch_bounds__(kSegThreads) void sparse_write_kernel(const uint16_t* __restrict__ a, int64_t n,
+                                                                   const float* __restrict__ thr_p, int64_t nseg,
+                                                                   const int64_t* __restrict__ offsets,
+                                                                   int64_t* __restrict__ idx_out,
+                                                                   uint16_t* __restrict__ val_out) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t seg = blockIdx.x * (int64_t)(kSegThreads / kWave) + (threadIdx.x >> 6);
+    if (seg >= nseg) return;
+    const float thr = rbf(*thr_p);
+    int64_t base = offsets[seg];
+    if (offsets[seg + 1] == base) return;          // nothing kept in this segment
+    for (int s = 0; s < kSegSteps; ++s) {
+        const int64_t c = seg * (kSeg / 8) + s * kWave + lane;
+        uint32_t e[8];
+        uint32_t mask = 0;
+        if (c * 8 < n) {
+            load_chunk(a, c, n, e);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) mask |= keep(e[j], thr) ? (1u << j) : 0u;
+        }
+        const uint32_t cnt = __popc(mask);
+        uint32_t inc = cnt;                          // inclusive prefix over lanes
+#pragma unroll
+        for (int o = 1; o < kWave; o <<= 1) {
+            const uint32_t up = (uint32_t)__shfl_up((int)inc, o, kWave);
+            if (lane >= o) inc += up;
+        }
+        int64_t w = base + (inc - cnt);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            if (mask & (1u << j)) {
+                idx_out[w] = c * 8 + j;
+                val_out[w] = (uint16_t)e[j];
+                ++w;
+            }
+        }
+        base += (uint32_t)__shfl((int)inc, kWave - 1, kWave);
+    }
+}
+
+// Segment offsets of an existing ascending index list: offsets[s] = first entry whose
+// index is >= s*kSeg.  Entry e fills the offsets of all segments that begin between its
+// predecessor's segment and its own.
+__global__ void seg_offsets_kernel(const int64_t* __restrict__ idx, int64_t nnz, int64_t nseg,
+                                   int64_t* __restrict__ offsets) {
+    const int64_t e = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+    if (e > nnz) return;
+    const int64_t prev = e == 0 ? -1 : idx[e - 1] / kSeg;
+    int64_t cur = e == nnz ? nseg : idx[e] / kSeg;
+    if (cur > nseg) cur = nseg;
+    for (int64_t s = prev + 1; s <= cur; ++s) offsets[s] = e;
+}
+
+// ---- dense restore ----------------------------------------------------------------------
+__global__ __launch_bounds__(kSegThreads) void sparse_restore_kernel(const int64_t* __restrict__ idx,
+                                                                     const uint16_t* __restrict__ val,
+                                                                     const int64_t* __restrict__ offsets,
+                                                                     int64_t nseg, int64_t n,
+                                                                     uint16_t* __restrict__ out) {
+    __shared__ __attribute__((aligned(16))) uint16_t stage[kSegThreads / kWave][kSeg];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x >> 6;
+    const int64_t seg = blockIdx.x * (int64_t)(kSegThreads / kWave) + wave;
+    const bool live = seg < nseg;
+    u32x4* st = reinterpret_cast<u32x4*>(stage[wave]);
+#pragma unroll
+    for (int s = 0; s < kSegSteps; ++s) st[s * kWave + lane] = u32x4{0, 0, 0, 0};
+    __syncthreads();
+    if (live) {
+        const int64_t e0 = offsets[seg], e1 = offsets[seg + 1];
+        const int64_t first = seg * kSeg;
+        for (int64_t e = e0 + lane; e < e1; e += kWave) {
+            const int64_t rel = idx[e] - first;
+            if (rel >= 0 && rel < kSeg) stage[wave][rel] = val[e];
+        }
+    }
+    __syncthreads();
+    if (live) {
+#pragma unroll
+        for (int s = 0; s < kSegSteps; ++s) {
+            const int64_t i0 = seg * kSeg + (int64_t)(s * kWave + lane) * 8;
+            if (i0 + 8 <= n) {
+                st16(out + i0, st[s * kWave + lane]);
+            } else {
+                for (int j = 0; j < 8 && i0 + j < n; ++j) out[i0 + j] = stage[wave][(s * kWave + lane) * 8 + j];
+            }
+        }
+    }
+}
+
+// ---- softmax backward ---------------------------------------------------------------------
+// o = bf16( (g - sum_row bf16(y*g)) * y ), the row sum accumulated in fp32
+// (operators/softmax_kernels.py:31-35).  One wave per row; rows of up to 64*8*CH
+// elements are held in registers so y and g are read once.
+template <int CH>
+__global__ __launch_bounds__(256) void softmax_bwd_kernel(const uint16_t* __restrict__ y, const uint16_t* __restrict__ g,
+                                                          uint16_t* __restrict__ o, int64_t rows, int n) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t row = blockIdx.x * 4ll + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int64_t base = row * n;
+    u32x4 yv[CH], gv[CH];
+    float acc = 0.0f;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int col = (c * kWave + lane) * 8;
+        yv[c] = u32x4{0, 0, 0, 0};
+        gv[c] = u32x4{0, 0, 0, 0};
+        if (col < n) {
+            yv[c] = ld16(y + base + col);
+            gv[c] = ld16(g + base + col);
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        float yf[8], gf[8];
+        unpack8(yv[c], yf);
+        unpack8(gv[c], gf);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc += rbf(yf[j] * gf[j]);
+    }
+    acc = wave_sum(acc);
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+        const int col = (c * kWave + lane) * 8;
+        if (col < n) {
+            float yf[8], gf[8], of[8];
+            unpack8(yv[c], yf);
+            unpack8(gv[c], gf);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) of[j] = (gf[j] - acc) * yf[j];
+            st16(o + base + col, pack8(of));
+        }
+    }
+}
+
+// any row length / alignment: element-wise accesses, two passes over the row
+__global__ __launch_bounds__(256) void softmax_bwd_generic_kernel(const uint16_t* __restrict__ y,
+                                                                  const uint16_t* __restrict__ g,
+                                                                  uint16_t* __restrict__ o, int64_t rows, int64_t n) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t row = blockIdx.x * 4ll + (threadIdx.x >> 6);
+    if (row >= rows) return;
+    const int64_t base = row * n;
+    float acc = 0.0f;
+    for (int64_t i = lane; i < n; i += kWave) acc += rbf(bf_to_f(y[base + i]) * bf_to_f(g[base + i]));
+    acc = wave_sum(acc);
+    for (int64_t i = lane; i < n; i += kWave)
+        o[base + i] = f_to_bf((bf_to_f(g[base + i]) - acc) * bf_to_f(y[base + i]));
+}
+
+}  // namespace hyc
+
+using namespace hyc;
+
+extern "C" int hyc_hist16(const void* a, int64_t n, uint32_t* hist, void* stream) {
+    if (n < 0 || n >= ((int64_t)1 << 32)) return HYC_ERR_SHAPE;
+    if (!hist || (n > 0 && !a)) return HYC_ERR_NULL;
+    if (n > 0 && !aligned16(a)) return HYC_ERR_ALIGN;
+    hipStream_t st = (hipStream_t)stream;
+    hipLaunchKernelGGL(fill_u32_kernel, dim3(64), dim3(1024), 0, st, hist, (int64_t)65536, 0u);
+    if (n > 0) {
+        int64_t blocks = cdiv(cdiv(n, 8), kHistThreads * 4);
+        if (blocks > 512) blocks = 512;
+        if (blocks < 1) blocks = 1;
+        hipLaunchKernelGGL(hist16_kernel, dim3((unsigned)blocks), dim3(kHistThreads), 0, st, (const uint16_t*)a, n, hist);
+    }
+    return check_launch();
+}
+
+extern "C" int hyc_hist_select(const uint32_t* hist, int64_t kth, float* threshold, void* stream) {
+    if (!hist || !threshold) return HYC_ERR_NULL;
+    if (kth < 1) return HYC_ERR_ARG;
+    hipLaunchKernelGGL(hist_select_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, hist, kth, threshold);
+    return check_launch();
+}
+
+extern "C" int64_t hyc_sparse_num_segments(int64_t n) { return n <= 0 ? 0 : cdiv(n, kSeg); }
+
+extern "C" int hyc_sparse_count(const void* a, int64_t n, const float* threshold, uint32_t* seg_counts,
+                                int64_t* seg_offsets, void* stream) {
+    if (n < 0) return HYC_ERR_SHAPE;
+    if (!seg_offsets || !threshold) return HYC_ERR_NULL;
+    const int64_t nseg = hyc_sparse_num_segments(n);
+    if (nseg > 0 && (!a || !seg_counts)) return HYC_ERR_NULL;
+    if (nseg > 0 && !aligned16(a)) return HYC_ERR_ALIGN;
+    if (cdiv(nseg, 4) > INT32_MAX) return HYC_ERR_SHAPE;
+    hipStream_t st = (hipStream_t)stream;
+    if (nseg > 0)
+        hipLaunchKernelGGL(sparse_count_kernel, dim3((unsigned)cdiv(nseg, 4)), dim3(kSegThreads), 0, st,
+                           (const uint16_t*)a, n, threshold, nseg, seg_counts);
+    hipLaunchKernelGGL(seg_scan_kernel, dim3(1), dim3(1024), 0, st, seg_counts, nseg, seg_offsets);
+    return check_launch();
+}
+
+extern "C" int hyc_sparse_write(const void* a, int64_t n, const float* threshold, const int64_t* seg_offsets,
+                                int64_t* indices, void* values, void* stream) {
+    if (n < 0) return HYC_ERR_SHAPE;
+    const int64_t nseg = hyc_sparse_num_segments(n);
+    if (nseg == 0) return HYC_OK;
+    if (!a || !threshold || !seg_offsets || !indices || !values) return HYC_ERR_NULL;
+    if (!aligned16(a)) return HYC_ERR_ALIGN;
+    hipLaunchKernelGGL(sparse_write_kernel, dim3((unsigned)cdiv(nseg, 4)), dim3(kSegThreads), 0, (hipStream_t)stream,
+                       (const uint16_t*)a, n, threshold, nseg, seg_offsets, indices, (uint16_t*)values);
+    return check_launch();
+}
+
+extern "C" int hyc_sparse_segment_offsets(const int64_t* indices, int64_t nnz, int64_t n, int64_t* seg_offsets,
+                                          void* stream) {
+    if (n < 0 || nnz < 0) return HYC_ERR_SHAPE;
+    if (!seg_offsets || (nnz > 0 && !indices)) return HYC_ERR_NULL;
+    const int64_t nseg = hyc_sparse_num_segments(n);
+    hipLaunchKernelGGL(seg_offsets_kernel, dim3((unsigned)cdiv(nnz + 1, 256)), dim3(256), 0, (hipStream_t)stream,
+                       indices, nnz, nseg, seg_offsets);
+    return check_launch();
+}
+
+extern "C" int hyc_sparse_restore(const int64_t* indices, const void* values, const int64_t* seg_offsets, int64_t n,
+                                  void* out, void* stream) {
+    if (n < 0) return HYC_ERR_SHAPE;
+    const int64_t nseg = hyc_sparse_num_segments(n);
+    if (nseg == 0) return HYC_OK;
+    if (!seg_offsets || !out) return HYC_ERR_NULL;
+    if (!aligned16(out)) return HYC_ERR_ALIGN;
+    hipLaunchKernelGGL(sparse_restore_kernel, dim3((unsigned)cdiv(nseg, 4)), dim3(kSegThreads), 0, (hipStream_t)stream,
+                       indices, (const uint16_t*)values, seg_offsets, nseg, n, (uint16_t*)out);
+    return check_launch();
+}
+
+extern "C" int hyc_softmax_bwd(const void* y, const void* grad_y, void* out, int64_t rows, int64_t n, void* stream) {
+    if (rows < 0 || n < 0) return HYC_ERR_SHAPE;
+    if (rows == 0 || n == 0) return HYC_OK;
+    if (!y || !grad_y || !out) return HYC_ERR_NULL;
+    if (cdiv(rows, 4) > INT32_MAX) return HYC_ERR_SHAPE;
+    const dim3 grid((unsigned)cdiv(rows, 4)), block(256);
+    hipStream_t st = (hipStream_t)stream;
+    const bool vec = (n % 8 == 0) && n <= 4096 && aligned16(y) && aligned16(grad_y) && aligned16(out);
+    const uint16_t* yp = (const uint16_t*)y;
+    const uint16_t* gp = (const uint16_t*)grad_y;
+    uint16_t* op = (uint16_t*)out;
+    if (!vec) hipLaunchKernelGGL(softmax_bwd_generic_kernel, grid, block, 0, st, yp, gp, op, rows, n);
+    else if (n <= 512) hipLaunchKernelGGL(softmax_bwd_kernel<1>, grid, block, 0, st, yp, gp, op, rows, (int)n);
+    else if (n <= 1024) hipLaunchKernelGGL(softmax_bwd_kernel<2>, grid, block, 0, st, yp, gp, op, rows, (int)n);
+    else if (n <= 2048) hipLaunchKernelGGL(softmax_bwd_kernel<4>, grid, block, 0, st, yp, gp, op, rows, (int)n);
+    else hipLaunchKernelGGL(softmax_bwd_kernel<8>, grid, block, 0, st, yp, gp, op, rows, (int)n);
+    return check_launch();
+}

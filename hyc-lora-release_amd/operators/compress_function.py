@@ -83,6 +83,102 @@ def _vec(t: torch.Tensor, n: int, name: str) -> torch.Tensor:
     return t
 
 
+def _require_per_channel(q_method: str) -> None:
+    if q_method == 'per-channel':
+        return
+    if q_method == 'per-tensor':
+        # The reference computes a 0-d step for 'per-tensor' and then fails inside its own
+        # kernel wrapper (s.stride(1) on a 0-d tensor); no layer ever asks for it.
+        raise NotImplementedError("q_method='per-tensor' is not supported; the layers use 'per-channel'")
+    raise ValueError(f"Unsupport Quantize Method: {q_method!r}")
+
+
+def _batch0_stats(x: torch.Tensor):
+    """(stats fp32 [3, N], N): min / max / sum of squares per channel over batch element 0."""
+    _lib.require_gpu(x)
+    if x.dtype != BF16:
+        x = x.to(BF16)
+    a = _Addr(x)
+    if a.N % 32:
+        raise ValueError(f"channel count must be a multiple of 32, got {a.N}")
+    if a.B == 0:
+        raise ValueError("statistics need at least one batch element")
+    stats = torch.empty((3, a.N), device=x.device, dtype=torch.float32)
+    _lib.call("hyc_channel_stats", a.t.data_ptr(), a.M, a.N, a.sm, a.hd, a.sh, stats.data_ptr(), _lib.stream_of(x))
+    return stats, a.N
+
+
+# ---------------------------------------------------------------------------------------
+# statistics (reference: operators/compress_function.py:30-105)
+# ---------------------------------------------------------------------------------------
+def _kth_value(x: torch.Tensor, kth: int) -> torch.Tensor:
+    """Exact kth-smallest (1-based) value of a bf16 tensor as a 0-d fp32 tensor."""
+    _lib.require_gpu(x)
+    n = x.numel()
+    if not 1 <= kth <= n:
+        raise RuntimeError(f"kthvalue(): selected number k out of range: k={kth}, numel={n}")
+    flat = x.reshape(-1)
+    if not flat.is_contiguous() or flat.data_ptr() % 16:
+        flat = flat.clone(memory_format=torch.contiguous_format)
+    hist = torch.empty(65536, device=x.device, dtype=torch.int32)
+    thr = torch.empty((), device=x.device, dtype=torch.float32)
+    st = _lib.stream_of(x)
+    _lib.call("hyc_hist16", flat.data_ptr(), n, hist.data_ptr(), st)
+    _lib.call("hyc_hist_select", hist.data_ptr(), kth, thr.data_ptr(), st)
+    return thr
+
+
+def get_statistics_softmax(x: torch.Tensor, outlier_ratio: float):
+    """Keep-threshold of an attention map: the int(numel*(1-ratio))-th smallest value,
+    0-d fp32.  Reference :30-32 (torch.kthvalue on an fp32 copy)."""
+    if x.dtype != BF16:
+        x = x.to(BF16)
+    return _kth_value(x, int(x.numel() * (1 - outlier_ratio)))
+
+
+def get_statistics_outlier(x: torch.Tensor, outlier_ratio: float):
+    """Same order statistic on |x|.  Reference :34-36 (not called by any layer)."""
+    return _kth_value(x.to(BF16).abs(), int(x.numel() * (1 - outlier_ratio)))
+
+
+def get_statistics_only_quant(x: torch.Tensor, q_bit: int = 8, q_method: str = 'per-tensor'):
+    """Per-channel step bf16 [1, N] from batch element 0.  Reference :45-59."""
+    _require_per_channel(q_method)
+    _check_bits(q_bit)
+    stats, n = _batch0_stats(x)
+    scale = torch.empty((1, n), device=x.device, dtype=BF16)
+    _lib.call("hyc_channel_select", stats.data_ptr(), n, 0, q_bit, 0, None, scale.data_ptr(), None,
+              _lib.stream_of(x))
+    return scale
+
+
+def get_statistics_only_quant_zero_point(x: torch.Tensor, q_bit: int = 8, q_method: str = 'per-tensor'):
+    """(step bf16 [1, N], zero point int8 [1, N]).  Reference :62-77."""
+    _require_per_channel(q_method)
+    _check_bits(q_bit)
+    stats, n = _batch0_stats(x)
+    scale = torch.empty((1, n), device=x.device, dtype=BF16)
+    zp = torch.empty((1, n), device=x.device, dtype=torch.int8)
+    _lib.call("hyc_channel_select", stats.data_ptr(), n, 0, q_bit, 0, None, scale.data_ptr(), zp.data_ptr(),
+              _lib.stream_of(x))
+    return scale, zp
+
+
+def get_statistics_channel_base(x: torch.Tensor, outlier_ratio: float, q_bit: int = 8, q_method: str = 'per-tensor'):
+    """(outlier channel indices int64 [k], step bf16 [1, N]) with k = int(N * ratio); the
+    step is that of the tensor with the outlier channels zeroed.  Reference :80-105.
+    No clone of x is made: the statistics of the zeroed tensor follow from those of x."""
+    _require_per_channel(q_method)
+    _check_bits(q_bit)
+    stats, n = _batch0_stats(x)
+    k = int(n * outlier_ratio)
+    idx = torch.empty((k,), device=x.device, dtype=torch.int64)
+    scale = torch.empty((1, n), device=x.device, dtype=BF16)
+    _lib.call("hyc_channel_select", stats.data_ptr(), n, k, q_bit, 1, idx.data_ptr() if k else None,
+              scale.data_ptr(), None, _lib.stream_of(x))
+    return idx, scale
+
+
 def _check_bits(quantize_bit: int) -> int:
     if quantize_bit not in (2, 4, 8):
         raise ValueError(f"quantize_bit must be 2, 4 or 8, got {quantize_bit}")
@@ -178,3 +274,108 @@ def compression_quantization_with_zero_point(x, s, z, quantize_bit=8, dtype=BF16
 def decompression_dequantization_with_zero_point(q, s, z, quantize_bit=8, is_head=False, num_heads=1, dtype=BF16):
     """Reference :278-306."""
     return _dequantize(q, s, z, None, None, quantize_bit, is_head, num_heads, dtype)
+
+
+# ---------------------------------------------------------------------------------------
+# attention-map compression (reference: operators/compress_function.py:309-317)
+# ---------------------------------------------------------------------------------------
+def _threshold_tensor(outlier, device) -> torch.Tensor:
+    if torch.is_tensor(outlier):
+        return outlier.to(device=device, dtype=torch.float32).reshape(())
+    return torch.tensor(float(outlier), device=device, dtype=torch.float32)
+
+
+def compress_attention_map(x: torch.Tensor, outlier):
+    """Kept entries of the flattened map: (indices int64 [nnz] ascending, values bf16 [nnz],
+    seg_offsets int64 [nseg + 1]).  An entry is kept when x > outlier (compared in bf16, as
+    torch does) and x != 0.  seg_offsets lets restore_attention_map skip the index search."""
+    _lib.require_gpu(x)
+    if x.dtype != BF16:
+        x = x.to(BF16)
+    flat = x.reshape(-1)
+    if not flat.is_contiguous() or flat.data_ptr() % 16:
+        flat = flat.clone(memory_format=torch.contiguous_format)
+    n = flat.numel()
+    thr = _threshold_tensor(outlier, x.device)
+    nseg = _lib.lib().hyc_sparse_num_segments(n)
+    counts = torch.empty(max(nseg, 1), device=x.device, dtype=torch.int32)
+    offsets = torch.empty(nseg + 1, device=x.device, dtype=torch.int64)
+    st = _lib.stream_of(x)
+    _lib.call("hyc_sparse_count", flat.data_ptr(), n, thr.data_ptr(), counts.data_ptr(), offsets.data_ptr(), st)
+    nnz = int(offsets[-1].item())      # the one host sync; to_sparse() has the same one
+    idx = torch.empty(nnz, device=x.device, dtype=torch.int64)
+    val = torch.empty(nnz, device=x.device, dtype=BF16)
+    if nnz:
+        _lib.call("hyc_sparse_write", flat.data_ptr(), n, thr.data_ptr(), offsets.data_ptr(), idx.data_ptr(),
+                  val.data_ptr(), st)
+    return idx, val, offsets
+
+
+def restore_attention_map(idx, val, seg_offsets, shape):
+    """Dense bf16 tensor of `shape`: zeros with val[i] at flat position idx[i]."""
+    _lib.require_gpu(idx, val)
+    n = 1
+    for d in shape:
+        n *= int(d)
+    idx = idx.reshape(-1).contiguous()
+    val = val.to(BF16).reshape(-1).contiguous()
+    st = _lib.stream_of(val)
+    if seg_offsets is None:
+        nseg = _lib.lib().hyc_sparse_num_segments(n)
+        seg_offsets = torch.empty(nseg + 1, device=val.device, dtype=torch.int64)
+        _lib.call("hyc_sparse_segment_offsets", idx.data_ptr(), idx.numel(), n, seg_offsets.data_ptr(), st)
+    out = torch.empty(n, device=val.device, dtype=BF16)
+    _lib.call("hyc_sparse_restore", idx.data_ptr(), val.data_ptr(), seg_offsets.data_ptr(), n, out.data_ptr(), st)
+    return out.reshape(tuple(shape))
+
+
+def compression_softmax(x: torch.Tensor, outlier):
+    """Sparse COO tensor of the flattened map, like (x * (x > outlier)).flatten().to_sparse().
+    Reference :309-313."""
+    idx, val, _ = compress_attention_map(x, outlier)
+    return torch.sparse_coo_tensor(idx.unsqueeze(0), val, (x.numel(),), is_coalesced=True)
+
+
+def decompression_softmax(x_sparse: torch.Tensor):
+    """Dense 1-D tensor, like x_sparse.to_dense().  Reference :316-317."""
+    if not x_sparse.is_coalesced():
+        x_sparse = x_sparse.coalesce()
+    return restore_attention_map(x_sparse.indices()[0], x_sparse.values(), None, x_sparse.shape)
+
+
+# ---------------------------------------------------------------------------------------
+# statistics + compress in one call (reference: operators/compress_function.py:346-368)
+# ---------------------------------------------------------------------------------------
+def compression_pack_channel_base(x, o_ratio, q_bit, q_method, it_num, it_num_thd, static_value):
+    """Outlier-channel extraction + quantisation; calibrates while it_num < it_num_thd."""
+    if it_num < it_num_thd:
+        o_channel_idx, scale = get_statistics_channel_base(x, o_ratio, q_bit, q_method)
+    else:
+        o_channel_idx, scale = static_value['outlier_channel_index'], static_value['scale']
+    o, q = outlier_subtraction_fuse_compression_quantization(x, scale, o_channel_idx, q_bit)
+    return o, q, o_channel_idx, scale
+
+
+def compression_pack_quant_base(x, q_bit, q_method, it_num, it_num_thd, static_value):
+    if it_num < it_num_thd:
+        scale = get_statistics_only_quant(x, q_bit, q_method)
+    else:
+        scale = static_value['scale']
+    return compression_quantization(x, scale, q_bit), scale
+
+
+def compression_pack_quant_zp_base(x, q_bit, q_method, it_num, it_num_thd, static_value):
+    if it_num < it_num_thd:
+        scale, zero_point = get_statistics_only_quant_zero_point(x, q_bit, q_method)
+    else:
+        scale, zero_point = static_value['scale'], static_value['zero_point']
+    return compression_quantization_with_zero_point(x, scale, zero_point, q_bit), scale, zero_point
+
+
+def compression_pack_softmax_base(x, o_ratio, it_num, it_num_thd, static_value):
+    """Attention-map compression -> (sparse COO tensor, threshold).  Reference :371-379."""
+    if it_num < it_num_thd:
+        outlier = get_statistics_softmax(x, o_ratio)
+    else:
+        outlier = static_value['outlier']
+    return compression_softmax(x, outlier), outlier

@@ -41,7 +41,8 @@ int hyc_abi_version(void);
 
 /* Launch-shape knobs for benchmarking (process-wide, not thread-safe against concurrent
  * launches).  Keys: "quant_rows_per_wave" (rows each wave walks in hyc_quant_pack /
- * hyc_unpack_dequant, default 16).  Unknown key or bad value: HYC_ERR_ARG.  No
+ * hyc_unpack_dequant, default 16), "fuse_rows_per_wave" (same for the fused LoRA-SiLU
+ * kernels, multiple of 16, default 64).  Unknown key or bad value: HYC_ERR_ARG.  No
  * counterpart in the reference (its launch shapes come from triton.autotune). */
 int hyc_set_tuning(const char *key, int value);
 
@@ -94,6 +95,172 @@ int hyc_unpack_dequant(const void *q, const void *scale, const void *zero_point,
                        int64_t B, int64_t M, int64_t N,
                        int64_t stride_b, int64_t stride_m, int64_t head_dim, int64_t stride_h,
                        int q_bit, void *stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Calibration statistics, step 1: per-channel minimum, maximum and sum of squares over the
+ * M rows of ONE batch element (the reference calibrates on batch element 0 only).
+ *
+ * Replaces the torch reductions in get_statistics_only_quant (operators/compress_function.py:50-54),
+ * get_statistics_only_quant_zero_point (:67-72) and get_statistics_channel_base (:86,93-97),
+ * together with the x.clone() the latter starts with (:81).
+ *
+ *   x      bf16 [M, N] of batch element 0, element (m, c) at
+ *          x + m*stride_m + (c / head_dim)*stride_h + (c % head_dim)
+ *   stats  fp32 [3, N] output: row 0 = min, row 1 = max (NaN propagates as in torch),
+ *          row 2 = sum of squares (fp32 accumulation in a fixed order).
+ */
+int hyc_channel_stats(const void *x, int64_t M, int64_t N, int64_t stride_m, int64_t head_dim,
+                      int64_t stride_h, float *stats, void *stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Calibration statistics, step 2: outlier channels and per-channel step / zero point.
+ *
+ * Replaces torch.topk + the bf16 scalar arithmetic of get_statistics_channel_base
+ * (operators/compress_function.py:86-105), get_statistics_only_quant (:50-59) and
+ * get_statistics_only_quant_zero_point (:67-77).
+ *
+ *   stats       fp32 [3, N] from hyc_channel_stats.
+ *   k           number of outlier channels (0 = none).  Chosen by bf16 norm
+ *               bf16(sqrt(sum of squares)) descending, ties by channel index ascending —
+ *               torch.topk leaves tie order unspecified, this rule is fixed.  N <= 32768
+ *               when k > 0.
+ *   outlier_idx int64 [k] output, in that order (NULL when k = 0).
+ *   scale       bf16 [N] output: bf16( bf16(max - min) / (2^q_bit - 1) ), with min = max = 0
+ *               for the chosen channels; if add_eps != 0 a zero step becomes bf16(0 + 1e-3)
+ *               (compress_function.py:104).
+ *   zero_point  int8 [N] output or NULL: -round_half_even(min / step) - 2^(q_bit-1), every
+ *               operation rounded to bf16, then converted like a C cast (:72,77).
+ */
+int hyc_channel_select(const float *stats, int64_t N, int64_t k, int q_bit, int add_eps,
+                       int64_t *outlier_idx, void *scale, int8_t *zero_point, void *stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Attention-map compression: exact k-th value.
+ *
+ * Replaces torch.kthvalue(x.float().flatten(), k) in get_statistics_softmax
+ * (operators/compress_function.py:30-32) without the fp32 copy and without sorting: a
+ * bf16 tensor has at most 65536 distinct values.
+ *
+ *   hyc_hist16      a bf16 [n] (n < 2^32, 16-byte aligned) -> hist uint32 [65536], cleared
+ *                   here first.  Bin = order-preserving key of the bit pattern (negative
+ *                   values first, NaN last).
+ *   hyc_hist_select kth is 1-based, 1 <= kth <= n (the caller checks the upper bound);
+ *                   *threshold (fp32, device) receives the kth-smallest value.
+ */
+int hyc_hist16(const void *a, int64_t n, uint32_t *hist, void *stream);
+int hyc_hist_select(const uint32_t *hist, int64_t kth, float *threshold, void *stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Attention-map compression: ordered compaction and dense restore.
+ *
+ * Replaces mask-multiply + flatten().to_sparse() in compression_softmax
+ * (operators/compress_function.py:309-313) and to_dense() in decompression_softmax
+ * (:316-317; models/llama/fused_llama_layer_intra_inter_full_fuse.py:414-415).
+ *
+ * An element is kept when a > bf16(threshold) and a != 0 (torch compares in bf16 and
+ * to_sparse drops zeros).  Output order is ascending flat index, as to_sparse gives.
+ * The flattened tensor is processed in segments of 4096 elements;
+ * hyc_sparse_num_segments(n) = ceil(n / 4096).
+ *
+ *   hyc_sparse_count   a bf16 [n]; threshold fp32 scalar ON THE DEVICE;
+ *                      seg_counts uint32 [nseg] scratch; seg_offsets int64 [nseg + 1] output:
+ *                      entries kept before each segment, last element = total kept (nnz).
+ *                      The caller reads nnz back to size the outputs, as to_sparse itself does.
+ *   hyc_sparse_write   same a / threshold / seg_offsets; indices int64 [nnz], values bf16 [nnz].
+ *   hyc_sparse_segment_offsets  rebuilds seg_offsets from an ascending index list (for sparse
+ *                      tensors that did not come from hyc_sparse_count).
+ *   hyc_sparse_restore out bf16 [n] (16-byte aligned): zeros, with values[i] at indices[i].
+ */
+int64_t hyc_sparse_num_segments(int64_t n);
+int hyc_sparse_count(const void *a, int64_t n, const float *threshold, uint32_t *seg_counts,
+                     int64_t *seg_offsets, void *stream);
+int hyc_sparse_write(const void *a, int64_t n, const float *threshold, const int64_t *seg_offsets,
+                     int64_t *indices, void *values, void *stream);
+int hyc_sparse_segment_offsets(const int64_t *indices, int64_t nnz, int64_t n, int64_t *seg_offsets,
+                               void *stream);
+int hyc_sparse_restore(const int64_t *indices, const void *values, const int64_t *seg_offsets,
+                       int64_t n, void *out, void *stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Softmax backward on a dense map: out = bf16((g - sum_row bf16(y*g)) * y), row sums in fp32.
+ *
+ * Replaces softmax_backward_kernel (operators/softmax_kernels.py:7-38).
+ *   y, grad_y, out   bf16 [rows, n], contiguous.
+ */
+int hyc_softmax_bwd(const void *y, const void *grad_y, void *out, int64_t rows, int64_t n, void *stream);
+
+/* ---------------------------------------------------------------------------------------
+ * RMSNorm forward: rstd = 1/sqrt(mean(x^2) + eps) in fp32, y = bf16(x * rstd * weight).
+ *
+ * Replaces _rms_norm_fwd_fused (operators/rmsnorm_kernels.py:10-54).
+ *   x, y    bf16 [rows, N] contiguous; N % 8 == 0, N <= 65536.
+ *   weight  [N], bf16 or fp32 (weight_is_fp32).   rstd  fp32 [rows] output.
+ */
+int hyc_rmsnorm_fwd(const void *x, const void *weight, int weight_is_fp32, void *y, float *rstd,
+                    int64_t rows, int64_t N, float eps, void *stream);
+
+/* ---------------------------------------------------------------------------------------
+ * RMSNorm backward: dx = (w*dy - (x^*c1 + c2)) * rstd with x^ = x*rstd, c1 = mean(x^*w*dy),
+ * c2 = mean(w*dy) — the reference keeps LayerNorm's c2 term and so does this; optionally
+ * dw = sum_rows dy*x^.
+ *
+ * Replaces _rms_norm_bwd_dx_fused (operators/rmsnorm_kernels.py:58-113) and, when dw is
+ * requested, _rms_norm_bwd_dwdb (operators/rmsnorm_updatable_kernels.py:117-137) — with a
+ * deterministic two-stage fp32 reduction instead of the spin-lock accumulation.
+ *   dy, x, dx  bf16 [rows, N] contiguous; N % 8 == 0, N <= 8192.
+ *   dw         [N] in the weight's dtype, or NULL.  When given, workspace must hold
+ *              hyc_rmsnorm_bwd_workspace(rows, N) bytes (fp32 partial rows).
+ */
+int64_t hyc_rmsnorm_bwd_workspace(int64_t rows, int64_t N);
+int hyc_rmsnorm_bwd(const void *dy, const void *x, const void *weight, int weight_is_fp32,
+                    const float *rstd, void *dx, void *dw, void *workspace, int64_t workspace_bytes,
+                    int64_t rows, int64_t N, void *stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Element-wise operators on n contiguous bf16 elements (16-byte aligned pointers).
+ *
+ *   hyc_silu_bwd  out = g * (sig * (1 + x*(1 - sig))), sig = bf16(sigmoid(x)), bf16 after
+ *                 every operation.  Replaces silu_backward_kernel (operators/silu_kernels.py:12-45).
+ *   hyc_silu_mul  out = (sig(x1) * x1) * x2.  Replaces triton_silu_hadamard_kernel (:73-106).
+ *   hyc_gelu_bwd  out = d/dx[tanh-GELU](x) * g, evaluated in fp32.  Replaces
+ *                 gelu_backward_kernel (operators/gelu_kernels.py:19-58).
+ */
+int hyc_silu_bwd(const void *x, const void *g, void *out, int64_t n, void *stream);
+int hyc_silu_mul(const void *x1, const void *x2, void *out, int64_t n, void *stream);
+int hyc_gelu_bwd(const void *x, const void *g, void *out, int64_t n, void *stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Fused LoRA-SiLU-Hadamard forward: quantises the two frozen-weight outputs for backward
+ * while producing the gated product.
+ *     q1 = pack(code(x1; s1)),  q2 = pack(code(x2; s2))           (same rule as hyc_quant_pack)
+ *     y1 = x1 + bf16(xa1 . b1); y2 = x2 + bf16(xa2 . b2)          (MFMA, fp32 accumulation)
+ *     o  = (y1 * bf16(sigmoid(y1))) * y2                          (bf16 after every operation)
+ *
+ * Replaces triton_fuse_silu_forward_kernel
+ * (operators/triton_fuse_lora_silu_hadamard_forward_kernels.py:28-149).
+ *   xa1, xa2 bf16 [T, R] contiguous (x @ lora_A);   b1, b2 bf16 [R, N] contiguous (lora_B);
+ *   x1, x2   bf16 [T, N] contiguous;                s1, s2 bf16 [N];
+ *   q1, q2   uint8 [T, N*q_bit/8];                  o      bf16 [T, N].
+ *   R: multiple of 4, 4..64 (the reference needs a power of two >= 16); N % 32 == 0; any T.
+ */
+int hyc_lora_silu_mul_fwd(const void *xa1, const void *b1, const void *x1, const void *s1,
+                          const void *xa2, const void *b2, const void *x2, const void *s2,
+                          void *q1, void *q2, void *o, int64_t T, int64_t N, int64_t R, int q_bit,
+                          void *stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Fused LoRA-SiLU-Hadamard backward: dequantises q1, q2, recomputes y1, y2 and the gated
+ * product o, and produces
+ *     grad_gate = (g * y2) * (sig * (1 + y1*(1 - sig))),   grad_up = g * (y1 * sig).
+ *
+ * Replaces triton_fuse_silu_backward_kernel
+ * (operators/triton_fuse_lora_silu_hadamard_backward_kernels.py:28-149).
+ *   grad_o, o, grad_gate, grad_up  bf16 [T, N] contiguous; the rest as in the forward.
+ */
+int hyc_lora_silu_mul_bwd(const void *xa1, const void *b1, const void *q1, const void *s1,
+                          const void *xa2, const void *b2, const void *q2, const void *s2,
+                          const void *grad_o, void *o, void *grad_gate, void *grad_up,
+                          int64_t T, int64_t N, int64_t R, int q_bit, void *stream);
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,126 @@
+"""GPU checks of the element-wise backward operators and RMSNorm against the CPU oracle
+(bf16 tolerance: max rel err <= 1e-2, cosine >= 0.9999) and against torch.autograd of the
+fp32 composite."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from helpers import BF16, assert_close_bf16
+from oracle import hyc_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import hyclora_amd  # noqa: F401
+    from hyclora_amd.operators import gelu_kernels, rmsnorm_kernels, rmsnorm_updatable_kernels, silu_kernels
+
+    class Ops:
+        silu = silu_kernels
+        gelu = gelu_kernels
+        norm = rmsnorm_kernels
+        normu = rmsnorm_updatable_kernels
+    return Ops
+
+
+def _pair(shape, seed, scale=2.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(BF16), torch.randn(*shape, generator=g).to(BF16)
+
+
+SHAPES = [(2, 64, 11008), (1, 7, 96), (3, 5, 41), (1, 1, 8)]
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+def test_silu_backward(ops, dev, shape):
+    x, g = _pair(shape, 1)
+    o = ops.silu.silu_backward(x.to(dev), g.to(dev))
+    assert_close_bf16(o, O.silu_bwd(x, g), what="silu_backward vs oracle")
+    xf = x.float().requires_grad_()
+    F.silu(xf).backward(g.float())
+    # five bf16 roundings in a row (2^-8 each) separate the reference's expression from fp32 autograd
+    assert_close_bf16(o, xf.grad, rel_tol=2e-2, what="silu_backward vs autograd")
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+def test_silu_hadamard(ops, dev, shape):
+    x1, x2 = _pair(shape, 2)
+    o = ops.silu.silu_hadamard(x1.to(dev), x2.to(dev))
+    assert_close_bf16(o, O.silu_mul(x1, x2), what="silu_hadamard vs oracle")
+    assert_close_bf16(o, F.silu(x1.float()) * x2.float(), what="silu_hadamard vs torch")
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+def test_gelu_backward(ops, dev, shape):
+    x, g = _pair(shape, 3)
+    o = ops.gelu.gelu_backward(x.to(dev), g.to(dev))
+    assert_close_bf16(o, O.gelu_bwd(x, g), what="gelu_backward vs oracle")
+    xf = x.float().requires_grad_()
+    F.gelu(xf, approximate="tanh").backward(g.float())
+    assert_close_bf16(o, xf.grad, what="gelu_backward vs autograd of tanh-GELU")
+
+
+def test_elementwise_extremes(ops, dev):
+    # saturated sigmoid / tanh must give the limits 0 and 1, not NaN.  (The GELU formula itself
+    # overflows to inf*0 beyond |x| ~ 1e19, in the reference as well, so it is probed up to 1e4.)
+    for top, fn, ref in ((3e38, ops.silu.silu_backward, O.silu_bwd), (1e4, ops.gelu.gelu_backward, O.gelu_bwd)):
+        x = torch.tensor([0.0, -0.0, 50.0, -50.0, 1e4, -1e4, top, -top] * 2, dtype=BF16).reshape(1, 2, 8)
+        g = torch.ones_like(x)
+        o = fn(x.to(dev), g.to(dev)).cpu().float()
+        r = ref(x, g).float()
+        assert torch.isfinite(o).all() and torch.allclose(o, r, atol=1e-2, rtol=1e-2)
+
+
+@pytest.mark.parametrize("n", [4096, 512, 96, 1024, 8192, 16384, 2048 + 64])
+@pytest.mark.parametrize("wdtype", [BF16, torch.float32])
+def test_rmsnorm_forward(ops, dev, n, wdtype):
+    g = torch.Generator().manual_seed(n)
+    x = (torch.randn(2, 33, n, generator=g) * 3).to(BF16)
+    w = (1 + 0.1 * torch.randn(n, generator=g)).to(wdtype)
+    y, mean, rstd, block, warps = ops.norm.rmsnorm_forward(x.to(dev), w.to(dev), 1e-5)
+    y_ref, rstd_ref = O.rmsnorm_fwd(x, w, 1e-5)
+    assert y.shape == x.shape and y.dtype == BF16 and rstd.shape == (66,) and rstd.dtype == torch.float32
+    assert block >= n and 1 <= warps <= 8 and mean.shape == (66,)
+    assert torch.allclose(rstd.cpu(), rstd_ref, rtol=1e-5, atol=0)
+    assert_close_bf16(y, y_ref, what="rmsnorm_forward vs oracle")
+    # independent: the textbook formula in fp64
+    xd = x.double()
+    ref = xd / torch.sqrt((xd * xd).mean(-1, keepdim=True) + 1e-5) * w.double()
+    assert_close_bf16(y, ref, what="rmsnorm_forward vs fp64 formula")
+
+
+@pytest.mark.parametrize("n", [4096, 512, 96, 1024, 8192])
+@pytest.mark.parametrize("rows", [(2, 33), (1, 1), (4, 300)])
+def test_rmsnorm_backward(ops, dev, n, rows):
+    g = torch.Generator().manual_seed(n + rows[1])
+    x = (torch.randn(*rows, n, generator=g) * 2).to(BF16)
+    dy = torch.randn(*rows, n, generator=g).to(BF16)
+    w = (1 + 0.1 * torch.randn(n, generator=g)).to(BF16)
+    xg, dyg, wg = x.to(dev), dy.to(dev), w.to(dev)
+    _, mean, rstd, block, warps = ops.norm.rmsnorm_forward(xg, wg, 1e-5)
+    dx, none = ops.norm.rmsnorm_backward(dyg, xg, wg, mean, rstd, True, 1e-5, warps, block)
+    assert none is None
+    dx_ref, dw_ref = O.rmsnorm_bwd(dy, x, w, rstd.cpu())
+    assert_close_bf16(dx, dx_ref, what="rmsnorm_backward dx vs oracle")
+    dx2, dw = ops.normu.rmsnorm_backward(dyg, xg, wg, mean, rstd, 1e-5, warps, block)
+    assert torch.equal(dx2, dx)
+    assert dw.dtype == w.dtype and dw.shape == (n,)
+    assert_close_bf16(dw, dw_ref, what="rmsnorm_backward dw vs oracle")
+    assert ops.norm.rmsnorm_backward(dyg, xg, wg, mean, rstd, False, 1e-5, warps, block) == (None, None)
+    # independent check of dw and of dx's x^-dependent part: autograd of true RMSNorm, to
+    # which the reference formula adds only the -mean(w*dy)*rstd term
+    xf = x.double().requires_grad_()
+    wf = w.double().requires_grad_()
+    yf = xf / torch.sqrt((xf * xf).mean(-1, keepdim=True) + 1e-5) * wf
+    yf.backward(dy.double())
+    assert_close_bf16(dw, wf.grad, what="dw vs autograd")
+    c2 = (w.double() * dy.double()).mean(-1, keepdim=True) * rstd.cpu().double().reshape(*rows, 1)
+    assert_close_bf16(dx, xf.grad - c2, what="dx vs autograd minus the LayerNorm mean term")
+
+
+def test_rmsnorm_errors(ops, dev):
+    with pytest.raises(RuntimeError):
+        ops.norm.rmsnorm_forward(torch.zeros(1, 1, 32776, dtype=BF16, device=dev), torch.ones(32776, dtype=BF16, device=dev), 1e-5)
+    with pytest.raises(ValueError):
+        ops.norm.rmsnorm_forward(torch.zeros(1, 1, 100, dtype=BF16, device=dev), torch.ones(100, dtype=BF16, device=dev), 1e-5)

@@ -1,0 +1,152 @@
+"""GPU parity of the attention-map path: exact threshold (k-th value), ordered compaction,
+dense restore and softmax backward, against the CPU oracle / torch library routines."""
+import pytest
+import torch
+
+from helpers import BF16, assert_close_bf16, same_bits
+from oracle import hyc_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def cf():
+    import hyclora_amd  # noqa: F401
+    from hyclora_amd.operators import compress_function
+    return compress_function
+
+
+@pytest.fixture(scope="module")
+def sk():
+    import hyclora_amd  # noqa: F401
+    from hyclora_amd.operators import softmax_kernels
+    return softmax_kernels
+
+
+def attention_map(seed, shape=(2, 4, 128, 128), causal=True):
+    """BASELINE configuration 3 in small: softmax of N(0,1)*8/sqrt(128) logits with a causal mask."""
+    g = torch.Generator().manual_seed(seed)
+    b, h, n, _ = shape
+    s = torch.randn(*shape, generator=g) * 8 / 128 ** 0.5
+    if causal:
+        s = s + torch.full((n, n), float("-inf")).triu(1)
+    return torch.softmax(s, dim=-1, dtype=torch.float32).to(BF16)
+
+
+@pytest.mark.parametrize("shape", [(2, 4, 128, 128), (1, 2, 100, 100), (1, 1, 8, 8), (2, 2, 256, 256)])
+@pytest.mark.parametrize("ratio", [0.05, 0.5, 0.001])
+def test_threshold_is_exact_order_statistic(cf, dev, shape, ratio):
+    a = attention_map(seed=shape[2], shape=shape)
+    thr = cf.get_statistics_softmax(a.to(dev), ratio)
+    assert thr.dtype == torch.float32 and thr.dim() == 0
+    assert thr.item() == O.softmax_threshold(a, ratio).item()
+    # independent of kthvalue: the value at that rank of a full sort
+    k = int(a.numel() * (1 - ratio))
+    assert thr.item() == torch.sort(a.float().flatten()).values[k - 1].item()
+
+
+def test_threshold_general_values(cf, dev):
+    # negative values, values >= 2 (outside the LDS-binned range), -0, inf
+    g = torch.Generator().manual_seed(0)
+    x = (torch.randn(3, 1000, generator=g) * 5).to(BF16)
+    x[0, :5] = torch.tensor([float("inf"), -float("inf"), -0.0, 0.0, 300.0]).to(BF16)
+    for k in (1, 2, 17, 1500, 2999, 3000):
+        got = cf._kth_value(x.to(dev), k).item()
+        assert got == torch.kthvalue(x.float().flatten(), k).values.item(), k
+    with pytest.raises(RuntimeError):
+        cf._kth_value(x.to(dev), 0)
+    with pytest.raises(RuntimeError):
+        cf._kth_value(x.to(dev), 3001)
+
+
+@pytest.mark.parametrize("shape", [(2, 4, 128, 128), (1, 2, 100, 100), (1, 1, 8, 8), (1, 3, 77, 77)])
+def test_compaction_and_restore(cf, dev, shape):
+    a = attention_map(seed=5, shape=shape)
+    thr = O.softmax_threshold(a, 0.05)
+    idx_ref, val_ref = O.softmax_compress(a, thr)
+    ag = a.to(dev)
+    idx, val, seg = cf.compress_attention_map(ag, thr.to(dev))
+    assert idx.dtype == torch.int64 and torch.equal(idx.cpu(), idx_ref)
+    assert same_bits(val.cpu(), val_ref)
+    dense_ref = O.softmax_restore(idx_ref, val_ref, a.shape)
+    assert same_bits(cf.restore_attention_map(idx, val, seg, a.shape).cpu(), dense_ref)
+    assert same_bits(cf.restore_attention_map(idx, val, None, a.shape).cpu(), dense_ref)
+    # reference-shaped API: a sparse COO tensor of the flattened map, and to_dense()
+    sp = cf.compression_softmax(ag, thr.to(dev))
+    ref_sp = (a * (a > thr)).flatten().to_sparse()
+    assert sp.layout == torch.sparse_coo and sp.shape == ref_sp.shape
+    assert torch.equal(sp.indices().cpu(), ref_sp.indices()) and same_bits(sp.values().cpu(), ref_sp.values())
+    assert same_bits(cf.decompression_softmax(sp).cpu(), ref_sp.to_dense())
+    assert same_bits(sp.to_dense().cpu(), ref_sp.to_dense())
+    # a sparse tensor that torch made restores through the same kernel
+    assert same_bits(cf.decompression_softmax(ref_sp.to(dev)).cpu(), ref_sp.to_dense())
+
+
+def test_threshold_is_compared_in_bf16_and_zeros_are_dropped(cf, dev):
+    a = torch.tensor([1.0078125, 1.0, 0.0, -0.0, 0.5, float("nan"), 1.015625, 2.0] * 8, dtype=BF16)
+    thr = torch.tensor(1.0058, dtype=torch.float32)        # rounds to bf16 1.0078125
+    idx_ref, val_ref = O.softmax_compress(a, thr)
+    idx, val, _ = cf.compress_attention_map(a.to(dev), thr.to(dev))
+    assert torch.equal(idx.cpu(), idx_ref) and same_bits(val.cpu(), val_ref)
+    assert idx_ref.numel() == 16                            # only 1.015625 and 2.0
+    # negative threshold: zeros pass the comparison but to_sparse drops them
+    thr = torch.tensor(-1.0)
+    idx_ref, val_ref = O.softmax_compress(a, thr)
+    idx, val, _ = cf.compress_attention_map(a.to(dev), -1.0)
+    assert torch.equal(idx.cpu(), idx_ref) and same_bits(val.cpu(), val_ref)
+    # nothing kept / everything kept
+    idx, val, seg = cf.compress_attention_map(a.to(dev), 1e9)
+    assert idx.numel() == 0 and (cf.restore_attention_map(idx, val, seg, a.shape) == 0).all()
+
+
+def test_pack_softmax_base_dispatch(cf, dev):
+    a = attention_map(seed=9).to(dev)
+    sp, thr = cf.compression_pack_softmax_base(a, 0.05, 0, 5, {'outlier': None})
+    sp2, thr2 = cf.compression_pack_softmax_base(a, 0.05, 5, 5, {'outlier': thr})
+    assert thr2 is thr and torch.equal(sp.indices(), sp2.indices())
+    nnz = sp.values().numel()
+    assert nnz <= int(a.numel() * 0.05) + 1
+
+
+@pytest.mark.parametrize("shape", [(2, 4, 128, 128), (1, 2, 100, 100), (1, 1, 1024, 1024), (1, 1, 8, 2048),
+                                   (1, 1, 4, 4096), (1, 1, 3, 8192), (1, 2, 5, 36)])
+def test_softmax_backward(sk, dev, shape):
+    g = torch.Generator().manual_seed(shape[-1])
+    y = torch.softmax(torch.randn(*shape, generator=g), dim=-1).to(BF16)
+    gr = torch.randn(*shape, generator=g).to(BF16)
+    o = sk.softmax_backward(y.to(dev), gr.to(dev))
+    assert o.dtype == BF16 and o.shape == y.shape
+    assert_close_bf16(o, O.softmax_bwd(y, gr), what="softmax_backward vs oracle")
+    # independent: autograd of softmax in fp64 at the same y
+    yf = y.double()
+    ref = (gr.double() - (yf * gr.double()).sum(-1, keepdim=True)) * yf
+    assert_close_bf16(o, ref, what="softmax_backward vs closed form")
+
+
+def test_full_size_config3_properties(cf, sk, dev):
+    # BASELINE configuration 3 at full size: [4,32,1024,1024], ratio 0.05
+    g = torch.Generator(device=dev).manual_seed(1)
+    s = torch.randn(4, 32, 1024, 1024, generator=g, device=dev, dtype=torch.float32) * (8 / 128 ** 0.5)
+    s += torch.full((1024, 1024), float("-inf"), device=dev).triu(1)
+    a = torch.softmax(s, dim=-1).to(BF16)
+    del s
+    n = a.numel()
+    k = int(n * (1 - 0.05))
+    assert k == 127506841
+    thr = cf.get_statistics_softmax(a, 0.05)
+    flat = a.flatten()
+    # rank property of an exact k-th value: #(< thr) < k <= #(<= thr)
+    below = int((flat < thr.to(BF16)).sum().item())
+    upto = int((flat <= thr.to(BF16)).sum().item())
+    assert below < k <= upto
+    idx, val, seg = cf.compress_attention_map(a, thr)
+    assert idx.numel() == n - upto and idx.numel() <= 6710887
+    assert bool((idx[1:] > idx[:-1]).all())
+    assert torch.equal(flat[idx], val)
+    dense = cf.restore_attention_map(idx, val, seg, a.shape)
+    assert torch.equal(dense, torch.where(a > thr.to(BF16), a, torch.zeros_like(a)))
+    grad = torch.randn(a.shape, generator=g, device=dev, dtype=torch.float32).to(BF16)
+    o = sk.softmax_backward(dense, grad)
+    # row 700 of a few heads against the oracle
+    rows = (slice(0, 4), slice(0, 2), slice(700, 704))
+    assert_close_bf16(o[rows], O.softmax_bwd(dense[rows].cpu(), grad[rows].cpu()), what="softmax bwd rows")
