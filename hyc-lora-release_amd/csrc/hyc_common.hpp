@@ -59,6 +59,15 @@ __device__ __forceinline__ u32x4 ld16_nt(const void* p) {
 __device__ __forceinline__ void st16_nt(void* p, u32x4 v) {
     __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
 }
+__device__ __forceinline__ u32x2 ld8_nt(const void* p) {
+    return __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(p));
+}
+__device__ __forceinline__ void st8_nt(void* p, u32x2 v) {
+    __builtin_nontemporal_store(v, reinterpret_cast<u32x2*>(p));
+}
+__device__ __forceinline__ void st4_nt(void* p, uint32_t v) {
+    __builtin_nontemporal_store(v, reinterpret_cast<uint32_t*>(p));
+}
 
 // ---- wave64 cross-lane -------------------------------------------------------------
 // DPP quad permutes: lane <- lane ^ 1 and lane <- lane ^ 2 inside each group of 4 lanes.

@@ -13,42 +13,78 @@
 
 namespace hyc {
 
-// 8 values -> 8 codes, one per byte of (lo, hi).
-template <int QBIT, bool ZP, bool FAST>
-__device__ __forceinline__ void codes_to_words(const float (&f)[8], const float (&s)[8], const float (&r)[8],
-                                               const float (&z)[8], uint32_t& lo, uint32_t& hi) {
-    int c[8];
+// Per-lane column constants of the quantiser: step, reciprocal, the input clamp of the
+// reciprocal path, and whether every one of the lane's 8 steps may use that path.
+template <int QBIT>
+struct QuantCols {
+    float s[8], r[8], xlo[8], xhi[8];
+    bool fast;
+    __device__ __forceinline__ void load(const uint16_t* scale, int col0, bool active) {
+        u32x4 sv = {0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};   // 1.0 for idle lanes
+        if (active) sv = ld16(scale + col0);
+        unpack8(sv, s);
+        fast = true;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        if constexpr (ZP) {
-            // zero-point form: IEEE quotient, then + z, then exact roundf
-            c[j] = hyc_code_from_t_exact(f[j] / s[j] + z[j], QBIT);
-        } else if constexpr (FAST) {
-            c[j] = hyc_code_from_t(hyc_quot_fast(f[j], s[j], r[j]), QBIT);
-        } else {
-            c[j] = hyc_code_from_t(f[j] / s[j], QBIT);
+        for (int j = 0; j < 8; ++j) {
+            r[j] = 1.0f / s[j];
+            xlo[j] = hyc_clamp_lo(s[j], QBIT);
+            xhi[j] = hyc_clamp_hi(s[j], QBIT);
+            fast = fast && hyc_scale_is_fast(s[j]);
         }
     }
-    lo = (uint32_t)c[0] | ((uint32_t)c[1] << 8) | ((uint32_t)c[2] << 16) | ((uint32_t)c[3] << 24);
-    hi = (uint32_t)c[4] | ((uint32_t)c[5] << 8) | ((uint32_t)c[6] << 16) | ((uint32_t)c[7] << 24);
+};
+
+// 8 values -> 8 codes, one per byte of (lo, hi).
+template <int QBIT, bool ZP, bool FAST>
+__device__ __forceinline__ void codes_to_words(const float (&f)[8], const QuantCols<QBIT>& q, const float (&z)[8],
+                                               uint32_t& lo, uint32_t& hi) {
+    if constexpr (FAST && !ZP) {
+        // signed codes; the offset 2^(q-1) is added to all four bytes of a word at once
+        // (sums of shifted two's-complement values, exact modulo 2^32)
+        uint32_t c[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) c[j] = (uint32_t)hyc_signed_code_fast(f[j], q.s[j], q.r[j], q.xlo[j], q.xhi[j]);
+        constexpr uint32_t bias = 0x01010101u * (1u << (QBIT - 1));
+        lo = c[0] + (c[1] << 8) + (c[2] << 16) + (c[3] << 24) + bias;
+        hi = c[4] + (c[5] << 8) + (c[6] << 16) + (c[7] << 24) + bias;
+    } else {
+        int c[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            if constexpr (ZP) {
+                // zero-point form: IEEE quotient, then + z, then exact roundf
+                c[j] = hyc_code_from_t_exact(f[j] / q.s[j] + z[j], QBIT);
+            } else {
+                c[j] = hyc_code_from_t(f[j] / q.s[j], QBIT);
+            }
+        }
+        lo = (uint32_t)c[0] | ((uint32_t)c[1] << 8) | ((uint32_t)c[2] << 16) | ((uint32_t)c[3] << 24);
+        hi = (uint32_t)c[4] | ((uint32_t)c[5] << 8) | ((uint32_t)c[6] << 16) | ((uint32_t)c[7] << 24);
+    }
 }
 
 // Merge the quad's code words into packed bytes and store this lane's share of them.
 // Every lane of the quad must call this (the exchange is a DPP quad permute); `active`
 // only gates the store.  qrow = first packed byte of the row.
-template <int QBIT>
+template <int QBIT, bool NT = false>
 __device__ __forceinline__ void store_packed(uint8_t* qrow, int chunk, bool active, uint32_t lo, uint32_t hi) {
     const int quad = chunk & 3;
     const int blk = chunk >> 2;
     if constexpr (QBIT == 8) {
-        if (active) st8(qrow + (int64_t)chunk * 8, u32x2{lo, hi});
+        if (active) {
+            if constexpr (NT) st8_nt(qrow + (int64_t)chunk * 8, u32x2{lo, hi});
+            else st8(qrow + (int64_t)chunk * 8, u32x2{lo, hi});
+        }
     } else if constexpr (QBIT == 4) {
         const int sub = quad >> 1;
         lo <<= 4 * sub;
         hi <<= 4 * sub;
         lo |= quad_xor2(lo);
         hi |= quad_xor2(hi);
-        if (active) *reinterpret_cast<uint32_t*>(qrow + blk * 16 + 8 * (quad & 1) + 4 * sub) = sub ? hi : lo;
+        if (active) {
+            if constexpr (NT) st4_nt(qrow + blk * 16 + 8 * (quad & 1) + 4 * sub, sub ? hi : lo);
+            else *reinterpret_cast<uint32_t*>(qrow + blk * 16 + 8 * (quad & 1) + 4 * sub) = sub ? hi : lo;
+        }
     } else {
         lo <<= 2 * quad;
         hi <<= 2 * quad;
@@ -56,7 +92,10 @@ __device__ __forceinline__ void store_packed(uint8_t* qrow, int chunk, bool acti
         hi |= quad_xor1(hi);
         lo |= quad_xor2(lo);
         hi |= quad_xor2(hi);
-        if (active && quad < 2) *reinterpret_cast<uint32_t*>(qrow + blk * 8 + 4 * quad) = quad ? hi : lo;
+        if (active && quad < 2) {
+            if constexpr (NT) st4_nt(qrow + blk * 8 + 4 * quad, quad ? hi : lo);
+            else *reinterpret_cast<uint32_t*>(qrow + blk * 8 + 4 * quad) = quad ? hi : lo;
+        }
     }
 }
 
@@ -78,24 +117,6 @@ struct PackedSlot {
         const uint32_t lo = (w.x >> shift) & mask, hi = (w.y >> shift) & mask;
 #pragma unroll
         for (int j = 0; j < 8; ++j) c[j] = (float)(((j < 4 ? lo : hi) >> (8 * (j & 3))) & 0xffu);
-    }
-};
-
-// Per-lane column constants of the quantiser: step, reciprocal, and whether every one of the
-// lane's 8 steps may use the reciprocal path.
-struct QuantCols {
-    float s[8], r[8];
-    bool fast;
-    __device__ __forceinline__ void load(const uint16_t* scale, int col0, bool active) {
-        u32x4 sv = {0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};   // 1.0 for idle lanes
-        if (active) sv = ld16(scale + col0);
-        unpack8(sv, s);
-        fast = true;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            r[j] = 1.0f / s[j];
-            fast = fast && hyc_scale_is_fast(s[j]);
-        }
     }
 };
 

@@ -82,6 +82,28 @@ HYC_HD int hyc_code_from_t(float t, int q_bit) {
     return (int)v + (1 << (q_bit - 1));
 }
 
+// Cheapest form of the rule for the reciprocal path, as a signed code in
+// [-2^(q-1), 2^(q-1)-1] (the caller adds the offset 2^(q-1) once per packed word).
+// Instead of clamping the quotient, the INPUT is clamped to [xlo, xhi] =
+// [(-2^(q-1) - 0.49) s, (2^(q-1) - 1 + 0.49) s]: inside that interval nothing changes, and
+// outside it the value lands 0.49 beyond the last code, which rounds to that code — the
+// same saturation, but infinities never reach the correction step and no second clamp is
+// needed.  A NaN input fails the comparison and becomes xlo, i.e. the lowest code (biased
+// code 0); a compare-and-select is used rather than fmaxf because fmaxf turns a
+// *signalling* NaN into a quiet NaN instead of dropping it.
+// The sign for the half-away rounding is taken from the clamped input (s > 0 here).
+HYC_HD float hyc_clamp_lo(float s, int q_bit) { return (-(float)(1 << (q_bit - 1)) - 0.49f) * s; }
+HYC_HD float hyc_clamp_hi(float s, int q_bit) { return ((float)(1 << (q_bit - 1)) - 1.0f + 0.49f) * s; }
+
+HYC_HD int hyc_signed_code_fast(float x, float s, float r, float xlo, float xhi) {
+    float xc = (x > xlo) ? x : xlo;
+    xc = fminf(xc, xhi);
+    const float q0 = xc * r;
+    const float rem = fmaf(-q0, s, xc);
+    const float q1 = fmaf(rem, r, q0);
+    return (int)(q1 + copysignf(0.5f, xc));
+}
+
 // Same rule with plain roundf semantics (trunc, then an exact fraction test), for
 // t = x/s + z: once an arbitrary zero point has been added the half-ulp argument above
 // no longer holds.

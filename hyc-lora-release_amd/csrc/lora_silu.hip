@@ -95,7 +95,7 @@ __device__ __forceinline__ float acc_elem(const f32x4& a, int v) {
 // ------------------------------------------------------------------------------------
 template <int QBIT, int KSTEPS, bool FAST>
 __device__ __forceinline__ void fuse_fwd_rows(const FuseArgs& a, int64_t row_begin, int64_t row_end, int lane, int chunk,
-                                              bool active, const QuantCols& c1, const QuantCols& c2,
+                                              bool active, const QuantCols<QBIT>& c1, const QuantCols<QBIT>& c2,
                                               const BOperand<KSTEPS>& B1, const BOperand<KSTEPS>& B2) {
     const int g = lane >> 4;
     const int row_bytes = a.N * QBIT / 8;
@@ -125,9 +125,9 @@ __device__ __forceinline__ void fuse_fwd_rows(const FuseArgs& a, int64_t row_beg
             uint32_t lo, hi;
             // rows past the end still take part in the quad exchange; their stores are masked
             const int64_t tq = t < row_end ? t : row_end - 1;
-            codes_to_words<QBIT, false, FAST>(f1, c1.s, c1.r, zero8, lo, hi);
+            codes_to_words<QBIT, false, FAST>(f1, c1, zero8, lo, hi);
             store_packed<QBIT>(a.q1 + tq * row_bytes, chunk, live, lo, hi);
-            codes_to_words<QBIT, false, FAST>(f2, c2.s, c2.r, zero8, lo, hi);
+            codes_to_words<QBIT, false, FAST>(f2, c2, zero8, lo, hi);
             store_packed<QBIT>(a.q2 + tq * row_bytes, chunk, live, lo, hi);
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
@@ -151,7 +151,7 @@ __global__ __launch_bounds__(kFuseThreads) void lora_silu_fwd_kernel(const FuseA
     const bool active = chunk < a.C;
     const int col0 = chunk * 8;
 
-    QuantCols c1, c2;
+    QuantCols<QBIT> c1, c2;
     c1.load(a.s1, col0, active);
     c2.load(a.s2, col0, active);
     BOperand<KSTEPS> B1, B2;

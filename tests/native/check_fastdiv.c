@@ -2,7 +2,8 @@
  *
  * For every bf16 step s accepted by hyc_scale_is_fast and every one of the 65536 bf16
  * inputs x (NaNs and infinities included), the integer code computed from
- * hyc_quot_fast(x, s, 1/s) must equal the code computed from the IEEE quotient x / s
+ * hyc_quot_fast(x, s, 1/s), and the one computed by hyc_signed_code_fast (input clamp
+ * instead of quotient clamp), must equal the code computed from the IEEE quotient x / s
  * with libm's roundf, for code widths 2, 4 and 8.  Prints the number of pairs examined
  * and the number of mismatches; exit status 0 iff there are none.
  *
@@ -41,9 +42,12 @@ int main(int argc, char **argv) {
             ++pairs;
             if (fabsf(ti) <= 512.0f && !(tf == ti)) ++inexact;
             int ok = 1;
-            for (int q = 2; q <= 8; q *= 2)
-                if (hyc_code_from_t(tf, q) != code_ieee(x, s, q) ||
-                    hyc_code_from_t_exact(ti, q) != code_ieee(x, s, q)) ok = 0;
+            for (int q = 2; q <= 8; q *= 2) {
+                const int want = code_ieee(x, s, q);
+                if (hyc_code_from_t(tf, q) != want || hyc_code_from_t_exact(ti, q) != want) ok = 0;
+                if (hyc_signed_code_fast(x, s, r, hyc_clamp_lo(s, q), hyc_clamp_hi(s, q)) + (1 << (q - 1)) != want)
+                    ok = 0;
+            }
             if (!ok) {
                 ++bad;
 #pragma omp critical

@@ -42,6 +42,8 @@ def test_special_values_and_degenerate_scales(cf, dev, q_bit):
     x = _rand((2, 40, 128), seed=11, scale=3.0)
     x[1, 0, :8] = torch.tensor([0.0, -0.0, float("inf"), float("-inf"), float("nan"), 1e-40, 3e38, -3e38]).to(BF16)
     x[1, 1, 64:72] = torch.tensor([0.5, -0.5, 1.5, -1.5, 2.5, -2.5, 3.5, -3.5]).to(BF16)
+    # signalling NaN bit patterns (0x7f81, 0xffa0): never produced by arithmetic, still code 0
+    x[1, 2, :2] = torch.tensor([0x7f81, 0xffa0 - 0x10000], dtype=torch.int16).view(BF16)
     s = O.scale_only_quant(x, q_bit)
     s[0, 64:72] = 1.0                      # exact ties t = +-k.5
     s[0, 5] = 0.0                          # zero step (constant channel, scale-only path): x/0
