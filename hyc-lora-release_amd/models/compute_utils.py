@@ -1,0 +1,86 @@
+"""Torch-side glue of the fused layers (reference: models/utils/compute_utils.py:7-51 and
+operators/rope_kernels.py:81-126).  The frozen-weight GEMMs, RoPE and the attention products are
+library / torch operations in the reference as well; only what surrounds them is compressed."""
+import torch
+
+
+def hidden_to_head_shape(x: torch.Tensor, num_heads: int):
+    bsz, seq_len, hidden = x.shape
+    return x.reshape(bsz, seq_len, num_heads, hidden // num_heads).transpose(1, 2)
+
+
+def head_to_hidden_shape(x: torch.Tensor):
+    bsz, _, seq_len, _ = x.shape
+    return x.transpose(1, 2).reshape(bsz, seq_len, -1).contiguous()
+
+
+def dense_weight(w: torch.Tensor, quant_state):
+    """Frozen weight as a dense [out, in] matrix.  quant_state None = already dense (the
+    benchmark configurations); otherwise NF4 via bitsandbytes, as in the reference."""
+    if quant_state is None:
+        return w
+    try:
+        import bitsandbytes.functional as BF
+    except ImportError as e:  # pragma: no cover - bitsandbytes is absent in this environment
+        raise RuntimeError("NF4 frozen weights need bitsandbytes; pass dense bf16 weights "
+                           "(quant_state=None) instead") from e
+    return BF.dequantize_nf4(w, quant_state)
+
+
+def lora_forward(w, w_quant_state, w_lora_a, w_lora_b, b, x):
+    """-> (x @ W^T [+ b] + (x @ A) @ B, the frozen part alone, x @ A).  Reference :18-25."""
+    wt = dense_weight(w, w_quant_state).t()
+    x = x.to(wt.dtype)
+    x_main = x @ wt
+    if b is not None:
+        x_main = x_main + b.to(wt.dtype)
+    x_lora_a = x @ w_lora_a.to(wt.dtype)
+    return x_main + x_lora_a @ w_lora_b.to(wt.dtype), x_main, x_lora_a
+
+
+def lora_backward(w, w_quant_state, w_lora_a, w_lora_b, x, x_lora_a, grad_y):
+    """-> (grad lora_A, grad lora_B, grad x).  Reference :28-36."""
+    wd = dense_weight(w, w_quant_state)          # [out, in]
+    dt = wd.dtype
+    grad_y = grad_y.to(dt)
+    w_lora_a, w_lora_b = w_lora_a.to(dt), w_lora_b.to(dt)
+    grad_mid = grad_y @ w_lora_b.mT
+    grad_a = x.to(dt).mT @ grad_mid
+    grad_b = x_lora_a.to(dt).mT @ grad_y
+    grad_x = grad_y @ wd
+    grad_x += grad_mid @ w_lora_a.mT
+    return grad_a, grad_b, grad_x
+
+
+def repeat_kv(h: torch.Tensor, n_rep: int):
+    if n_rep == 1:
+        return h
+    b, kv, s, d = h.shape
+    return h[:, :, None, :, :].expand(b, kv, n_rep, s, d).reshape(b, kv * n_rep, s, d)
+
+
+def repeat_kv_backward(g: torch.Tensor, n_rep: int):
+    if n_rep == 1:
+        return g
+    b, hq, s, d = g.shape
+    return g.reshape(b, hq // n_rep, n_rep, s, d).sum(dim=2)
+
+
+def _rope(x, cos, sin, sign):
+    # x: [B, S, H, D]; cos/sin: [..., S_max, D] with the two halves equal (HF layout) - only the
+    # first half is read, as the reference kernel does (rope_kernels.py:56-59)
+    cos, sin = cos.squeeze(), sin.squeeze()
+    seq, half = x.shape[1], x.shape[-1] // 2
+    assert seq <= cos.shape[0]
+    c = cos[:seq, :half][None, :, None, :]
+    s = sin[:seq, :half][None, :, None, :] * sign
+    x1, x2 = x[..., :half].to(s.dtype), x[..., half:].to(s.dtype)
+    return torch.cat([x1 * c - x2 * s, x2 * c + x1 * s], dim=-1).to(x.dtype)
+
+
+def rope_forward(x, cos, sin):
+    return _rope(x, cos, sin, 1.0)
+
+
+def rope_backward(dy, cos, sin):
+    return _rope(dy, cos, sin, -1.0)

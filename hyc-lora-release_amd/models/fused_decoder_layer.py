@@ -1,0 +1,439 @@
+"""A LoRA decoder layer (RMSNorm - attention - RMSNorm - gated MLP) as one autograd.Function that
+saves *compressed* activations for backward.
+
+Restates what the reference spreads over twelve near-identical files
+(models/{llama,mistral,llama_flash_attn}/fused_*_layer_{intra,intra_inter,intra_inter_full_fuse}.py)
+as one function with three switches:
+
+  mode        'intra'                 every saved activation is quantised as is; q, k (after RoPE) and
+                                      v are saved in head shape; silu(gate) and the gated product are
+                                      saved too                      (fused_llama_layer_intra.py:95-310)
+              'intra_inter'           only the frozen-weight outputs (x@W, "main") are quantised; the
+                                      LoRA part is recomputed from the saved x@A in backward
+                                                                     (fused_llama_layer_intra_inter.py)
+              'intra_inter_full_fuse' as above, with the gate/up quantisation, LoRA add, SiLU and
+                                      product in one fused kernel each way
+                                                      (fused_llama_layer_intra_inter_full_fuse.py:218-235,359-371)
+  attention   'map'   softmax map is materialised, thresholded and saved sparse (:159-176,414-432)
+              'sdpa'  no map is saved; attention is recomputed in backward; q/k main use a zero point
+                      (llama_flash_attn/fused_llama_layer_intra_inter.py:118-180 - the flash-attn
+                      kernels themselves are replaced by torch's scaled_dot_product_attention)
+  norm weights receive gradients when they require grad (rmsnorm_updatable_kernels.py:173-220).
+
+Deliberate differences from the reference:
+  * the activations handed to the channel-base compressor are not cloned first (the kernels do not
+    modify their input);
+  * backward restores the input-norm outliers with the *input-norm* channel list; the reference's
+    intra_inter / full_fuse files pass the post-attention list there
+    (fused_llama_layer_intra_inter_full_fuse.py:484), which its own 'intra' file does not (:492);
+  * RMSNorm eps is a parameter (default 1e-5, the value the reference hard-codes, :99,203).
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+
+import torch
+import torch.nn.functional as F
+
+from ..operators.compress_function import (compress_attention_map, compression_pack_channel_base,
+                                           compression_pack_quant_base, compression_pack_quant_zp_base,
+                                           decompression_dequantization,
+                                           decompression_dequantization_with_zero_point,
+                                           get_statistics_only_quant, get_statistics_softmax,
+                                           outlier_addition_fuse_decompression_dequantization,
+                                           restore_attention_map, update_dict)
+from ..operators.rmsnorm_kernels import _backward as _rmsnorm_backward
+from ..operators.rmsnorm_kernels import rmsnorm_forward
+from ..operators.silu_kernels import silu_backward, silu_hadamard
+from ..operators.softmax_kernels import softmax_backward
+from ..operators.triton_fuse_lora_silu_hadamard_backward_kernels import triton_fuse_silu_backward
+from ..operators.triton_fuse_lora_silu_hadamard_forward_kernels import triton_fuse_silu_forward
+from .compute_utils import (head_to_hidden_shape, hidden_to_head_shape, lora_backward, lora_forward,
+                            repeat_kv, repeat_kv_backward, rope_backward, rope_forward)
+
+MODES = ("intra", "intra_inter", "intra_inter_full_fuse")
+
+
+@dataclass(frozen=True)
+class LayerSpec:
+    mode: str = "intra_inter_full_fuse"
+    attention: str = "map"          # 'map' | 'sdpa'
+    eps: float = 1e-5
+
+    def __post_init__(self):
+        if self.mode not in MODES:
+            raise ValueError(f"layer_type must be one of {MODES}, got {self.mode!r}")
+        if self.attention not in ("map", "sdpa"):
+            raise ValueError(f"attention must be 'map' or 'sdpa', got {self.attention!r}")
+
+    def stat_slots(self):
+        """(static_value key, field) of every calibration statistic the layer returns, in order."""
+        slots = [("x", "outlier_channel_index"), ("x", "scale"), ("x_norm_1", "scale"),
+                 ("q", "scale"), ("k", "scale"), ("v", "scale")]
+        if self.attention == "map":
+            slots.append(("a", "outlier"))
+        else:
+            slots += [("q", "zero_point"), ("k", "zero_point")]
+        slots += [("o", "scale"), ("x_medium", "outlier_channel_index"), ("x_medium", "scale"),
+                  ("x_norm_2", "scale"), ("gate", "scale"), ("up", "scale")]
+        if self.mode == "intra":
+            slots += [("fn", "scale"), ("hadamard", "scale")]
+        return slots
+
+    def empty_static_value(self):
+        sv = {}
+        for key, field in self.stat_slots():
+            sv.setdefault(key, {})[field] = None
+        return sv
+
+
+_PROJ = ("q", "k", "v", "o", "gate", "up", "down")
+
+
+class FusedDecoderLayerFunc(torch.autograd.Function):
+    """Inputs follow the reference's Func.apply order (…full_fuse.py:31-93) with the LayerSpec appended."""
+
+    @staticmethod
+    def forward(ctx, x, norm_weight_1, norm_bias_1, cos, sin,
+                w_q, b_q, qs_q, a_q, bb_q, w_k, b_k, qs_k, a_k, bb_k,
+                w_v, b_v, qs_v, a_v, bb_v, w_o, b_o, qs_o, a_o, bb_o,
+                norm_weight_2, norm_bias_2,
+                w_gate, b_gate, qs_gate, a_gate, bb_gate, w_up, b_up, qs_up, a_up, bb_up,
+                w_down, b_down, qs_down, a_down, bb_down,
+                attention_mask, num_heads, head_dim, num_key_value_heads,
+                iteration, iteration_threshold, static_value, softmax_outlier_ratio,
+                layernorm_outlier_ratio, q_bit, spec):
+        W = dict(q=(w_q, b_q, qs_q, a_q, bb_q), k=(w_k, b_k, qs_k, a_k, bb_k), v=(w_v, b_v, qs_v, a_v, bb_v),
+                 o=(w_o, b_o, qs_o, a_o, bb_o), gate=(w_gate, b_gate, qs_gate, a_gate, bb_gate),
+                 up=(w_up, b_up, qs_up, a_up, bb_up), down=(w_down, b_down, qs_down, a_down, bb_down))
+        it, thd, sv = iteration, iteration_threshold, static_value
+        calib = it < thd
+        n_rep = num_heads // num_key_value_heads
+        stats, saved = {}, {}
+
+        def proj(name, inp):
+            w, b, qs, la, lb = W[name]
+            return lora_forward(w, qs, la, lb, b, inp)
+
+        def quant(name, t, key=None):
+            q, s = compression_pack_quant_base(t, q_bit, 'per-channel', it, thd, sv[key or name])
+            stats[(key or name, "scale")] = s
+            saved[name + "_q"], saved[name + "_s"] = q, s
+
+        def quant_zp(name, t, key):
+            q, s, z = compression_pack_quant_zp_base(t, q_bit, 'per-channel', it, thd, sv[key])
+            stats[(key, "scale")], stats[(key, "zero_point")] = s, z
+            saved[name + "_q"], saved[name + "_s"], saved[name + "_z"] = q, s, z
+
+        def channel_base(name, t):
+            o, q, idx, s = compression_pack_channel_base(t, layernorm_outlier_ratio, q_bit, 'per-channel', it, thd,
+                                                         sv[name])
+            stats[(name, "outlier_channel_index")], stats[(name, "scale")] = idx, s
+            saved[name + "_o"], saved[name + "_q"], saved[name + "_s"], saved[name + "_idx"] = o, q, s, idx
+
+        # ---- attention block -------------------------------------------------------------------
+        x_norm_1, _, rstd_1, block_size, num_warps = rmsnorm_forward(x, norm_weight_1, spec.eps)
+        saved["rstd_1"] = rstd_1
+        channel_base("x", x)
+        q, q_main, saved["q_lora_a"] = proj("q", x_norm_1)
+        k, k_main, saved["k_lora_a"] = proj("k", x_norm_1)
+        v, v_main, saved["v_lora_a"] = proj("v", x_norm_1)
+        quant("x_norm_1", x_norm_1)
+        del x_norm_1
+        if spec.mode != "intra":
+            if spec.attention == "sdpa":
+                quant_zp("q_main", q_main, "q")
+                quant_zp("k_main", k_main, "k")
+            else:
+                quant("q_main", q_main, "q")
+                quant("k_main", k_main, "k")
+            quant("v_main", v_main, "v")
+        del q_main, k_main, v_main
+
+        q = hidden_to_head_shape(q, num_heads)
+        k = hidden_to_head_shape(k, num_key_value_heads)
+        v = hidden_to_head_shape(v, num_key_value_heads)
+        q = rope_forward(q.transpose(1, 2), cos, sin).transpose(1, 2)
+        k = rope_forward(k.transpose(1, 2), cos, sin).transpose(1, 2)
+        k = repeat_kv(k, n_rep)
+        v = repeat_kv(v, n_rep)
+        if spec.mode == "intra":
+            (quant_zp if spec.attention == "sdpa" else quant)("q_rope", q, "q")
+            (quant_zp if spec.attention == "sdpa" else quant)("k_rope", k, "k")
+            quant("v_rep", v, "v")
+
+        if spec.attention == "map":
+            s = q @ k.transpose(-2, -1) / math.sqrt(head_dim)
+            del q, k
+            if attention_mask is not None:
+                s = s + attention_mask
+            a = torch.softmax(s, dim=-1, dtype=v.dtype)
+            del s
+            thr = get_statistics_softmax(a, softmax_outlier_ratio) if calib else sv['a']['outlier']
+            stats[("a", "outlier")] = thr
+            saved["a_idx"], saved["a_val"], saved["a_seg"] = compress_attention_map(a, thr)
+            ctx.a_shape = tuple(a.shape)
+            o = a @ v
+            del a, v
+        else:
+            o = F.scaled_dot_product_attention(q, k, v, attn_mask=attention_mask, is_causal=attention_mask is None)
+            del q, k, v
+        o = head_to_hidden_shape(o)
+        o_final, _, saved["o_lora_a"] = proj("o", o)
+        quant("o", o)
+        del o
+        x_medium = x + o_final
+        del o_final
+
+        # ---- MLP block ---------------------------------------------------------------------------
+        x_norm_2, _, rstd_2, block_size, num_warps = rmsnorm_forward(x_medium, norm_weight_2, spec.eps)
+        saved["rstd_2"] = rstd_2
+        channel_base("x_medium", x_medium)
+        if spec.mode == "intra_inter_full_fuse":
+            from .compute_utils import dense_weight
+            wg, wu = dense_weight(w_gate, qs_gate).t(), dense_weight(w_up, qs_up).t()
+            x_norm_2 = x_norm_2.to(wg.dtype)
+            gate_main = x_norm_2 @ wg if b_gate is None else x_norm_2 @ wg + b_gate.to(wg.dtype)
+            up_main = x_norm_2 @ wu if b_up is None else x_norm_2 @ wu + b_up.to(wu.dtype)
+            gate_lora_a = x_norm_2 @ a_gate.to(wg.dtype)
+            up_lora_a = x_norm_2 @ a_up.to(wu.dtype)
+            if calib:
+                gate_s = get_statistics_only_quant(gate_main, q_bit, 'per-channel')
+                up_s = get_statistics_only_quant(up_main, q_bit, 'per-channel')
+            else:
+                gate_s, up_s = sv['gate']['scale'], sv['up']['scale']
+            stats[("gate", "scale")], stats[("up", "scale")] = gate_s, up_s
+            gate_q, up_q, hadamard = triton_fuse_silu_forward(gate_lora_a, bb_gate, gate_main, gate_s,
+                                                              up_lora_a, bb_up, up_main, up_s, q_bit)
+            saved.update(gate_main_q=gate_q, gate_main_s=gate_s, up_main_q=up_q, up_main_s=up_s)
+            del gate_main, up_main
+        else:
+            gate, gate_main, gate_lora_a = proj("gate", x_norm_2)
+            up, up_main, up_lora_a = proj("up", x_norm_2)
+            if spec.mode == "intra_inter":
+                quant("gate_main", gate_main, "gate")
+                quant("up_main", up_main, "up")
+                hadamard = silu_hadamard(gate, up)
+            else:
+                fn = F.silu(gate)
+                quant("gate", gate)
+                hadamard = up * fn
+                quant("up", up)
+                quant("fn", fn)
+                del fn
+            del gate, up, gate_main, up_main
+        saved["gate_lora_a"], saved["up_lora_a"] = gate_lora_a, up_lora_a
+        quant("x_norm_2", x_norm_2)
+        del x_norm_2
+        down, _, saved["down_lora_a"] = proj("down", hadamard)
+        if spec.mode == "intra":
+            quant("hadamard", hadamard)
+        del hadamard
+        x_out = x_medium + down
+
+        ctx.names = list(saved.keys())
+        ctx.save_for_backward(*saved.values(), cos, sin, norm_weight_1, norm_weight_2,
+                              *(t for n in _PROJ for t in (W[n][0], W[n][1], W[n][3], W[n][4])))
+        ctx.quant_states = {n: W[n][2] for n in _PROJ}
+        ctx.spec, ctx.q_bit = spec, q_bit
+        ctx.num_heads, ctx.num_key_value_heads, ctx.head_dim = num_heads, num_key_value_heads, head_dim
+        ctx.block_size, ctx.num_warps = block_size, num_warps
+        ctx.has_mask = attention_mask is not None
+        ctx.attention_mask = attention_mask
+        ctx.norm_grads = (norm_weight_1.requires_grad, norm_weight_2.requires_grad)
+        out_stats = tuple(stats[slot] for slot in spec.stat_slots())
+        ctx.mark_non_differentiable(*[t for t in out_stats if torch.is_tensor(t)])
+        return (x_out,) + out_stats
+
+    @staticmethod
+    def backward(ctx, grad_output, *_unused):
+        spec, q_bit = ctx.spec, ctx.q_bit
+        tensors = list(ctx.saved_tensors)
+        ns = len(ctx.names)
+        S = dict(zip(ctx.names, tensors[:ns]))
+        cos, sin, norm_weight_1, norm_weight_2 = tensors[ns:ns + 4]
+        rest = tensors[ns + 4:]
+        W = {n: (rest[4 * i], rest[4 * i + 1], ctx.quant_states[n], rest[4 * i + 2], rest[4 * i + 3])
+             for i, n in enumerate(_PROJ)}
+        H, KV, D = ctx.num_heads, ctx.num_key_value_heads, ctx.head_dim
+        n_rep = H // KV
+        G = {}                                           # LoRA gradients
+
+        def deq(name, **kw):
+            if name + "_z" in S:
+                return decompression_dequantization_with_zero_point(S[name + "_q"], S[name + "_s"], S[name + "_z"],
+                                                                    q_bit, **kw)
+            return decompression_dequantization(S[name + "_q"], S[name + "_s"], q_bit, **kw)
+
+        def back(name, inp, inp_lora_a, grad_y):
+            w, _, qs, la, lb = W[name]
+            ga, gb, gx = lora_backward(w, qs, la, lb, inp, inp_lora_a, grad_y)
+            G[name] = (ga, gb)
+            return gx
+
+        def lora_part(name):
+            return S[name + "_lora_a"] @ W[name][4].to(S[name + "_lora_a"].dtype)
+
+        def norm_backward(dy, xin, weight, rstd, want_dw):
+            return _rmsnorm_backward(dy, xin, weight, rstd, want_dw=want_dw)
+
+        # ---- MLP block ---------------------------------------------------------------------------
+        if spec.mode == "intra_inter_full_fuse":
+            from .compute_utils import dense_weight
+            w, _, qs, la, lb = W["down"]
+            wd = dense_weight(w, qs)
+            la, lb = la.to(wd.dtype), lb.to(wd.dtype)
+            g = grad_output.to(wd.dtype)
+            grad_b_down = S["down_lora_a"].to(wd.dtype).mT @ g
+            grad_down = g @ wd
+            grad_mid = g @ lb.mT
+            grad_down += grad_mid @ la.mT
+            hadamard, grad_fn, grad_h2 = triton_fuse_silu_backward(
+                S["gate_lora_a"], W["gate"][4], S["gate_main_q"], S["gate_main_s"],
+                S["up_lora_a"], W["up"][4], S["up_main_q"], S["up_main_s"], grad_down, q_bit)
+            G["down"] = (hadamard.to(wd.dtype).mT @ grad_mid, grad_b_down)
+            del hadamard, grad_down
+        else:
+            if spec.mode == "intra_inter":
+                gate = deq("gate_main") + lora_part("gate")
+                up = deq("up_main") + lora_part("up")
+                fn = F.silu(gate)
+                hadamard = up * fn
+            else:
+                hadamard, up, fn, gate = deq("hadamard"), deq("up"), deq("fn"), deq("gate")
+            grad_down = back("down", hadamard, S["down_lora_a"], grad_output)
+            del hadamard
+            grad_h1 = grad_down * up
+            grad_h2 = grad_down * fn
+            grad_fn = silu_backward(gate, grad_h1)
+            del grad_down, up, fn, gate, grad_h1
+        x_norm_2 = deq("x_norm_2")
+        grad_x2 = back("gate", x_norm_2, S["gate_lora_a"], grad_fn)
+        grad_x2 = grad_x2 + back("up", x_norm_2, S["up_lora_a"], grad_h2)
+        del x_norm_2, grad_fn, grad_h2
+        x_medium = outlier_addition_fuse_decompression_dequantization(
+            S["x_medium_q"], S["x_medium_s"], S["x_medium_o"], S["x_medium_idx"], q_bit)
+        grad_norm_2, grad_nw2 = norm_backward(grad_x2, x_medium, norm_weight_2, S["rstd_2"], ctx.norm_grads[1])
+        del x_medium, grad_x2
+        grad_medium = grad_norm_2 + grad_output
+
+        # ---- attention block -------------------------------------------------------------------
+        grad_o = back("o", deq("o"), S["o_lora_a"], grad_medium)
+        grad_o = hidden_to_head_shape(grad_o, H)
+
+        def rebuilt(name, heads):
+            """q/k/v in head shape as the forward attention saw them (before repeat_kv)."""
+            main = deq(name + "_main")
+            t = hidden_to_head_shape(main + lora_part(name).to(main.dtype), heads)
+            if name != "v":
+                t = rope_forward(t.transpose(1, 2), cos, sin).transpose(1, 2)
+            return t
+
+        if spec.mode == "intra":
+            q, k, v = (deq(n, is_head=True, num_heads=H) for n in ("q_rope", "k_rope", "v_rep"))
+        else:
+            q, k, v = rebuilt("q", H), repeat_kv(rebuilt("k", KV), n_rep), repeat_kv(rebuilt("v", KV), n_rep)
+
+        if spec.attention == "map":
+            a = restore_attention_map(S["a_idx"], S["a_val"], S["a_seg"], ctx.a_shape)
+            grad_v = a.transpose(-2, -1) @ grad_o
+            grad_a = grad_o @ v.transpose(-2, -1)
+            del v, grad_o
+            grad_s = softmax_backward(a, grad_a)
+            del a, grad_a
+            grad_s = grad_s / math.sqrt(D)
+            grad_k = grad_s.transpose(-2, -1) @ q
+            grad_q = grad_s @ k
+            del grad_s, q, k
+        else:
+            with torch.enable_grad():
+                q_, k_, v_ = (t.detach().requires_grad_() for t in (q, k, v))
+                o_ = F.scaled_dot_product_attention(q_, k_, v_, attn_mask=ctx.attention_mask,
+                                                    is_causal=not ctx.has_mask)
+                grad_q, grad_k, grad_v = torch.autograd.grad(o_, (q_, k_, v_), grad_o)
+            del q, k, v, q_, k_, v_, o_, grad_o
+        grad_v = repeat_kv_backward(grad_v, n_rep)
+        grad_k = repeat_kv_backward(grad_k, n_rep)
+        grad_q = rope_backward(grad_q.transpose(1, 2), cos, sin).transpose(1, 2)
+        grad_k = rope_backward(grad_k.transpose(1, 2), cos, sin).transpose(1, 2)
+        grad_q, grad_k, grad_v = (head_to_hidden_shape(t) for t in (grad_q, grad_k, grad_v))
+
+        x_norm_1 = deq("x_norm_1")
+        grad_x = back("q", x_norm_1, S["q_lora_a"], grad_q)
+        grad_x += back("k", x_norm_1, S["k_lora_a"], grad_k)
+        grad_x += back("v", x_norm_1, S["v_lora_a"], grad_v)
+        del x_norm_1, grad_q, grad_k, grad_v
+        x = outlier_addition_fuse_decompression_dequantization(S["x_q"], S["x_s"], S["x_o"], S["x_idx"], q_bit)
+        grad_norm_1, grad_nw1 = norm_backward(grad_x, x, norm_weight_1, S["rstd_1"], ctx.norm_grads[0])
+        grad_input = grad_norm_1 + grad_medium
+
+        def lora_grads(name):
+            return (None, None, None) + G[name]
+
+        return ((grad_input, grad_nw1, None, None, None)
+                + lora_grads("q") + lora_grads("k") + lora_grads("v") + lora_grads("o")
+                + (grad_nw2, None)
+                + lora_grads("gate") + lora_grads("up") + lora_grads("down")
+                + (None,) * 11)
+
+
+def _weight_of(module):
+    """Weight of a LoRA adapter container (`module.default.weight`, PEFT) or of a plain Linear."""
+    inner = getattr(module, "default", module)
+    return inner.weight
+
+
+class FusedDecoderLayer(torch.nn.Module):
+    """Module wrapper: owns the calibration state (`iteration`, `static_value`) and feeds the
+    Function.  Same call signature as the reference's modules (…full_fuse.py:582-614)."""
+
+    layer_type = "intra_inter_full_fuse"
+    attention = "map"
+
+    def __init__(self, eps: float = 1e-5):
+        super().__init__()
+        self.spec = LayerSpec(self.layer_type, self.attention, eps)
+        self.iteration = 0
+        self.static_value = self.spec.empty_static_value()
+        self.use_hyclora = False
+
+    def set_hyclora_config(self, hyclora_config):
+        self.hyclora_config = hyclora_config
+        self.use_hyclora = hyclora_config.use_hyclora
+        self.iteration_threshold = hyclora_config.iteration_threshold
+        self.softmax_outlier_ratio = hyclora_config.softmax_outlier_ratio
+        self.layernorm_outlier_ratio = hyclora_config.layernorm_outlier_ratio
+        self.q_bit = hyclora_config.q_bit
+
+    def forward(self, input, norm_weight_1, norm_bias_1, cos, sin,
+                q_proj_base, q_proj_lora_a, q_proj_lora_b, k_proj_base, k_proj_lora_a, k_proj_lora_b,
+                v_proj_base, v_proj_lora_a, v_proj_lora_b, o_proj_base, o_proj_lora_a, o_proj_lora_b,
+                norm_weight_2, norm_bias_2,
+                gate_proj_base, gate_proj_lora_a, gate_proj_lora_b, up_proj_base, up_proj_lora_a, up_proj_lora_b,
+                down_proj_base, down_proj_lora_a, down_proj_lora_b,
+                attention_mask, num_heads, head_dim, num_key_value_heads):
+        def five(base, la, lb):
+            w = base.weight
+            return (w, getattr(base, "bias", None), getattr(w, "quant_state", None),
+                    _weight_of(la).T, _weight_of(lb).T)
+
+        outs = FusedDecoderLayerFunc.apply(
+            input, norm_weight_1, norm_bias_1, cos, sin,
+            *five(q_proj_base, q_proj_lora_a, q_proj_lora_b), *five(k_proj_base, k_proj_lora_a, k_proj_lora_b),
+            *five(v_proj_base, v_proj_lora_a, v_proj_lora_b), *five(o_proj_base, o_proj_lora_a, o_proj_lora_b),
+            norm_weight_2, norm_bias_2,
+            *five(gate_proj_base, gate_proj_lora_a, gate_proj_lora_b), *five(up_proj_base, up_proj_lora_a, up_proj_lora_b),
+            *five(down_proj_base, down_proj_lora_a, down_proj_lora_b),
+            attention_mask, num_heads, head_dim, num_key_value_heads,
+            self.iteration, self.iteration_threshold, self.static_value,
+            self.softmax_outlier_ratio, self.layernorm_outlier_ratio, self.q_bit, self.spec)
+        y, stat_values = outs[0], outs[1:]
+        if self.iteration < self.iteration_threshold:
+            fresh = {}
+            for (key, field), value in zip(self.spec.stat_slots(), stat_values):
+                fresh.setdefault(key, {})[field] = value
+            for key, fields in fresh.items():
+                self.static_value[key] = update_dict(self.static_value[key], fields, self.iteration)
+        self.iteration += 1
+        return y

@@ -1,0 +1,22 @@
+"""Long-sequence Llama layers: no attention map is materialised or saved, q/k main are quantised
+with a zero point, norm weights receive gradients
+(models/llama_flash_attn/fused_llama_layer_{intra,intra_inter}.py).  The flash-attn varlen kernels
+of the reference are replaced by torch's scaled_dot_product_attention (its ROCm flash/CK backend);
+backward recomputes the attention instead of calling a saved-LSE backward kernel."""
+from .fused_decoder_layer import FusedDecoderLayer
+
+
+class FusedLlamaLayerIntra(FusedDecoderLayer):
+    layer_type = "intra"
+    attention = "sdpa"
+
+
+class FusedLlamaLayerIntraInter(FusedDecoderLayer):
+    layer_type = "intra_inter"
+    attention = "sdpa"
+
+
+class FusedLlamaLayerIntraInterFullFuse(FusedDecoderLayer):
+    """Not present in the reference's flash variant; the fused MLP kernels apply unchanged."""
+    layer_type = "intra_inter_full_fuse"
+    attention = "sdpa"

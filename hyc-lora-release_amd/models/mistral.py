@@ -1,0 +1,33 @@
+"""Mistral decoder layers (grouped-query attention: 32 query / 8 key-value heads); class names as in
+the reference (models/mistral/fused_mistral_layer_*.py).  The computation is the generic layer: the
+reference's Mistral files differ from the Llama ones only in always calling repeat_kv and in a dtype
+cast of lora_B (fused_mistral_layer_intra_inter_full_fuse.py:226-227), both covered there."""
+from .fused_decoder_layer import FusedDecoderLayer
+
+
+class FusedMistralLayerIntra(FusedDecoderLayer):
+    layer_type = "intra"
+
+
+class FusedMistralLayerIntraInter(FusedDecoderLayer):
+    layer_type = "intra_inter"
+
+
+class FusedMistralLayerIntraInterFullFuse(FusedDecoderLayer):
+    layer_type = "intra_inter_full_fuse"
+
+
+LAYER_TYPES = {
+    "intra": FusedMistralLayerIntra,
+    "intra_inter": FusedMistralLayerIntraInter,
+    "intra_inter_full_fuse": FusedMistralLayerIntraInterFullFuse,
+}
+
+
+def make_fused_mistral_layer(hyclora_config):
+    try:
+        layer = LAYER_TYPES[hyclora_config.layer_type]()
+    except KeyError:
+        raise ValueError(f"Unknown layer type: {hyclora_config.layer_type}") from None
+    layer.set_hyclora_config(hyclora_config)
+    return layer

@@ -179,7 +179,7 @@ def pack_codes(c: torch.Tensor, q_bit: int) -> torch.Tensor:
     n = c.shape[-1]
     assert n % 32 == 0
     blk = c.reshape(*c.shape[:-1], n // 32, epp, w).to(torch.int32)
-    out = torch.zeros(*c.shape[:-1], n // 32, w, dtype=torch.int32)
+    out = torch.zeros(*c.shape[:-1], n // 32, w, dtype=torch.int32, device=c.device)
     for i in range(epp):
         out |= blk[..., i, :] << (q_bit * i)
     return out.reshape(*c.shape[:-1], n // epp).to(torch.uint8)
@@ -191,7 +191,7 @@ def unpack_codes(p: torch.Tensor, q_bit: int) -> torch.Tensor:
     w = 32 // epp
     nb = p.shape[-1]
     blk = p.reshape(*p.shape[:-1], nb // w, 1, w).to(torch.int32)
-    shifts = (torch.arange(epp, dtype=torch.int32) * q_bit).reshape(epp, 1)
+    shifts = (torch.arange(epp, dtype=torch.int32, device=p.device) * q_bit).reshape(epp, 1)
     c = (blk >> shifts) & (2 ** q_bit - 1)
     return c.reshape(*p.shape[:-1], nb * epp).to(torch.uint8)
 
@@ -252,7 +252,7 @@ def softmax_compress(a: torch.Tensor, thr) -> Tuple[torch.Tensor, torch.Tensor]:
 
 def softmax_restore(idx, vals, shape) -> torch.Tensor:
     """to_dense().reshape(shape) (compress_function.py:316-317)."""
-    out = torch.zeros(math.prod(shape), dtype=vals.dtype)
+    out = torch.zeros(math.prod(shape), dtype=vals.dtype, device=vals.device)
     out[idx] = vals
     return out.reshape(shape)
 

@@ -1,0 +1,196 @@
+"""Oracle restatement of one fused decoder layer: forward, what is saved (compressed), and the
+hand-written backward that recomputes from the compressed activations.  TEST INFRASTRUCTURE ONLY.
+
+Follows models/llama/fused_llama_layer_intra_inter_full_fuse.py:95-285 (forward) and :358-494
+(backward), fused_llama_layer_intra_inter.py:352-383 and fused_llama_layer_intra.py:373-455 for the
+other two layer types, using only plain torch operations and the element-level oracle functions of
+hyc_oracle.py (device-agnostic: runs wherever the input tensors live).  One deviation, shared with
+the implementation under test: the input-norm outliers are restored with the input-norm channel list
+(the reference's intra_inter/full_fuse files pass the post-attention list, :484).
+
+Calibration is always "fresh" (iteration < threshold): statistics are computed from the tensors at hand.
+"""
+import math
+
+import torch
+import torch.nn.functional as F
+
+from . import hyc_oracle as O
+
+
+def _heads(x, h):
+    b, s, d = x.shape
+    return x.reshape(b, s, h, d // h).transpose(1, 2)
+
+
+def _hidden(x):
+    b, _, s, _ = x.shape
+    return x.transpose(1, 2).reshape(b, s, -1).contiguous()
+
+
+def _repeat(x, n):
+    if n == 1:
+        return x
+    b, kv, s, d = x.shape
+    return x[:, :, None].expand(b, kv, n, s, d).reshape(b, kv * n, s, d)
+
+
+def _repeat_bwd(g, n):
+    if n == 1:
+        return g
+    b, h, s, d = g.shape
+    return g.reshape(b, h // n, n, s, d).sum(dim=2)
+
+
+def _rope(x, cos, sin, sign=1.0):
+    # operators/rope_kernels.py:56-78: first-half cos/sin, rotate the two halves; backward = -sin
+    cos, sin = cos.squeeze(), sin.squeeze()
+    seq, half = x.shape[1], x.shape[-1] // 2
+    c = cos[:seq, :half][None, :, None, :]
+    s = sin[:seq, :half][None, :, None, :] * sign
+    x1, x2 = x[..., :half].to(s.dtype), x[..., half:].to(s.dtype)
+    return torch.cat([x1 * c - x2 * s, x2 * c + x1 * s], dim=-1).to(x.dtype)
+
+
+def layer_forward_backward(x, nw1, nw2, cos, sin, weights, mask, heads, kv_heads, grad_out, *, mode, q_bit,
+                           softmax_ratio, layernorm_ratio, eps=1e-5):
+    """weights: name -> (W [out,in], A [r,in], B [out,r]) for q,k,v,o,gate,up,down (plain tensors).
+    Returns (x_out, grads) with grads = {'x': .., (name,'A'): .., (name,'B'): ..}."""
+    hd = x.shape[-1] // heads
+    n_rep = heads // kv_heads
+    At = {n: w[1].t() for n, w in weights.items()}      # [in, r]
+    Bt = {n: w[2].t() for n, w in weights.items()}      # [r, out]
+    Wt = {n: w[0].t() for n, w in weights.items()}      # [in, out]
+
+    def lora_fwd(n, inp):                                # compute_utils.py:18-25
+        main = inp @ Wt[n]
+        xa = inp @ At[n]
+        return main + xa @ Bt[n], main, xa
+
+    def lora_bwd(n, inp, xa, gy):                        # compute_utils.py:28-36
+        gmid = gy @ Bt[n].mT
+        ga = inp.mT @ gmid
+        gb = xa.mT @ gy
+        gx = gy @ Wt[n].T
+        gx = gx + gmid @ At[n].T
+        return ga, gb, gx
+
+    def cq(t):                                           # compression_pack_quant_base, calibrating
+        s = O.scale_only_quant(t, q_bit)
+        return O.compress(t, s, q_bit), s
+
+    def ccb(t):                                          # compression_pack_channel_base, calibrating
+        idx, s = O.channel_stats(t, layernorm_ratio, q_bit)
+        xo, q = O.compress_channel_base(t, s, idx, q_bit)
+        return xo, q, idx, s
+
+    # ------------------------------ forward ------------------------------
+    xn1, rstd1 = O.rmsnorm_fwd(x, nw1, eps)
+    x_sv = ccb(x)
+    q, q_main, q_xa = lora_fwd("q", xn1)
+    k, k_main, k_xa = lora_fwd("k", xn1)
+    v, v_main, v_xa = lora_fwd("v", xn1)
+    xn1_sv = cq(xn1)
+    if mode != "intra":
+        q_sv, k_sv, v_sv = cq(q_main), cq(k_main), cq(v_main)
+    q, k, v = _heads(q, heads), _heads(k, kv_heads), _heads(v, kv_heads)
+    q = _rope(q.transpose(1, 2), cos, sin).transpose(1, 2)
+    k = _rope(k.transpose(1, 2), cos, sin).transpose(1, 2)
+    k, v = _repeat(k, n_rep), _repeat(v, n_rep)
+    if mode == "intra":
+        q_sv, k_sv, v_sv = cq(q), cq(k), cq(v)           # 4-D inputs are read as [B, S, H*D]
+    s = q @ k.transpose(-2, -1) / math.sqrt(hd)
+    if mask is not None:
+        s = s + mask
+    a = torch.softmax(s, dim=-1, dtype=v.dtype)
+    thr = O.softmax_threshold(a, softmax_ratio)
+    a_idx, a_val = O.softmax_compress(a, thr)
+    a_shape = a.shape
+    o = _hidden(a @ v)
+    o_final, _, o_xa = lora_fwd("o", o)
+    o_sv = cq(o)
+    xm = x + o_final
+    xn2, rstd2 = O.rmsnorm_fwd(xm, nw2, eps)
+    xm_sv = ccb(xm)
+    if mode == "intra_inter_full_fuse":
+        gate_main, up_main = xn2 @ Wt["gate"], xn2 @ Wt["up"]
+        gate_xa, up_xa = xn2 @ At["gate"], xn2 @ At["up"]
+        gs, us = O.scale_only_quant(gate_main, q_bit), O.scale_only_quant(up_main, q_bit)
+        gq, uq, had = O.fused_fwd(gate_xa, Bt["gate"], gate_main, gs, up_xa, Bt["up"], up_main, us, q_bit)
+        had = had.to(x.device)
+    else:
+        gate, gate_main, gate_xa = lora_fwd("gate", xn2)
+        up, up_main, up_xa = lora_fwd("up", xn2)
+        if mode == "intra_inter":
+            gate_sv, up_sv = cq(gate_main), cq(up_main)
+            had = O.silu_mul(gate, up)
+        else:
+            fn = F.silu(gate)
+            gate_sv = cq(gate)
+            had = up * fn
+            up_sv, fn_sv = cq(up), cq(fn)
+    xn2_sv = cq(xn2)
+    down, _, down_xa = lora_fwd("down", had)
+    if mode == "intra":
+        had_sv = cq(had)
+    x_out = xm + down
+
+    # ------------------------------ backward ------------------------------
+    G = {}
+    dq = lambda sv, **kw: O.decompress(sv[0], sv[1], q_bit, **kw).to(x.device)
+    go = grad_out
+    if mode == "intra_inter_full_fuse":
+        G[("down", "B")] = down_xa.mT @ go
+        g_down = go @ Wt["down"].T
+        g_mid = go @ Bt["down"].T
+        g_down = g_down + g_mid @ At["down"].T
+        had_r, g_fn, g_h2 = O.fused_bwd(gate_xa, Bt["gate"], gq, gs, up_xa, Bt["up"], uq, us, g_down, q_bit)
+        G[("down", "A")] = had_r.mT @ g_mid
+    else:
+        if mode == "intra_inter":
+            gate = dq(gate_sv) + gate_xa @ Bt["gate"]
+            up = dq(up_sv) + up_xa @ Bt["up"]
+            fn = F.silu(gate)
+            had_r = up * fn
+        else:
+            had_r, up, fn, gate = dq(had_sv), dq(up_sv), dq(fn_sv), dq(gate_sv)
+        G[("down", "A")], G[("down", "B")], g_down = lora_bwd("down", had_r, down_xa, go)
+        g_h1, g_h2 = g_down * up, g_down * fn
+        g_fn = O.silu_bwd(gate, g_h1)
+    xn2_r = dq(xn2_sv)
+    G[("gate", "A")], G[("gate", "B")], g1 = lora_bwd("gate", xn2_r, gate_xa, g_fn)
+    G[("up", "A")], G[("up", "B")], g2 = lora_bwd("up", xn2_r, up_xa, g_h2)
+    g_gate_up = g2 + g1
+    xm_r = O.decompress_channel_base(xm_sv[1], xm_sv[3], xm_sv[0], xm_sv[2], q_bit)
+    g_norm2, G["nw2"] = O.rmsnorm_bwd(g_gate_up, xm_r, nw2, rstd2)
+    g_medium = g_norm2 + go
+    G[("o", "A")], G[("o", "B")], g_o = lora_bwd("o", dq(o_sv), o_xa, g_medium)
+    g_o = _heads(g_o, heads)
+    a_r = O.softmax_restore(a_idx, a_val, a_shape)
+    if mode == "intra":
+        q_r, k_r, v_r = (dq(sv, is_head=True, num_heads=heads) for sv in (q_sv, k_sv, v_sv))
+    else:
+        v_r = _repeat(_heads(dq(v_sv) + v_xa @ Bt["v"], kv_heads), n_rep)
+        q_r = _heads(dq(q_sv) + q_xa @ Bt["q"], heads)
+        q_r = _rope(q_r.transpose(1, 2), cos, sin).transpose(1, 2)
+        k_r = _heads(dq(k_sv) + k_xa @ Bt["k"], kv_heads)
+        k_r = _repeat(_rope(k_r.transpose(1, 2), cos, sin).transpose(1, 2), n_rep)
+    g_v = a_r.transpose(-2, -1) @ g_o
+    g_a = g_o @ v_r.transpose(-2, -1)
+    g_v = _repeat_bwd(g_v, n_rep)
+    g_s = O.softmax_bwd(a_r, g_a) / math.sqrt(hd)
+    g_k = _repeat_bwd(g_s.transpose(-2, -1) @ q_r, n_rep)
+    g_q = g_s @ k_r
+    g_q = _rope(g_q.transpose(1, 2), cos, sin, -1.0).transpose(1, 2)
+    g_k = _rope(g_k.transpose(1, 2), cos, sin, -1.0).transpose(1, 2)
+    g_q, g_k, g_v = _hidden(g_q), _hidden(g_k), _hidden(g_v)
+    xn1_r = dq(xn1_sv)
+    G[("q", "A")], G[("q", "B")], gx = lora_bwd("q", xn1_r, q_xa, g_q)
+    G[("k", "A")], G[("k", "B")], gt = lora_bwd("k", xn1_r, k_xa, g_k)
+    gx = gx + gt
+    G[("v", "A")], G[("v", "B")], gt = lora_bwd("v", xn1_r, v_xa, g_v)
+    gx = gx + gt
+    x_r = O.decompress_channel_base(x_sv[1], x_sv[3], x_sv[0], x_sv[2], q_bit)
+    g_norm1, G["nw1"] = O.rmsnorm_bwd(gx, x_r, nw1, rstd1)
+    G["x"] = g_norm1 + g_medium
+    return x_out, G

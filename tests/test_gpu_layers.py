@@ -1,0 +1,271 @@
+"""GPU checks of the fused decoder layers: forward output and all gradients against an uncompressed
+bf16 torch-autograd layer of the same architecture (whose RMSNorm backward is the reference's formula,
+via the oracle), for the three layer types, Llama (MHA) and Mistral (GQA) head layouts, the
+map-free attention variant, the calibration state machine and the saved-activation footprint."""
+import math
+from types import SimpleNamespace
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from helpers import BF16, rel_err_and_cos
+from oracle import hyc_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+class Lin:
+    def __init__(self, weight, bias=None):
+        self.weight, self.bias = weight, bias
+
+
+def make_layer_inputs(dev, seed, B=2, S=64, hidden=256, heads=4, kv_heads=4, inter=512, rank=16):
+    g = torch.Generator(device=dev).manual_seed(seed)
+    rn = lambda *s, sc=1.0: (torch.randn(*s, generator=g, device=dev) * sc).to(BF16)
+    hd = hidden // heads
+    dims = dict(q=(hidden, hidden), k=(kv_heads * hd, hidden), v=(kv_heads * hd, hidden), o=(hidden, hidden),
+                gate=(inter, hidden), up=(inter, hidden), down=(hidden, inter))
+    P = {}
+    for n, (out_f, in_f) in dims.items():
+        base = Lin(rn(out_f, in_f, sc=1.0 / math.sqrt(in_f)))
+        la = Lin(rn(rank, in_f, sc=1.0 / math.sqrt(in_f)).requires_grad_())
+        lb = Lin(rn(out_f, rank, sc=0.05).requires_grad_())
+        P[n] = (base, la, lb)
+    x = rn(B, S, hidden)
+    x[..., 7] *= 30           # an outlier channel, as real residual streams have
+    x.requires_grad_()
+    nw1 = (1 + 0.1 * torch.randn(hidden, generator=g, device=dev)).to(BF16).requires_grad_()
+    nw2 = (1 + 0.1 * torch.randn(hidden, generator=g, device=dev)).to(BF16).requires_grad_()
+    pos = torch.arange(S, device=dev, dtype=torch.float32)
+    inv = 1.0 / (10000 ** (torch.arange(0, hd, 2, device=dev, dtype=torch.float32) / hd))
+    ang = torch.cat([pos[:, None] * inv[None, :]] * 2, dim=-1)
+    cos, sin = ang.cos().to(BF16)[None], ang.sin().to(BF16)[None]
+    mask = torch.full((S, S), float("-inf"), device=dev).triu(1).to(BF16)[None, None]
+    grad = rn(B, S, hidden)
+    return SimpleNamespace(P=P, x=x, nw1=nw1, nw2=nw2, cos=cos, sin=sin, mask=mask, grad=grad,
+                           heads=heads, kv_heads=kv_heads, hd=hd)
+
+
+class RefRMSNorm(torch.autograd.Function):
+    """RMSNorm whose backward is the reference's formula (rmsnorm_kernels.py:92-100), from the oracle."""
+    @staticmethod
+    def forward(ctx, x, w):
+        y, rstd = O.rmsnorm_fwd(x, w, 1e-5)
+        ctx.save_for_backward(x, w, rstd)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, w, rstd = ctx.saved_tensors
+        return O.rmsnorm_bwd(dy, x, w, rstd)
+
+
+def reference_layer(t):
+    from hyclora_amd.models.compute_utils import hidden_to_head_shape, head_to_hidden_shape, repeat_kv, rope_forward
+    P = t.P
+
+    def proj(n, inp):
+        base, la, lb = P[n]
+        return inp @ base.weight.t() + (inp @ la.weight.t()) @ lb.weight.t()
+
+    xn1 = RefRMSNorm.apply(t.x, t.nw1)
+    q = hidden_to_head_shape(proj("q", xn1), t.heads)
+    k = hidden_to_head_shape(proj("k", xn1), t.kv_heads)
+    v = hidden_to_head_shape(proj("v", xn1), t.kv_heads)
+    q = rope_forward(q.transpose(1, 2), t.cos, t.sin).transpose(1, 2)
+    k = rope_forward(k.transpose(1, 2), t.cos, t.sin).transpose(1, 2)
+    k, v = repeat_kv(k, t.heads // t.kv_heads), repeat_kv(v, t.heads // t.kv_heads)
+    s = q @ k.transpose(-2, -1) / math.sqrt(t.hd) + t.mask
+    a = torch.softmax(s, dim=-1, dtype=BF16)
+    o = head_to_hidden_shape(a @ v)
+    xm = t.x + proj("o", o)
+    xn2 = RefRMSNorm.apply(xm, t.nw2)
+    had = F.silu(proj("gate", xn2)) * proj("up", xn2)
+    return xm + proj("down", had)
+
+
+def grads_of(t, out):
+    params = [t.x, t.nw1, t.nw2] + [m.weight for n in ("q", "k", "v", "o", "gate", "up", "down") for m in t.P[n][1:]]
+    for p in params:
+        p.grad = None
+    out.backward(t.grad)
+    return [p.grad.clone() if p.grad is not None else None for p in params]
+
+
+def run_fused(layer, t, use_mask=True):
+    P = t.P
+    args = [t.x, t.nw1, None, t.cos, t.sin]
+    for n in ("q", "k", "v", "o"):
+        args += list(P[n])
+    args += [t.nw2, None]
+    for n in ("gate", "up", "down"):
+        args += list(P[n])
+    args += [t.mask if use_mask else None, t.heads, t.hd, t.kv_heads]
+    return layer(*args)
+
+
+def config(layer_type, q_bit, sm_ratio=0.999, ln_ratio=0.005, thr=5):
+    return SimpleNamespace(use_hyclora=True, layer_type=layer_type, iteration_threshold=thr,
+                           softmax_outlier_ratio=sm_ratio, layernorm_outlier_ratio=ln_ratio, q_bit=q_bit)
+
+
+# Cosine floor of the gradients against the UNCOMPRESSED layer, per code width.  These are sanity
+# bounds, not parity bounds: the reference's scheme (symmetric codes with a min-max step taken from
+# batch element 0, no zero point) clips one-sided activations such as silu(gate) even at 8 bits.
+# Parity of the layer logic is checked tightly against the oracle layer below.
+COS_FLOOR = {8: 0.95, 4: 0.93, 2: 0.4}
+
+
+@pytest.mark.parametrize("layer_type", ["intra", "intra_inter", "intra_inter_full_fuse"])
+@pytest.mark.parametrize("q_bit", [8, 4, 2])
+@pytest.mark.parametrize("family", ["llama", "mistral"])
+def test_layer_matches_uncompressed_autograd(dev, layer_type, q_bit, family):
+    import hyclora_amd  # noqa: F401
+    from hyclora_amd.models import llama, mistral
+    kv = 4 if family == "llama" else 2
+    t = make_layer_inputs(dev, seed=q_bit + len(layer_type), kv_heads=kv)
+    make = llama.make_fused_llama_layer if family == "llama" else mistral.make_fused_mistral_layer
+    layer = make(config(layer_type, q_bit))
+    assert type(layer).__name__.startswith("FusedLlama" if family == "llama" else "FusedMistral")
+    ref_out = reference_layer(t)
+    ref_grads = grads_of(t, ref_out)
+    out = run_fused(layer, t)
+    rel, cos = rel_err_and_cos(out, ref_out)
+    assert rel <= 1e-2 and cos >= 0.9999, f"forward: rel {rel:.2e} cos {cos:.6f}"   # forward is not compressed
+    grads = grads_of(t, out)
+    names = ["x", "norm_w1", "norm_w2"] + [f"{n}.lora_{ab}" for n in ("q", "k", "v", "o", "gate", "up", "down") for ab in "AB"]
+    for name, gq, gr in zip(names, grads, ref_grads):
+        if name.startswith("norm_w"):
+            assert gq is None or gq.shape == gr.shape       # map variant: norm weights are frozen in the reference
+            continue
+        assert gq is not None and gq.shape == gr.shape, name
+        rel, cos = rel_err_and_cos(gq, gr)
+        assert cos >= COS_FLOOR[q_bit], f"{layer_type} q{q_bit} grad {name}: rel {rel:.2e} cos {cos:.5f}"
+
+
+@pytest.mark.parametrize("layer_type", ["intra", "intra_inter", "intra_inter_full_fuse"])
+@pytest.mark.parametrize("q_bit", [8, 4, 2])
+@pytest.mark.parametrize("kv_heads", [4, 2])
+def test_layer_matches_oracle_layer(dev, layer_type, q_bit, kv_heads):
+    """Same compression semantics on both sides: the fused layer (HIP kernels) against the oracle's
+    restatement of the reference layer (plain torch + oracle element functions, same device so the
+    GEMMs agree).  What is saved, how it is restored and the order of the recomputation must match."""
+    import hyclora_amd  # noqa: F401
+    from hyclora_amd.models import llama
+    from oracle import layer_oracle
+    t = make_layer_inputs(dev, seed=17 + q_bit, kv_heads=kv_heads)
+    layer = llama.make_fused_llama_layer(config(layer_type, q_bit, sm_ratio=0.05))
+    out = run_fused(layer, t)
+    grads = grads_of(t, out)
+    weights = {n: tuple(m.weight.detach() for m in t.P[n]) for n in t.P}
+    with torch.no_grad():
+        ref_out, G = layer_oracle.layer_forward_backward(
+            t.x.detach(), t.nw1.detach(), t.nw2.detach(), t.cos, t.sin, weights, t.mask, t.heads, t.kv_heads,
+            t.grad, mode=layer_type, q_bit=q_bit, softmax_ratio=0.05, layernorm_ratio=0.005)
+    rel, cos = rel_err_and_cos(out, ref_out)
+    assert rel <= 1e-2 and cos >= 0.9999
+    expect = [G["x"], None, None]
+    for n in ("q", "k", "v", "o", "gate", "up", "down"):
+        expect += [G[(n, "A")].sum(0).t(), G[(n, "B")].sum(0).t()]
+    names = ["x", "norm_w1", "norm_w2"] + [f"{n}.lora_{ab}" for n in ("q", "k", "v", "o", "gate", "up", "down") for ab in "AB"]
+    for name, got, want in zip(names, grads, expect):
+        if want is None:
+            continue
+        rel, cos = rel_err_and_cos(got, want)
+        # the two sides run the same GEMMs, but a recomputed bf16 value that differs in its last bit
+        # can flip a code, and one flipped 2-bit code is a quarter of the range
+        rel_tol = 0.2 if q_bit == 2 else 2e-2
+        assert rel <= rel_tol and cos >= 0.999, f"{layer_type} q{q_bit} kv{kv_heads} grad {name}: rel {rel:.2e} cos {cos:.5f}"
+
+
+def test_sdpa_variant_and_norm_weight_grads(dev):
+    import hyclora_amd  # noqa: F401
+    from hyclora_amd.models import llama_flash_attn as lf
+    t = make_layer_inputs(dev, seed=3)
+    ref_out = reference_layer(t)
+    ref_grads = grads_of(t, ref_out)
+    for cls in (lf.FusedLlamaLayerIntraInter, lf.FusedLlamaLayerIntra, lf.FusedLlamaLayerIntraInterFullFuse):
+        layer = cls()
+        layer.set_hyclora_config(config(layer.layer_type, 8))
+        out = run_fused(layer, t, use_mask=False)            # causal attention without a materialised mask
+        rel, cos = rel_err_and_cos(out, ref_out)
+        assert rel <= 1e-2 and cos >= 0.9999
+        grads = grads_of(t, out)
+        for i, (gq, gr) in enumerate(zip(grads, ref_grads)):
+            assert gq is not None
+            rel, cos = rel_err_and_cos(gq, gr)
+            assert cos >= COS_FLOOR[8], f"{cls.__name__} grad #{i}: rel {rel:.2e} cos {cos:.5f}"
+        assert layer.static_value['q']['zero_point'] is not None and 'a' not in layer.static_value
+
+
+def test_calibration_state_machine(dev):
+    import hyclora_amd  # noqa: F401
+    from hyclora_amd.models import FusedLlamaLayerIntraInterFullFuse
+    t = make_layer_inputs(dev, seed=11)
+    layer = FusedLlamaLayerIntraInterFullFuse()
+    layer.set_hyclora_config(config("intra_inter_full_fuse", 4, thr=2))
+    assert layer.static_value['x']['scale'] is None
+    run_fused(layer, t)
+    s0 = layer.static_value['gate']['scale'].clone()
+    idx0 = layer.static_value['x']['outlier_channel_index'].clone()
+    assert layer.iteration == 1 and 7 in idx0.tolist()
+    t2 = make_layer_inputs(dev, seed=12)
+    run_fused(layer, t2)                                      # second calibration step: running mean
+    assert layer.iteration == 2
+    s1 = layer.static_value['gate']['scale']
+    assert s1.dtype == BF16 and not torch.equal(s1, s0)
+    frozen = {k: {f: (v.clone() if torch.is_tensor(v) else v) for f, v in d.items()} for k, d in layer.static_value.items()}
+    out = run_fused(layer, t)                                 # past the threshold: statistics are frozen
+    out.backward(t.grad)
+    assert layer.iteration == 3
+    for k, d in layer.static_value.items():
+        for f, v in d.items():
+            assert torch.equal(v, frozen[k][f]), (k, f)
+    with pytest.raises(ValueError):
+        from hyclora_amd.models.llama import make_fused_llama_layer
+        make_fused_llama_layer(config("no_such_type", 4))
+
+
+def _saved_activation_bytes(fn):
+    seen = {}
+
+    def pack(t):
+        if not isinstance(t, torch.nn.Parameter) and not getattr(t, "_is_weight", False):
+            seen[(t.data_ptr(), t.numel() * t.element_size())] = t.numel() * t.element_size()
+        return t
+
+    with torch.autograd.graph.saved_tensors_hooks(pack, lambda t: t):
+        fn()
+    return sum(seen.values())
+
+
+def test_saved_activation_footprint(dev):
+    # configuration 5 in small: map-free attention, q_bit 4; the compressed layer must keep far fewer
+    # activation bytes alive than the uncompressed bf16 layer
+    import hyclora_amd  # noqa: F401
+    from hyclora_amd.models import llama_flash_attn as lf
+    t = make_layer_inputs(dev, seed=5, B=1, S=256, hidden=512, heads=8, kv_heads=8, inter=1376)
+    weights = {id(m.weight) for n in t.P for m in t.P[n]} | {id(t.nw1), id(t.nw2), id(t.cos), id(t.sin)}
+    layer = lf.FusedLlamaLayerIntraInter()
+    layer.set_hyclora_config(config("intra_inter", 4))
+    holder = {}
+
+    def count(fn):
+        total = 0
+
+        def pack(x):
+            nonlocal total
+            base = x._base if x._base is not None else x
+            if id(x) not in weights and id(base) not in weights and not any(x.data_ptr() == m.weight.data_ptr() for n in t.P for m in t.P[n]):
+                total += x.numel() * x.element_size()
+            return x
+        with torch.autograd.graph.saved_tensors_hooks(pack, lambda x: x):
+            holder["out"] = fn()
+        return total
+
+    fused_bytes = count(lambda: run_fused(layer, t, use_mask=False))
+    B, S, Hd, I, R = 1, 256, 512, 1376, 16
+    T = B * S
+    baseline = 8 * T * Hd * 2 + 4 * T * I * 2 + 7 * T * R * 2          # the bf16 save list of the uncompressed layer
+    assert fused_bytes < 0.4 * baseline, (fused_bytes, baseline)
