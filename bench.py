@@ -42,9 +42,130 @@ def parse():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU-oracle timing (for profiler runs)")
-    ap.add_argument("--only", choices=["all", "roundtrip", "quant", "fused", "copy"], default="all",
+    ap.add_argument("--only", choices=["all", "roundtrip", "quant", "fused", "copy", "layers"], default="all",
                     help="restrict the run to one part (for profiler runs)")
     return ap.parse_args()
+
+
+def bench_layers(torch, dev):
+    """Forward+backward of one decoder layer with random-init bf16 weights N(0, 0.02) and LoRA r=16 on
+    all seven linears: the compressed layer of this package against an uncompressed bf16
+    torch-autograd layer of the same architecture, with the activation bytes each keeps for backward."""
+    import math
+    from types import SimpleNamespace
+
+    import torch.nn.functional as F
+
+    from hyclora_amd.models import llama, llama_flash_attn, mistral
+    from hyclora_amd.models.compute_utils import (head_to_hidden_shape, hidden_to_head_shape, repeat_kv,
+                                                  rope_forward)
+    BF16 = torch.bfloat16
+    gen = torch.Generator(device=dev).manual_seed(1)
+
+    class Lin:
+        def __init__(self, w):
+            self.weight, self.bias = w, None
+
+    def make(B, S, hidden, heads, kv, inter, theta, rank=16):
+        rn = lambda *s, sc: (torch.randn(*s, generator=gen, device=dev) * sc).to(BF16)
+        hd = hidden // heads
+        dims = dict(q=(hidden, hidden), k=(kv * hd, hidden), v=(kv * hd, hidden), o=(hidden, hidden),
+                    gate=(inter, hidden), up=(inter, hidden), down=(hidden, inter))
+        P = {}
+        for n, (o_f, i_f) in dims.items():
+            a = torch.empty(rank, i_f, device=dev)
+            torch.nn.init.kaiming_uniform_(a, a=math.sqrt(5), generator=gen)
+            P[n] = (Lin(rn(o_f, i_f, sc=0.02)), Lin(a.to(BF16).requires_grad_()), Lin(rn(o_f, rank, sc=1e-3).requires_grad_()))
+        x = rn(B, S, hidden, sc=1.0).requires_grad_()
+        nw1 = torch.ones(hidden, device=dev, dtype=BF16)
+        nw2 = torch.ones(hidden, device=dev, dtype=BF16)
+        pos = torch.arange(S, device=dev, dtype=torch.float32)
+        inv = 1.0 / (theta ** (torch.arange(0, hd, 2, device=dev, dtype=torch.float32) / hd))
+        ang = torch.cat([pos[:, None] * inv[None, :]] * 2, dim=-1)
+        return SimpleNamespace(P=P, x=x, nw1=nw1, nw2=nw2, cos=ang.cos().to(BF16)[None], sin=ang.sin().to(BF16)[None],
+                               grad=rn(B, S, hidden, sc=1.0), heads=heads, kv=kv, hd=hd, S=S)
+
+    def run_fused(layer, t, mask):
+        args = [t.x, t.nw1, None, t.cos, t.sin]
+        for n in ("q", "k", "v", "o"):
+            args += list(t.P[n])
+        args += [t.nw2, None]
+        for n in ("gate", "up", "down"):
+            args += list(t.P[n])
+        return layer(*args, mask, t.heads, t.hd, t.kv)
+
+    def run_plain(t, mask, sdpa):
+        def proj(n, inp):
+            base, la, lb = t.P[n]
+            return inp @ base.weight.t() + (inp @ la.weight.t()) @ lb.weight.t()
+        rms = lambda v, w: (v.float() * torch.rsqrt(v.float().pow(2).mean(-1, keepdim=True) + 1e-5)).to(BF16) * w
+        xn = rms(t.x, t.nw1)
+        q, k, v = (hidden_to_head_shape(proj(n, xn), h) for n, h in (("q", t.heads), ("k", t.kv), ("v", t.kv)))
+        q = rope_forward(q.transpose(1, 2), t.cos, t.sin).transpose(1, 2)
+        k = rope_forward(k.transpose(1, 2), t.cos, t.sin).transpose(1, 2)
+        k, v = repeat_kv(k, t.heads // t.kv), repeat_kv(v, t.heads // t.kv)
+        if sdpa:
+            o = F.scaled_dot_product_attention(q, k, v, is_causal=True)
+        else:
+            a = torch.softmax(q @ k.transpose(-2, -1) / math.sqrt(t.hd) + mask, dim=-1, dtype=BF16)
+            o = a @ v
+        xm = t.x + proj("o", head_to_hidden_shape(o))
+        xn2 = rms(xm, t.nw2)
+        return xm + proj("down", F.silu(proj("gate", xn2)) * proj("up", xn2))
+
+    def measure(fn, t, steps=5, warmup=2):
+        weights = {m.weight.data_ptr() for n in t.P for m in t.P[n]} | {t.nw1.data_ptr(), t.nw2.data_ptr(), t.cos.data_ptr(), t.sin.data_ptr()}
+        seen = {}
+
+        def pack(v):
+            if v.data_ptr() not in weights:
+                seen[(v.data_ptr(), v.numel())] = v.numel() * v.element_size()
+            return v
+        with torch.autograd.graph.saved_tensors_hooks(pack, lambda v: v):
+            y = fn()                                  # what the forward keeps alive for backward
+        saved = sum(seen.values())
+        y.backward(t.grad)
+        for _ in range(warmup):
+            fn().backward(t.grad)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            fn().backward(t.grad)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / steps, saved
+
+    cfg = lambda lt, q: SimpleNamespace(use_hyclora=True, layer_type=lt, iteration_threshold=2,
+                                        softmax_outlier_ratio=0.05, layernorm_outlier_ratio=0.005, q_bit=q)
+    out = {}
+    cases = [("config2_llama7b_b4_s1024_full_fuse", dict(B=4, S=1024, hidden=4096, heads=32, kv=32, inter=11008, theta=1e4),
+              llama.make_fused_llama_layer, "intra_inter_full_fuse", [4], False),
+             ("config4_mistral7b_b2_s2048_full_fuse", dict(B=2, S=2048, hidden=4096, heads=32, kv=8, inter=14336, theta=1e6),
+              mistral.make_fused_mistral_layer, "intra_inter_full_fuse", [2, 4, 8], False),
+             ("config5_llama7b_b1_s8192_mapfree_intra_inter", dict(B=1, S=8192, hidden=4096, heads=32, kv=32, inter=11008, theta=1e4),
+              None, "intra_inter", [4], True)]
+    for name, dims, maker, lt, qbits, sdpa in cases:
+        t = make(**dims)
+        mask = None if sdpa else torch.full((t.S, t.S), float("-inf"), device=dev).triu(1).to(BF16)[None, None]
+        ms_p, saved_p = measure(lambda: run_plain(t, mask, sdpa), t)
+        entry = {"bf16_uncompressed": {"fwd_bwd_ms": ms_p, "saved_activation_MB": saved_p / 1e6}}
+        for q in qbits:
+            if maker is None:
+                layer = llama_flash_attn.FusedLlamaLayerIntraInter()
+                layer.set_hyclora_config(cfg(lt, q))
+            else:
+                layer = maker(cfg(lt, q))
+            for _ in range(3):                       # run past calibration so the steady state is timed
+                run_fused(layer, t, mask).backward(t.grad)
+            ms_f, saved_f = measure(lambda: run_fused(layer, t, mask), t)
+            entry[f"compressed_q{q}"] = {"fwd_bwd_ms": ms_f, "saved_activation_MB": saved_f / 1e6,
+                                         "saved_vs_bf16": saved_p / max(saved_f, 1)}
+            del layer
+        out[name] = entry
+        del t, mask
+        torch.cuda.empty_cache()
+    return out
 
 
 def main():
@@ -239,12 +360,21 @@ def main():
         kernels["softmax_bwd"] = {"ms": ms, "GBps": 6 * Ea / ms / 1e6}
         del a, g_a, idx_a, val_a
 
+    # ---- whole decoder layers (BASELINE configurations 2, 4, 5): fwd+bwd ms and saved bytes ----
+    layers = None
+    want_cpu = args.only == "all" and not args.skip_cpu
+    if want_cpu:
+        x_cpu, s_cpu = xs[0].cpu(), scale.cpu().reshape(1, -1)
+    if args.only in ("all", "layers"):
+        for buffers in (xs, qs, xh):
+            buffers.clear()
+        torch.cuda.empty_cache()
+        layers = bench_layers(torch, dev)
+
     # ---- CPU baseline: the oracle on the host cores, same tensor --------------------------------
     cpu = None
-    if args.only == "all" and not args.skip_cpu:
+    if want_cpu:
         from oracle import hyc_oracle as O
-        x_cpu = xs[0].cpu()
-        s_cpu = scale.cpu().reshape(1, -1)
         torch.set_num_threads(os.cpu_count() or 1)
         O.decompress(O.compress(x_cpu[:1, :64], s_cpu, QB), s_cpu, QB)      # warm-up
         t0 = time.perf_counter()
@@ -280,6 +410,7 @@ def main():
         "cpu_baseline": cpu,
         "fused": fused,
         "kernels": kernels,
+        "layers": layers,
     }
     print(json.dumps(line))
 

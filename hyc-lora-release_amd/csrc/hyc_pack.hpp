@@ -13,11 +13,12 @@
 
 namespace hyc {
 
-// Per-lane column constants of the quantiser: step, reciprocal, the input clamp of the
-// reciprocal path, and whether every one of the lane's 8 steps may use that path.
+// Per-lane column constants of the quantiser: step, reciprocal, the upper input clamp of the
+// reciprocal path (the lower one is -xhi - s), and whether every one of the lane's 8 steps
+// may use that path.
 template <int QBIT>
 struct QuantCols {
-    float s[8], r[8], xlo[8], xhi[8];
+    float s[8], r[8], xhi[8];
     bool fast;
     __device__ __forceinline__ void load(const uint16_t* scale, int col0, bool active) {
         u32x4 sv = {0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};   // 1.0 for idle lanes
@@ -27,7 +28,6 @@ struct QuantCols {
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             r[j] = 1.0f / s[j];
-            xlo[j] = hyc_clamp_lo(s[j], QBIT);
             xhi[j] = hyc_clamp_hi(s[j], QBIT);
             fast = fast && hyc_scale_is_fast(s[j]);
         }
@@ -43,7 +43,7 @@ __device__ __forceinline__ void codes_to_words(const float (&f)[8], const QuantC
         // (sums of shifted two's-complement values, exact modulo 2^32)
         uint32_t c[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) c[j] = (uint32_t)hyc_signed_code_fast(f[j], q.s[j], q.r[j], q.xlo[j], q.xhi[j]);
+        for (int j = 0; j < 8; ++j) c[j] = (uint32_t)hyc_signed_code_fast(f[j], q.s[j], q.r[j], hyc_clamp_lo_from_hi(q.xhi[j], q.s[j]), q.xhi[j]);
         constexpr uint32_t bias = 0x01010101u * (1u << (QBIT - 1));
         lo = c[0] + (c[1] << 8) + (c[2] << 16) + (c[3] << 24) + bias;
         hi = c[4] + (c[5] << 8) + (c[6] << 16) + (c[7] << 24) + bias;

@@ -92,8 +92,11 @@ HYC_HD int hyc_code_from_t(float t, int q_bit) {
 // code 0); a compare-and-select is used rather than fmaxf because fmaxf turns a
 // *signalling* NaN into a quiet NaN instead of dropping it.
 // The sign for the half-away rounding is taken from the clamped input (s > 0 here).
-HYC_HD float hyc_clamp_lo(float s, int q_bit) { return (-(float)(1 << (q_bit - 1)) - 0.49f) * s; }
+// The lower bound is derived from the upper one (lo - 0.49 = -(hi + 0.49) - 1), so a kernel
+// that is short of registers keeps only xhi and recomputes xlo = -xhi - s on the fly.
 HYC_HD float hyc_clamp_hi(float s, int q_bit) { return ((float)(1 << (q_bit - 1)) - 1.0f + 0.49f) * s; }
+HYC_HD float hyc_clamp_lo_from_hi(float xhi, float s) { return -xhi - s; }
+HYC_HD float hyc_clamp_lo(float s, int q_bit) { return hyc_clamp_lo_from_hi(hyc_clamp_hi(s, q_bit), s); }
 
 HYC_HD int hyc_signed_code_fast(float x, float s, float r, float xlo, float xhi) {
     float xc = (x > xlo) ? x : xlo;
