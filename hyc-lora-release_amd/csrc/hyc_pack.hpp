@@ -63,40 +63,60 @@ __device__ __forceinline__ void codes_to_words(const float (&f)[8], const QuantC
     }
 }
 
-// Merge the quad's code words into packed bytes and store this lane's share of them.
-// Every lane of the quad must call this (the exchange is a DPP quad permute); `active`
-// only gates the store.  qrow = first packed byte of the row.
-template <int QBIT, bool NT = false>
-__device__ __forceinline__ void store_packed(uint8_t* qrow, int chunk, bool active, uint32_t lo, uint32_t hi) {
+// Merge the quad's code words into packed bytes; on return (lo, hi) hold what this lane stores:
+// q=8 both dwords, q=4 and q=2 one dword (returned in lo).  Every lane of the quad must call this
+// (the exchange is a DPP quad permute).
+template <int QBIT>
+__device__ __forceinline__ void merge_packed(int chunk, uint32_t& lo, uint32_t& hi) {
     const int quad = chunk & 3;
-    const int blk = chunk >> 2;
-    if constexpr (QBIT == 8) {
-        if (active) {
-            if constexpr (NT) st8_nt(qrow + (int64_t)chunk * 8, u32x2{lo, hi});
-            else st8(qrow + (int64_t)chunk * 8, u32x2{lo, hi});
-        }
-    } else if constexpr (QBIT == 4) {
+    if constexpr (QBIT == 4) {
         const int sub = quad >> 1;
         lo <<= 4 * sub;
         hi <<= 4 * sub;
         lo |= quad_xor2(lo);
         hi |= quad_xor2(hi);
-        if (active) {
-            if constexpr (NT) st4_nt(qrow + blk * 16 + 8 * (quad & 1) + 4 * sub, sub ? hi : lo);
-            else *reinterpret_cast<uint32_t*>(qrow + blk * 16 + 8 * (quad & 1) + 4 * sub) = sub ? hi : lo;
-        }
-    } else {
+        lo = sub ? hi : lo;
+    } else if constexpr (QBIT == 2) {
         lo <<= 2 * quad;
         hi <<= 2 * quad;
         lo |= quad_xor1(lo);
         hi |= quad_xor1(hi);
         lo |= quad_xor2(lo);
         hi |= quad_xor2(hi);
-        if (active && quad < 2) {
-            if constexpr (NT) st4_nt(qrow + blk * 8 + 4 * quad, quad ? hi : lo);
-            else *reinterpret_cast<uint32_t*>(qrow + blk * 8 + 4 * quad) = quad ? hi : lo;
-        }
+        lo = (quad & 1) ? hi : lo;
     }
+}
+
+// Byte offset inside a packed row of what merge_packed left in this lane, and whether this
+// lane stores at all (at q=2 only two lanes of the quad do).
+template <int QBIT>
+__device__ __forceinline__ int packed_store_offset(int chunk) {
+    const int quad = chunk & 3, blk = chunk >> 2;
+    if constexpr (QBIT == 8) return chunk * 8;
+    else if constexpr (QBIT == 4) return blk * 16 + 8 * (quad & 1) + 4 * (quad >> 1);
+    else return blk * 8 + 4 * (quad & 1);
+}
+template <int QBIT>
+__device__ __forceinline__ bool packed_store_lane(int chunk) { return QBIT != 2 || (chunk & 3) < 2; }
+
+template <int QBIT, bool NT = false>
+__device__ __forceinline__ void store_merged(uint8_t* qrow, int chunk, bool active, uint32_t lo, uint32_t hi) {
+    if (!(active && packed_store_lane<QBIT>(chunk))) return;
+    uint8_t* p = qrow + packed_store_offset<QBIT>(chunk);
+    if constexpr (QBIT == 8) {
+        if constexpr (NT) st8_nt(p, u32x2{lo, hi});
+        else st8(p, u32x2{lo, hi});
+    } else {
+        if constexpr (NT) st4_nt(p, lo);
+        else *reinterpret_cast<uint32_t*>(p) = lo;
+    }
+}
+
+// merge + store in one step
+template <int QBIT, bool NT = false>
+__device__ __forceinline__ void store_packed(uint8_t* qrow, int chunk, bool active, uint32_t lo, uint32_t hi) {
+    merge_packed<QBIT>(chunk, lo, hi);
+    store_merged<QBIT, NT>(qrow, chunk, active, lo, hi);
 }
 
 // Where a chunk's codes sit inside a packed row: the 8 bytes at `offset`, each shifted

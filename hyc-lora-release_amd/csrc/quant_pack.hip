@@ -23,6 +23,8 @@
 // on the dequantiser, whose stores otherwise evict useful lines.  The packed codes are stored
 // non-temporally but LOADED normally: neighbouring lanes read the same 8 bytes and rely on
 // the cache to merge those requests.
+#include <type_traits>
+
 #include "hyc_pack.hpp"
 
 namespace hyc {
@@ -117,30 +119,49 @@ __device__ __forceinline__ int64_t chunk_offset(int col0, int head_dim, int64_t 
 // ------------------------------------------------------------------------------------
 // quantise + pack
 // ------------------------------------------------------------------------------------
-template <int QBIT, bool ZP, bool OUTL, bool FAST>
+// Loads the lane's chunk of kRowUnroll consecutive rows starting at the cursor (rows at or past
+// row1 are skipped) and advances the cursor.
+template <bool FULL>
+__device__ __forceinline__ void load_rows(const QuantArgs& a, RowCursor& cur, int64_t t0, int64_t row1, bool active,
+                                          int64_t coff, u32x4 (&v)[kRowUnroll]) {
+#pragma unroll
+    for (int u = 0; u < kRowUnroll; ++u) {
+        if constexpr (FULL) {
+            v[u] = ld16_nt(a.x + cur.off + coff);
+        } else {
+            v[u] = u32x4{0, 0, 0, 0};
+            if (active && t0 + u < row1) v[u] = ld16_nt(a.x + cur.off + coff);
+        }
+        cur.next(a.M, a.stride_b, a.stride_m);
+    }
+}
+
+// Order of memory operations inside the strip loop: the loads of the NEXT row group are issued
+// before the stores of the current one.  The hardware counts loads and stores with one in-order
+// counter (vmcnt), so waiting for loads that were issued after stores also waits for those stores;
+// issuing the loads first lets the wave wait for its data while its stores are still in flight.
+// The loaded registers are free by then (the codes of the current group are already packed), so
+// this costs no extra registers.
+//
+// FULL = the wave's tile lies completely inside the tensor (all 64 lanes active, the strip is a
+// whole number of row groups).  That variant has no predicates or branches around its memory
+// operations, which is what lets the compiler count outstanding operations exactly and emit
+// s_waitcnt vmcnt(<stores in flight>) instead of vmcnt(0) at the top of the loop.
+template <int QBIT, bool ZP, bool OUTL, bool FAST, bool FULL>
 __device__ __forceinline__ void quant_rows(const QuantArgs& a, int64_t row0, int64_t row1, bool active, int chunk,
                                            int64_t coff, const QuantCols<QBIT>& qc, const float (&z)[8],
                                            const OutlierLane& ol) {
     const int row_bytes = a.N * QBIT / 8;
     if (row0 >= row1) return;
     RowCursor cur(row0, a.M, a.stride_b, a.stride_m);
-    for (int64_t t0 = row0; t0 < row1; t0 += kRowUnroll) {
-        u32x4 v[kRowUnroll];
-        uint16_t* xrow[kRowUnroll];
+    u32x4 v[kRowUnroll];
+    load_rows<FULL>(a, cur, row0, row1, active, coff, v);
+    auto compute = [&](int64_t t0, uint32_t (&lo)[kRowUnroll], uint32_t (&hi)[kRowUnroll]) {
 #pragma unroll
         for (int u = 0; u < kRowUnroll; ++u) {
             const int64_t t = t0 + u;
-            xrow[u] = a.x + cur.off + coff;
-            v[u] = u32x4{0, 0, 0, 0};
-            if (active && t < row1) v[u] = ld16_nt(xrow[u]);
-            cur.next(a.M, a.stride_b, a.stride_m);
-        }
-#pragma unroll
-        for (int u = 0; u < kRowUnroll; ++u) {
-            const int64_t t = t0 + u;
-            if (t >= row1) break;          // uniform across the wave
             if constexpr (OUTL) {
-                if (ol.mask) {
+                if (ol.mask && (FULL || (active && t < row1))) {
                     uint32_t d[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
 #pragma unroll
                     for (int j = 0; j < 8; ++j) {
@@ -148,7 +169,10 @@ __device__ __forceinline__ void quant_rows(const QuantArgs& a, int64_t row0, int
                             const uint32_t sh = 16 * (j & 1);
                             a.xo[t * a.k + outlier_pos(ol, j)] = (uint16_t)(d[j >> 1] >> sh);
                             d[j >> 1] &= ~(0xffffu << sh);
-                            if (a.zero_input) xrow[u][j] = 0;
+                            if (a.zero_input) {
+                                const RowCursor here(t, a.M, a.stride_b, a.stride_m);
+                                a.x[here.off + coff + j] = 0;
+                            }
                         }
                     }
                     v[u] = u32x4{d[0], d[1], d[2], d[3]};
@@ -156,11 +180,34 @@ __device__ __forceinline__ void quant_rows(const QuantArgs& a, int64_t row0, int
             }
             float f[8];
             unpack8(v[u], f);
-            uint32_t lo, hi;
-            codes_to_words<QBIT, ZP, FAST>(f, qc, z, lo, hi);
-            store_packed<QBIT, true>(a.q + t * row_bytes, chunk, active, lo, hi);
+            codes_to_words<QBIT, ZP, FAST>(f, qc, z, lo[u], hi[u]);
+            merge_packed<QBIT>(chunk, lo[u], hi[u]);       // rows past row1 hold zeros; never stored
         }
+    };
+    auto store = [&](int64_t t0, const uint32_t (&lo)[kRowUnroll], const uint32_t (&hi)[kRowUnroll]) {
+#pragma unroll
+        for (int u = 0; u < kRowUnroll; ++u) {
+            const int64_t t = t0 + u;
+            store_merged<QBIT, true>(a.q + t * row_bytes, chunk, FULL || (active && t < row1), lo[u], hi[u]);
+        }
+    };
+    // The first group is peeled so that the loop is always entered with "4 loads, then 4 stores"
+    // outstanding, the same state its back edge carries; otherwise the wait at the loop top has
+    // to cover the entry case (loads only) and ends up waiting for the stores as well.
+    uint32_t lo[kRowUnroll], hi[kRowUnroll];
+    int64_t t0 = row0;
+    compute(t0, lo, hi);
+    if (t0 + kRowUnroll < row1) {
+        load_rows<FULL>(a, cur, t0 + kRowUnroll, row1, active, coff, v);
+        store(t0, lo, hi);
+        for (t0 += kRowUnroll; t0 + kRowUnroll < row1; t0 += kRowUnroll) {
+            compute(t0, lo, hi);
+            load_rows<FULL>(a, cur, t0 + kRowUnroll, row1, active, coff, v);
+            store(t0, lo, hi);
+        }
+        compute(t0, lo, hi);                                   // last group: nothing left to load
     }
+    store(t0, lo, hi);
 }
 
 template <int QBIT, bool ZP, bool OUTL>
@@ -189,11 +236,15 @@ __global__ __launch_bounds__(kQuantThreads) void quant_pack_kernel(const QuantAr
     int64_t row1 = row0 + a.rows_per_wave;
     if (row1 > a.T) row1 = a.T;
 
+    const bool full = (col_tile + 1) * kWave <= a.C && row1 - row0 == a.rows_per_wave &&
+                      a.rows_per_wave % kRowUnroll == 0;      // uniform across the wave
     // one slow column anywhere in the wave sends the whole wave down the IEEE-division path
     if (ZP || __ballot(!qc.fast) != 0ull)
-        quant_rows<QBIT, ZP, OUTL, false>(a, row0, row1, active, chunk, coff, qc, z, ol);
+        quant_rows<QBIT, ZP, OUTL, false, false>(a, row0, row1, active, chunk, coff, qc, z, ol);
+    else if (full)
+        quant_rows<QBIT, ZP, OUTL, true, true>(a, row0, row1, active, chunk, coff, qc, z, ol);
     else
-        quant_rows<QBIT, ZP, OUTL, true>(a, row0, row1, active, chunk, coff, qc, z, ol);
+        quant_rows<QBIT, ZP, OUTL, true, false>(a, row0, row1, active, chunk, coff, qc, z, ol);
 }
 
 // ------------------------------------------------------------------------------------
@@ -233,52 +284,84 @@ __global__ __launch_bounds__(kQuantThreads) void unpack_dequant_kernel(const Qua
     const PackedSlot<QBIT> slot(chunk);
 
     if (row0 >= row1) return;
-    RowCursor cur(row0, a.M, a.stride_b, a.stride_m);
-    for (int64_t t0 = row0; t0 < row1; t0 += kRowUnroll) {
+    const bool full = (col_tile + 1) * kWave <= a.C && row1 - row0 == a.rows_per_wave &&
+                      a.rows_per_wave % kRowUnroll == 0;      // uniform: no predicate needed anywhere
+    auto run = [&](auto full_tag) {
+        constexpr bool FULL = decltype(full_tag)::value;
+        RowCursor cur(row0, a.M, a.stride_b, a.stride_m);
         u32x2 w[kRowUnroll];
+        auto load_codes = [&](int64_t t0) {
 #pragma unroll
-        for (int u = 0; u < kRowUnroll; ++u) {
-            const int64_t t = t0 + u;
-            w[u] = u32x2{0, 0};
-            if (active && t < row1) w[u] = ld8(a.q + t * row_bytes + slot.offset);
-        }
-#pragma unroll
-        for (int u = 0; u < kRowUnroll; ++u) {
-            const int64_t t = t0 + u;
-            if (t >= row1) break;
-            float c[8], f[8];
-            slot.decode(w[u], c);
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                if constexpr (ZP) {
-                    // bf16 arithmetic step by step: (c - 2^(q-1)) is exact, minus z rounds to bf16
-                    f[j] = rbf((c[j] - kHalf) - z[j]) * s[j];
+            for (int u = 0; u < kRowUnroll; ++u) {
+                if constexpr (FULL) {
+                    w[u] = ld8(a.q + (t0 + u) * row_bytes + slot.offset);
                 } else {
-                    // not fma(c, s, -2^(q-1) s): that loses the sign of zero and turns an
-                    // infinite step into NaN where the reference's product does not
-                    f[j] = (c[j] - kHalf) * s[j];
+                    w[u] = u32x2{0, 0};
+                    if (active && t0 + u < row1) w[u] = ld8(a.q + (t0 + u) * row_bytes + slot.offset);
                 }
             }
-            u32x4 o = pack8(f);
-            uint16_t* xrow = a.x + cur.off + coff;
-            cur.next(a.M, a.stride_b, a.stride_m);
-            if constexpr (OUTL) {
-                if (ol.mask) {
-                    uint32_t d[4] = {o.x, o.y, o.z, o.w};
+        };
+        u32x4 o[kRowUnroll];
+        uint16_t* xrow[kRowUnroll];
+        auto compute = [&](int64_t t0) {
 #pragma unroll
-                    for (int j = 0; j < 8; ++j) {
-                        if (ol.mask & (1u << j)) {
-                            const uint32_t sh = 16 * (j & 1);
-                            const uint32_t val = a.xo[t * a.k + outlier_pos(ol, j)];
-                            d[j >> 1] = (d[j >> 1] & ~(0xffffu << sh)) | (val << sh);
-                        }
+            for (int u = 0; u < kRowUnroll; ++u) {
+                const int64_t t = t0 + u;
+                float c[8], f[8];
+                slot.decode(w[u], c);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    if constexpr (ZP) {
+                        // bf16 arithmetic step by step: (c - 2^(q-1)) is exact, minus z rounds to bf16
+                        f[j] = rbf((c[j] - kHalf) - z[j]) * s[j];
+                    } else {
+                        // not fma(c, s, -2^(q-1) s): that loses the sign of zero and turns an
+                        // infinite step into NaN where the reference's product does not
+                        f[j] = (c[j] - kHalf) * s[j];
                     }
-                    o = u32x4{d[0], d[1], d[2], d[3]};
+                }
+                o[u] = pack8(f);
+                xrow[u] = a.x + cur.off + coff;
+                cur.next(a.M, a.stride_b, a.stride_m);
+                if constexpr (OUTL) {
+                    if (ol.mask && (FULL || (active && t < row1))) {
+                        uint32_t d[4] = {o[u].x, o[u].y, o[u].z, o[u].w};
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) {
+                            if (ol.mask & (1u << j)) {
+                                const uint32_t sh = 16 * (j & 1);
+                                const uint32_t val = a.xo[t * a.k + outlier_pos(ol, j)];
+                                d[j >> 1] = (d[j >> 1] & ~(0xffffu << sh)) | (val << sh);
+                            }
+                        }
+                        o[u] = u32x4{d[0], d[1], d[2], d[3]};
+                    }
                 }
             }
-            if (active) st16_nt(xrow, o);
+        };
+        auto store = [&](int64_t t0) {
+#pragma unroll
+            for (int u = 0; u < kRowUnroll; ++u)
+                if (FULL || (active && t0 + u < row1)) st16_nt(xrow[u], o[u]);
+        };
+        // next group's loads go out before this group's stores (see quant_rows)
+        load_codes(row0);
+        int64_t t0 = row0;
+        compute(t0);                              // first group peeled, as in quant_rows
+        if (t0 + kRowUnroll < row1) {
+            load_codes(t0 + kRowUnroll);
+            store(t0);
+            for (t0 += kRowUnroll; t0 + kRowUnroll < row1; t0 += kRowUnroll) {
+                compute(t0);
+                load_codes(t0 + kRowUnroll);
+                store(t0);
+            }
+            compute(t0);
         }
-    }
+        store(t0);
+    };
+    if (full) run(std::true_type{});
+    else run(std::false_type{});
 }
 
 // ------------------------------------------------------------------------------------
