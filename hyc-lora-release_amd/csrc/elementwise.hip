@@ -45,8 +45,8 @@ __global__ __launch_bounds__(kEwThreads) void binary_kernel(const uint16_t* __re
     for (int u = 0; u < kEwUnroll; ++u) {
         const int64_t c = c0 + u * kEwThreads;
         if (c < chunks) {
-            av[u] = ld16(a + c * 8);
-            bv[u] = ld16(b + c * 8);
+            av[u] = ld16_nt(a + c * 8);
+            bv[u] = ld16_nt(b + c * 8);
         }
     }
 #pragma unroll
@@ -58,7 +58,7 @@ __global__ __launch_bounds__(kEwThreads) void binary_kernel(const uint16_t* __re
             unpack8(bv[u], bf);
 #pragma unroll
             for (int j = 0; j < 8; ++j) of[j] = op(af[j], bf[j]);
-            st16(o + c * 8, pack8(of));
+            st16_nt(o + c * 8, pack8(of));
         }
     }
     if (blockIdx.x == 0 && threadIdx.x < (n & 7)) {       // ragged tail

@@ -43,7 +43,7 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_fwd_kernel(const uint16_
     for (int c = 0; c < CH; ++c) {
         const int col = (c * kWave + lane) * 8;
         xv[c] = u32x4{0, 0, 0, 0};
-        if (col < N) xv[c] = ld16(xr + col);
+        if (col < N) xv[c] = ld16_nt(xr + col);
     }
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
@@ -64,7 +64,7 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_fwd_kernel(const uint16_
             load_w8<W32>(w, col, wf);
 #pragma unroll
             for (int j = 0; j < 8; ++j) o[j] = (f[j] * rstd) * wf[j];
-            st16(y + row * N + col, pack8(o));
+            st16_nt(y + row * N + col, pack8(o));
         }
     }
 }
@@ -108,18 +108,14 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_bwd_kernel(const uint16_
                                                                    int64_t rows, int N) {
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x >> 6;
-    float wf[CH][8];
+    // The weight is re-read per row (8 KiB at N=4096, cache-resident) rather than held in
+    // registers: together with the dw accumulators it would cost an occupancy step.
     float dwacc[DW ? CH : 1][8];
+    if constexpr (DW) {
 #pragma unroll
-    for (int c = 0; c < CH; ++c) {
-        const int col = (c * kWave + lane) * 8;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) wf[c][j] = 0.0f;
-        if (col < N) load_w8<W32>(w, col, wf[c]);
-        if constexpr (DW) {
+        for (int c = 0; c < CH; ++c)
 #pragma unroll
             for (int j = 0; j < 8; ++j) dwacc[c][j] = 0.0f;
-        }
     }
     const float inv_n = 1.0f / (float)N;
     for (int64_t row = (int64_t)blockIdx.x * kNormWaves + wave; row < rows; row += (int64_t)gridDim.x * kNormWaves) {
@@ -131,19 +127,21 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_bwd_kernel(const uint16_
             xv[c] = u32x4{0, 0, 0, 0};
             gv[c] = u32x4{0, 0, 0, 0};
             if (col < N) {
-                xv[c] = ld16(x + row * N + col);
-                gv[c] = ld16(dy + row * N + col);
+                xv[c] = ld16_nt(x + row * N + col);
+                gv[c] = ld16_nt(dy + row * N + col);
             }
         }
         float s1 = 0.0f, s2 = 0.0f;
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
-            float xf[8], gf[8];
+            const int col = (c * kWave + lane) * 8;
+            float xf[8], gf[8], wf[8] = {0, 0, 0, 0, 0, 0, 0, 0};
             unpack8(xv[c], xf);
             unpack8(gv[c], gf);
+            if (col < N) load_w8<W32>(w, col, wf);
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                const float xh = xf[j] * rstd, wdy = wf[c][j] * gf[j];
+                const float xh = xf[j] * rstd, wdy = wf[j] * gf[j];
                 s1 = fmaf(xh, wdy, s1);
                 s2 += wdy;
                 if constexpr (DW) dwacc[c][j] = fmaf(gf[j], xh, dwacc[c][j]);
@@ -154,15 +152,16 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_bwd_kernel(const uint16_
         for (int c = 0; c < CH; ++c) {
             const int col = (c * kWave + lane) * 8;
             if (col < N) {
-                float xf[8], gf[8], o[8];
+                float xf[8], gf[8], wf[8], o[8];
                 unpack8(xv[c], xf);
                 unpack8(gv[c], gf);
+                load_w8<W32>(w, col, wf);
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
-                    const float xh = xf[j] * rstd, wdy = wf[c][j] * gf[j];
+                    const float xh = xf[j] * rstd, wdy = wf[j] * gf[j];
                     o[j] = (wdy - (xh * c1 + c2)) * rstd;
                 }
-                st16(dx + row * N + col, pack8(o));
+                st16_nt(dx + row * N + col, pack8(o));
             }
         }
     }

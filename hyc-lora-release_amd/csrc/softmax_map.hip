@@ -146,29 +146,37 @@ __global__ __launch_bounds__(kSegThreads) void sparse_count_kernel(const uint16_
     if (lane == 0) counts[seg] = cnt;
 }
 
-// Single workgroup: offsets[s] = sum of counts[0..s), offsets[nseg] = total.
+// Single workgroup: offsets[s] = sum of counts[0..s), offsets[nseg] = total.  The counts are
+// walked in tiles of 1024 (one per thread, coalesced); each tile is scanned with wave shuffles
+// plus one LDS step across the 16 waves, and a running total carries from tile to tile.
 __global__ __launch_bounds__(1024) void seg_scan_kernel(const uint32_t* __restrict__ counts, int64_t nseg,
                                                         int64_t* __restrict__ offsets) {
-    __shared__ long long incl[1024];
-    const int t = threadIdx.x;
-    const int64_t per = cdiv(nseg, 1024);
-    const int64_t b = t * per, e = b + per < nseg ? b + per : nseg;
-    long long sum = 0;
-    for (int64_t i = b; i < e; ++i) sum += counts[i];
-    incl[t] = sum;
+    __shared__ uint32_t wave_tot[16];
+    __shared__ long long carry;
+    const int t = threadIdx.x, lane = t & (kWave - 1), wave = t >> 6;
+    if (t == 0) carry = 0;
     __syncthreads();
-    for (int o = 1; o < 1024; o <<= 1) {
-        const long long add = t >= o ? incl[t - o] : 0;
+    for (int64_t base = 0; base < nseg; base += 1024) {
+        const int64_t i = base + t;
+        const uint32_t c = i < nseg ? counts[i] : 0u;
+        uint32_t inc = c;                                   // inclusive scan inside the wave
+#pragma unroll
+        for (int o = 1; o < kWave; o <<= 1) {
+            const uint32_t up = (uint32_t)__shfl_up((int)inc, o, kWave);
+            if (lane >= o) inc += up;
+        }
+        if (lane == kWave - 1) wave_tot[wave] = inc;
         __syncthreads();
-        incl[t] += add;
+        uint32_t before = 0;                                // totals of the waves in front
+#pragma unroll
+        for (int w = 0; w < 16; ++w) before += w < wave ? wave_tot[w] : 0u;
+        const long long run = carry;
+        if (i < nseg) offsets[i] = run + before + (inc - c);
+        __syncthreads();
+        if (t == 1023) carry = run + before + inc;
         __syncthreads();
     }
-    long long run = incl[t] - sum;
-    for (int64_t i = b; i < e; ++i) {
-        offsets[i] = run;
-        run += counts[i];
-    }
-    if (t == 1023) offsets[nseg] = incl[1023];
+    if (t == 0) offsets[nseg] = carry;
 }
 
 __global__ __launch_bounds__(kSegThreads) void sparse_write_kernel(const uint16_t* __restrict__ a, int64_t n,
@@ -253,7 +261,7 @@ __global__ __launch_bounds__(kSegThreads) void sparse_restore_kernel(const int64
         for (int s = 0; s < kSegSteps; ++s) {
             const int64_t i0 = seg * kSeg + (int64_t)(s * kWave + lane) * 8;
             if (i0 + 8 <= n) {
-                st16(out + i0, st[s * kWave + lane]);
+                st16_nt(out + i0, st[s * kWave + lane]);
             } else {
                 for (int j = 0; j < 8 && i0 + j < n; ++j) out[i0 + j] = stage[wave][(s * kWave + lane) * 8 + j];
             }
@@ -280,8 +288,8 @@ __global__ __launch_bounds__(256) void softmax_bwd_kernel(const uint16_t* __rest
         yv[c] = u32x4{0, 0, 0, 0};
         gv[c] = u32x4{0, 0, 0, 0};
         if (col < n) {
-            yv[c] = ld16(y + base + col);
-            gv[c] = ld16(g + base + col);
+            yv[c] = ld16_nt(y + base + col);
+            gv[c] = ld16_nt(g + base + col);
         }
     }
 #pragma unroll
@@ -302,7 +310,7 @@ __global__ __launch_bounds__(256) void softmax_bwd_kernel(const uint16_t* __rest
             unpack8(gv[c], gf);
 #pragma unroll
             for (int j = 0; j < 8; ++j) of[j] = (gf[j] - acc) * yf[j];
-            st16(o + base + col, pack8(of));
+            st16_nt(o + base + col, pack8(of));
         }
     }
 }
