@@ -31,9 +31,9 @@ sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of quant_pack_kernel<4,false,false> on the benchmark tensor, measured with
-# rocprofv3 --pmc FETCH_SIZE (44 136 KiB raw, x1.9995 from the copy-kernel calibration) and
-# WRITE_SIZE (22 016 KiB, x1.0): 88 248 KiB read + 22 016 KiB written.
-MEASURED_TRAFFIC_BYTES = (88248 + 22016) * 1024
+# rocprofv3 --pmc FETCH_SIZE (44 196 KiB raw, x1.9995 from the copy-kernel calibration) and
+# WRITE_SIZE (22 016 KiB, x1.0): 88 368 KiB read + 22 016 KiB written.
+MEASURED_TRAFFIC_BYTES = (88368 + 22016) * 1024
 
 
 def parse():

@@ -156,7 +156,7 @@ __device__ __forceinline__ void quant_rows(const QuantArgs& a, int64_t row0, int
     RowCursor cur(row0, a.M, a.stride_b, a.stride_m);
     u32x4 v[kRowUnroll];
     load_rows<FULL>(a, cur, row0, row1, active, coff, v);
-    auto compute = [&](int64_t t0, uint32_t (&lo)[kRowUnroll], uint32_t (&hi)[kRowUnroll]) {
+    auto compute = [&](u32x4 (&v)[kRowUnroll], int64_t t0, uint32_t (&lo)[kRowUnroll], uint32_t (&hi)[kRowUnroll]) {
 #pragma unroll
         for (int u = 0; u < kRowUnroll; ++u) {
             const int64_t t = t0 + u;
@@ -196,16 +196,16 @@ __device__ __forceinline__ void quant_rows(const QuantArgs& a, int64_t row0, int
     // to cover the entry case (loads only) and ends up waiting for the stores as well.
     uint32_t lo[kRowUnroll], hi[kRowUnroll];
     int64_t t0 = row0;
-    compute(t0, lo, hi);
+    compute(v, t0, lo, hi);
     if (t0 + kRowUnroll < row1) {
         load_rows<FULL>(a, cur, t0 + kRowUnroll, row1, active, coff, v);
         store(t0, lo, hi);
         for (t0 += kRowUnroll; t0 + kRowUnroll < row1; t0 += kRowUnroll) {
-            compute(t0, lo, hi);
+            compute(v, t0, lo, hi);
             load_rows<FULL>(a, cur, t0 + kRowUnroll, row1, active, coff, v);
             store(t0, lo, hi);
         }
-        compute(t0, lo, hi);                                   // last group: nothing left to load
+        compute(v, t0, lo, hi);                                // last group: nothing left to load
     }
     store(t0, lo, hi);
 }
