@@ -358,6 +358,8 @@ def main():
         kernels["softmax_restore"] = {"ms": ms, "GBps": (2 * Ea + 10 * nnz) / ms / 1e6}
         ms, _ = timed(lambda i: softmax_kernels.softmax_backward(a, g_a), 10, 2)
         kernels["softmax_bwd"] = {"ms": ms, "GBps": 6 * Ea / ms / 1e6}
+        ms, _ = timed(lambda i: softmax_kernels.softmax_backward_from_compressed(idx_a, val_a, seg_a, g_a), 10, 2)
+        kernels["softmax_restore_bwd_one_pass"] = {"ms": ms, "GBps": (6 * Ea + 10 * nnz) / ms / 1e6}
         del a, g_a, idx_a, val_a
 
     # ---- whole decoder layers (BASELINE configurations 2, 4, 5): fwd+bwd ms and saved bytes ----

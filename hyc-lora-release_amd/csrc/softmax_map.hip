@@ -269,6 +269,72 @@ __global__ __launch_bounds__(kSegThreads) void sparse_restore_kernel(const int64
     }
 }
 
+// ---- restore + softmax backward in one pass ----------------------------------------------
+// From the compressed map (idx, val, seg_offsets) and the upstream gradient g, writes
+//   a  = the restored dense map (optional, the caller needs it for grad_v = a^T @ grad_o) and
+//   o  = (g - sum_row bf16(a*g)) * a
+// without reading a dense map back from HBM.  One wave rebuilds one 4096-element segment in LDS
+// exactly like sparse_restore_kernel; the segment holds 4096/n whole rows (n = 512 .. 4096), and
+// each row is SPR = n/512 wave-wide steps, so its sum is a plain wave reduction.
+template <int SPR>
+__global__ __launch_bounds__(kSegThreads) void softmax_bwd_restore_kernel(const int64_t* __restrict__ idx,
+                                                                          const uint16_t* __restrict__ val,
+                                                                          const int64_t* __restrict__ offsets,
+                                                                          const uint16_t* __restrict__ g, int64_t nseg,
+                                                                          uint16_t* __restrict__ a_out,
+                                                                          uint16_t* __restrict__ o_out) {
+    __shared__ __attribute__((aligned(16))) uint16_t stage[kSegThreads / kWave][kSeg];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x >> 6;
+    const int64_t seg = blockIdx.x * (int64_t)(kSegThreads / kWave) + wave;
+    const bool live = seg < nseg;
+    u32x4* st = reinterpret_cast<u32x4*>(stage[wave]);
+#pragma unroll
+    for (int s = 0; s < kSegSteps; ++s) st[s * kWave + lane] = u32x4{0, 0, 0, 0};
+    __syncthreads();
+    if (live) {
+        const int64_t e0 = offsets[seg], e1 = offsets[seg + 1];
+        const int64_t first = seg * kSeg;
+        for (int64_t e = e0 + lane; e < e1; e += kWave) {
+            const int64_t rel = idx[e] - first;
+            if (rel >= 0 && rel < kSeg) stage[wave][rel] = val[e];
+        }
+    }
+    __syncthreads();
+    if (!live) return;
+#pragma unroll
+    for (int r = 0; r < kSegSteps / SPR; ++r) {             // rows of this segment
+        u32x4 yv[SPR], gv[SPR];
+        float acc = 0.0f;
+#pragma unroll
+        for (int s = 0; s < SPR; ++s) {
+            const int c = (r * SPR + s) * kWave + lane;      // chunk inside the segment
+            yv[s] = st[c];
+            gv[s] = ld16_nt(g + seg * kSeg + (int64_t)c * 8);
+        }
+#pragma unroll
+        for (int s = 0; s < SPR; ++s) {
+            float yf[8], gf[8];
+            unpack8(yv[s], yf);
+            unpack8(gv[s], gf);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc += rbf(yf[j] * gf[j]);
+        }
+        acc = wave_sum(acc);
+#pragma unroll
+        for (int s = 0; s < SPR; ++s) {
+            const int c = (r * SPR + s) * kWave + lane;
+            float yf[8], gf[8], of[8];
+            unpack8(yv[s], yf);
+            unpack8(gv[s], gf);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) of[j] = (gf[j] - acc) * yf[j];
+            st16_nt(o_out + seg * kSeg + (int64_t)c * 8, pack8(of));
+            if (a_out) st16_nt(a_out + seg * kSeg + (int64_t)c * 8, yv[s]);
+        }
+    }
+}
+
 // ---- softmax backward ---------------------------------------------------------------------
 // o = bf16( (g - sum_row bf16(y*g)) * y ), the row sum accumulated in fp32
 // (operators/softmax_kernels.py:31-35).  One wave per row; rows of up to 64*8*CH
@@ -424,5 +490,29 @@ extern "C" int hyc_softmax_bwd(const void* y, const void* grad_y, void* out, int
     else if (n <= 1024) hipLaunchKernelGGL(softmax_bwd_kernel<2>, grid, block, 0, st, yp, gp, op, rows, (int)n);
     else if (n <= 2048) hipLaunchKernelGGL(softmax_bwd_kernel<4>, grid, block, 0, st, yp, gp, op, rows, (int)n);
     else hipLaunchKernelGGL(softmax_bwd_kernel<8>, grid, block, 0, st, yp, gp, op, rows, (int)n);
+    return check_launch();
+}
+
+extern "C" int hyc_softmax_bwd_restore(const int64_t* indices, const void* values, const int64_t* seg_offsets,
+                                       const void* grad_y, void* a_out, void* out, int64_t rows, int64_t n,
+                                       void* stream) {
+    if (rows < 0 || n < 0) return HYC_ERR_SHAPE;
+    if (n != 512 && n != 1024 && n != 2048 && n != 4096) return HYC_ERR_SHAPE;
+    if (rows == 0) return HYC_OK;
+    if ((rows * n) % kSeg != 0) return HYC_ERR_SHAPE;
+    if (!seg_offsets || !grad_y || !out) return HYC_ERR_NULL;
+    if (!aligned16(grad_y) || !aligned16(out) || (a_out && !aligned16(a_out))) return HYC_ERR_ALIGN;
+    const int64_t nseg = rows * n / kSeg;
+    if (cdiv(nseg, 4) > INT32_MAX) return HYC_ERR_SHAPE;
+    const dim3 grid((unsigned)cdiv(nseg, 4)), block(kSegThreads);
+    hipStream_t st = (hipStream_t)stream;
+    const uint16_t* vp = (const uint16_t*)values;
+    const uint16_t* gp = (const uint16_t*)grad_y;
+    uint16_t* ap = (uint16_t*)a_out;
+    uint16_t* op = (uint16_t*)out;
+    if (n == 512) hipLaunchKernelGGL(softmax_bwd_restore_kernel<1>, grid, block, 0, st, indices, vp, seg_offsets, gp, nseg, ap, op);
+    else if (n == 1024) hipLaunchKernelGGL(softmax_bwd_restore_kernel<2>, grid, block, 0, st, indices, vp, seg_offsets, gp, nseg, ap, op);
+    else if (n == 2048) hipLaunchKernelGGL(softmax_bwd_restore_kernel<4>, grid, block, 0, st, indices, vp, seg_offsets, gp, nseg, ap, op);
+    else hipLaunchKernelGGL(softmax_bwd_restore_kernel<8>, grid, block, 0, st, indices, vp, seg_offsets, gp, nseg, ap, op);
     return check_launch();
 }

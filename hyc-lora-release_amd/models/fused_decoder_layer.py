@@ -42,11 +42,11 @@ from ..operators.compress_function import (compress_attention_map, compression_p
                                            decompression_dequantization_with_zero_point,
                                            get_statistics_only_quant, get_statistics_softmax,
                                            outlier_addition_fuse_decompression_dequantization,
-                                           restore_attention_map, update_dict)
+                                           update_dict)
 from ..operators.rmsnorm_kernels import _backward as _rmsnorm_backward
 from ..operators.rmsnorm_kernels import rmsnorm_forward
 from ..operators.silu_kernels import silu_backward, silu_hadamard
-from ..operators.softmax_kernels import softmax_backward
+from ..operators.softmax_kernels import softmax_backward_from_compressed
 from ..operators.triton_fuse_lora_silu_hadamard_backward_kernels import triton_fuse_silu_backward
 from ..operators.triton_fuse_lora_silu_hadamard_forward_kernels import triton_fuse_silu_forward
 from .compute_utils import (head_to_hidden_shape, hidden_to_head_shape, lora_backward, lora_forward,
@@ -336,12 +336,14 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             q, k, v = rebuilt("q", H), repeat_kv(rebuilt("k", KV), n_rep), repeat_kv(rebuilt("v", KV), n_rep)
 
         if spec.attention == "map":
-            a = restore_attention_map(S["a_idx"], S["a_val"], S["a_seg"], ctx.a_shape)
-            grad_v = a.transpose(-2, -1) @ grad_o
+            # grad_a first, then the restored map and the softmax backward come out of one pass over
+            # the compressed map (the reference restores, then reads the dense map twice more)
             grad_a = grad_o @ v.transpose(-2, -1)
-            del v, grad_o
-            grad_s = softmax_backward(a, grad_a)
-            del a, grad_a
+            del v
+            a, grad_s = softmax_backward_from_compressed(S["a_idx"], S["a_val"], S["a_seg"], grad_a)
+            del grad_a
+            grad_v = a.transpose(-2, -1) @ grad_o
+            del a, grad_o
             grad_s = grad_s / math.sqrt(D)
             grad_k = grad_s.transpose(-2, -1) @ q
             grad_q = grad_s @ k

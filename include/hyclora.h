@@ -190,6 +190,22 @@ int hyc_sparse_restore(const int64_t *indices, const void *values, const int64_t
 int hyc_softmax_bwd(const void *y, const void *grad_y, void *out, int64_t rows, int64_t n, void *stream);
 
 /* ---------------------------------------------------------------------------------------
+ * Dense restore and softmax backward in one pass over the compressed map: saves reading the
+ * restored map back (1 of the 4 dense passes of restore + backward).
+ *
+ * Replaces a_o.to_dense() followed by softmax_backward(a, grad_a)
+ * (models/llama/fused_llama_layer_intra_inter_full_fuse.py:414-415,432; operators/softmax_kernels.py:7-38).
+ *   indices / values / seg_offsets  as produced by hyc_sparse_count + hyc_sparse_write for a map of
+ *                                   rows*n elements;
+ *   grad_y, out   bf16 [rows, n];   a_out  bf16 [rows, n] or NULL (the restored map);
+ *   n in {512, 1024, 2048, 4096} and rows*n a multiple of 4096; other shapes: HYC_ERR_SHAPE (use
+ *   hyc_sparse_restore + hyc_softmax_bwd).
+ */
+int hyc_softmax_bwd_restore(const int64_t *indices, const void *values, const int64_t *seg_offsets,
+                            const void *grad_y, void *a_out, void *out, int64_t rows, int64_t n,
+                            void *stream);
+
+/* ---------------------------------------------------------------------------------------
  * RMSNorm forward: rstd = 1/sqrt(mean(x^2) + eps) in fp32, y = bf16(x * rstd * weight).
  *
  * Replaces _rms_norm_fwd_fused (operators/rmsnorm_kernels.py:10-54).

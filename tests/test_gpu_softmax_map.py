@@ -123,6 +123,32 @@ def test_softmax_backward(sk, dev, shape):
     assert_close_bf16(o, ref, what="softmax_backward vs closed form")
 
 
+@pytest.mark.parametrize("shape", [(1, 2, 16, 512), (2, 2, 8, 1024), (1, 1, 1024, 1024), (1, 3, 4, 2048), (1, 1, 5, 4096),
+                                   (1, 2, 100, 100), (1, 1, 3, 8192), (1, 1, 7, 512)])
+@pytest.mark.parametrize("ratio", [0.05, 0.0])
+def test_softmax_backward_from_compressed(cf, sk, dev, shape, ratio):
+    """restore + backward in one pass == the two separate kernels, bit for bit (the last three shapes
+    take the two-kernel route: row length not supported / element count not a multiple of 4096)."""
+    g = torch.Generator().manual_seed(shape[-1] + shape[-2])
+    a = torch.softmax(torch.randn(*shape, generator=g) * 3, dim=-1).to(BF16)
+    gr = torch.randn(*shape, generator=g).to(BF16)
+    thr = cf.get_statistics_softmax(a.to(dev), ratio) if ratio else torch.tensor(2.0, device=dev)  # 2.0: keeps nothing
+    idx, val, seg = cf.compress_attention_map(a.to(dev), thr)
+    dense = cf.restore_attention_map(idx, val, seg, shape)
+    want = sk.softmax_backward(dense, gr.to(dev))
+    a_out, o = sk.softmax_backward_from_compressed(idx, val, seg, gr.to(dev))
+    assert same_bits(a_out, dense) and same_bits(o, want)
+    none, o2 = sk.softmax_backward_from_compressed(idx, val, seg, gr.to(dev), want_map=False)
+    assert none is None and same_bits(o2, want)
+    # against the oracle, from the oracle's own compressed form
+    i_o, v_o = O.softmax_compress(a, thr.cpu())
+    ref = O.softmax_bwd(O.softmax_restore(i_o, v_o, a.shape), gr)
+    if ratio:
+        assert_close_bf16(o, ref, what="fused restore+bwd vs oracle")
+    else:                                     # nothing kept: the gradient is exactly zero
+        assert i_o.numel() == 0 and not bool(o.cpu().float().abs().max()) and not bool(ref.float().abs().max())
+
+
 def test_full_size_config3_properties(cf, sk, dev):
     # BASELINE configuration 3 at full size: [4,32,1024,1024], ratio 0.05
     g = torch.Generator(device=dev).manual_seed(1)
@@ -150,3 +176,5 @@ def test_full_size_config3_properties(cf, sk, dev):
     # row 700 of a few heads against the oracle
     rows = (slice(0, 4), slice(0, 2), slice(700, 704))
     assert_close_bf16(o[rows], O.softmax_bwd(dense[rows].cpu(), grad[rows].cpu()), what="softmax bwd rows")
+    a2, o2 = sk.softmax_backward_from_compressed(idx, val, seg, grad)
+    assert torch.equal(a2, dense) and torch.equal(o2, o)
