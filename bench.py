@@ -57,8 +57,13 @@ def bench_layers(torch, dev):
     import torch.nn.functional as F
 
     from hyclora_amd.models import llama, llama_flash_attn, mistral
-    from hyclora_amd.models.compute_utils import (head_to_hidden_shape, hidden_to_head_shape, repeat_kv,
-                                                  rope_forward)
+    from hyclora_amd.models.compute_utils import head_to_hidden_shape, hidden_to_head_shape, repeat_kv
+
+    def rope_forward(x, cos, sin):            # differentiable torch rotation for the uncompressed autograd arm
+        half, cos, sin = x.shape[-1] // 2, cos.squeeze(), sin.squeeze()
+        c, s = cos[None, :x.shape[1], None, :half], sin[None, :x.shape[1], None, :half]
+        x1, x2 = x[..., :half], x[..., half:]
+        return torch.cat([x1 * c - x2 * s, x2 * c + x1 * s], dim=-1)
     BF16 = torch.bfloat16
     gen = torch.Generator(device=dev).manual_seed(1)
 

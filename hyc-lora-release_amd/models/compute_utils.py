@@ -1,6 +1,7 @@
 """Torch-side glue of the fused layers (reference: models/utils/compute_utils.py:7-51 and
-operators/rope_kernels.py:81-126).  The frozen-weight GEMMs, RoPE and the attention products are
-library / torch operations in the reference as well; only what surrounds them is compressed."""
+operators/rope_kernels.py:81-126).  The frozen-weight GEMMs and the attention products are library /
+torch operations in the reference as well; only what surrounds them is compressed.  RoPE is the
+in-place HIP kernel of operators/rope_kernels.py, re-exported here."""
 import torch
 
 
@@ -66,21 +67,4 @@ def repeat_kv_backward(g: torch.Tensor, n_rep: int):
     return g.reshape(b, hq // n_rep, n_rep, s, d).sum(dim=2)
 
 
-def _rope(x, cos, sin, sign):
-    # x: [B, S, H, D]; cos/sin: [..., S_max, D] with the two halves equal (HF layout) - only the
-    # first half is read, as the reference kernel does (rope_kernels.py:56-59)
-    cos, sin = cos.squeeze(), sin.squeeze()
-    seq, half = x.shape[1], x.shape[-1] // 2
-    assert seq <= cos.shape[0]
-    c = cos[:seq, :half][None, :, None, :]
-    s = sin[:seq, :half][None, :, None, :] * sign
-    x1, x2 = x[..., :half].to(s.dtype), x[..., half:].to(s.dtype)
-    return torch.cat([x1 * c - x2 * s, x2 * c + x1 * s], dim=-1).to(x.dtype)
-
-
-def rope_forward(x, cos, sin):
-    return _rope(x, cos, sin, 1.0)
-
-
-def rope_backward(dy, cos, sin):
-    return _rope(dy, cos, sin, -1.0)
+from ..operators.rope_kernels import rope_backward, rope_forward  # noqa: E402,F401  (in place, HIP)

@@ -408,6 +408,37 @@ class FusedDecoderLayer(torch.nn.Module):
         self.layernorm_outlier_ratio = hyclora_config.layernorm_outlier_ratio
         self.q_bit = hyclora_config.q_bit
 
+    # The reference keeps `iteration` and `static_value` as plain attributes (…full_fuse.py:574-580),
+    # so a checkpoint taken after calibration restarts calibrating.  Here they travel with
+    # state_dict() as the module's extra state: ints, None and tensors only, loadable with
+    # torch.load(weights_only=True).
+    def get_extra_state(self):
+        return {"iteration": int(self.iteration),
+                "static_value": {key: {f: (v.detach().clone() if torch.is_tensor(v) else v) for f, v in fields.items()}
+                                 for key, fields in self.static_value.items()}}
+
+    def set_extra_state(self, state):
+        if not state:
+            return
+        want = self.spec.empty_static_value()
+        got = state["static_value"]
+        if set(got) != set(want) or any(set(got[k]) != set(want[k]) for k in want):
+            raise ValueError(f"calibration state of another layer type: has {sorted(got)}, "
+                             f"{self.spec.mode}/{self.spec.attention} needs {sorted(want)}")
+        self.iteration = int(state["iteration"])
+        self.static_value = {key: {f: (v.detach().clone() if torch.is_tensor(v) else v) for f, v in fields.items()}
+                             for key, fields in got.items()}
+
+    def _apply(self, fn, *args, **kwargs):
+        # .to(device)/.cuda() move the statistics with the module; their dtypes are part of the
+        # format (bf16 steps, fp32 threshold, int64 channels) and survive .half()/.float()
+        super()._apply(fn, *args, **kwargs)
+        for fields in self.static_value.values():
+            for f, v in fields.items():
+                if torch.is_tensor(v):
+                    fields[f] = fn(v).to(v.dtype)
+        return self
+
     def forward(self, input, norm_weight_1, norm_bias_1, cos, sin,
                 q_proj_base, q_proj_lora_a, q_proj_lora_b, k_proj_base, k_proj_lora_a, k_proj_lora_b,
                 v_proj_base, v_proj_lora_a, v_proj_lora_b, o_proj_base, o_proj_lora_a, o_proj_lora_b,

@@ -233,6 +233,22 @@ int hyc_rmsnorm_bwd(const void *dy, const void *x, const void *weight, int weigh
                     int64_t rows, int64_t N, void *stream);
 
 /* ---------------------------------------------------------------------------------------
+ * Rotary position embedding, in place: for every (b, s, h) the head x[b,s,h,:] = (x1 | x2) becomes
+ * (x1*cos[s] - x2*sin[s] | x2*cos[s] + x1*sin[s]); backward != 0 uses -sin.
+ *
+ * Replaces _rope_embedding / rope_forward / rope_backward (operators/rope_kernels.py:36-78, :81-126).
+ *   x        bf16, element (b,s,h,d) at x + b*stride_b + s*stride_s + h*stride_h + d; head_dim % 16 == 0;
+ *            strides multiples of 8 elements (a [B,S,H,D] tensor: S*H*D, H*D, D; a [B,H,S,D] tensor
+ *            is rotated in place with H*S*D, D, S*D).
+ *   cos, sin angle tables, row s at + s*stride_{cos,sin} elements; only the first head_dim/2 entries of a
+ *            row are read.  bf16 tables (table_is_fp32 == 0): bf16 rounding after every multiply and
+ *            add, as bf16 Triton arithmetic; fp32 tables: fp32 arithmetic, one rounding on the store.
+ */
+int hyc_rope(void *x, const void *cos, const void *sin, int table_is_fp32, int64_t B, int64_t S, int64_t H,
+             int64_t head_dim, int64_t stride_b, int64_t stride_s, int64_t stride_h, int64_t stride_cos,
+             int64_t stride_sin, int backward, void *stream);
+
+/* ---------------------------------------------------------------------------------------
  * Element-wise operators on n contiguous bf16 elements (16-byte aligned pointers).
  *
  *   hyc_silu_bwd  out = g * (sig * (1 + x*(1 - sig))), sig = bf16(sigmoid(x)), bf16 after

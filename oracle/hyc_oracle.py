@@ -22,6 +22,9 @@ Pinning status (what independent evidence holds each function in place):
     formula (which keeps LayerNorm's mean term) and is pinned only against a
     float64 evaluation of that same formula and against autograd for inputs where the
     extra term vanishes: "parity unpinned" for the c2 term beyond reading the source.
+  * rope: pinned against the textbook rotate-half form x*cos + rotate_half(x)*sin with
+    full-width tables, against an explicit complex-number rotation in float64, and by
+    norm preservation / forward-then-backward identity (tests/test_oracle_rope.py).
 The reference ships no tests, golden vectors or CPU implementation of its Triton
 kernels, so there is nothing of its own to check against.
 """
@@ -262,6 +265,24 @@ def softmax_bwd(y: torch.Tensor, g: torch.Tensor) -> torch.Tensor:
     yg = (y.to(BF16) * g.to(BF16)).float()
     ssum = yg.sum(dim=-1, keepdim=True)
     return ((g.float() - ssum) * y.float()).to(BF16)
+
+
+# --------------------------------------------------------------------------------------
+# rotary position embedding
+# --------------------------------------------------------------------------------------
+def rope(x, cos, sin, backward=False):
+    """x [B,S,H,D] -> rotated copy.  Halves (x1|x2) -> (x1*c - x2*s | x2*c + x1*s) with c, s the FIRST
+    half of table row s (rope_kernels.py:54-59, :72-78); backward negates s (:61-63).  x is
+    converted to the table's dtype and every product and sum is a tensor operation of that dtype
+    (bf16 tables: rounded after each operation; fp32 tables: fp32), result rounded to x's dtype."""
+    cos, sin = cos.squeeze(), sin.squeeze()
+    S, half = x.shape[1], x.shape[-1] // 2
+    c = cos[:S, :half][None, :, None, :]
+    s = sin[:S, :half][None, :, None, :]
+    if backward:
+        s = -s
+    x1, x2 = x[..., :half].to(c.dtype), x[..., half:].to(c.dtype)
+    return torch.cat([x1 * c - x2 * s, x2 * c + x1 * s], dim=-1).to(x.dtype)
 
 
 # --------------------------------------------------------------------------------------

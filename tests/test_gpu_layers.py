@@ -62,7 +62,8 @@ class RefRMSNorm(torch.autograd.Function):
 
 
 def reference_layer(t):
-    from hyclora_amd.models.compute_utils import hidden_to_head_shape, head_to_hidden_shape, repeat_kv, rope_forward
+    from hyclora_amd.models.compute_utils import hidden_to_head_shape, head_to_hidden_shape, repeat_kv
+    rope_forward = O.rope                      # differentiable torch ops; the HIP operator works in place
     P = t.P
 
     def proj(n, inp):
@@ -225,6 +226,36 @@ def test_calibration_state_machine(dev):
     with pytest.raises(ValueError):
         from hyclora_amd.models.llama import make_fused_llama_layer
         make_fused_llama_layer(config("no_such_type", 4))
+
+
+def test_calibration_state_survives_a_checkpoint(dev, tmp_path):
+    """Calibrate, save state_dict, load it into a fresh module (weights_only loader): the resumed
+    layer is past calibration and reproduces the original's next step bit for bit."""
+    import hyclora_amd  # noqa: F401
+    from hyclora_amd.models import FusedLlamaLayerIntraInterFullFuse
+    t = make_layer_inputs(dev, seed=21)
+    layer = FusedLlamaLayerIntraInterFullFuse()
+    layer.set_hyclora_config(config("intra_inter_full_fuse", 4, thr=2))
+    run_fused(layer, t)
+    run_fused(layer, make_layer_inputs(dev, seed=22))
+    torch.save(layer.state_dict(), tmp_path / "layer.pt")
+    resumed = FusedLlamaLayerIntraInterFullFuse()
+    resumed.set_hyclora_config(config("intra_inter_full_fuse", 4, thr=2))
+    resumed.load_state_dict(torch.load(tmp_path / "layer.pt", weights_only=True, map_location="cpu"))
+    assert resumed.iteration == 2
+    assert resumed.static_value['x']['outlier_channel_index'].device.type == "cpu"   # as saved ...
+    resumed.to(dev)                                                                  # ... moved with the module
+    for k, d in layer.static_value.items():
+        for f, v in d.items():
+            assert torch.equal(resumed.static_value[k][f], v) and resumed.static_value[k][f].dtype == v.dtype, (k, f)
+    t3 = make_layer_inputs(dev, seed=23)
+    want = run_fused(layer, t3)
+    want.backward(torch.ones_like(want))
+    g_want = t3.x.grad.clone()
+    t3.x.grad = None
+    got = run_fused(resumed, t3)
+    got.backward(torch.ones_like(got))
+    assert torch.equal(got, want) and torch.equal(t3.x.grad, g_want)
 
 
 def _saved_activation_bytes(fn):
