@@ -44,10 +44,13 @@ def parse():
     ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU-oracle timing (for profiler runs)")
     ap.add_argument("--only", choices=["all", "roundtrip", "quant", "fused", "copy", "layers"], default="all",
                     help="restrict the run to one part (for profiler runs)")
+    ap.add_argument("--layer-case", default="", help="with --only layers: run only the cases whose name contains this")
+    ap.add_argument("--layer-arm", choices=["both", "plain", "compressed"], default="both",
+                    help="with --only layers: run only one arm (for profiler runs)")
     return ap.parse_args()
 
 
-def bench_layers(torch, dev):
+def bench_layers(torch, dev, only_case="", arm="both"):
     """Forward+backward of one decoder layer with random-init bf16 weights N(0, 0.02) and LoRA r=16 on
     all seven linears: the compressed layer of this package against an uncompressed bf16
     torch-autograd layer of the same architecture, with the activation bytes each keeps for backward."""
@@ -151,11 +154,15 @@ def bench_layers(torch, dev):
              ("config5_llama7b_b1_s8192_mapfree_intra_inter", dict(B=1, S=8192, hidden=4096, heads=32, kv=32, inter=11008, theta=1e4),
               None, "intra_inter", [4], True)]
     for name, dims, maker, lt, qbits, sdpa in cases:
+        if only_case not in name:
+            continue
         t = make(**dims)
         mask = None if sdpa else torch.full((t.S, t.S), float("-inf"), device=dev).triu(1).to(BF16)[None, None]
-        ms_p, saved_p = measure(lambda: run_plain(t, mask, sdpa), t)
-        entry = {"bf16_uncompressed": {"fwd_bwd_ms": ms_p, "saved_activation_MB": saved_p / 1e6}}
-        for q in qbits:
+        entry, saved_p = {}, 0
+        if arm != "compressed":
+            ms_p, saved_p = measure(lambda: run_plain(t, mask, sdpa), t)
+            entry["bf16_uncompressed"] = {"fwd_bwd_ms": ms_p, "saved_activation_MB": saved_p / 1e6}
+        for q in (qbits if arm != "plain" else []):
             if maker is None:
                 layer = llama_flash_attn.FusedLlamaLayerIntraInter()
                 layer.set_hyclora_config(cfg(lt, q))
@@ -165,7 +172,7 @@ def bench_layers(torch, dev):
                 run_fused(layer, t, mask).backward(t.grad)
             ms_f, saved_f = measure(lambda: run_fused(layer, t, mask), t)
             entry[f"compressed_q{q}"] = {"fwd_bwd_ms": ms_f, "saved_activation_MB": saved_f / 1e6,
-                                         "saved_vs_bf16": saved_p / max(saved_f, 1)}
+                                         "saved_vs_bf16": saved_p / max(saved_f, 1) if saved_p else None}
             del layer
         out[name] = entry
         del t, mask
@@ -376,7 +383,7 @@ def main():
         for buffers in (xs, qs, xh):
             buffers.clear()
         torch.cuda.empty_cache()
-        layers = bench_layers(torch, dev)
+        layers = bench_layers(torch, dev, args.layer_case, args.layer_arm)
 
     # ---- CPU baseline: the oracle on the host cores, same tensor --------------------------------
     cpu = None

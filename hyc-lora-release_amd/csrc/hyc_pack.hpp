@@ -13,12 +13,11 @@
 
 namespace hyc {
 
-// Per-lane column constants of the quantiser: step, reciprocal, the upper input clamp of the
-// reciprocal path (the lower one is -xhi - s), and whether every one of the lane's 8 steps
-// may use that path.
+// Per-lane column constants of the quantiser: step, enlarged reciprocal (hyc_recip_nudged),
+// and whether every one of the lane's 8 steps may use the reciprocal path.
 template <int QBIT>
 struct QuantCols {
-    float s[8], r[8], xhi[8];
+    float s[8], rn[8];
     bool fast;
     __device__ __forceinline__ void load(const uint16_t* scale, int col0, bool active) {
         u32x4 sv = {0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};   // 1.0 for idle lanes
@@ -27,26 +26,42 @@ struct QuantCols {
         fast = true;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            r[j] = 1.0f / s[j];
-            xhi[j] = hyc_clamp_hi(s[j], QBIT);
+            rn[j] = hyc_recip_nudged(s[j]);
             fast = fast && hyc_scale_is_fast(s[j]);
         }
     }
 };
+
+// Device form of hyc_code_word_fast: the same fused multiply-add, with the clamp done by one
+// v_med3_f32.  With a NaN among its operands the instruction returns
+// min(min(src0, src1), src2), each min dropping a NaN operand; with the lower bound in src2 a
+// NaN therefore comes out as the lower bound (code 0), like the host form.  The operand order
+// matters for exactly that case, hence inline assembly instead of the commutative builtin.
+template <int QBIT>
+__device__ __forceinline__ uint32_t code_word_fast_dev(float x, float rn) {
+    const float m = fmaf(x, rn, HYC_MAGIC + (float)(1 << (QBIT - 1)));
+    float mc;
+    asm("v_med3_f32 %0, %1, %2, %3" : "=v"(mc) : "v"(m), "v"(HYC_MAGIC + (float)((1 << QBIT) - 1)), "v"(HYC_MAGIC));
+    return __float_as_uint(mc);
+}
+
+// low bytes of four dwords -> one dword (byte j from w_j)
+__device__ __forceinline__ uint32_t low_bytes(uint32_t w0, uint32_t w1, uint32_t w2, uint32_t w3) {
+    const uint32_t w01 = __builtin_amdgcn_perm(w1, w0, 0x0c0c0400u);   // selector 0-3: bytes of 2nd operand, 4-7: of 1st
+    const uint32_t w23 = __builtin_amdgcn_perm(w3, w2, 0x0c0c0400u);
+    return __builtin_amdgcn_perm(w23, w01, 0x05040100u);
+}
 
 // 8 values -> 8 codes, one per byte of (lo, hi).
 template <int QBIT, bool ZP, bool FAST>
 __device__ __forceinline__ void codes_to_words(const float (&f)[8], const QuantCols<QBIT>& q, const float (&z)[8],
                                                uint32_t& lo, uint32_t& hi) {
     if constexpr (FAST && !ZP) {
-        // signed codes; the offset 2^(q-1) is added to all four bytes of a word at once
-        // (sums of shifted two's-complement values, exact modulo 2^32)
-        uint32_t c[8];
+        uint32_t w[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) c[j] = (uint32_t)hyc_signed_code_fast(f[j], q.s[j], q.r[j], hyc_clamp_lo_from_hi(q.xhi[j], q.s[j]), q.xhi[j]);
-        constexpr uint32_t bias = 0x01010101u * (1u << (QBIT - 1));
-        lo = c[0] + (c[1] << 8) + (c[2] << 16) + (c[3] << 24) + bias;
-        hi = c[4] + (c[5] << 8) + (c[6] << 16) + (c[7] << 24) + bias;
+        for (int j = 0; j < 8; ++j) w[j] = code_word_fast_dev<QBIT>(f[j], q.rn[j]);
+        lo = low_bytes(w[0], w[1], w[2], w[3]);
+        hi = low_bytes(w[4], w[5], w[6], w[7]);
     } else {
         int c[8];
 #pragma unroll

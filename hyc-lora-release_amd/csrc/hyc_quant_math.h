@@ -5,12 +5,14 @@
 // is   t = fp32(x) / fp32(s) (+ z);  r = roundf(t);  r = clamp(r, -2^(q-1), 2^(q-1)-1);
 //      code = r + 2^(q-1).
 // x and s are bf16.  An IEEE fp32 division costs ~10 VALU operations per element on
-// CDNA, which would make the quantiser ALU-bound before it is HBM-bound.  Because the
-// divisor is constant per column, the kernels keep r = 1/s per column and recover the
-// correctly rounded quotient with one multiply and two fused multiply-adds
-// (hyc_quot_fast).  That this equals the IEEE quotient bit for bit — for every bf16 x
-// and every bf16 s accepted by hyc_scale_is_fast — is established exhaustively on the
-// CPU by tests/native/check_fastdiv.c, which includes this very header.
+// CDNA, and the quantiser is then bound by the vector ALU rather than by HBM.  Because x
+// and s carry 8-bit significands, the real quotient x/s is either exactly a half-integer
+// or at least ~2^-16 (relative) away from one, so the code is a function of the real
+// quotient alone, and a slightly enlarged reciprocal per column reproduces it with one
+// fused multiply-add (hyc_code_fast).  That the codes equal those of the IEEE division
+// followed by roundf — for every bf16 x and every bf16 s accepted by hyc_scale_is_fast —
+// is established exhaustively on the CPU by tests/native/check_fastdiv.c, which includes
+// this very header.
 #ifndef HYC_QUANT_MATH_H
 #define HYC_QUANT_MATH_H
 
@@ -23,11 +25,6 @@
 #else
 #define HYC_HD static inline
 #endif
-
-// Quotients are pre-clamped to +-HYC_QCLAMP before the correction step so that
-// infinities cannot turn into NaN there.  Any |t| >= 512 saturates every supported
-// code width even after adding a zero point in [-128, 127].
-#define HYC_QCLAMP 1024.0f
 
 HYC_HD float hyc_bits_to_f32(uint32_t u) {
     float f;
@@ -54,20 +51,8 @@ HYC_HD uint16_t hyc_f32_to_bf16(float f) {
 
 // A column may use the reciprocal path when its step is an ordinary positive number
 // whose reciprocal is an ordinary number too.  Everything else (0, negative, tiny,
-// huge, inf, NaN) takes the IEEE division.
+// huge, inf, NaN) takes the IEEE division (hyc_code_from_t).
 HYC_HD int hyc_scale_is_fast(float s) { return (s >= 1e-18f) && (s <= 1e18f); }
-
-// x/s from r = 1/s (itself the IEEE reciprocal), valid when hyc_scale_is_fast(s): one
-// Newton-style correction of x*r with an exact remainder.  The integer code derived
-// from the result equals the code derived from the IEEE quotient for every bf16 x
-// (the quotient itself may differ in the sign of zero and for subnormal x, where the
-// code is 2^(q-1) either way).  Beyond +-512 only the sign matters; NaN x gives NaN.
-HYC_HD float hyc_quot_fast(float x, float s, float r) {
-    float q0 = x * r;
-    q0 = fminf(fmaxf(q0, -HYC_QCLAMP), HYC_QCLAMP);
-    float rem = fmaf(-q0, s, x);
-    return fmaf(rem, r, q0);
-}
 
 // roundf + clamp + offset.  t is clamped first (the bounds are integers, so clamping
 // before rounding is the same as after); fmaxf maps NaN to the lower bound, i.e. code 0.
@@ -82,30 +67,33 @@ HYC_HD int hyc_code_from_t(float t, int q_bit) {
     return (int)v + (1 << (q_bit - 1));
 }
 
-// Cheapest form of the rule for the reciprocal path, as a signed code in
-// [-2^(q-1), 2^(q-1)-1] (the caller adds the offset 2^(q-1) once per packed word).
-// Instead of clamping the quotient, the INPUT is clamped to [xlo, xhi] =
-// [(-2^(q-1) - 0.49) s, (2^(q-1) - 1 + 0.49) s]: inside that interval nothing changes, and
-// outside it the value lands 0.49 beyond the last code, which rounds to that code — the
-// same saturation, but infinities never reach the correction step and no second clamp is
-// needed.  A NaN input fails the comparison and becomes xlo, i.e. the lowest code (biased
-// code 0); a compare-and-select is used rather than fmaxf because fmaxf turns a
-// *signalling* NaN into a quiet NaN instead of dropping it.
-// The sign for the half-away rounding is taken from the clamped input (s > 0 here).
-// The lower bound is derived from the upper one (lo - 0.49 = -(hi + 0.49) - 1), so a kernel
-// that is short of registers keeps only xhi and recomputes xlo = -xhi - s on the fly.
-HYC_HD float hyc_clamp_hi(float s, int q_bit) { return ((float)(1 << (q_bit - 1)) - 1.0f + 0.49f) * s; }
-HYC_HD float hyc_clamp_lo_from_hi(float xhi, float s) { return -xhi - s; }
-HYC_HD float hyc_clamp_lo(float s, int q_bit) { return hyc_clamp_lo_from_hi(hyc_clamp_hi(s, q_bit), s); }
+// The reciprocal path.  rn = (1/s) * (1 + 2^-18) is kept per column.  x * rn is the real
+// quotient pushed away from zero by a relative 2^-18 (give or take the ~2^-23 of rounding
+// rn and the product): an exact tie k + 0.5 lands strictly beyond the tie on the side
+// roundf sends it to, and a quotient that is not a tie cannot be pushed across one (the
+// nearest tie is >= 2^-16 away, relatively, for |x/s| <= 128.5).  After that no ties are
+// left, so any round-to-nearest gives roundf's answer, and the cheapest one is the rounding
+// of the fused multiply-add itself: adding 1.5 * 2^23 forces the sum's unit in the last place
+// to 1, which leaves the integer - offset 2^(q-1) included - in the low mantissa bits.
+// Clamping that float to [HYC_MAGIC, HYC_MAGIC + 2^q - 1] saturates the code (the bounds are
+// integers, so clamping after rounding equals clamping before); infinities and overflowing
+// products clamp like any large value, and a NaN, which fails the comparison, becomes the
+// lower bound: code 0, as in the reference.  The code is the low byte of the result.
+#define HYC_MAGIC 12582912.0f            /* 1.5 * 2^23 */
+#define HYC_RECIP_NUDGE 1.000003814697265625f   /* 1 + 2^-18 */
 
-HYC_HD int hyc_signed_code_fast(float x, float s, float r, float xlo, float xhi) {
-    float xc = (x > xlo) ? x : xlo;
-    xc = fminf(xc, xhi);
-    const float q0 = xc * r;
-    const float rem = fmaf(-q0, s, xc);
-    const float q1 = fmaf(rem, r, q0);
-    return (int)(q1 + copysignf(0.5f, xc));
+HYC_HD float hyc_recip_nudged(float s) { return (1.0f / s) * HYC_RECIP_NUDGE; }
+
+// Host form (compare-and-select so that signalling NaNs are dropped too); the kernels do the
+// clamp with one v_med3_f32.  Returns the float whose low byte is the biased code.
+HYC_HD uint32_t hyc_code_word_fast(float x, float rn, int q_bit) {
+    const float lo = HYC_MAGIC, hi = HYC_MAGIC + (float)((1 << q_bit) - 1);
+    float m = fmaf(x, rn, HYC_MAGIC + (float)(1 << (q_bit - 1)));
+    m = (m > lo) ? m : lo;
+    m = fminf(m, hi);
+    return hyc_f32_to_bits(m);
 }
+HYC_HD int hyc_code_fast(float x, float rn, int q_bit) { return (int)(hyc_code_word_fast(x, rn, q_bit) & 0xffu); }
 
 // Same rule with plain roundf semantics (trunc, then an exact fraction test), for
 // t = x/s + z: once an arbitrary zero point has been added the half-ulp argument above

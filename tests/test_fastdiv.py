@@ -1,5 +1,5 @@
-"""Runs the exhaustive host-side proof that the quantiser's reciprocal-based quotient gives
-the same integer codes as IEEE division for every bf16 input and every accepted bf16 step
+"""Runs the exhaustive host-side proof that the quantiser's reciprocal-based code rule gives
+the same integer codes as IEEE division + roundf for every bf16 input and every accepted bf16 step
 (tests/native/check_fastdiv.c; about 10^9 pairs, ~15 s on 8 cores)."""
 import subprocess
 from pathlib import Path

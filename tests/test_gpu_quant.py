@@ -57,6 +57,27 @@ def test_special_values_and_degenerate_scales(cf, dev, q_bit):
 
 
 @pytest.mark.parametrize("q_bit", QBITS)
+def test_every_bf16_pattern_against_a_spread_of_steps(cf, dev, q_bit):
+    """All 65536 bf16 bit patterns (both NaN kinds, infinities, subnormals) as x, one per row, against
+    64 steps per wave-width of columns: the reciprocal path's whole range, its edges, and steps outside
+    it.  Covers on the device what the exhaustive CPU check covers for the shared arithmetic, plus the
+    device-only clamp instruction."""
+    pats = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(BF16)        # every pattern
+    g = torch.Generator().manual_seed(q_bit)
+    steps = torch.cat([
+        torch.tensor([1e-18, 1.0001e-18, 9.9e17, 1e18, 1e-19, 2e18, 1.0, 0.5, 3.0, 0.1, 7.0, 1e-3, 0.0, -1.0,
+                      float("inf"), 2 ** -126]),
+        torch.exp(torch.rand(48, generator=g) * 80 - 40)]).to(BF16)                  # log-uniform 4e-18 .. 2e17
+    x = pats[None, :, None].expand(1, 65536, 64).contiguous()
+    p = cf.compression_quantization(x.to(dev), steps.to(dev), q_bit)
+    want = O.compress(x, steps, q_bit)
+    if not torch.equal(p.cpu(), want):
+        bad = (O.unpack_codes(p.cpu(), q_bit) != O.unpack_codes(want, q_bit)).nonzero()
+        r, c = bad[0, -2].item(), bad[0, -1].item()
+        raise AssertionError(f"{bad.shape[0]} codes differ; first: x pattern {r:#06x}, step {steps[c].item()!r}")
+
+
+@pytest.mark.parametrize("q_bit", QBITS)
 def test_zero_point_path(cf, dev, q_bit):
     x = (_rand((2, 70, 256), seed=5).float() + 0.7).to(BF16)
     s, z8 = O.scale_zero_point(x, q_bit)
