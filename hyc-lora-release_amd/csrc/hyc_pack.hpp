@@ -26,7 +26,7 @@ struct QuantCols {
         fast = true;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            rn[j] = hyc_recip_nudged(s[j]);
+            rn[j] = __builtin_amdgcn_rcpf(s[j]) * HYC_RECIP_NUDGE;   // within HYC_RECIP_SLACK of hyc_recip_nudged
             fast = fast && hyc_scale_is_fast(s[j]);
         }
     }

@@ -84,6 +84,13 @@ HYC_HD int hyc_code_from_t(float t, int q_bit) {
 
 HYC_HD float hyc_recip_nudged(float s) { return (1.0f / s) * HYC_RECIP_NUDGE; }
 
+// The kernels take the reciprocal from the hardware approximation (v_rcp_f32, 1 ulp) instead of
+// an IEEE division.  The code is monotone in rn, so it is enough that both ends of a band of
+// relative half-width HYC_RECIP_SLACK around hyc_recip_nudged(s) give the right codes; the
+// exhaustive checker tests exactly those two ends, and the band is 4x wider than the error of
+// the approximation plus the rounding of the product.
+#define HYC_RECIP_SLACK 4.76837158203125e-07f    /* 2^-21 */
+
 // Host form (compare-and-select so that signalling NaNs are dropped too); the kernels do the
 // clamp with one v_med3_f32.  Returns the float whose low byte is the biased code.
 HYC_HD uint32_t hyc_code_word_fast(float x, float rn, int q_bit) {

@@ -29,12 +29,22 @@
 
 namespace hyc {
 
-constexpr int kQuantWaves = 4;      // waves per workgroup
+#ifndef HYC_Q_WAVES
+#define HYC_Q_WAVES 4
+#endif
+#ifndef HYC_Q_UNROLL
+#define HYC_Q_UNROLL 4
+#endif
+constexpr int kQuantWaves = HYC_Q_WAVES;      // waves per workgroup
 constexpr int kQuantThreads = kQuantWaves * kWave;
-constexpr int kRowUnroll = 4;       // independent 128-bit loads in flight per lane
+#ifndef HYC_D_UNROLL
+#define HYC_D_UNROLL 2
+#endif
+constexpr int kRowUnroll = HYC_Q_UNROLL;       // quantiser: independent 128-bit loads in flight per lane
+constexpr int kDeqUnroll = HYC_D_UNROLL;       // dequantiser: rows per group
 
 static int g_quant_rows_per_wave = 8;     // strip heights; see hyc_set_tuning
-static int g_dequant_rows_per_wave = 4;
+static int g_dequant_rows_per_wave = 2;
 
 struct QuantArgs {
     uint16_t* x;            // bf16 activations (input of quantise / output of dequantise)
@@ -285,14 +295,14 @@ __global__ __launch_bounds__(kQuantThreads) void unpack_dequant_kernel(const Qua
 
     if (row0 >= row1) return;
     const bool full = (col_tile + 1) * kWave <= a.C && row1 - row0 == a.rows_per_wave &&
-                      a.rows_per_wave % kRowUnroll == 0;      // uniform: no predicate needed anywhere
+                      a.rows_per_wave % kDeqUnroll == 0;      // uniform: no predicate needed anywhere
     auto run = [&](auto full_tag) {
         constexpr bool FULL = decltype(full_tag)::value;
         RowCursor cur(row0, a.M, a.stride_b, a.stride_m);
-        u32x2 w[kRowUnroll];
+        u32x2 w[kDeqUnroll];
         auto load_codes = [&](int64_t t0) {
 #pragma unroll
-            for (int u = 0; u < kRowUnroll; ++u) {
+            for (int u = 0; u < kDeqUnroll; ++u) {
                 if constexpr (FULL) {
                     w[u] = ld8(a.q + (t0 + u) * row_bytes + slot.offset);
                 } else {
@@ -301,11 +311,11 @@ __global__ __launch_bounds__(kQuantThreads) void unpack_dequant_kernel(const Qua
                 }
             }
         };
-        u32x4 o[kRowUnroll];
-        uint16_t* xrow[kRowUnroll];
+        u32x4 o[kDeqUnroll];
+        uint16_t* xrow[kDeqUnroll];
         auto compute = [&](int64_t t0) {
 #pragma unroll
-            for (int u = 0; u < kRowUnroll; ++u) {
+            for (int u = 0; u < kDeqUnroll; ++u) {
                 const int64_t t = t0 + u;
                 float c[8], f[8];
                 slot.decode(w[u], c);
@@ -341,19 +351,19 @@ __global__ __launch_bounds__(kQuantThreads) void unpack_dequant_kernel(const Qua
         };
         auto store = [&](int64_t t0) {
 #pragma unroll
-            for (int u = 0; u < kRowUnroll; ++u)
+            for (int u = 0; u < kDeqUnroll; ++u)
                 if (FULL || (active && t0 + u < row1)) st16_nt(xrow[u], o[u]);
         };
         // next group's loads go out before this group's stores (see quant_rows)
         load_codes(row0);
         int64_t t0 = row0;
         compute(t0);                              // first group peeled, as in quant_rows
-        if (t0 + kRowUnroll < row1) {
-            load_codes(t0 + kRowUnroll);
+        if (t0 + kDeqUnroll < row1) {
+            load_codes(t0 + kDeqUnroll);
             store(t0);
-            for (t0 += kRowUnroll; t0 + kRowUnroll < row1; t0 += kRowUnroll) {
+            for (t0 += kDeqUnroll; t0 + kDeqUnroll < row1; t0 += kDeqUnroll) {
                 compute(t0);
-                load_codes(t0 + kRowUnroll);
+                load_codes(t0 + kDeqUnroll);
                 store(t0);
             }
             compute(t0);

@@ -5,6 +5,8 @@
  * (one fused multiply-add with the enlarged reciprocal, clamp, low byte), and the codes the
  * division paths compute (hyc_code_from_t, hyc_code_from_t_exact), must equal the code
  * computed from the IEEE quotient x / s with libm's roundf, for code widths 2, 4 and 8.
+ * hyc_code_fast is also evaluated with the reciprocal moved to either end of the band
+ * +-HYC_RECIP_SLACK (relative), which bounds what an approximate reciprocal can return.
  * Also reports how close an enlarged quotient inside the code range ever comes to a
  * half-integer (it must stay clear of one, or the rounding mode of the addition would matter).
  * Prints the number of pairs examined and the number of mismatches; exit status 0 iff none.
@@ -47,6 +49,9 @@ int main(int argc, char **argv) {
                 const int want = code_ieee(x, s, q);
                 if (hyc_code_from_t(ti, q) != want || hyc_code_from_t_exact(ti, q) != want) ok = 0;
                 if (hyc_code_fast(x, rn, q) != want) ok = 0;
+                /* both ends of the band that covers an approximate hardware reciprocal */
+                if (hyc_code_fast(x, rn * (1.0f - HYC_RECIP_SLACK), q) != want) ok = 0;
+                if (hyc_code_fast(x, rn * (1.0f + HYC_RECIP_SLACK), q) != want) ok = 0;
             }
             const double tn = (double)x * (double)rn;
             if (fabs(tn) <= 129.0) {
