@@ -39,7 +39,7 @@ constexpr int kTileRows = 16;
 // backward kernel fetched every code line twice: +45 MB of HBM reads on [4096 x 11008].)
 template <int QBIT> constexpr int kColTilesPerGroup = 8 / QBIT;
 
-static int g_fuse_rows_per_wave = 32;
+static int g_fuse_rows_per_wave[2] = {32, 48};   // backward, forward; see hyc_set_tuning
 
 struct FuseArgs {
     const uint16_t* xa1; const uint16_t* b1; const uint16_t* s1;
@@ -128,8 +128,7 @@ __device__ __forceinline__ void fuse_fwd_rows(const FuseArgs& a, int64_t row_beg
     const int g = lane >> 4;
     const int row_bytes = a.N * QBIT / 8;
     const float zero8[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    for (int64_t row0 = row_begin; row0 < row_end; row0 += kTileRows) {
-        u32x4 xv1[4], xv2[4];
+    auto load_x = [&](int64_t row0, u32x4 (&xv1)[4], u32x4 (&xv2)[4]) {
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
             const int64_t t = row0 + 4 * g + v;
@@ -140,6 +139,10 @@ __device__ __forceinline__ void fuse_fwd_rows(const FuseArgs& a, int64_t row_beg
                 xv2[v] = ld16_nt(a.x2 + t * a.N + chunk * 8);
             }
         }
+    };
+    for (int64_t row0 = row_begin; row0 < row_end; row0 += kTileRows) {
+        u32x4 xv1[4], xv2[4];
+        load_x(row0, xv1, xv2);
         uint32_t L1[4][4], L2[4][4];
         lora_tile_bf16<KSTEPS>(a.xa1, a.R, row0, row_end, lane, B1, L1);
         lora_tile_bf16<KSTEPS>(a.xa2, a.R, row0, row_end, lane, B2, L2);
@@ -323,7 +326,7 @@ static int fuse_launch(FuseArgs& a, int64_t T, int64_t N, int64_t R, int q_bit, 
     a.N = (int)N;
     a.C = (int)(N / 8);
     a.R = (int)R;
-    a.rows_per_wave = g_fuse_rows_per_wave;
+    a.rows_per_wave = g_fuse_rows_per_wave[fwd ? 1 : 0];
     const int ct = 8 / q_bit;                                  // kColTilesPerGroup
     a.col_tiles = (int)cdiv(cdiv(N, kTileCols), ct);           // workgroups along the columns
     const int64_t row_tiles = cdiv(T, (int64_t)(kFuseWaves / ct) * a.rows_per_wave);
@@ -339,7 +342,7 @@ static int fuse_launch(FuseArgs& a, int64_t T, int64_t N, int64_t R, int q_bit, 
 int tune_fuse(const char* key, int value) {
     if (strcmp(key, "fuse_rows_per_wave") == 0) {
         if (value < kTileRows || value > 65536 || value % kTileRows != 0) return HYC_ERR_ARG;
-        g_fuse_rows_per_wave = value;
+        g_fuse_rows_per_wave[0] = g_fuse_rows_per_wave[1] = value;
         return HYC_OK;
     }
     return 1;

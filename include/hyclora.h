@@ -42,7 +42,8 @@ int hyc_abi_version(void);
 /* Launch-shape knobs for benchmarking (process-wide, not thread-safe against concurrent
  * launches).  Keys: "quant_rows_per_wave" (rows each wave walks in hyc_quant_pack,
  * default 8), "dequant_rows_per_wave" (same for hyc_unpack_dequant, default 2),
- * "fuse_rows_per_wave" (same for the fused LoRA-SiLU kernels, multiple of 16, default 32).  Unknown key or bad value: HYC_ERR_ARG.  No
+ * "fuse_rows_per_wave" (same for both fused LoRA-SiLU kernels, multiple of 16; defaults 48 forward,
+ * 32 backward).  Unknown key or bad value: HYC_ERR_ARG.  No
  * counterpart in the reference (its launch shapes come from triton.autotune). */
 int hyc_set_tuning(const char *key, int value);
 
