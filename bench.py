@@ -413,6 +413,13 @@ def main():
         kernels["softmax_restore"] = {"ms": ms, "GBps": (2 * Ea + 10 * nnz) / ms / 1e6}
         ms, _ = timed(lambda i: softmax_kernels.softmax_backward(a, g_a), 10, 2)
         kernels["softmax_bwd"] = {"ms": ms, "GBps": 6 * Ea / ms / 1e6}
+        causal = torch.full((1024, 1024), float("-inf"), device=dev).triu(1).to(BF16)[None, None]
+        ms, _ = timed(lambda i: softmax_kernels.softmax_forward(g_a, 0.0884, causal), 10, 2)
+        kernels["softmax_fwd_scale_mask"] = {"ms": ms, "GBps": 4 * Ea / ms / 1e6}
+        ms, _ = timed(lambda i: softmax_kernels.softmax_forward(g_a, 0.0884, causal, threshold=thr), 10, 2)
+        kernels["softmax_fwd_scale_mask_count"] = {"ms": ms, "GBps": 4 * Ea / ms / 1e6}
+        ms, _ = timed(lambda i: torch.softmax(g_a / 11.3137 + causal, dim=-1, dtype=BF16), 10, 2)
+        kernels["softmax_fwd_scale_mask"]["torch_three_passes_ms"] = ms
         ms, _ = timed(lambda i: softmax_kernels.softmax_backward_from_compressed(idx_a, val_a, seg_a, g_a), 10, 2)
         kernels["softmax_restore_bwd_one_pass"] = {"ms": ms, "GBps": (6 * Ea + 10 * nnz) / ms / 1e6}
         del a, g_a, idx_a, val_a

@@ -21,6 +21,7 @@ constexpr int kHistLdsBins = 16384;   // keys 0x8000..0xBFFF: bf16 values in [+0
 constexpr int kSeg = 4096;            // elements per compaction segment (one wave)
 constexpr int kSegThreads = 256;      // 4 segments per workgroup
 constexpr int kSegSteps = kSeg / (kWave * 8);
+constexpr int kStageEntries = 1024;   // kept entries of a segment that sparse_write gathers in LDS
 
 // Monotonic 16-bit key of a bf16 bit pattern: ascending key = ascending value, NaN last
 // (torch.kthvalue orders NaN above everything).
@@ -146,37 +147,50 @@ __global__ __launch_bounds__(kSegThreads) void sparse_count_kernel(const uint16_
     if (lane == 0) counts[seg] = cnt;
 }
 
-// Single workgroup: offsets[s] = sum of counts[0..s), offsets[nseg] = total.  The counts are
-// walked in tiles of 1024 (one per thread, coalesced); each tile is scanned with wave shuffles
-// plus one LDS step across the 16 waves, and a running total carries from tile to tile.
+// offsets[s] = sum of counts[0..s), offsets[nseg] = total.  Workgroup b scans the 1024 counts of
+// its own tile (one per thread: wave shuffles plus one LDS step across the 16 waves) and finds
+// the sum of everything in front of the tile by itself, adding up counts[0 .. 1024 b) with all its
+// threads: redundant reads of a few hundred KB from L2 instead of a second launch or a chain of
+// workgroups waiting for each other.  Launch with max(1, ceil(nseg / 1024)) workgroups.
 __global__ __launch_bounds__(1024) void seg_scan_kernel(const uint32_t* __restrict__ counts, int64_t nseg,
                                                         int64_t* __restrict__ offsets) {
+    __shared__ long long part[16];
     __shared__ uint32_t wave_tot[16];
-    __shared__ long long carry;
     const int t = threadIdx.x, lane = t & (kWave - 1), wave = t >> 6;
-    if (t == 0) carry = 0;
-    __syncthreads();
-    for (int64_t base = 0; base < nseg; base += 1024) {
-        const int64_t i = base + t;
-        const uint32_t c = i < nseg ? counts[i] : 0u;
-        uint32_t inc = c;                                   // inclusive scan inside the wave
+    const int64_t base = (int64_t)blockIdx.x * 1024;
+    long long front = 0;
+    int64_t f = t;
+    for (; f + 7 * 1024 < base; f += 8 * 1024) {           // eight independent loads in flight
+        uint32_t v[8];
 #pragma unroll
-        for (int o = 1; o < kWave; o <<= 1) {
-            const uint32_t up = (uint32_t)__shfl_up((int)inc, o, kWave);
-            if (lane >= o) inc += up;
-        }
-        if (lane == kWave - 1) wave_tot[wave] = inc;
-        __syncthreads();
-        uint32_t before = 0;                                // totals of the waves in front
+        for (int u = 0; u < 8; ++u) v[u] = counts[f + u * 1024];
 #pragma unroll
-        for (int w = 0; w < 16; ++w) before += w < wave ? wave_tot[w] : 0u;
-        const long long run = carry;
-        if (i < nseg) offsets[i] = run + before + (inc - c);
-        __syncthreads();
-        if (t == 1023) carry = run + before + inc;
-        __syncthreads();
+        for (int u = 0; u < 8; ++u) front += v[u];
     }
-    if (t == 0) offsets[nseg] = carry;
+    for (; f < base; f += 1024) front += counts[f];
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) front += __shfl_xor(front, o, kWave);
+    const int64_t i = base + t;
+    const uint32_t c = i < nseg ? counts[i] : 0u;
+    uint32_t inc = c;                                       // inclusive scan inside the wave
+#pragma unroll
+    for (int o = 1; o < kWave; o <<= 1) {
+        const uint32_t up = (uint32_t)__shfl_up((int)inc, o, kWave);
+        if (lane >= o) inc += up;
+    }
+    if (lane == 0) part[wave] = front;
+    if (lane == kWave - 1) wave_tot[wave] = inc;
+    __syncthreads();
+    long long at = 0;
+    uint32_t before = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) {
+        at += part[w];
+        before += w < wave ? wave_tot[w] : 0u;
+        total += wave_tot[w];
+    }
+    if (i < nseg) offsets[i] = at + before + (inc - c);
+    if (t == 0 && base + 1024 >= nseg) offsets[nseg] = at + total;
 }
 
 __global__ __launch_bounds__(kSegThreads) void sparse_write_kernel(const uint16_t* __restrict__ a, int64_t n,
@@ -184,38 +198,77 @@ __global__ __launch_bounds__(kSegThreads) void sparse_write_kernel(const uint16_
                                                                    const int64_t* __restrict__ offsets,
                                                                    int64_t* __restrict__ idx_out,
                                                                    uint16_t* __restrict__ val_out) {
+    __shared__ uint32_t stage[kSegThreads / kWave][kStageEntries];
     const int lane = threadIdx.x & (kWave - 1);
     const int64_t seg = blockIdx.x * (int64_t)(kSegThreads / kWave) + (threadIdx.x >> 6);
     if (seg >= nseg) return;
     const float thr = rbf(*thr_p);
-    int64_t base = offsets[seg];
+    const int64_t base = offsets[seg];
     if (offsets[seg + 1] == base) return;          // nothing kept in this segment
+    // all of the segment's loads are issued before anything depends on them
+    uint32_t e[kSegSteps][8];
+    uint32_t mask[kSegSteps], inc[kSegSteps];
+#pragma unroll
     for (int s = 0; s < kSegSteps; ++s) {
         const int64_t c = seg * (kSeg / 8) + s * kWave + lane;
-        uint32_t e[8];
-        uint32_t mask = 0;
+        mask[s] = 0;
         if (c * 8 < n) {
-            load_chunk(a, c, n, e);
+            load_chunk(a, c, n, e[s]);
 #pragma unroll
-            for (int j = 0; j < 8; ++j) mask |= keep(e[j], thr) ? (1u << j) : 0u;
+            for (int j = 0; j < 8; ++j) mask[s] |= keep(e[s][j], thr) ? (1u << j) : 0u;
         }
-        const uint32_t cnt = __popc(mask);
-        uint32_t inc = cnt;                          // inclusive prefix over lanes
+    }
+#pragma unroll
+    for (int s = 0; s < kSegSteps; ++s) {            // independent inclusive prefixes over the lanes
+        uint32_t v = __popc(mask[s]);
 #pragma unroll
         for (int o = 1; o < kWave; o <<= 1) {
-            const uint32_t up = (uint32_t)__shfl_up((int)inc, o, kWave);
-            if (lane >= o) inc += up;
+            const uint32_t up = (uint32_t)__shfl_up((int)v, o, kWave);
+            if (lane >= o) v += up;
         }
-        int64_t w = base + (inc - cnt);
+        inc[s] = v;
+    }
+    uint32_t before[kSegSteps], total = 0;            // kept entries in the steps in front
+#pragma unroll
+    for (int s = 0; s < kSegSteps; ++s) {
+        before[s] = total;
+        total += (uint32_t)__shfl((int)inc[s], kWave - 1, kWave);
+    }
+    if (total <= kStageEntries) {
+        // usual case (a few percent kept): gather the wave's entries in LDS in output order, then
+        // write them with contiguous stores - one 512-byte run of indices per instruction instead
+        // of a handful of scattered 8-byte stores
+        uint32_t* st = stage[threadIdx.x >> 6];
+#pragma unroll
+        for (int s = 0; s < kSegSteps; ++s) {
+            uint32_t w = before[s] + (inc[s] - __popc(mask[s]));
+            const uint32_t rel = (uint32_t)(s * kWave + lane) * 8;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                if (mask[s] & (1u << j)) st[w++] = ((rel + j) << 16) | (e[s][j] & 0xffffu);
+            }
+        }
+        __builtin_amdgcn_wave_barrier();               // LDS writes of this wave are visible to its lanes
+        const int64_t first = seg * (int64_t)kSeg;
+        for (uint32_t k = lane; k < total; k += kWave) {
+            const uint32_t v = st[k];
+            idx_out[base + k] = first + (v >> 16);
+            val_out[base + k] = (uint16_t)v;
+        }
+        return;
+    }
+#pragma unroll
+    for (int s = 0; s < kSegSteps; ++s) {             // dense segment: store straight from registers
+        const int64_t c = seg * (kSeg / 8) + s * kWave + lane;
+        int64_t w = base + before[s] + (inc[s] - __popc(mask[s]));
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            if (mask & (1u << j)) {
+            if (mask[s] & (1u << j)) {
                 idx_out[w] = c * 8 + j;
-                val_out[w] = (uint16_t)e[j];
+                val_out[w] = (uint16_t)e[s][j];
                 ++w;
             }
         }
-        base += (uint32_t)__shfl((int)inc, kWave - 1, kWave);
     }
 }
 
@@ -266,6 +319,95 @@ __global__ __launch_bounds__(kSegThreads) void sparse_restore_kernel(const int64
                 for (int j = 0; j < 8 && i0 + j < n; ++j) out[i0 + j] = stage[wave][(s * kWave + lane) * 8 + j];
             }
         }
+    }
+}
+
+// ---- scaled, masked softmax forward (+ kept-entry count) ------------------------------------
+// a = bf16(softmax_fp32(t)),  t = bf16(bf16(s * scale) + mask)   (the mask term only if given):
+// the three torch passes "matmul / sqrt(d)", "+ attention_mask", "softmax(dtype=bf16)"
+// (models/llama/fused_llama_layer_intra_inter_full_fuse.py:159-167) in one read and one write.
+// One wave per row, the row held in registers (CH chunks of 8 per lane).  Row r uses mask row
+// (r / rows_per_batch) * mask_stride_b + (r % mask_rows) * mask_stride_row.
+// COUNT: a wave walks the 4096/n rows of one compaction segment and also leaves the number of
+// entries the compaction will keep (a > threshold, a != 0) in counts[segment], which saves
+// hyc_sparse_count's pass over the map.
+template <int CH, bool COUNT>
+__global__ __launch_bounds__(256) void softmax_fwd_kernel(const uint16_t* __restrict__ s, const uint16_t* __restrict__ mask,
+                                                          uint16_t* __restrict__ out, int64_t rows, int n, float scale,
+                                                          int mask_rows, int64_t rows_per_batch, int64_t mask_stride_b,
+                                                          int64_t mask_stride_row, const float* __restrict__ thr_p,
+                                                          uint32_t* __restrict__ counts, int rows_per_wave) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t w = blockIdx.x * 4ll + (threadIdx.x >> 6);
+    const int64_t row_begin = w * rows_per_wave;
+    if (row_begin >= rows) return;
+    float thr = 0.0f;
+    if constexpr (COUNT) thr = rbf(*thr_p);
+    uint32_t cnt = 0;
+    for (int r = 0; r < rows_per_wave; ++r) {
+        const int64_t row = row_begin + r;
+        if (row >= rows) break;
+        const int64_t base = row * n;
+        const uint16_t* mrow = nullptr;
+        if (mask) mrow = mask + (row / rows_per_batch) * mask_stride_b + (row % mask_rows) * mask_stride_row;
+        u32x4 sv[CH], mv[CH];
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int col = (c * kWave + lane) * 8;
+            sv[c] = u32x4{0, 0, 0, 0};
+            mv[c] = u32x4{0, 0, 0, 0};
+            if (col < n) {
+                sv[c] = ld16_nt(s + base + col);
+                if (mrow) mv[c] = ld16(mrow + col);
+            }
+        }
+        float t[CH][8];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int col = (c * kWave + lane) * 8;
+            float mf[8];
+            unpack8(sv[c], t[c]);
+            unpack8(mv[c], mf);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                float v = rbf(t[c][j] * scale);
+                if (mrow) v = rbf(v + mf[j]);
+                t[c][j] = col < n ? v : -INFINITY;
+                mx = fmaxf(mx, t[c][j]);
+            }
+        }
+        mx = wave_max(mx);
+        float sum = 0.0f;
+#pragma unroll
+        for (int c = 0; c < CH; ++c)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                t[c][j] = __expf(t[c][j] - mx);
+                sum += t[c][j];
+            }
+        sum = wave_sum(sum);
+        const float inv = __builtin_amdgcn_rcpf(sum);
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            const int col = (c * kWave + lane) * 8;
+            if (col < n) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) t[c][j] *= inv;
+                const u32x4 ov = pack8(t[c]);
+                st16_nt(out + base + col, ov);
+                if constexpr (COUNT) {
+                    const uint32_t d[4] = {ov.x, ov.y, ov.z, ov.w};
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) cnt += keep((d[j >> 1] >> (16 * (j & 1))) & 0xffffu, thr) ? 1u : 0u;
+                }
+            }
+        }
+    }
+    if constexpr (COUNT) {
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) cnt += (uint32_t)__shfl_xor((int)cnt, o, kWave);
+        if (lane == 0) counts[w] = cnt;
     }
 }
 
@@ -436,7 +578,7 @@ extern "C" int hyc_sparse_count(const void* a, int64_t n, const float* threshold
     if (nseg > 0)
         hipLaunchKernelGGL(sparse_count_kernel, dim3((unsigned)cdiv(nseg, 4)), dim3(kSegThreads), 0, st,
                            (const uint16_t*)a, n, threshold, nseg, seg_counts);
-    hipLaunchKernelGGL(seg_scan_kernel, dim3(1), dim3(1024), 0, st, seg_counts, nseg, seg_offsets);
+    hipLaunchKernelGGL(seg_scan_kernel, dim3((unsigned)(nseg > 1024 ? cdiv(nseg, 1024) : 1)), dim3(1024), 0, st, seg_counts, nseg, seg_offsets);
     return check_launch();
 }
 
@@ -514,5 +656,55 @@ extern "C" int hyc_softmax_bwd_restore(const int64_t* indices, const void* value
     else if (n == 1024) hipLaunchKernelGGL(softmax_bwd_restore_kernel<2>, grid, block, 0, st, indices, vp, seg_offsets, gp, nseg, ap, op);
     else if (n == 2048) hipLaunchKernelGGL(softmax_bwd_restore_kernel<4>, grid, block, 0, st, indices, vp, seg_offsets, gp, nseg, ap, op);
     else hipLaunchKernelGGL(softmax_bwd_restore_kernel<8>, grid, block, 0, st, indices, vp, seg_offsets, gp, nseg, ap, op);
+    return check_launch();
+}
+
+extern "C" int hyc_softmax_fwd(const void* s, const void* mask, void* out, int64_t rows, int64_t n, float scale,
+                               int64_t mask_rows, int64_t rows_per_batch, int64_t mask_stride_b, int64_t mask_stride_row,
+                               const float* threshold, uint32_t* seg_counts, int64_t* seg_offsets, void* stream) {
+    if (rows < 0 || n < 0) return HYC_ERR_SHAPE;
+    if (n % 8 != 0 || n > 8192) return HYC_ERR_SHAPE;
+    const bool count = threshold || seg_counts || seg_offsets;
+    if (count && !(threshold && seg_counts && seg_offsets)) return HYC_ERR_NULL;
+    if (count && (n < 512 || kSeg % n != 0 || (rows * n) % kSeg != 0)) return HYC_ERR_SHAPE;
+    if (rows == 0 || n == 0) {
+        if (count) hipLaunchKernelGGL(seg_scan_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, seg_counts, (int64_t)0, seg_offsets);
+        return count ? check_launch() : HYC_OK;
+    }
+    if (!s || !out) return HYC_ERR_NULL;
+    if (!aligned16(s) || !aligned16(out)) return HYC_ERR_ALIGN;
+    if (mask) {
+        if (!aligned16(mask) || mask_stride_b % 8 || mask_stride_row % 8) return HYC_ERR_ALIGN;
+        if (mask_rows <= 0 || rows_per_batch <= 0 || mask_stride_row < n) return HYC_ERR_SHAPE;
+    } else {
+        mask_rows = rows_per_batch = 1;
+    }
+    const int rpw = count ? (int)(kSeg / n) : 1;
+    const int64_t waves = cdiv(rows, (int64_t)rpw);
+    if (cdiv(waves, 4) > INT32_MAX) return HYC_ERR_SHAPE;
+    const dim3 grid((unsigned)cdiv(waves, 4)), block(256);
+    hipStream_t st = (hipStream_t)stream;
+    const uint16_t* sp = (const uint16_t*)s;
+    const uint16_t* mp = (const uint16_t*)mask;
+    uint16_t* op = (uint16_t*)out;
+#define HYC_SMF(CH)                                                                                                     \
+    do {                                                                                                                \
+        if (count)                                                                                                      \
+            hipLaunchKernelGGL((softmax_fwd_kernel<CH, true>), grid, block, 0, st, sp, mp, op, rows, (int)n, scale,      \
+                               (int)mask_rows, rows_per_batch, mask_stride_b, mask_stride_row, threshold, seg_counts, rpw); \
+        else                                                                                                            \
+            hipLaunchKernelGGL((softmax_fwd_kernel<CH, false>), grid, block, 0, st, sp, mp, op, rows, (int)n, scale,     \
+                               (int)mask_rows, rows_per_batch, mask_stride_b, mask_stride_row, threshold, seg_counts, rpw); \
+    } while (0)
+    if (n <= 512) HYC_SMF(1);
+    else if (n <= 1024) HYC_SMF(2);
+    else if (n <= 2048) HYC_SMF(4);
+    else if (n <= 4096) HYC_SMF(8);
+    else HYC_SMF(16);
+#undef HYC_SMF
+    if (count) {
+        const int64_t nseg = rows * n / kSeg;
+        hipLaunchKernelGGL(seg_scan_kernel, dim3((unsigned)(nseg > 1024 ? cdiv(nseg, 1024) : 1)), dim3(1024), 0, st, seg_counts, nseg, seg_offsets);
+    }
     return check_launch();
 }

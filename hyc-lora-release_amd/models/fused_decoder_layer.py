@@ -46,7 +46,7 @@ from ..operators.compress_function import (compress_attention_map, compression_p
 from ..operators.rmsnorm_kernels import _backward as _rmsnorm_backward
 from ..operators.rmsnorm_kernels import rmsnorm_forward
 from ..operators.silu_kernels import silu_backward, silu_hadamard
-from ..operators.softmax_kernels import softmax_backward_from_compressed
+from ..operators.softmax_kernels import softmax_backward_from_compressed, softmax_forward
 from ..operators.triton_fuse_lora_silu_hadamard_backward_kernels import triton_fuse_silu_backward
 from ..operators.triton_fuse_lora_silu_hadamard_forward_kernels import triton_fuse_silu_forward
 from .compute_utils import (head_to_hidden_shape, hidden_to_head_shape, lora_backward, lora_forward,
@@ -164,15 +164,30 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             quant("v_rep", v, "v")
 
         if spec.attention == "map":
-            s = q @ k.transpose(-2, -1) / math.sqrt(head_dim)
+            s = q @ k.transpose(-2, -1)
             del q, k
-            if attention_mask is not None:
-                s = s + attention_mask
-            a = torch.softmax(s, dim=-1, dtype=v.dtype)
+            # scale, mask and softmax in one pass over the scores, in place; once the threshold is
+            # frozen the same pass also counts the entries the compaction keeps
+            m = attention_mask
+            if m is not None and not (m.dim() == 4 and m.shape[1] == 1 and m.shape[0] in (1, s.shape[0])
+                                      and tuple(m.shape[2:]) == tuple(s.shape[2:])):
+                m = m.expand(s.shape[0], 1, *s.shape[2:]) if m.dim() == 4 and m.shape[1] == 1 else None
+            seg = None
+            if s.dtype == torch.bfloat16 and s.shape[-1] % 8 == 0 and s.shape[-1] <= 8192 and \
+                    (attention_mask is None or m is not None):
+                if calib:
+                    a = softmax_forward(s, 1.0 / math.sqrt(head_dim), m, inplace=True)
+                else:
+                    a, seg = softmax_forward(s, 1.0 / math.sqrt(head_dim), m, threshold=sv['a']['outlier'], inplace=True)
+            else:
+                s = s / math.sqrt(head_dim)
+                if attention_mask is not None:
+                    s = s + attention_mask
+                a = torch.softmax(s, dim=-1, dtype=v.dtype)
             del s
             thr = get_statistics_softmax(a, softmax_outlier_ratio) if calib else sv['a']['outlier']
             stats[("a", "outlier")] = thr
-            saved["a_idx"], saved["a_val"], saved["a_seg"] = compress_attention_map(a, thr)
+            saved["a_idx"], saved["a_val"], saved["a_seg"] = compress_attention_map(a, thr, seg)
             ctx.a_shape = tuple(a.shape)
             o = a @ v
             del a, v

@@ -285,10 +285,12 @@ def _threshold_tensor(outlier, device) -> torch.Tensor:
     return torch.tensor(float(outlier), device=device, dtype=torch.float32)
 
 
-def compress_attention_map(x: torch.Tensor, outlier):
+def compress_attention_map(x: torch.Tensor, outlier, seg_offsets=None):
     """Kept entries of the flattened map: (indices int64 [nnz] ascending, values bf16 [nnz],
     seg_offsets int64 [nseg + 1]).  An entry is kept when x > outlier (compared in bf16, as
-    torch does) and x != 0.  seg_offsets lets restore_attention_map skip the index search."""
+    torch does) and x != 0.  seg_offsets lets restore_attention_map skip the index search.
+    `seg_offsets` may be passed in when the producer of x already counted (softmax_forward with a
+    threshold): the counting pass is skipped."""
     _lib.require_gpu(x)
     if x.dtype != BF16:
         x = x.to(BF16)
@@ -298,10 +300,15 @@ def compress_attention_map(x: torch.Tensor, outlier):
     n = flat.numel()
     thr = _threshold_tensor(outlier, x.device)
     nseg = _lib.lib().hyc_sparse_num_segments(n)
-    counts = torch.empty(max(nseg, 1), device=x.device, dtype=torch.int32)
-    offsets = torch.empty(nseg + 1, device=x.device, dtype=torch.int64)
     st = _lib.stream_of(x)
-    _lib.call("hyc_sparse_count", flat.data_ptr(), n, thr.data_ptr(), counts.data_ptr(), offsets.data_ptr(), st)
+    if seg_offsets is not None:
+        if seg_offsets.numel() != nseg + 1 or seg_offsets.dtype != torch.int64:
+            raise ValueError("seg_offsets does not belong to a map of this size")
+        offsets = seg_offsets
+    else:
+        counts = torch.empty(max(nseg, 1), device=x.device, dtype=torch.int32)
+        offsets = torch.empty(nseg + 1, device=x.device, dtype=torch.int64)
+        _lib.call("hyc_sparse_count", flat.data_ptr(), n, thr.data_ptr(), counts.data_ptr(), offsets.data_ptr(), st)
     nnz = int(offsets[-1].item())      # the one host sync; to_sparse() has the same one
     idx = torch.empty(nnz, device=x.device, dtype=torch.int64)
     val = torch.empty(nnz, device=x.device, dtype=BF16)

@@ -47,3 +47,52 @@ def softmax_backward_from_compressed(idx, val, seg_offsets, grad_y, want_map=Tru
               seg_offsets.data_ptr(), grad_y.data_ptr(), _lib.ptr(a), o.data_ptr(), numel // n, n,
               _lib.stream_of(grad_y))
     return a, o
+
+
+COUNTED_ROW_LENGTHS = FUSED_ROW_LENGTHS
+
+
+def softmax_forward(s, scale, mask=None, threshold=None, inplace=False):
+    """bf16 softmax over the last dimension of  bf16(bf16(s * scale) + mask)  in one pass: what the
+    reference computes with three torch kernels (q @ k^T / sqrt(d), + attention_mask, softmax;
+    fused_llama_layer_intra_inter_full_fuse.py:159-167).
+
+    s: bf16 [..., rows, n] scores straight from the matmul; scale: Python float (1 / sqrt(head_dim));
+    mask: None or an additive bf16 mask broadcastable as [B or 1, 1, S, n] against s [B, H, S, n];
+    inplace: overwrite s.  With `threshold` (0-d tensor, the frozen keep-threshold) the per-segment
+    offsets of the compaction are produced in the same pass and returned as the second value (None
+    when the row length does not allow it); pass them to compress_attention_map."""
+    _lib.require_gpu(s)
+    if s.dtype != torch.bfloat16:
+        raise NotImplementedError("softmax_forward computes on bfloat16 scores")
+    n = s.shape[-1]
+    if n % 8 or n > 8192:
+        raise ValueError(f"row length {n}: must be a multiple of 8, at most 8192")
+    if not s.is_contiguous() or s.data_ptr() % 16:
+        s, inplace = s.contiguous(), True                     # a private copy may be overwritten
+    out = s if inplace else torch.empty_like(s)
+    rows = s.numel() // n if n else 0
+    mptr, mask_rows, rows_per_batch, msb, msr = None, 1, 1, 0, 0
+    if mask is not None:
+        _lib.require_gpu(mask)
+        if s.dim() != 4 or mask.dim() != 4 or mask.shape[1] != 1 or mask.shape[-1] != n or \
+                mask.shape[2] != s.shape[2] or mask.shape[0] not in (1, s.shape[0]):
+            raise ValueError(f"mask {tuple(mask.shape)} is not [B or 1, 1, S, n] for scores {tuple(s.shape)}")
+        if mask.dtype != torch.bfloat16:
+            mask = mask.to(torch.bfloat16)
+        if mask.stride(-1) != 1 or mask.stride(2) % 8 or mask.stride(0) % 8 or mask.data_ptr() % 16:
+            mask = mask.contiguous()
+        mptr, mask_rows, rows_per_batch = mask.data_ptr(), s.shape[2], s.shape[1] * s.shape[2]
+        msb, msr = (mask.stride(0) if mask.shape[0] > 1 else 0), mask.stride(2)
+    counts = offsets = thr = None
+    if threshold is not None and n in COUNTED_ROW_LENGTHS and s.numel() % 4096 == 0 and s.numel():
+        from .compress_function import _threshold_tensor
+        thr = _threshold_tensor(threshold, s.device)
+        nseg = s.numel() // 4096
+        counts = torch.empty(nseg, device=s.device, dtype=torch.int32)
+        offsets = torch.empty(nseg + 1, device=s.device, dtype=torch.int64)
+    _lib.call("hyc_softmax_fwd", s.data_ptr(), mptr, out.data_ptr(), rows, n, float(scale), mask_rows, rows_per_batch,
+              msb, msr, _lib.ptr(thr), _lib.ptr(counts), _lib.ptr(offsets), _lib.stream_of(s))
+    if threshold is not None:
+        return out, offsets
+    return out

@@ -191,6 +191,28 @@ int hyc_sparse_restore(const int64_t *indices, const void *values, const int64_t
 int hyc_softmax_bwd(const void *y, const void *grad_y, void *out, int64_t rows, int64_t n, void *stream);
 
 /* ---------------------------------------------------------------------------------------
+ * Scaled, masked softmax forward over the last dimension, optionally with the kept-entry count
+ * of the compaction that follows:
+ *     t = bf16(bf16(s * scale) + mask)   (mask term only if mask != NULL);   out = bf16(softmax_fp32(t)).
+ *
+ * Replaces the three torch passes  s = q @ k^T / sqrt(head_dim);  s = s + attention_mask;
+ * a = torch.softmax(s, dim=-1, dtype=v.dtype)
+ * (models/llama/fused_llama_layer_intra_inter_full_fuse.py:159-167; the scalar division is a
+ * multiplication by the fp32 reciprocal in torch's device kernel, hence `scale`).
+ *   s, out    bf16 [rows, n] contiguous, 16-byte aligned (out may alias s); n % 8 == 0, n <= 8192.
+ *   mask      bf16 or NULL; row r adds mask[(r / rows_per_batch) * mask_stride_b +
+ *             (r % mask_rows) * mask_stride_row + 0..n-1]  (a [B,1,S,S] mask over [B,H,S,S] scores:
+ *             mask_rows = S, rows_per_batch = H*S, strides S*S and S; stride_b = 0 broadcasts).
+ *   threshold, seg_counts, seg_offsets   all NULL, or all given: then seg_counts / seg_offsets are
+ *             filled exactly as hyc_sparse_count(out, rows*n, threshold, ...) would fill them, without
+ *             another pass over the map.  Needs n in {512,1024,2048,4096} and rows*n % 4096 == 0
+ *             (otherwise HYC_ERR_SHAPE: call hyc_sparse_count afterwards instead).
+ */
+int hyc_softmax_fwd(const void *s, const void *mask, void *out, int64_t rows, int64_t n, float scale,
+                    int64_t mask_rows, int64_t rows_per_batch, int64_t mask_stride_b, int64_t mask_stride_row,
+                    const float *threshold, uint32_t *seg_counts, int64_t *seg_offsets, void *stream);
+
+/* ---------------------------------------------------------------------------------------
  * Dense restore and softmax backward in one pass over the compressed map: saves reading the
  * restored map back (1 of the 4 dense passes of restore + backward).
  *

@@ -17,6 +17,8 @@ Pinning status (what independent evidence holds each function in place):
     operations; pinned by closed forms and planted outlier channels.
   * softmax_threshold / softmax_compress / softmax_restore: pinned against
     torch.sort / torch.nonzero on small inputs.
+  * softmax_fwd: pinned to tolerance against a float64 softmax of the same rounded logits,
+    by unit row sums, exact zeros under a -inf mask and shift invariance.
   * softmax_bwd, rmsnorm_fwd, silu_*, gelu_bwd, fused_*: pinned to tolerance against
     torch.autograd of the fp32 composite.  rmsnorm_bwd follows the reference's
     formula (which keeps LayerNorm's mean term) and is pinned only against a
@@ -258,6 +260,16 @@ def softmax_restore(idx, vals, shape) -> torch.Tensor:
     out = torch.zeros(math.prod(shape), dtype=vals.dtype, device=vals.device)
     out[idx] = vals
     return out.reshape(shape)
+
+
+def softmax_fwd(s: torch.Tensor, scale: float, mask=None) -> torch.Tensor:
+    """bf16(softmax_fp32(bf16(bf16(s * scale) + mask))): `q @ k^T / sqrt(d)` (a multiplication by the
+    fp32 reciprocal in torch's device kernel), `+ attention_mask`, `torch.softmax(dtype=bf16)` with
+    its fp32 internals (fused_llama_layer_intra_inter_full_fuse.py:159-167)."""
+    t = (s.to(BF16).float() * torch.tensor(scale, dtype=F32)).to(BF16)
+    if mask is not None:
+        t = t + mask.to(BF16)
+    return torch.softmax(t.float(), dim=-1).to(BF16)
 
 
 def softmax_bwd(y: torch.Tensor, g: torch.Tensor) -> torch.Tensor:

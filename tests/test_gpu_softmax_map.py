@@ -149,6 +149,61 @@ def test_softmax_backward_from_compressed(cf, sk, dev, shape, ratio):
         assert i_o.numel() == 0 and not bool(o.cpu().float().abs().max()) and not bool(ref.float().abs().max())
 
 
+@pytest.mark.parametrize("shape", [(2, 4, 128, 128), (1, 2, 64, 1024), (2, 2, 24, 512), (1, 1, 8, 2048), (1, 1, 4, 4096),
+                                   (1, 1, 3, 8192), (1, 3, 40, 40), (1, 2, 7, 1000)])
+@pytest.mark.parametrize("masked", ["causal", "batch", None])
+def test_softmax_forward(sk, dev, shape, masked):
+    b, h, m, n = shape
+    g = torch.Generator().manual_seed(n + m)
+    s = (torch.randn(*shape, generator=g) * 20).to(BF16)
+    mask = None
+    if masked == "causal":                         # [1,1,S,n] additive, -inf above the diagonal band
+        mask = torch.zeros(1, 1, m, n)
+        mask[0, 0] = torch.full((m, n), float("-inf")).triu(n - m + 1)
+        mask = mask.to(BF16)
+    elif masked == "batch":                        # [B,1,S,n] with the dtype's minimum, as HF builds it
+        mask = torch.where(torch.rand(b, 1, m, n, generator=g) < 0.3, torch.finfo(BF16).min, 0.0).to(BF16)
+        mask[..., 0] = 0
+    scale = 1.0 / 128 ** 0.5
+    want = O.softmax_fwd(s, scale, mask)
+    got = sk.softmax_forward(s.to(dev), scale, None if mask is None else mask.to(dev))
+    assert got.dtype == BF16 and got.shape == s.shape
+    assert_close_bf16(got, want, what="softmax_forward vs oracle")
+    # independent: float64 softmax of the same bf16 logits; rows sum to one; masked entries are exactly zero
+    t = (s.float() * torch.tensor(scale)).to(BF16)
+    if mask is not None:
+        t = t + mask
+    ref = torch.softmax(t.double(), dim=-1)
+    assert_close_bf16(got, ref, what="softmax_forward vs float64")
+    assert (got.float().sum(-1).cpu() - 1).abs().max() < 2e-2
+    if masked == "causal":
+        assert not bool(got.cpu()[mask.expand_as(s) == float("-inf")].float().abs().max())
+    # in place
+    sd = s.to(dev)
+    same = sk.softmax_forward(sd, scale, None if mask is None else mask.to(dev), inplace=True)
+    assert same.data_ptr() == sd.data_ptr() and same_bits(same, got)
+
+
+@pytest.mark.parametrize("shape", [(1, 2, 16, 512), (2, 2, 8, 1024), (1, 1, 6, 2048), (1, 3, 4, 4096), (1, 1, 3, 8192), (1, 2, 40, 40)])
+def test_softmax_forward_counts_for_the_compaction(cf, sk, dev, shape):
+    """With a frozen threshold the forward pass hands the compaction its segment offsets: same
+    compressed map as the separate counting pass (for row lengths that do not allow it the second
+    value is None and the compaction counts by itself)."""
+    g = torch.Generator().manual_seed(shape[-1])
+    s = (torch.randn(*shape, generator=g) * 8).to(BF16).to(dev)
+    a = sk.softmax_forward(s, 0.25)
+    thr = cf.get_statistics_softmax(a, 0.05)
+    a2, seg = sk.softmax_forward(s, 0.25, threshold=thr)
+    assert same_bits(a2, a)
+    idx, val, seg_ref = cf.compress_attention_map(a, thr)
+    if shape[-1] in (512, 1024, 2048, 4096):
+        assert seg is not None and torch.equal(seg, seg_ref)
+    else:
+        assert seg is None
+    idx2, val2, seg2 = cf.compress_attention_map(a2, thr, seg)
+    assert torch.equal(idx2, idx) and same_bits(val2, val) and torch.equal(seg2, seg_ref)
+
+
 def test_full_size_config3_properties(cf, sk, dev):
     # BASELINE configuration 3 at full size: [4,32,1024,1024], ratio 0.05
     g = torch.Generator(device=dev).manual_seed(1)
