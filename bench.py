@@ -394,6 +394,15 @@ def main():
         _, sc = cf.get_statistics_channel_base(x_h[0], 0.005, QB, 'per-channel')
         ms, _ = timed(lambda i: cf.outlier_subtraction_fuse_compression_quantization(x_h[i % 4], sc, idx, QB), Kx, Wx)
         kernels["quant_pack_q4_outlier_4096"] = {"ms": ms, "GBps": T * H * 2.5 / ms / 1e6}
+        sy = cf.get_statistics_only_quant(y, QB, 'per-channel')
+        tbl = rmsnorm_kernels.outlier_table(idx, H)
+        ms, _ = timed(lambda i: rmsnorm_kernels.rmsnorm_forward_compress(x_h[i % 4], w_h, 1e-5, QB, scale_y=sy, scale_x=sc,
+                                                                         outlier_idx=idx, table=tbl), Kx, Wx)
+        ms3, _ = timed(lambda i: (rmsnorm_kernels.rmsnorm_forward(x_h[i % 4], w_h, 1e-5),
+                                  cf.outlier_subtraction_fuse_compression_quantization(x_h[i % 4], sc, idx, QB),
+                                  cf.compression_quantization(x_h[(i + 1) % 4], sy, QB)), Kx, Wx)
+        kernels["rmsnorm_fwd_compress_4096"] = {"ms": ms, "GBps": T * H * (4 + 2 * QB / 8) / ms / 1e6,
+                                                "three_separate_kernels_ms": ms3}
         ms, _ = timed(lambda i: cf.get_statistics_channel_base(x_h[i % 4], 0.005, QB, 'per-channel'), Kx, Wx)
         kernels["calibration_stats_4096"] = {"ms": ms}
         # attention map (configuration 3 shape): compaction, restore, softmax backward

@@ -44,7 +44,7 @@ from ..operators.compress_function import (compress_attention_map, compression_p
                                            outlier_addition_fuse_decompression_dequantization,
                                            update_dict)
 from ..operators.rmsnorm_kernels import _backward as _rmsnorm_backward
-from ..operators.rmsnorm_kernels import rmsnorm_forward
+from ..operators.rmsnorm_kernels import rmsnorm_forward, rmsnorm_forward_compress
 from ..operators.silu_kernels import silu_backward, silu_hadamard
 from ..operators.softmax_kernels import softmax_backward_from_compressed, softmax_forward
 from ..operators.triton_fuse_lora_silu_hadamard_backward_kernels import triton_fuse_silu_backward
@@ -132,14 +132,31 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             stats[(name, "outlier_channel_index")], stats[(name, "scale")] = idx, s
             saved[name + "_o"], saved[name + "_q"], saved[name + "_s"], saved[name + "_idx"] = o, q, s, idx
 
+        def norm_block(xname, nname, t, w):
+            """RMSNorm of t plus the compressed copies of t (channel base) and of the output.  With
+            frozen statistics all three come out of one pass over t; while calibrating the steps of
+            the output depend on the output, so the separate operators run (returns done=False and
+            the caller quantises the output itself)."""
+            n = t.shape[-1]
+            if calib or t.dtype != torch.bfloat16 or t.dim() != 3 or n % 32 or n > 8192:
+                y, _, rstd, _, _ = rmsnorm_forward(t, w, spec.eps)
+                channel_base(xname, t)
+                return y, rstd, False
+            idx, sx, sn = sv[xname]['outlier_channel_index'], sv[xname]['scale'], sv[nname]['scale']
+            y, rstd, q_y, q_x, x_out = rmsnorm_forward_compress(t, w, spec.eps, q_bit, scale_y=sn, scale_x=sx,
+                                                                outlier_idx=idx)
+            stats[(xname, "outlier_channel_index")], stats[(xname, "scale")], stats[(nname, "scale")] = idx, sx, sn
+            saved[xname + "_o"], saved[xname + "_q"], saved[xname + "_s"], saved[xname + "_idx"] = x_out, q_x, sx, idx
+            saved[nname + "_q"], saved[nname + "_s"] = q_y, sn
+            return y, rstd, True
+
         # ---- attention block -------------------------------------------------------------------
-        x_norm_1, _, rstd_1, block_size, num_warps = rmsnorm_forward(x, norm_weight_1, spec.eps)
-        saved["rstd_1"] = rstd_1
-        channel_base("x", x)
+        x_norm_1, saved["rstd_1"], norm_1_done = norm_block("x", "x_norm_1", x, norm_weight_1)
         q, q_main, saved["q_lora_a"] = proj("q", x_norm_1)
         k, k_main, saved["k_lora_a"] = proj("k", x_norm_1)
         v, v_main, saved["v_lora_a"] = proj("v", x_norm_1)
-        quant("x_norm_1", x_norm_1)
+        if not norm_1_done:
+            quant("x_norm_1", x_norm_1)
         del x_norm_1
         if spec.mode != "intra":
             if spec.attention == "sdpa":
@@ -202,9 +219,7 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
         del o_final
 
         # ---- MLP block ---------------------------------------------------------------------------
-        x_norm_2, _, rstd_2, block_size, num_warps = rmsnorm_forward(x_medium, norm_weight_2, spec.eps)
-        saved["rstd_2"] = rstd_2
-        channel_base("x_medium", x_medium)
+        x_norm_2, saved["rstd_2"], norm_2_done = norm_block("x_medium", "x_norm_2", x_medium, norm_weight_2)
         if spec.mode == "intra_inter_full_fuse":
             from .compute_utils import dense_weight
             wg, wu = dense_weight(w_gate, qs_gate).t(), dense_weight(w_up, qs_up).t()
@@ -239,7 +254,8 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
                 del fn
             del gate, up, gate_main, up_main
         saved["gate_lora_a"], saved["up_lora_a"] = gate_lora_a, up_lora_a
-        quant("x_norm_2", x_norm_2)
+        if not norm_2_done:
+            quant("x_norm_2", x_norm_2)
         del x_norm_2
         down, _, saved["down_lora_a"] = proj("down", hadamard)
         if spec.mode == "intra":
@@ -253,7 +269,6 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
         ctx.quant_states = {n: W[n][2] for n in _PROJ}
         ctx.spec, ctx.q_bit = spec, q_bit
         ctx.num_heads, ctx.num_key_value_heads, ctx.head_dim = num_heads, num_key_value_heads, head_dim
-        ctx.block_size, ctx.num_warps = block_size, num_warps
         ctx.has_mask = attention_mask is not None
         ctx.attention_mask = attention_mask
         ctx.norm_grads = (norm_weight_1.requires_grad, norm_weight_2.requires_grad)

@@ -73,3 +73,60 @@ def rmsnorm_backward(dy, x, w, m, v, needs_inputs_grad, eps, num_warps, BLOCK_SI
         return None, None
     dx, _ = _backward(dy, x, w, v, want_dw=False)
     return dx, None
+
+
+def outlier_table(outlier_idx, n):
+    """uint16 [n] lookup for rmsnorm_forward_compress: 1 + list position for an outlier channel, else
+    0.  Worth caching while the channel list is frozen."""
+    _lib.require_gpu(outlier_idx)
+    idx = outlier_idx.reshape(-1).to(torch.int64).contiguous()
+    table = torch.empty((n,), dtype=torch.int16, device=idx.device)
+    _lib.call("hyc_outlier_table", idx.data_ptr() if idx.numel() else None, idx.numel(), n, table.data_ptr(),
+              _lib.stream_of(idx))
+    return table
+
+
+def rmsnorm_forward_compress(x, weight, eps, q_bit, scale_y=None, scale_x=None, outlier_idx=None, table=None):
+    """RMSNorm forward that also produces, from the same read of x, the packed codes of the
+    normalised output (steps `scale_y`) and the channel-base compressed input (steps `scale_x`,
+    outlier channels `outlier_idx`): what rmsnorm_forward + compression_pack_quant_base(y) +
+    compression_pack_channel_base(x) produce with frozen statistics, bit for bit
+    (fused_llama_layer_intra_inter_full_fuse.py:97-126).
+
+    -> (y, rstd, q_y or None, q_x or None, x_outlier or None)."""
+    _lib.require_gpu(x, weight)
+    if x.dtype != torch.bfloat16 or x.dim() != 3:
+        raise NotImplementedError("rmsnorm_forward_compress takes bfloat16 [batch, seq, hidden] activations")
+    if q_bit not in (2, 4, 8):
+        raise ValueError(f"q_bit must be 2, 4 or 8, got {q_bit}")
+    x = x.contiguous()
+    b, m, n = x.shape
+    if n % 32 or n > 8192:
+        raise ValueError(f"hidden size {n}: must be a multiple of 32, at most 8192")
+    rows = b * m
+    dev = x.device
+    y = torch.empty_like(x)
+    rstd = torch.empty((rows,), dtype=torch.float32, device=dev)
+    w, w32 = _weight(weight)
+
+    def steps(sc):
+        sc = sc.reshape(-1).to(torch.bfloat16).contiguous()
+        if sc.numel() != n:
+            raise ValueError(f"{sc.numel()} steps for {n} channels")
+        return sc
+    q_y = q_x = x_out = None
+    k = 0
+    if scale_y is not None:
+        scale_y = steps(scale_y)
+        q_y = torch.empty((b, m, n * q_bit // 8), dtype=torch.uint8, device=dev)
+    if scale_x is not None:
+        scale_x = steps(scale_x)
+        q_x = torch.empty((b, m, n * q_bit // 8), dtype=torch.uint8, device=dev)
+        k = 0 if outlier_idx is None else outlier_idx.numel()
+        x_out = torch.empty((b, m, k), dtype=torch.bfloat16, device=dev)
+        if k and table is None:
+            table = outlier_table(outlier_idx, n)
+    _lib.call("hyc_rmsnorm_fwd_compress", x.data_ptr(), w.data_ptr(), w32, y.data_ptr(), rstd.data_ptr(), rows, n,
+              float(eps), q_bit, _lib.ptr(scale_y), _lib.ptr(q_y), _lib.ptr(scale_x), _lib.ptr(q_x),
+              _lib.ptr(table) if k else None, k, _lib.ptr(x_out) if k else None, _lib.stream_of(x))
+    return y, rstd, q_y, q_x, x_out

@@ -256,6 +256,30 @@ int hyc_rmsnorm_bwd(const void *dy, const void *x, const void *weight, int weigh
                     int64_t rows, int64_t N, void *stream);
 
 /* ---------------------------------------------------------------------------------------
+ * RMSNorm forward fused with the compressions a decoder layer applies around it: the row is read
+ * once and yields the normalised output, its quantised copy and the channel-base compressed copy
+ * of the input.
+ *
+ * Replaces the sequence rmsnorm_forward(x, w, eps); compression_pack_channel_base(x, ...);
+ * compression_pack_quant_base(x_norm, ...) with frozen statistics
+ * (models/llama/fused_llama_layer_intra_inter_full_fuse.py:97-126; kernels
+ * operators/rmsnorm_kernels.py:10-54 and operators/compress_function_kernel.py:46-112).  Results are
+ * bit-identical to hyc_rmsnorm_fwd followed by hyc_quant_pack on y and on x.
+ *   x, y        bf16 [rows, N] contiguous; N % 32 == 0, N <= 8192;  rstd fp32 [rows].
+ *   scale_y,q_y steps bf16 [N] and packed codes uint8 [rows, N*q_bit/8] of y; q_y NULL: skipped.
+ *   scale_x,q_x the same for x with the outlier channels zeroed; q_x NULL: skipped.
+ *   outlier_table uint16 [N] from hyc_outlier_table (1 + list position of an outlier channel, else 0),
+ *   k           number of outlier channels, x_outlier bf16 [rows, k] (column order = list order).
+ *
+ * hyc_outlier_table builds that table from a channel list (int64 [k], k <= 65535).
+ */
+int hyc_outlier_table(const int64_t *outlier_idx, int64_t k, int64_t N, uint16_t *table, void *stream);
+int hyc_rmsnorm_fwd_compress(const void *x, const void *weight, int weight_is_fp32, void *y, float *rstd,
+                             int64_t rows, int64_t N, float eps, int q_bit, const void *scale_y, void *q_y,
+                             const void *scale_x, void *q_x, const uint16_t *outlier_table, int64_t k,
+                             void *x_outlier, void *stream);
+
+/* ---------------------------------------------------------------------------------------
  * Rotary position embedding, in place: for every (b, s, h) the head x[b,s,h,:] = (x1 | x2) becomes
  * (x1*cos[s] - x2*sin[s] | x2*cos[s] + x1*sin[s]); backward != 0 uses -sin.
  *

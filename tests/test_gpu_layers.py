@@ -228,6 +228,33 @@ def test_calibration_state_machine(dev):
         make_fused_llama_layer(config("no_such_type", 4))
 
 
+@pytest.mark.parametrize("layer_type", ["intra", "intra_inter", "intra_inter_full_fuse"])
+@pytest.mark.parametrize("q_bit", [4, 2])
+def test_frozen_statistics_path_equals_calibrating_path(dev, layer_type, q_bit):
+    """Once the statistics are frozen the layer switches to kernels that fuse more (norm + both
+    compressions in one pass, softmax that also counts for the compaction).  On the same input the
+    frozen statistics equal the fresh ones, so the two code paths must agree bit for bit."""
+    import hyclora_amd  # noqa: F401
+    from hyclora_amd.models.llama import make_fused_llama_layer
+    t = make_layer_inputs(dev, seed=31, S=128, hidden=512, heads=4, kv_heads=4, inter=1024)   # rows of 128: not counted in the softmax pass
+    t2 = make_layer_inputs(dev, seed=32, S=512, hidden=256, heads=2, kv_heads=2, inter=512)   # rows of 512: counted
+    for tt in (t, t2):
+        layer = make_fused_llama_layer(config(layer_type, q_bit, sm_ratio=0.05, thr=1))
+        outs = []
+        for it in range(2):
+            y = run_fused(layer, tt)
+            y.backward(tt.grad)
+            outs.append((y.detach().clone(), tt.x.grad.clone(), [m.weight.grad.clone() for n in tt.P for m in tt.P[n][1:]]))
+            tt.x.grad = None
+            for n in tt.P:
+                for m in tt.P[n][1:]:
+                    m.weight.grad = None
+        assert layer.iteration == 2
+        assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+        for a, b in zip(outs[0][2], outs[1][2]):
+            assert torch.equal(a, b)
+
+
 def test_calibration_state_survives_a_checkpoint(dev, tmp_path):
     """Calibrate, save state_dict, load it into a fresh module (weights_only loader): the resumed
     layer is past calibration and reproduces the original's next step bit for bit."""

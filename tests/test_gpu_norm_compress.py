@@ -1,0 +1,71 @@
+"""GPU parity of the fused RMSNorm-forward + compression kernel: its outputs must equal, bit for
+bit, those of the separate operators (which are themselves checked against the oracle), and the
+oracle's compressed forms directly."""
+import pytest
+import torch
+
+from helpers import BF16, activation_with_outlier_channels, assert_close_bf16, same_bits
+from oracle import hyc_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import hyclora_amd  # noqa: F401
+    from hyclora_amd.operators import compress_function, rmsnorm_kernels
+
+    class Ops:
+        cf = compress_function
+        norm = rmsnorm_kernels
+    return Ops
+
+
+@pytest.mark.parametrize("q_bit", [2, 4, 8])
+@pytest.mark.parametrize("shape", [(2, 37, 4096), (1, 5, 512), (3, 4, 96), (1, 9, 8192), (2, 3, 1024 + 32)])
+@pytest.mark.parametrize("wdtype", [BF16, torch.float32])
+def test_fused_equals_separate_operators(ops, dev, q_bit, shape, wdtype):
+    x, planted = activation_with_outlier_channels(seed=shape[-1] + q_bit, shape=shape, frac=0.01)
+    g = torch.Generator().manual_seed(1)
+    w = (1 + 0.1 * torch.randn(shape[-1], generator=g)).to(wdtype)
+    xd, wd = x.to(dev), w.to(dev)
+    # frozen statistics, as after calibration
+    idx, s_x = ops.cf.get_statistics_channel_base(xd, 0.01, q_bit, 'per-channel')
+    y_ref, _, rstd_ref, _, _ = ops.norm.rmsnorm_forward(xd, wd, 1e-5)
+    s_y = ops.cf.get_statistics_only_quant(y_ref, q_bit, 'per-channel')
+    xo_ref, qx_ref = ops.cf.outlier_subtraction_fuse_compression_quantization(xd, s_x, idx, q_bit)
+    qy_ref = ops.cf.compression_quantization(y_ref, s_y, q_bit)
+
+    y, rstd, q_y, q_x, x_out = ops.norm.rmsnorm_forward_compress(xd, wd, 1e-5, q_bit, scale_y=s_y, scale_x=s_x, outlier_idx=idx)
+    assert same_bits(y, y_ref) and torch.equal(rstd, rstd_ref)
+    assert torch.equal(q_y, qy_ref) and torch.equal(q_x, qx_ref) and same_bits(x_out, xo_ref)
+    # against the oracle's own forms of the two compressions
+    xo_o, qx_o = O.compress_channel_base(x, s_x.cpu(), idx.cpu(), q_bit)
+    assert torch.equal(q_x.cpu(), qx_o) and same_bits(x_out.cpu(), xo_o)
+    assert torch.equal(q_y.cpu(), O.compress(y_ref.cpu(), s_y.cpu(), q_bit))
+    y_o, _ = O.rmsnorm_fwd(x, w, 1e-5)
+    assert_close_bf16(y, y_o, what="fused rmsnorm y vs oracle")
+    # parts can be switched off
+    y2, _, q_y2, q_x2, xo2 = ops.norm.rmsnorm_forward_compress(xd, wd, 1e-5, q_bit, scale_y=s_y)
+    assert same_bits(y2, y_ref) and torch.equal(q_y2, qy_ref) and q_x2 is None and xo2 is None
+    y3, _, q_y3, q_x3, xo3 = ops.norm.rmsnorm_forward_compress(xd, wd, 1e-5, q_bit, scale_x=s_x)   # no outlier channels
+    assert q_y3 is None and xo3.shape[-1] == 0
+    assert torch.equal(q_x3, ops.cf.compression_quantization(xd, s_x, q_bit))
+
+
+def test_outlier_table_and_errors(ops, dev):
+    idx = torch.tensor([5, 0, 31, 7], device=dev)
+    t = ops.norm.outlier_table(idx, 32).cpu().tolist()
+    want = [0] * 32
+    want[5], want[0], want[31], want[7] = 1, 2, 3, 4
+    assert t == want
+    x = torch.zeros(1, 2, 40, device=dev, dtype=BF16)
+    w = torch.ones(40, device=dev, dtype=BF16)
+    with pytest.raises(ValueError):
+        ops.norm.rmsnorm_forward_compress(x, w, 1e-5, 4, scale_y=torch.ones(40, device=dev, dtype=BF16))   # N % 32
+    x = torch.zeros(1, 2, 64, device=dev, dtype=BF16)
+    w = torch.ones(64, device=dev, dtype=BF16)
+    with pytest.raises(ValueError):
+        ops.norm.rmsnorm_forward_compress(x, w, 1e-5, 3, scale_y=torch.ones(64, device=dev, dtype=BF16))
+    with pytest.raises(ValueError):
+        ops.norm.rmsnorm_forward_compress(x, w, 1e-5, 4, scale_y=torch.ones(32, device=dev, dtype=BF16))
