@@ -675,7 +675,7 @@ extern "C" int hyc_softmax_fwd(const void* s, const void* mask, void* out, int64
     if (!aligned16(s) || !aligned16(out)) return HYC_ERR_ALIGN;
     if (mask) {
         if (!aligned16(mask) || mask_stride_b % 8 || mask_stride_row % 8) return HYC_ERR_ALIGN;
-        if (mask_rows <= 0 || rows_per_batch <= 0 || mask_stride_row < n) return HYC_ERR_SHAPE;
+        if (mask_rows <= 0 || rows_per_batch <= 0 || (mask_stride_row != 0 && mask_stride_row < n)) return HYC_ERR_SHAPE;
     } else {
         mask_rows = rows_per_batch = 1;
     }

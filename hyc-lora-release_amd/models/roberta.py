@@ -1,0 +1,338 @@
+"""RoBERTa encoder layers (post-LayerNorm, GELU MLP) with compressed saved activations; class names,
+argument order and calibration behaviour of the reference
+(models/roberta/fused_roberta_layer_{intra,intra_inter}.py).
+
+One autograd.Function serves both layer types:
+  intra        keeps the quantised tensors the backward needs as they are (q, k, v in head shape after
+               the LoRA add, up, gelu(up));
+  intra_inter  keeps only the frozen-weight parts of q, k, v, up and rebuilds the rest in backward
+               from the saved LoRA-A products (…intra_inter.py:90-121, :367-371, :411-423).
+"""
+import math
+
+import torch
+
+from ..operators.compress_function import (compress_attention_map, compression_pack_channel_base,
+                                           compression_pack_quant_base, decompression_dequantization,
+                                           get_statistics_softmax,
+                                           outlier_addition_fuse_decompression_dequantization, update_dict)
+from ..operators.gelu_kernels import gelu_backward
+from ..operators.layernorm_kernels import layernorm_backward, layernorm_forward
+from ..operators.softmax_kernels import softmax_backward_from_compressed, softmax_forward
+from .compute_utils import head_to_hidden_shape, hidden_to_head_shape, lora_backward, lora_forward
+
+MODES = ("intra", "intra_inter")
+_PROJ = ("q", "k", "v", "o", "up", "down")
+_EPS = 1e-5
+
+
+def stat_slots(mode):
+    """(static_value key, field) of every calibration statistic the layer returns, in the reference's
+    order (…intra_inter.py:277-282; the intra file adds gelu(up), :296)."""
+    slots = [("x", "scale"), ("q", "scale"), ("k", "scale"), ("v", "scale"), ("a", "outlier"), ("o", "scale"),
+             ("o_final", "outlier_channel_index"), ("o_final", "scale"), ("x_medium", "scale"), ("up", "scale")]
+    if mode == "intra":
+        slots.append(("fn", "scale"))
+    return slots + [("down", "outlier_channel_index"), ("down", "scale")]
+
+
+def _weight_of(lora_linear):
+    inner = getattr(lora_linear, "default", lora_linear)       # peft wraps adapters in a ModuleDict
+    return inner.weight
+
+
+class FusedRobertaLayerFunc(torch.autograd.Function):
+    """Inputs follow the reference's Func.apply order (…intra_inter.py:26-85) with the mode appended."""
+
+    @staticmethod
+    def forward(ctx, x,
+                w_q, b_q, qs_q, a_q, bb_q, w_k, b_k, qs_k, a_k, bb_k, w_v, b_v, qs_v, a_v, bb_v,
+                w_o, b_o, qs_o, a_o, bb_o, norm_weight_1, norm_bias_1,
+                w_up, b_up, qs_up, a_up, bb_up, w_down, b_down, qs_down, a_down, bb_down,
+                norm_weight_2, norm_bias_2, attention_mask, num_heads, head_dim,
+                iteration, iteration_threshold, static_value, softmax_outlier_ratio, layernorm_outlier_ratio,
+                q_bit, mode):
+        if mode not in MODES:
+            raise ValueError(f"layer_type must be one of {MODES}, got {mode!r}")
+        W = dict(q=(w_q, b_q, qs_q, a_q, bb_q), k=(w_k, b_k, qs_k, a_k, bb_k), v=(w_v, b_v, qs_v, a_v, bb_v),
+                 o=(w_o, b_o, qs_o, a_o, bb_o), up=(w_up, b_up, qs_up, a_up, bb_up),
+                 down=(w_down, b_down, qs_down, a_down, bb_down))
+        it, thd, sv = iteration, iteration_threshold, static_value
+        calib = it < thd
+        saved, stats = {}, {}
+
+        def proj(name, inp):
+            w, b, qs, la, lb = W[name]
+            return lora_forward(w, qs, la, lb, b, inp)
+
+        def quant(name, t, key=None):
+            q, s = compression_pack_quant_base(t, q_bit, 'per-channel', it, thd, sv[key or name])
+            stats[(key or name, "scale")] = s
+            saved[name + "_q"], saved[name + "_s"] = q, s
+
+        def channel_base(name, t):
+            o, q, idx, s = compression_pack_channel_base(t, layernorm_outlier_ratio, q_bit, 'per-channel', it, thd,
+                                                         sv[name])
+            stats[(name, "outlier_channel_index")], stats[(name, "scale")] = idx, s
+            saved[name + "_o"], saved[name + "_q"], saved[name + "_s"], saved[name + "_idx"] = o, q, s, idx
+
+        # ---- attention block -------------------------------------------------------------------
+        q, q_main, saved["q_lora_a"] = proj("q", x)
+        k, k_main, saved["k_lora_a"] = proj("k", x)
+        v, v_main, saved["v_lora_a"] = proj("v", x)
+        quant("x", x)
+        if mode == "intra_inter":
+            quant("q_main", q_main, "q")
+            quant("k_main", k_main, "k")
+            quant("v_main", v_main, "v")
+        del q_main, k_main, v_main
+        q, k, v = (hidden_to_head_shape(t, num_heads) for t in (q, k, v))
+        if mode == "intra":
+            quant("q", q)
+            quant("k", k)
+        s = q @ k.transpose(-2, -1)
+        del q, k
+        m = attention_mask
+        fits = m is None or (m.dim() == 4 and m.shape[1] == 1 and m.shape[0] in (1, s.shape[0]) and
+                             m.shape[-1] == s.shape[-1] and m.shape[2] in (1, s.shape[2]))
+        if s.dtype == torch.bfloat16 and s.shape[-1] % 8 == 0 and s.shape[-1] <= 8192 and fits:
+            if m is not None and m.shape[2] == 1:                # padding mask [B,1,1,S]: one row for all queries
+                m = m.expand(m.shape[0], 1, s.shape[2], s.shape[3])
+            seg = None
+            if calib:
+                a = softmax_forward(s, 1.0 / math.sqrt(head_dim), m, inplace=True)
+            else:
+                a, seg = softmax_forward(s, 1.0 / math.sqrt(head_dim), m, threshold=sv['a']['outlier'], inplace=True)
+        else:
+            seg = None
+            s = s / math.sqrt(head_dim)
+            if attention_mask is not None:
+                s = s + attention_mask
+            a = torch.softmax(s, dim=-1, dtype=v.dtype)
+        del s
+        o = a @ v
+        thr = get_statistics_softmax(a, softmax_outlier_ratio) if calib else sv['a']['outlier']
+        stats[("a", "outlier")] = thr
+        saved["a_idx"], saved["a_val"], saved["a_seg"] = compress_attention_map(a, thr, seg)
+        ctx.a_shape = tuple(a.shape)
+        del a
+        if mode == "intra":
+            quant("v", v)
+        del v
+        o = head_to_hidden_shape(o)
+        o_final, _, saved["o_lora_a"] = proj("o", o)
+        quant("o", o)
+        del o
+
+        # ---- first LayerNorm (post-norm: on the residual sum) ----------------------------------
+        o_final += x
+        x_medium, saved["mean_1"], saved["rstd_1"], _, _ = layernorm_forward(o_final, norm_weight_1, norm_bias_1, _EPS)
+        channel_base("o_final", o_final)
+        del o_final
+
+        # ---- MLP block ---------------------------------------------------------------------------
+        up, up_main, saved["up_lora_a"] = proj("up", x_medium)
+        quant("x_medium", x_medium)
+        if mode == "intra_inter":
+            quant("up_main", up_main, "up")
+        del up_main
+        fn = torch.nn.functional.gelu(up)
+        if mode == "intra":
+            quant("up", up)
+        del up
+        down, _, saved["down_lora_a"] = proj("down", fn)
+        down += x_medium
+        if mode == "intra":
+            quant("fn", fn)
+        del fn, x_medium
+        x_out, saved["mean_2"], saved["rstd_2"], block_size, num_warps = layernorm_forward(down, norm_weight_2, norm_bias_2, _EPS)
+        channel_base("down", down)
+        del down
+
+        ctx.names = list(saved.keys())
+        ctx.save_for_backward(*saved.values(), norm_weight_1, norm_bias_1, norm_weight_2, norm_bias_2,
+                              *(t for n in _PROJ for t in (W[n][0], W[n][3], W[n][4])))
+        ctx.quant_states = {n: W[n][2] for n in _PROJ}
+        ctx.mode, ctx.q_bit, ctx.num_heads, ctx.head_dim = mode, q_bit, num_heads, head_dim
+        ctx.block_size, ctx.num_warps = block_size, num_warps
+        out_stats = tuple(stats[slot] for slot in stat_slots(mode))
+        ctx.mark_non_differentiable(*[t for t in out_stats if torch.is_tensor(t)])
+        return (x_out,) + out_stats
+
+    @staticmethod
+    def backward(ctx, grad_output, *_unused):
+        mode, q_bit, H, D = ctx.mode, ctx.q_bit, ctx.num_heads, ctx.head_dim
+        tensors = list(ctx.saved_tensors)
+        ns = len(ctx.names)
+        S = dict(zip(ctx.names, tensors[:ns]))
+        nw1, nb1, nw2, nb2 = tensors[ns:ns + 4]
+        rest = tensors[ns + 4:]
+        W = {n: (rest[3 * i], ctx.quant_states[n], rest[3 * i + 1], rest[3 * i + 2]) for i, n in enumerate(_PROJ)}
+        G = {}
+
+        def deq(name, **kw):
+            return decompression_dequantization(S[name + "_q"], S[name + "_s"], q_bit, **kw)
+
+        def deq_cb(name):
+            return outlier_addition_fuse_decompression_dequantization(S[name + "_q"], S[name + "_s"], S[name + "_o"],
+                                                                      S[name + "_idx"], q_bit)
+
+        def back(name, inp, inp_lora_a, grad_y):
+            w, qs, la, lb = W[name]
+            G[name + "_a"], G[name + "_b"], gx = lora_backward(w, qs, la, lb, inp, inp_lora_a, grad_y)
+            return gx
+
+        def rebuilt(name):
+            main = deq(name + "_main")
+            return main + S[name + "_lora_a"].to(main.dtype) @ W[name][3].to(main.dtype)
+
+        grad_output = grad_output.to(torch.bfloat16)
+        grad_ln2, _, _ = layernorm_backward(grad_output, deq_cb("down"), nw2, nb2, S["mean_2"], S["rstd_2"], True, _EPS,
+                                            ctx.num_warps, ctx.block_size)
+        if mode == "intra":
+            fn, up = deq("fn"), deq("up")
+        else:
+            up = rebuilt("up")
+            fn = torch.nn.functional.gelu(up)
+        grad_down = back("down", fn, S["down_lora_a"], grad_ln2)
+        del fn
+        grad_fn = gelu_backward(up, grad_down)
+        del up, grad_down
+        grad_up = back("up", deq("x_medium"), S["up_lora_a"], grad_fn)
+        grad_medium = grad_ln2 + grad_up
+        del grad_ln2, grad_up, grad_fn
+        grad_ln1, _, _ = layernorm_backward(grad_medium, deq_cb("o_final"), nw1, nb1, S["mean_1"], S["rstd_1"], True, _EPS,
+                                            ctx.num_warps, ctx.block_size)
+        del grad_medium
+        grad_o = hidden_to_head_shape(back("o", deq("o"), S["o_lora_a"], grad_ln1), H)
+
+        if mode == "intra":
+            v = deq("v", is_head=True, num_heads=H)
+        else:
+            v = hidden_to_head_shape(rebuilt("v"), H)
+        grad_a = grad_o @ v.transpose(-2, -1)
+        del v
+        a, grad_s = softmax_backward_from_compressed(S["a_idx"], S["a_val"], S["a_seg"], grad_a)
+        del grad_a
+        grad_v = a.transpose(-2, -1) @ grad_o
+        del a, grad_o
+        if mode == "intra":
+            q, k = deq("q", is_head=True, num_heads=H), deq("k", is_head=True, num_heads=H)
+        else:
+            q, k = hidden_to_head_shape(rebuilt("q"), H), hidden_to_head_shape(rebuilt("k"), H)
+        grad_s = grad_s / math.sqrt(D)
+        grad_k = grad_s.transpose(-2, -1) @ q
+        grad_q = grad_s @ k
+        del grad_s, q, k
+        grad_q, grad_k, grad_v = (head_to_hidden_shape(t) for t in (grad_q, grad_k, grad_v))
+
+        x = deq("x")
+        grad_x = back("q", x, S["q_lora_a"], grad_q)
+        grad_x += back("k", x, S["k_lora_a"], grad_k)
+        grad_x += back("v", x, S["v_lora_a"], grad_v)
+        grad_input = grad_x + grad_ln1
+
+        def five(n):
+            return (None, None, None, G[n + "_a"], G[n + "_b"])
+        return (grad_input, *five("q"), *five("k"), *five("v"), *five("o"), None, None,
+                *five("up"), *five("down"), None, None) + (None,) * 10
+
+
+class FusedRobertaLayer(torch.nn.Module):
+    """Module wrapper: owns the calibration state and feeds the Function.  Same call signature as the
+    reference's modules (…intra_inter.py:538-568); the state travels with state_dict()."""
+
+    layer_type = "intra_inter"
+
+    def __init__(self):
+        super().__init__()
+        self.iteration = 0
+        self.static_value = self._empty()
+        self.use_hyclora = False
+
+    def _empty(self):
+        sv = {}
+        for key, field in stat_slots(self.layer_type):
+            sv.setdefault(key, {})[field] = None
+        return sv
+
+    def set_hyclora_config(self, hyclora_config):
+        self.hyclora_config = hyclora_config
+        self.use_hyclora = hyclora_config.use_hyclora
+        self.iteration_threshold = hyclora_config.iteration_threshold
+        self.softmax_outlier_ratio = hyclora_config.softmax_outlier_ratio
+        self.layernorm_outlier_ratio = hyclora_config.layernorm_outlier_ratio
+        self.q_bit = hyclora_config.q_bit
+
+    def get_extra_state(self):
+        return {"iteration": int(self.iteration),
+                "static_value": {key: {f: (v.detach().clone() if torch.is_tensor(v) else v) for f, v in fields.items()}
+                                 for key, fields in self.static_value.items()}}
+
+    def set_extra_state(self, state):
+        if not state:
+            return
+        want, got = self._empty(), state["static_value"]
+        if set(got) != set(want) or any(set(got[k]) != set(want[k]) for k in want):
+            raise ValueError(f"calibration state of another layer type: has {sorted(got)}, needs {sorted(want)}")
+        self.iteration = int(state["iteration"])
+        self.static_value = {key: {f: (v.detach().clone() if torch.is_tensor(v) else v) for f, v in fields.items()}
+                             for key, fields in got.items()}
+
+    def _apply(self, fn, *args, **kwargs):
+        super()._apply(fn, *args, **kwargs)
+        for fields in self.static_value.values():
+            for f, v in fields.items():
+                if torch.is_tensor(v):
+                    fields[f] = fn(v).to(v.dtype)
+        return self
+
+    def forward(self, input,
+                q_proj_base, q_proj_lora_a, q_proj_lora_b, k_proj_base, k_proj_lora_a, k_proj_lora_b,
+                v_proj_base, v_proj_lora_a, v_proj_lora_b, o_proj_base, o_proj_lora_a, o_proj_lora_b,
+                norm_weight_1, norm_bias_1,
+                up_proj_base, up_proj_lora_a, up_proj_lora_b, down_proj_base, down_proj_lora_a, down_proj_lora_b,
+                norm_weight_2, norm_bias_2, attention_mask, num_heads, head_dim):
+        def five(base, la, lb):
+            w = base.weight
+            return (w, getattr(base, "bias", None), getattr(w, "quant_state", None), _weight_of(la).T, _weight_of(lb).T)
+
+        outs = FusedRobertaLayerFunc.apply(
+            input, *five(q_proj_base, q_proj_lora_a, q_proj_lora_b), *five(k_proj_base, k_proj_lora_a, k_proj_lora_b),
+            *five(v_proj_base, v_proj_lora_a, v_proj_lora_b), *five(o_proj_base, o_proj_lora_a, o_proj_lora_b),
+            norm_weight_1, norm_bias_1,
+            *five(up_proj_base, up_proj_lora_a, up_proj_lora_b), *five(down_proj_base, down_proj_lora_a, down_proj_lora_b),
+            norm_weight_2, norm_bias_2, attention_mask, num_heads, head_dim,
+            self.iteration, self.iteration_threshold, self.static_value,
+            self.softmax_outlier_ratio, self.layernorm_outlier_ratio, self.q_bit, self.layer_type)
+        y, stat_values = outs[0], outs[1:]
+        if self.iteration < self.iteration_threshold:
+            fresh = {}
+            for (key, field), value in zip(stat_slots(self.layer_type), stat_values):
+                fresh.setdefault(key, {})[field] = value
+            for key, fields in fresh.items():
+                self.static_value[key] = update_dict(self.static_value[key], fields, self.iteration)
+        self.iteration += 1
+        return y
+
+
+class FusedRobertaLayerIntra(FusedRobertaLayer):
+    layer_type = "intra"
+
+
+class FusedRobertaLayerIntraInter(FusedRobertaLayer):
+    layer_type = "intra_inter"
+
+
+LAYER_TYPES = {"intra": FusedRobertaLayerIntra, "intra_inter": FusedRobertaLayerIntraInter}
+
+
+def make_fused_roberta_layer(hyclora_config):
+    """Pick the class by `layer_type` and configure it (what the reference's model file does per
+    encoder layer)."""
+    try:
+        layer = LAYER_TYPES[hyclora_config.layer_type]()
+    except KeyError:
+        raise ValueError(f"Unknown layer type: {hyclora_config.layer_type}") from None
+    layer.set_hyclora_config(hyclora_config)
+    return layer

@@ -202,7 +202,8 @@ int hyc_softmax_bwd(const void *y, const void *grad_y, void *out, int64_t rows, 
  *   s, out    bf16 [rows, n] contiguous, 16-byte aligned (out may alias s); n % 8 == 0, n <= 8192.
  *   mask      bf16 or NULL; row r adds mask[(r / rows_per_batch) * mask_stride_b +
  *             (r % mask_rows) * mask_stride_row + 0..n-1]  (a [B,1,S,S] mask over [B,H,S,S] scores:
- *             mask_rows = S, rows_per_batch = H*S, strides S*S and S; stride_b = 0 broadcasts).
+ *             mask_rows = S, rows_per_batch = H*S, strides S*S and S; a stride of 0 broadcasts: stride_b = 0 one
+ *             mask for all batches, stride_row = 0 one mask row for all queries, as a padding mask).
  *   threshold, seg_counts, seg_offsets   all NULL, or all given: then seg_counts / seg_offsets are
  *             filled exactly as hyc_sparse_count(out, rows*n, threshold, ...) would fill them, without
  *             another pass over the map.  Needs n in {512,1024,2048,4096} and rows*n % 4096 == 0
@@ -254,6 +255,23 @@ int64_t hyc_rmsnorm_bwd_workspace(int64_t rows, int64_t N);
 int hyc_rmsnorm_bwd(const void *dy, const void *x, const void *weight, int weight_is_fp32,
                     const float *rstd, void *dx, void *dw, void *workspace, int64_t workspace_bytes,
                     int64_t rows, int64_t N, void *stream);
+
+/* ---------------------------------------------------------------------------------------
+ * LayerNorm over the last dimension (the encoder layers' norm).
+ *
+ * hyc_layernorm_fwd replaces _layer_norm_fwd_fused / layernorm_forward
+ * (operators/layernorm_kernels.py:9-56, :125-147): mean and rstd = 1/sqrt(var + eps) in fp32 (variance
+ * from the centred values), y = (x - mean)*rstd*w + b rounded once to bf16.
+ * hyc_layernorm_bwd replaces _layer_norm_bwd_dx_fused / layernorm_backward (:60-121, :150-198):
+ * dx = (w*dy - (x^*c1 + c2))*rstd with c1 = mean(x^ * w*dy), c2 = mean(w*dy).  The reference computes
+ * dw / db partials under a spin lock and discards them (returns (dx, None, None)); so there are none here.
+ *   x, y, dy, dx  bf16 [rows, N] contiguous, 16-byte aligned; N % 8 == 0, N <= 8192.
+ *   weight, bias  [N], both bf16 (params_are_fp32 == 0) or both fp32;  mean, rstd  fp32 [rows].
+ */
+int hyc_layernorm_fwd(const void *x, const void *weight, const void *bias, int params_are_fp32, void *y,
+                      float *mean, float *rstd, int64_t rows, int64_t N, float eps, void *stream);
+int hyc_layernorm_bwd(const void *dy, const void *x, const void *weight, int params_are_fp32,
+                      const float *mean, const float *rstd, void *dx, int64_t rows, int64_t N, void *stream);
 
 /* ---------------------------------------------------------------------------------------
  * RMSNorm forward fused with the compressions a decoder layer applies around it: the row is read

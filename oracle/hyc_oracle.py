@@ -24,6 +24,8 @@ Pinning status (what independent evidence holds each function in place):
     formula (which keeps LayerNorm's mean term) and is pinned only against a
     float64 evaluation of that same formula and against autograd for inputs where the
     extra term vanishes: "parity unpinned" for the c2 term beyond reading the source.
+  * layernorm_fwd / layernorm_bwd: pinned against torch.nn.functional.layer_norm and its
+    autograd in float64 (an independent library routine), tests/test_oracle_layernorm.py.
   * rope: pinned against the textbook rotate-half form x*cos + rotate_half(x)*sin with
     full-width tables, against an explicit complex-number rotation in float64, and by
     norm preservation / forward-then-backward identity (tests/test_oracle_rope.py).
@@ -322,6 +324,29 @@ def rmsnorm_bwd(dy, x, w, rstd):
     dx = ((wdy - (xhat * c1 + c2)) * rstd.reshape(-1, 1)).to(dy.dtype).reshape(dy.shape)
     dw = (dyf * xhat).sum(dim=0).to(w.dtype)
     return dx, dw
+
+
+def layernorm_fwd(x, w, b, eps):
+    """(y bf16, mean fp32 [rows], rstd fp32 [rows]): mean and centred variance in fp32,
+    y = (x - mean)*rstd*w + b rounded once (layernorm_kernels.py:27-56)."""
+    xf = x.float()
+    mean = xf.sum(-1, keepdim=True) / x.shape[-1]
+    d = xf - mean
+    var = (d * d).sum(-1, keepdim=True) / x.shape[-1]
+    rstd = 1.0 / torch.sqrt(var + eps)
+    y = (d * rstd) * w.float() + b.float()
+    return y.to(x.dtype), mean.reshape(-1), rstd.reshape(-1)
+
+
+def layernorm_bwd(dy, x, w, mean, rstd):
+    """dx = (w*dy - (x^*c1 + c2))*rstd, c1 = mean(x^*w*dy), c2 = mean(w*dy), fp32 (layernorm_kernels.py:92-104)."""
+    n = x.shape[-1]
+    shp = x.shape[:-1] + (1,)
+    xh = (x.float() - mean.reshape(shp)) * rstd.reshape(shp)
+    wdy = w.float() * dy.float()
+    c1 = (xh * wdy).sum(-1, keepdim=True) / n
+    c2 = wdy.sum(-1, keepdim=True) / n
+    return ((wdy - (xh * c1 + c2)) * rstd.reshape(shp)).to(dy.dtype)
 
 
 def _sig_bf16(x):

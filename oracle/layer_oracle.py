@@ -194,3 +194,120 @@ def layer_forward_backward(x, nw1, nw2, cos, sin, weights, mask, heads, kv_heads
     g_norm1, G["nw1"] = O.rmsnorm_bwd(gx, x_r, nw1, rstd1)
     G["x"] = g_norm1 + g_medium
     return x_out, G
+
+
+def roberta_layer_forward_backward(x, weights, ln1, ln2, mask, heads, grad_out, *, mode, q_bit, softmax_ratio,
+                                   layernorm_ratio, eps=1e-5):
+    """Encoder (post-LayerNorm, GELU) layer: models/roberta/fused_roberta_layer_intra_inter.py:86-200
+    (forward), :362-455 (backward) and fused_roberta_layer_intra.py:86-205, :373-440.
+    weights: name -> (W [out,in], bias [out] or None, A [r,in], B [out,r]) for q,k,v,o,up,down;
+    ln1 / ln2: (weight, bias).  Returns (x_out, grads) like layer_forward_backward."""
+    hd = x.shape[-1] // heads
+    Wt = {n: w[0].t() for n, w in weights.items()}
+    bias = {n: w[1] for n, w in weights.items()}
+    At = {n: w[2].t() for n, w in weights.items()}
+    Bt = {n: w[3].t() for n, w in weights.items()}
+
+    def lora_fwd(n, inp):
+        main = inp @ Wt[n]
+        if bias[n] is not None:
+            main = main + bias[n]
+        xa = inp @ At[n]
+        return main + xa @ Bt[n], main, xa
+
+    def lora_bwd(n, inp, xa, gy):
+        gmid = gy @ Bt[n].mT
+        ga = inp.mT @ gmid
+        gb = xa.mT @ gy
+        gx = gy @ Wt[n].T
+        gx = gx + gmid @ At[n].T
+        return ga, gb, gx
+
+    def cq(t):
+        s = O.scale_only_quant(t, q_bit)
+        return O.compress(t, s, q_bit), s
+
+    def ccb(t):
+        idx, s = O.channel_stats(t, layernorm_ratio, q_bit)
+        xo, q = O.compress_channel_base(t, s, idx, q_bit)
+        return xo, q, idx, s
+
+    dq = lambda sv, **kw: O.decompress(sv[0], sv[1], q_bit, **kw).to(x.device)
+
+    # ------------------------------ forward ------------------------------
+    q, q_main, q_xa = lora_fwd("q", x)
+    k, k_main, k_xa = lora_fwd("k", x)
+    v, v_main, v_xa = lora_fwd("v", x)
+    x_sv = cq(x)
+    if mode == "intra_inter":
+        q_sv, k_sv, v_sv = cq(q_main), cq(k_main), cq(v_main)
+    q, k, v = _heads(q, heads), _heads(k, heads), _heads(v, heads)
+    if mode == "intra":
+        q_sv, k_sv = cq(q), cq(k)
+    a = O.softmax_fwd(q @ k.transpose(-2, -1), 1.0 / math.sqrt(hd), mask)
+    o = a @ v
+    thr = O.softmax_threshold(a, softmax_ratio)
+    a_idx, a_val = O.softmax_compress(a, thr)
+    a_shape = a.shape
+    if mode == "intra":
+        v_sv = cq(v)
+    o = _hidden(o)
+    o_final, _, o_xa = lora_fwd("o", o)
+    o_sv = cq(o)
+    o_final = o_final + x
+    x_medium, mean1, rstd1 = O.layernorm_fwd(o_final, ln1[0], ln1[1], eps)
+    of_sv = ccb(o_final)
+    up, up_main, up_xa = lora_fwd("up", x_medium)
+    xm_sv = cq(x_medium)
+    if mode == "intra_inter":
+        up_sv = cq(up_main)
+    fn = F.gelu(up)
+    if mode == "intra":
+        up_sv = cq(up)
+    down, _, down_xa = lora_fwd("down", fn)
+    down = down + x_medium
+    if mode == "intra":
+        fn_sv = cq(fn)
+    x_out, mean2, rstd2 = O.layernorm_fwd(down, ln2[0], ln2[1], eps)
+    down_sv = ccb(down)
+
+    # ------------------------------ backward ------------------------------
+    G = {}
+    go = grad_out
+    down_r = O.decompress_channel_base(down_sv[1], down_sv[3], down_sv[0], down_sv[2], q_bit)
+    g_ln2 = O.layernorm_bwd(go, down_r, ln2[0], mean2, rstd2)
+    if mode == "intra":
+        fn_r, up_r = dq(fn_sv), dq(up_sv)
+    else:
+        up_r = dq(up_sv) + up_xa @ Bt["up"]
+        fn_r = F.gelu(up_r)
+    G[("down", "A")], G[("down", "B")], g_down = lora_bwd("down", fn_r, down_xa, g_ln2)
+    g_fn = O.gelu_bwd(up_r, g_down)
+    G[("up", "A")], G[("up", "B")], g_up = lora_bwd("up", dq(xm_sv), up_xa, g_fn)
+    g_medium = g_ln2 + g_up
+    of_r = O.decompress_channel_base(of_sv[1], of_sv[3], of_sv[0], of_sv[2], q_bit)
+    g_ln1 = O.layernorm_bwd(g_medium, of_r, ln1[0], mean1, rstd1)
+    G[("o", "A")], G[("o", "B")], g_o = lora_bwd("o", dq(o_sv), o_xa, g_ln1)
+    g_o = _heads(g_o, heads)
+    a_r = O.softmax_restore(a_idx, a_val, a_shape)
+    if mode == "intra":
+        v_r = dq(v_sv, is_head=True, num_heads=heads)
+        q_r, k_r = dq(q_sv, is_head=True, num_heads=heads), dq(k_sv, is_head=True, num_heads=heads)
+    else:
+        v_r = _heads(dq(v_sv) + v_xa @ Bt["v"], heads)
+        q_r = _heads(dq(q_sv) + q_xa @ Bt["q"], heads)
+        k_r = _heads(dq(k_sv) + k_xa @ Bt["k"], heads)
+    g_v = a_r.transpose(-2, -1) @ g_o
+    g_a = g_o @ v_r.transpose(-2, -1)
+    g_s = O.softmax_bwd(a_r, g_a) / math.sqrt(hd)
+    g_k = g_s.transpose(-2, -1) @ q_r
+    g_q = g_s @ k_r
+    g_q, g_k, g_v = _hidden(g_q), _hidden(g_k), _hidden(g_v)
+    x_r = dq(x_sv)
+    G[("q", "A")], G[("q", "B")], gx = lora_bwd("q", x_r, q_xa, g_q)
+    G[("k", "A")], G[("k", "B")], gt = lora_bwd("k", x_r, k_xa, g_k)
+    gx = gx + gt
+    G[("v", "A")], G[("v", "B")], gt = lora_bwd("v", x_r, v_xa, g_v)
+    gx = gx + gt
+    G["x"] = gx + g_ln1
+    return x_out, G

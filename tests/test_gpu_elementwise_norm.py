@@ -124,3 +124,45 @@ def test_rmsnorm_errors(ops, dev):
         ops.norm.rmsnorm_forward(torch.zeros(1, 1, 32776, dtype=BF16, device=dev), torch.ones(32776, dtype=BF16, device=dev), 1e-5)
     with pytest.raises(ValueError):
         ops.norm.rmsnorm_forward(torch.zeros(1, 1, 100, dtype=BF16, device=dev), torch.ones(100, dtype=BF16, device=dev), 1e-5)
+
+
+@pytest.fixture(scope="module")
+def ln():
+    import hyclora_amd  # noqa: F401
+    from hyclora_amd.operators import layernorm_kernels
+    return layernorm_kernels
+
+
+@pytest.mark.parametrize("n", [768, 1024, 96, 4096, 8192, 2048 + 64])
+@pytest.mark.parametrize("pdtype", [BF16, torch.float32])
+def test_layernorm_forward_backward(ln, dev, n, pdtype):
+    g = torch.Generator().manual_seed(n)
+    shape = (3, 11, n)
+    x = (torch.randn(*shape, generator=g) * 2 + 0.5).to(BF16)
+    w = (1 + 0.2 * torch.randn(n, generator=g)).to(pdtype)
+    b = (0.1 * torch.randn(n, generator=g)).to(pdtype)
+    dy = torch.randn(*shape, generator=g).to(BF16)
+    y, mean, rstd, bs, nw = ln.layernorm_forward(x.to(dev), w.to(dev), b.to(dev), 1e-5)
+    y_o, mean_o, rstd_o = O.layernorm_fwd(x, w, b, 1e-5)
+    assert y.dtype == BF16 and y.shape == x.shape and mean.shape == (33,) and bs >= n
+    assert_close_bf16(y, y_o, what="layernorm_forward vs oracle")
+    assert torch.allclose(mean.cpu(), mean_o, atol=1e-5) and torch.allclose(rstd.cpu(), rstd_o, rtol=1e-5)
+    ref = F.layer_norm(x.double(), (n,), w.double(), b.double(), 1e-5)
+    assert_close_bf16(y, ref, what="layernorm_forward vs torch layer_norm")
+    dx, dw, db = ln.layernorm_backward(dy.to(dev), x.to(dev), w.to(dev), b.to(dev), mean, rstd, True, 1e-5, nw, bs)
+    assert dw is None and db is None
+    assert_close_bf16(dx, O.layernorm_bwd(dy, x, w, mean_o, rstd_o), what="layernorm_backward vs oracle")
+    xd = x.double().requires_grad_()
+    F.layer_norm(xd, (n,), w.double(), b.double(), 1e-5).backward(dy.double())
+    assert_close_bf16(dx, xd.grad, what="layernorm_backward vs autograd")
+    assert ln.layernorm_backward(dy.to(dev), x.to(dev), w.to(dev), b.to(dev), mean, rstd, False, 1e-5, nw, bs) == (None, None, None)
+
+
+def test_layernorm_errors(ln, dev):
+    w = torch.ones(20, device=dev, dtype=BF16)
+    with pytest.raises(RuntimeError):
+        ln.layernorm_forward(torch.zeros(2, 20, device=dev, dtype=BF16), w, w, 1e-5)             # N % 8
+    with pytest.raises(NotImplementedError):
+        ln.layernorm_forward(torch.zeros(2, 24, device=dev), torch.ones(24, device=dev), torch.ones(24, device=dev), 1e-5)
+    with pytest.raises(Exception):
+        ln.layernorm_forward(torch.zeros(2, 24, dtype=BF16), torch.ones(24, dtype=BF16), torch.ones(24, dtype=BF16), 1e-5)

@@ -1,0 +1,143 @@
+"""GPU tests of the encoder (RoBERTa) layers: against the oracle's restatement of the reference layer,
+against an uncompressed torch-autograd layer (sanity bound), the calibration state machine, and the
+frozen-statistics code path against the calibrating one."""
+import math
+from types import SimpleNamespace
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from helpers import BF16, rel_err_and_cos
+from test_gpu_layers import Lin, config
+
+pytestmark = pytest.mark.gpu
+
+NAMES = ("q", "k", "v", "o", "up", "down")
+
+
+def make_inputs(dev, seed, B=2, S=64, hidden=256, heads=4, inter=512, rank=16, padding=True):
+    g = torch.Generator(device=dev).manual_seed(seed)
+    rn = lambda *s, sc=1.0: (torch.randn(*s, generator=g, device=dev) * sc).to(BF16)
+    dims = dict(q=(hidden, hidden), k=(hidden, hidden), v=(hidden, hidden), o=(hidden, hidden),
+                up=(inter, hidden), down=(hidden, inter))
+    P = {}
+    for n, (out_f, in_f) in dims.items():
+        base = Lin(rn(out_f, in_f, sc=1.0 / math.sqrt(in_f)), rn(out_f, sc=0.1))
+        la = Lin(rn(rank, in_f, sc=1.0 / math.sqrt(in_f)).requires_grad_())
+        lb = Lin(rn(out_f, rank, sc=0.05).requires_grad_())
+        P[n] = (base, la, lb)
+    x = rn(B, S, hidden)
+    x[..., 5] *= 20
+    x.requires_grad_()
+    ln = [((1 + 0.1 * torch.randn(hidden, generator=g, device=dev)).to(BF16),
+           (0.1 * torch.randn(hidden, generator=g, device=dev)).to(BF16)) for _ in range(2)]
+    mask = None
+    if padding:                                   # HF extended padding mask [B,1,1,S]: the last tokens of batch 1 are padding
+        mask = torch.zeros(B, 1, 1, S, device=dev)
+        mask[1, ..., S - S // 4:] = torch.finfo(BF16).min
+        mask = mask.to(BF16)
+    return SimpleNamespace(P=P, x=x, ln=ln, mask=mask, grad=rn(B, S, hidden), heads=heads, hd=hidden // heads)
+
+
+def run_fused(layer, t):
+    args = [t.x]
+    for n in ("q", "k", "v", "o"):
+        args += list(t.P[n])
+    args += [t.ln[0][0], t.ln[0][1]]
+    for n in ("up", "down"):
+        args += list(t.P[n])
+    args += [t.ln[1][0], t.ln[1][1], t.mask, t.heads, t.hd]
+    return layer(*args)
+
+
+def reference_layer(t):
+    def proj(n, inp):
+        base, la, lb = t.P[n]
+        return inp @ base.weight.t() + base.bias + (inp @ la.weight.t()) @ lb.weight.t()
+
+    def heads(v):
+        b, s, d = v.shape
+        return v.reshape(b, s, t.heads, d // t.heads).transpose(1, 2)
+    q, k, v = heads(proj("q", t.x)), heads(proj("k", t.x)), heads(proj("v", t.x))
+    s = q @ k.transpose(-2, -1) / math.sqrt(t.hd)
+    if t.mask is not None:
+        s = s + t.mask
+    o = (torch.softmax(s, dim=-1, dtype=BF16) @ v).transpose(1, 2).reshape(t.x.shape)
+    hidden = t.x.shape[-1]
+    xm = F.layer_norm(proj("o", o) + t.x, (hidden,), t.ln[0][0], t.ln[0][1], 1e-5)
+    return F.layer_norm(proj("down", F.gelu(proj("up", xm))) + xm, (hidden,), t.ln[1][0], t.ln[1][1], 1e-5)
+
+
+def grads_of(t, out):
+    params = [t.x] + [m.weight for n in NAMES for m in t.P[n][1:]]
+    for p in params:
+        p.grad = None
+    out.backward(t.grad)
+    return [p.grad.clone() for p in params]
+
+
+@pytest.mark.parametrize("layer_type", ["intra", "intra_inter"])
+@pytest.mark.parametrize("q_bit", [8, 4, 2])
+@pytest.mark.parametrize("padding", [True, False])
+def test_roberta_layer_matches_oracle_layer(dev, layer_type, q_bit, padding):
+    import hyclora_amd  # noqa: F401
+    from hyclora_amd.models import roberta
+    from oracle import layer_oracle
+    t = make_inputs(dev, seed=40 + q_bit, padding=padding)
+    layer = roberta.make_fused_roberta_layer(config(layer_type, q_bit, sm_ratio=0.05))
+    out = run_fused(layer, t)
+    grads = grads_of(t, out)
+    weights = {n: (t.P[n][0].weight, t.P[n][0].bias, t.P[n][1].weight.detach(), t.P[n][2].weight.detach()) for n in NAMES}
+    with torch.no_grad():
+        ref_out, G = layer_oracle.roberta_layer_forward_backward(
+            t.x.detach(), weights, t.ln[0], t.ln[1], t.mask, t.heads, t.grad, mode=layer_type, q_bit=q_bit,
+            softmax_ratio=0.05, layernorm_ratio=0.005)
+    rel, cos = rel_err_and_cos(out, ref_out)
+    assert rel <= 1e-2 and cos >= 0.9999
+    expect = [G["x"]]
+    for n in NAMES:
+        expect += [G[(n, "A")].sum(0).t(), G[(n, "B")].sum(0).t()]
+    names = ["x"] + [f"{n}.lora_{ab}" for n in NAMES for ab in "AB"]
+    for name, got, want in zip(names, grads, expect):
+        rel, cos = rel_err_and_cos(got, want)
+        rel_tol = 0.2 if q_bit == 2 else 2e-2            # one flipped 2-bit code is a quarter of the range
+        assert rel <= rel_tol and cos >= 0.999, f"{layer_type} q{q_bit} grad {name}: rel {rel:.2e} cos {cos:.5f}"
+
+
+@pytest.mark.parametrize("layer_type", ["intra", "intra_inter"])
+def test_roberta_layer_close_to_uncompressed_autograd(dev, layer_type):
+    import hyclora_amd  # noqa: F401
+    from hyclora_amd.models import roberta
+    t = make_inputs(dev, seed=50)
+    ref_out = reference_layer(t)
+    ref_grads = grads_of(t, ref_out)
+    layer = roberta.make_fused_roberta_layer(config(layer_type, 8))
+    out = run_fused(layer, t)
+    rel, cos = rel_err_and_cos(out, ref_out)
+    assert rel <= 2e-2 and cos >= 0.9999                  # forward is not compressed
+    for i, (got, want) in enumerate(zip(grads_of(t, out), ref_grads)):
+        rel, cos = rel_err_and_cos(got, want)
+        assert cos >= 0.9, f"{layer_type} grad #{i}: rel {rel:.2e} cos {cos:.5f}"    # sanity bound only: the scheme (step from batch element 0, no zero point) clips; parity is the oracle test above
+
+
+def test_roberta_calibration_freezes_and_paths_agree(dev, tmp_path):
+    import hyclora_amd  # noqa: F401
+    from hyclora_amd.models import roberta
+    t = make_inputs(dev, seed=60, S=512, hidden=256, heads=2)     # rows of 512: the frozen path counts in the softmax pass
+    layer = roberta.make_fused_roberta_layer(config("intra_inter", 4, sm_ratio=0.05, thr=1))
+    assert layer.static_value["down"]["scale"] is None
+    y0 = run_fused(layer, t)
+    g0 = grads_of(t, y0)
+    assert layer.iteration == 1 and 5 in layer.static_value["o_final"]["outlier_channel_index"].tolist()
+    y1 = run_fused(layer, t)                                       # frozen statistics == fresh ones on the same input
+    g1 = grads_of(t, y1)
+    assert torch.equal(y0, y1) and all(torch.equal(a, b) for a, b in zip(g0, g1))
+    torch.save(layer.state_dict(), tmp_path / "enc.pt")
+    resumed = roberta.make_fused_roberta_layer(config("intra_inter", 4, sm_ratio=0.05, thr=1))
+    resumed.load_state_dict(torch.load(tmp_path / "enc.pt", weights_only=True))
+    assert resumed.iteration == 2
+    y2 = run_fused(resumed, t)
+    assert torch.equal(y2, y1)
+    with pytest.raises(ValueError):
+        roberta.make_fused_roberta_layer(config("intra_inter_full_fuse", 4))
