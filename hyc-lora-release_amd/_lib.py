@@ -43,6 +43,7 @@ _SIGNATURES = {
     "hyc_sparse_segment_offsets": (_I, [_P, _L, _L, _P, _P]),
     "hyc_sparse_restore": (_I, [_P, _P, _P, _L, _P, _P]),
     "hyc_softmax_bwd": (_I, [_P, _P, _P, _L, _L, _P]),
+    "hyc_nf4_dequant": (_I, [_P, _P, _I, _P, _P, _P, _L, _P, _P, _L, _L, _P]),
     "hyc_layernorm_fwd": (_I, [_P, _P, _P, _I, _P, _P, _P, _L, _L, ctypes.c_float, _P]),
     "hyc_layernorm_bwd": (_I, [_P, _P, _P, _I, _P, _P, _P, _L, _L, _P]),
     "hyc_outlier_table": (_I, [_P, _L, _L, _P, _P]),

@@ -4,6 +4,8 @@ torch operations in the reference as well; only what surrounds them is compresse
 in-place HIP kernel of operators/rope_kernels.py, re-exported here."""
 import torch
 
+from ..operators.nf4 import dequantize_nf4
+
 
 def hidden_to_head_shape(x: torch.Tensor, num_heads: int):
     bsz, seq_len, hidden = x.shape
@@ -16,16 +18,12 @@ def head_to_hidden_shape(x: torch.Tensor):
 
 
 def dense_weight(w: torch.Tensor, quant_state):
-    """Frozen weight as a dense [out, in] matrix.  quant_state None = already dense (the
-    benchmark configurations); otherwise NF4 via bitsandbytes, as in the reference."""
+    """Frozen weight as a dense [out, in] matrix.  quant_state None = already dense (the benchmark
+    configurations); otherwise a bitsandbytes-format NF4 weight, dequantised by the HIP kernel (the
+    reference calls BF.dequantize_nf4 at the same place, compute_utils.py:19, :29)."""
     if quant_state is None:
         return w
-    try:
-        import bitsandbytes.functional as BF
-    except ImportError as e:  # pragma: no cover - bitsandbytes is absent in this environment
-        raise RuntimeError("NF4 frozen weights need bitsandbytes; pass dense bf16 weights "
-                           "(quant_state=None) instead") from e
-    return BF.dequantize_nf4(w, quant_state)
+    return dequantize_nf4(w, quant_state)
 
 
 def lora_forward(w, w_quant_state, w_lora_a, w_lora_b, b, x):

@@ -257,6 +257,22 @@ int hyc_rmsnorm_bwd(const void *dy, const void *x, const void *weight, int weigh
                     int64_t rows, int64_t N, void *stream);
 
 /* ---------------------------------------------------------------------------------------
+ * NF4 block-wise weight dequantisation to bf16, bitsandbytes 0.43.2 layout (the version the
+ * reference pins in requirements.txt:3).
+ *
+ * Replaces BF.dequantize_nf4(w, quant_state) (models/utils/compute_utils.py:19, :29):
+ *   out[i] = bf16(table[code_i] * absmax[i / blocksize]),  code of an even i in the high nibble of
+ *   packed[i / 2];  nested != 0 ("double quant"): absmax is uint8 [n / blocksize] and the block's
+ *   statistic is code2[absmax[b]] * absmax2[b / blocksize2] + *offset (fp32; offset is a device
+ *   scalar, NULL = 0);  nested == 0: absmax is fp32.
+ *   table  fp32 [16] (the NF4 code book; the quant state carries it), code2 fp32 [256];
+ *   n even, blocksize % 8 == 0; packed 4-byte aligned, out 16-byte aligned.
+ */
+int hyc_nf4_dequant(const void *packed, const void *absmax, int nested, const float *code2, const float *absmax2,
+                    const float *offset, int64_t blocksize2, const float *table, void *out, int64_t n, int64_t blocksize,
+                    void *stream);
+
+/* ---------------------------------------------------------------------------------------
  * LayerNorm over the last dimension (the encoder layers' norm).
  *
  * hyc_layernorm_fwd replaces _layer_norm_fwd_fused / layernorm_forward

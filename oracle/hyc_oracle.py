@@ -26,6 +26,10 @@ Pinning status (what independent evidence holds each function in place):
     extra term vanishes: "parity unpinned" for the c2 term beyond reading the source.
   * layernorm_fwd / layernorm_bwd: pinned against torch.nn.functional.layer_norm and its
     autograd in float64 (an independent library routine), tests/test_oracle_layernorm.py.
+  * nf4_dequant: bitsandbytes (0.43.2, pinned in the reference's requirements.txt) is not installed,
+    so its published format is restated; pinned by the published NF4 code book, hand-computed
+    bytes (nibble order, nested statistics) and exact round trips of on-grid weights
+    (tests/test_oracle_nf4.py).  "parity unpinned" against bitsandbytes' own output.
   * rope: pinned against the textbook rotate-half form x*cos + rotate_half(x)*sin with
     full-width tables, against an explicit complex-number rotation in float64, and by
     norm preservation / forward-then-backward identity (tests/test_oracle_rope.py).
@@ -417,3 +421,60 @@ def fused_bwd(xa1, b1, q1, s1, xa2, b2, q2, s2, grad_o, q_bit):
     gh2 = g * sil
     grad_gate = gh1 * (sig * (1.0 + y1 * (1.0 - sig)))
     return o, grad_gate, gh2
+
+
+# --------------------------------------------------------------------------------------
+# NF4 frozen weights (bitsandbytes 0.43.2 is not importable here: its published format is restated)
+# --------------------------------------------------------------------------------------
+NF4_TABLE = torch.tensor([-1.0, -0.6961928009986877, -0.5250730514526367, -0.39491748809814453, -0.28444138169288635,
+                          -0.18477343022823334, -0.09105003625154495, 0.0, 0.07958029955625534, 0.16093020141124725,
+                          0.24611230194568634, 0.33791524171829224, 0.44070982933044434, 0.5626170039176941,
+                          0.7229568362236023, 1.0], dtype=F32)
+
+
+def nf4_absmax(absmax, nested=None):
+    """fp32 block statistics; nested = (code2 fp32 [256], absmax2 fp32, blocksize2, offset) for double
+    quantisation: code2[absmax] * absmax2[block / blocksize2] + offset
+    (bitsandbytes functional.py dequantize_4bit: dequantize_blockwise(absmax, state2) + offset)."""
+    if nested is None:
+        return absmax.float()
+    code2, absmax2, bs2, offset = nested
+    idx = torch.arange(absmax.numel()) // bs2
+    return code2.float()[absmax.long()] * absmax2.float()[idx] + float(offset)
+
+
+def nf4_dequant(packed, absmax, shape, blocksize=64, nested=None, table=NF4_TABLE):
+    """bf16 weight of `shape`: element 2i from the HIGH nibble of byte i, 2i+1 from the low one
+    (bitsandbytes csrc/kernels.cu kDequantizeBlockwise, NF4 branch); value = table[code] * absmax[i / blocksize]
+    in fp32, rounded to bf16 (what models/utils/compute_utils.py:19 gets from BF.dequantize_nf4)."""
+    p = packed.reshape(-1).long()
+    codes = torch.stack([p >> 4, p & 15], dim=1).reshape(-1)
+    am = nf4_absmax(absmax.reshape(-1), nested)
+    vals = table.float()[codes] * am[torch.arange(codes.numel()) // blocksize]
+    return vals.to(BF16).reshape(shape)
+
+
+def nf4_quantize(w, blocksize=64, code2=None, blocksize2=256):
+    """Test-data generator (not a restatement of bitsandbytes' quantiser): nearest NF4 level of
+    w / absmax per block; with code2, the statistics are themselves quantised to 8 bits around their
+    mean.  -> (packed uint8 [n/2], absmax fp32 [nblocks] or uint8 codes, nested tuple or None)."""
+    flat = w.float().reshape(-1)
+    n = flat.numel()
+    nb = -(-n // blocksize)
+    pad = torch.zeros(nb * blocksize)
+    pad[:n] = flat
+    blocks = pad.reshape(nb, blocksize)
+    absmax = blocks.abs().amax(dim=1).clamp_min(1e-12)
+    codes = ((blocks / absmax[:, None])[..., None] - NF4_TABLE).abs().argmin(dim=-1).reshape(-1)[:n]
+    packed = ((codes[0::2] << 4) | codes[1::2]).to(torch.uint8)
+    if code2 is None:
+        return packed, absmax, None
+    offset = absmax.mean()
+    rest = absmax - offset
+    nb2 = -(-nb // blocksize2)
+    pad2 = torch.zeros(nb2 * blocksize2)
+    pad2[:nb] = rest
+    b2 = pad2.reshape(nb2, blocksize2)
+    absmax2 = b2.abs().amax(dim=1).clamp_min(1e-12)
+    c2 = ((b2 / absmax2[:, None])[..., None] - code2.float()).abs().argmin(dim=-1).reshape(-1)[:nb]
+    return packed, c2.to(torch.uint8), (code2, absmax2, blocksize2, offset)
