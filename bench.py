@@ -43,7 +43,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=1000,
                     help="untimed steps; ~50 ms of work lets the GPU reach its steady clocks (20 steps do not)")
     ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU-oracle timing (for profiler runs)")
-    ap.add_argument("--only", choices=["all", "roundtrip", "quant", "fused", "copy", "layers"], default="all",
+    ap.add_argument("--only", choices=["all", "roundtrip", "quant", "fused", "copy", "layers", "stack"], default="all",
                     help="restrict the run to one part (for profiler runs)")
     ap.add_argument("--layer-case", default="", help="with --only layers: run only the cases whose name contains this")
     ap.add_argument("--layer-arm", choices=["both", "plain", "compressed"], default="both",
@@ -178,6 +178,144 @@ def bench_layers(torch, dev, only_case="", arm="both"):
         out[name] = entry
         del t, mask
         torch.cuda.empty_cache()
+    return out
+
+
+def bench_stack(torch, dev, n_layers=4, steps=5):
+    """The reference's memory / throughput harness (run_memory_throughput.py:178-191: allocated memory
+    before the first forward and after the forward of steps 0 and 1; run_memory_throughput.sh: Llama-2-7B,
+    batch 4, seq 512, intra_inter, q_bit 2, NF4 frozen weights, LoRA r=16) on a stack of decoder layers
+    with random NF4 weights: the compressed layers of this package against an uncompressed bf16
+    torch-autograd stack that dequantises the same NF4 weights at every use."""
+    import math
+    from types import SimpleNamespace
+
+    import torch.nn.functional as F
+
+    from hyclora_amd.models import llama
+    from hyclora_amd.models.compute_utils import dense_weight, head_to_hidden_shape, hidden_to_head_shape
+    from hyclora_amd.operators import nf4
+    BF16 = torch.bfloat16
+    gen = torch.Generator(device=dev).manual_seed(2)
+    B, S, hidden, heads, inter, rank = 4, 512, 4096, 32, 11008, 16
+    hd = hidden // heads
+    code2 = torch.cat([-torch.logspace(-7, 0, 127).flip(0), torch.zeros(2), torch.logspace(-7, 0, 127)]).sort().values.to(dev)
+
+    class Lin:
+        def __init__(self, w, qs=None):
+            self.weight, self.bias = w, None
+            if qs is not None:
+                self.weight.quant_state = qs
+
+    def nf4_weight(out_f, in_f):
+        n = out_f * in_f
+        packed = torch.randint(0, 256, (n // 2, 1), generator=gen, device=dev, dtype=torch.uint8)
+        nb = n // 64
+        state2 = SimpleNamespace(absmax=torch.full((-(-nb // 256),), 0.01, device=dev), code=code2, blocksize=256)
+        qs = nf4.make_quant_state(torch.randint(0, 256, (nb,), generator=gen, device=dev, dtype=torch.uint8), (out_f, in_f),
+                                  offset=torch.tensor(0.03, device=dev), state2=state2)
+        return Lin(packed, qs)
+
+    dims = dict(q=(hidden, hidden), k=(hidden, hidden), v=(hidden, hidden), o=(hidden, hidden),
+                gate=(inter, hidden), up=(inter, hidden), down=(hidden, inter))
+    layers = []
+    for _ in range(n_layers):
+        P = {}
+        for n, (o_f, i_f) in dims.items():
+            a = torch.empty(rank, i_f, device=dev)
+            torch.nn.init.kaiming_uniform_(a, a=math.sqrt(5), generator=gen)
+            P[n] = (nf4_weight(o_f, i_f), Lin(a.to(BF16).requires_grad_()),
+                    Lin((torch.randn(o_f, rank, generator=gen, device=dev) * 1e-3).to(BF16).requires_grad_()))
+        layers.append(SimpleNamespace(P=P, nw1=torch.ones(hidden, device=dev, dtype=BF16), nw2=torch.ones(hidden, device=dev, dtype=BF16)))
+    pos = torch.arange(S, device=dev, dtype=torch.float32)
+    inv = 1.0 / (1e4 ** (torch.arange(0, hd, 2, device=dev, dtype=torch.float32) / hd))
+    ang = torch.cat([pos[:, None] * inv[None, :]] * 2, dim=-1)
+    cos, sin = ang.cos().to(BF16)[None], ang.sin().to(BF16)[None]
+    mask = torch.full((S, S), float("-inf"), device=dev).triu(1).to(BF16)[None, None]
+    x0 = (torch.randn(B, S, hidden, generator=gen, device=dev)).to(BF16).requires_grad_()
+
+    def rope(x):
+        half = hd // 2
+        c, s_ = cos[0][None, :, None, :half], sin[0][None, :, None, :half]
+        x1, x2 = x[..., :half], x[..., half:]
+        return torch.cat([x1 * c - x2 * s_, x2 * c + x1 * s_], dim=-1)
+
+    class FrozenNF4Matmul(torch.autograd.Function):
+        """x @ dequant(W)^T that keeps only the packed weight for backward and dequantises again
+        there, like bitsandbytes' 4-bit matmul in an uncompressed QLoRA run."""
+        @staticmethod
+        def forward(ctx, inp, base):
+            ctx.base = base
+            return inp @ dense_weight(base.weight, base.weight.quant_state).t()
+
+        @staticmethod
+        def backward(ctx, gy):
+            return gy @ dense_weight(ctx.base.weight, ctx.base.weight.quant_state), None
+
+    def plain_layer(L, x):
+        def proj(n, inp):
+            base, la, lb = L.P[n]
+            return FrozenNF4Matmul.apply(inp, base) + (inp @ la.weight.t()) @ lb.weight.t()
+        rms = lambda v, w: (v.float() * torch.rsqrt(v.float().pow(2).mean(-1, keepdim=True) + 1e-5)).to(BF16) * w
+        xn = rms(x, L.nw1)
+        q, k, v = (hidden_to_head_shape(proj(n, xn), heads) for n in ("q", "k", "v"))
+        q = rope(q.transpose(1, 2)).transpose(1, 2)
+        k = rope(k.transpose(1, 2)).transpose(1, 2)
+        a = torch.softmax(q @ k.transpose(-2, -1) / math.sqrt(hd) + mask, dim=-1, dtype=BF16)
+        xm = x + proj("o", head_to_hidden_shape(a @ v))
+        xn2 = rms(xm, L.nw2)
+        return xm + proj("down", F.silu(proj("gate", xn2)) * proj("up", xn2))
+
+    cfg = SimpleNamespace(use_hyclora=True, layer_type="intra_inter", iteration_threshold=2, softmax_outlier_ratio=0.05,
+                          layernorm_outlier_ratio=0.005, q_bit=2)
+    fused = [llama.make_fused_llama_layer(cfg) for _ in layers]
+
+    def fused_layer(i, x):
+        L = layers[i]
+        args = [x, L.nw1, None, cos, sin]
+        for n in ("q", "k", "v", "o"):
+            args += list(L.P[n])
+        args += [L.nw2, None]
+        for n in ("gate", "up", "down"):
+            args += list(L.P[n])
+        return fused[i](*args, mask, heads, hd, heads)
+
+    def forward(arm):
+        x = x0
+        for i, L in enumerate(layers):
+            x = fused_layer(i, x) if arm == "compressed" else plain_layer(L, x)
+        return x.float().pow(2).mean()
+
+    out = {"layers": n_layers, "batch": B, "seq_len": S, "q_bit": 2, "layer_type": "intra_inter", "weights": "NF4, double-quantised statistics"}
+    mib = lambda: torch.cuda.memory_allocated() / 2 ** 20
+    import gc
+    for arm in ("plain", "compressed"):
+        gc.collect()
+        x0.grad = None
+        for L in layers:
+            for n in L.P:
+                L.P[n][1].weight.grad = L.P[n][2].weight.grad = None
+        torch.cuda.synchronize()
+        torch.cuda.empty_cache()
+        static = mib()
+        after = []
+        for it in range(3):                                   # steps 0 and 1 as in the reference, 2 = first frozen step
+            loss = forward(arm)
+            after.append(mib() - static)
+            loss.backward()
+            del loss
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            forward(arm).backward()
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / steps
+        out[arm] = {"static_MiB": static, "allocated_after_forward_minus_static_MiB": after,
+                    "fwd_bwd_ms": ms, "sequences_per_s": B / (ms * 1e-3)}
+    out["activation_memory_ratio"] = out["plain"]["allocated_after_forward_minus_static_MiB"][1] / \
+        out["compressed"]["allocated_after_forward_minus_static_MiB"][1]
     return out
 
 
@@ -443,6 +581,12 @@ def main():
             buffers.clear()
         torch.cuda.empty_cache()
         layers = bench_layers(torch, dev, args.layer_case, args.layer_arm)
+    stack = None
+    if args.only in ("all", "stack"):
+        for buffers in (xs, qs, xh):
+            buffers.clear()
+        torch.cuda.empty_cache()
+        stack = bench_stack(torch, dev)
 
     # ---- CPU baseline: the oracle on the host cores, same tensor --------------------------------
     cpu = None
@@ -485,6 +629,7 @@ def main():
         "fused": fused,
         "kernels": kernels,
         "layers": layers,
+        "stack": stack,
     }
     print(json.dumps(line))
 
