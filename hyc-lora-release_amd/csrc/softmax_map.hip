@@ -21,6 +21,9 @@ constexpr int kHistLdsBins = 16384;   // keys 0x8000..0xBFFF: bf16 values in [+0
 constexpr int kSeg = 4096;            // elements per compaction segment (one wave)
 constexpr int kSegThreads = 256;      // 4 segments per workgroup
 constexpr int kSegSteps = kSeg / (kWave * 8);
+#ifndef HYC_SW_WAVES
+#define HYC_SW_WAVES 4
+#endif
 constexpr int kStageEntries = 1024;   // kept entries of a segment that sparse_write gathers in LDS
 
 // Monotonic 16-bit key of a bf16 bit pattern: ascending key = ascending value, NaN last
@@ -111,6 +114,19 @@ __device__ __forceinline__ bool keep(uint32_t bits, float thr) {
     return v > thr && v != 0.0f;
 }
 
+// Inclusive prefix sum over the 64 lanes with DPP moves only (no LDS traffic): a shift-and-add scan
+// inside each row of 16 lanes (lanes without a source add 0), then the last lane of row 0 / 2 is
+// added to row 1 / 3, then lane 31 (sum of rows 0-1) to rows 2-3.
+__device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v) {
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x111, 0xf, 0xf, true);    // row_shr:1
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x112, 0xf, 0xf, true);    // row_shr:2
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x114, 0xf, 0xf, true);    // row_shr:4
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x118, 0xf, 0xf, true);    // row_shr:8
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x142, 0xa, 0xf, false);   // row_bcast:15 -> rows 1, 3
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x143, 0xc, 0xf, false);   // row_bcast:31 -> rows 2, 3
+    return v;
+}
+
 // Loads the 8 elements of chunk `c` of the flattened tensor, zero-filling past n.
 __device__ __forceinline__ void load_chunk(const uint16_t* a, int64_t c, int64_t n, uint32_t (&e)[8]) {
     const int64_t i0 = c * 8;
@@ -122,6 +138,21 @@ __device__ __forceinline__ void load_chunk(const uint16_t* a, int64_t c, int64_t
 #pragma unroll
         for (int j = 0; j < 8; ++j) e[j] = (i0 + j < n) ? a[i0 + j] : 0u;
     }
+}
+
+// The same chunk as four dwords (element 2p in the low half of dword p).
+__device__ __forceinline__ u32x4 load_chunk_packed(const uint16_t* a, int64_t c, int64_t n) {
+    const int64_t i0 = c * 8;
+    if (i0 + 8 <= n) return ld16(a + i0);
+    uint32_t d[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+        if (i0 + j < n) d[j >> 1] |= (uint32_t)a[i0 + j] << (16 * (j & 1));
+    return u32x4{d[0], d[1], d[2], d[3]};
+}
+__device__ __forceinline__ uint32_t chunk_elem(const u32x4& v, int j) {
+    const uint32_t d = (j >> 1) == 0 ? v.x : ((j >> 1) == 1 ? v.y : ((j >> 1) == 2 ? v.z : v.w));
+    return (j & 1) ? d >> 16 : d & 0xffffu;
 }
 
 __global__ __launch_bounds__(kSegThreads) void sparse_count_kernel(const uint16_t* __restrict__ a, int64_t n,
@@ -193,7 +224,8 @@ __global__ __launch_bounds__(1024) void seg_scan_kernel(const uint32_t* __restri
     if (t == 0 && base + 1024 >= nseg) offsets[nseg] = at + total;
 }
 
-__global__ __launch_bounds__(kSegThreads) void sparse_write_kernel(const uint16_t* __restrict__ a, int64_t n,
+__global__ __launch_bounds__(kSegThreads) __attribute__((amdgpu_waves_per_eu(HYC_SW_WAVES)))
+void sparse_write_kernel(const uint16_t* __restrict__ a, int64_t n,
                                                                    const float* __restrict__ thr_p, int64_t nseg,
                                                                    const int64_t* __restrict__ offsets,
                                                                    int64_t* __restrict__ idx_out,
@@ -205,28 +237,25 @@ __global__ __launch_bounds__(kSegThreads) void sparse_write_kernel(const uint16_
     const float thr = rbf(*thr_p);
     const int64_t base = offsets[seg];
     if (offsets[seg + 1] == base) return;          // nothing kept in this segment
-    // all of the segment's loads are issued before anything depends on them
-    uint32_t e[kSegSteps][8];
+    // all of the segment's loads are issued before anything depends on them; the chunks stay packed
+    // (4 registers each) so that enough waves fit on a SIMD
+    u32x4 e[kSegSteps];
     uint32_t mask[kSegSteps], inc[kSegSteps];
 #pragma unroll
     for (int s = 0; s < kSegSteps; ++s) {
         const int64_t c = seg * (kSeg / 8) + s * kWave + lane;
-        mask[s] = 0;
-        if (c * 8 < n) {
-            load_chunk(a, c, n, e[s]);
+        e[s] = u32x4{0, 0, 0, 0};
+        if (c * 8 < n) e[s] = load_chunk_packed(a, c, n);
+    }
 #pragma unroll
-            for (int j = 0; j < 8; ++j) mask[s] |= keep(e[s][j], thr) ? (1u << j) : 0u;
-        }
+    for (int s = 0; s < kSegSteps; ++s) {
+        mask[s] = 0;                                  // elements past n were loaded as zeros and are never kept
+#pragma unroll
+        for (int j = 0; j < 8; ++j) mask[s] |= keep(chunk_elem(e[s], j), thr) ? (1u << j) : 0u;
     }
 #pragma unroll
     for (int s = 0; s < kSegSteps; ++s) {            // independent inclusive prefixes over the lanes
-        uint32_t v = __popc(mask[s]);
-#pragma unroll
-        for (int o = 1; o < kWave; o <<= 1) {
-            const uint32_t up = (uint32_t)__shfl_up((int)v, o, kWave);
-            if (lane >= o) v += up;
-        }
-        inc[s] = v;
+        inc[s] = wave_inclusive_scan(__popc(mask[s]));
     }
     uint32_t before[kSegSteps], total = 0;            // kept entries in the steps in front
 #pragma unroll
@@ -245,7 +274,7 @@ __global__ __launch_bounds__(kSegThreads) void sparse_write_kernel(const uint16_
             const uint32_t rel = (uint32_t)(s * kWave + lane) * 8;
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                if (mask[s] & (1u << j)) st[w++] = ((rel + j) << 16) | (e[s][j] & 0xffffu);
+                if (mask[s] & (1u << j)) st[w++] = ((rel + j) << 16) | chunk_elem(e[s], j);
             }
         }
         __builtin_amdgcn_wave_barrier();               // LDS writes of this wave are visible to its lanes
@@ -265,7 +294,7 @@ __global__ __launch_bounds__(kSegThreads) void sparse_write_kernel(const uint16_
         for (int j = 0; j < 8; ++j) {
             if (mask[s] & (1u << j)) {
                 idx_out[w] = c * 8 + j;
-                val_out[w] = (uint16_t)e[s][j];
+                val_out[w] = (uint16_t)chunk_elem(e[s], j);
                 ++w;
             }
         }
