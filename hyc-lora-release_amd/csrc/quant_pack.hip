@@ -37,6 +37,9 @@ namespace hyc {
 #endif
 constexpr int kQuantWaves = HYC_Q_WAVES;      // waves per workgroup
 constexpr int kQuantThreads = kQuantWaves * kWave;
+#ifndef HYC_QO_WAVES
+#define HYC_QO_WAVES 4
+#endif
 #ifndef HYC_D_UNROLL
 #define HYC_D_UNROLL 2
 #endif
@@ -221,7 +224,8 @@ __device__ __forceinline__ void quant_rows(const QuantArgs& a, int64_t row0, int
 }
 
 template <int QBIT, bool ZP, bool OUTL>
-__global__ __launch_bounds__(kQuantThreads) void quant_pack_kernel(const QuantArgs a) {
+__global__ __launch_bounds__(kQuantThreads) __attribute__((amdgpu_waves_per_eu(OUTL ? HYC_QO_WAVES : 4)))
+void quant_pack_kernel(const QuantArgs a) {
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int col_tile = blockIdx.x % a.col_tiles;
