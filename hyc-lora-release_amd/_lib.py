@@ -50,7 +50,7 @@ _SIGNATURES = {
     "hyc_rmsnorm_fwd_compress": (_I, [_P, _P, _I, _P, _P, _L, _L, ctypes.c_float, _I, _P, _P, _P, _P, _P, _L, _P, _P]),
     "hyc_rope": (_I, [_P, _P, _P, _I, _L, _L, _L, _L, _L, _L, _L, _L, _L, _I, _P]),
     "hyc_softmax_fwd": (_I, [_P, _P, _P, _L, _L, ctypes.c_float, _L, _L, _L, _L, _P, _P, _P, _P]),
-    "hyc_softmax_bwd_restore": (_I, [_P, _P, _P, _P, _P, _P, _L, _L, _P]),
+    "hyc_softmax_bwd_restore": (_I, [_P, _P, _P, _P, _P, _P, _L, _L, ctypes.c_float, _P]),
     "hyc_rmsnorm_fwd": (_I, [_P, _P, _I, _P, _P, _L, _L, ctypes.c_float, _P]),
     "hyc_rmsnorm_bwd_workspace": (_L, [_L, _L]),
     "hyc_rmsnorm_bwd": (_I, [_P, _P, _P, _I, _P, _P, _P, _P, _L, _L, _L, _P]),

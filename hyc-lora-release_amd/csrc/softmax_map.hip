@@ -443,7 +443,7 @@ __global__ __launch_bounds__(256) void softmax_fwd_kernel(const uint16_t* __rest
 // ---- restore + softmax backward in one pass ----------------------------------------------
 // From the compressed map (idx, val, seg_offsets) and the upstream gradient g, writes
 //   a  = the restored dense map (optional, the caller needs it for grad_v = a^T @ grad_o) and
-//   o  = (g - sum_row bf16(a*g)) * a
+//   o  = bf16((g - sum_row bf16(a*g)) * a) * out_scale     (the layer's grad_s / sqrt(head_dim) folded in)
 // without reading a dense map back from HBM.  One wave rebuilds one 4096-element segment in LDS
 // exactly like sparse_restore_kernel; the segment holds 4096/n whole rows (n = 512 .. 4096), and
 // each row is SPR = n/512 wave-wide steps, so its sum is a plain wave reduction.
@@ -453,7 +453,7 @@ __global__ __launch_bounds__(kSegThreads) void softmax_bwd_restore_kernel(const 
                                                                           const int64_t* __restrict__ offsets,
                                                                           const uint16_t* __restrict__ g, int64_t nseg,
                                                                           uint16_t* __restrict__ a_out,
-                                                                          uint16_t* __restrict__ o_out) {
+                                                                          uint16_t* __restrict__ o_out, float out_scale) {
     __shared__ __attribute__((aligned(16))) uint16_t stage[kSegThreads / kWave][kSeg];
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x >> 6;
@@ -499,7 +499,7 @@ __global__ __launch_bounds__(kSegThreads) void softmax_bwd_restore_kernel(const 
             unpack8(yv[s], yf);
             unpack8(gv[s], gf);
 #pragma unroll
-            for (int j = 0; j < 8; ++j) of[j] = (gf[j] - acc) * yf[j];
+            for (int j = 0; j < 8; ++j) of[j] = rbf((gf[j] - acc) * yf[j]) * out_scale;   // bf16 result, then the bf16 scaling
             st16_nt(o_out + seg * kSeg + (int64_t)c * 8, pack8(of));
             if (a_out) st16_nt(a_out + seg * kSeg + (int64_t)c * 8, yv[s]);
         }
@@ -666,7 +666,7 @@ extern "C" int hyc_softmax_bwd(const void* y, const void* grad_y, void* out, int
 
 extern "C" int hyc_softmax_bwd_restore(const int64_t* indices, const void* values, const int64_t* seg_offsets,
                                        const void* grad_y, void* a_out, void* out, int64_t rows, int64_t n,
-                                       void* stream) {
+                                       float out_scale, void* stream) {
     if (rows < 0 || n < 0) return HYC_ERR_SHAPE;
     if (n != 512 && n != 1024 && n != 2048 && n != 4096) return HYC_ERR_SHAPE;
     if (rows == 0) return HYC_OK;
@@ -681,10 +681,10 @@ extern "C" int hyc_softmax_bwd_restore(const int64_t* indices, const void* value
     const uint16_t* gp = (const uint16_t*)grad_y;
     uint16_t* ap = (uint16_t*)a_out;
     uint16_t* op = (uint16_t*)out;
-    if (n == 512) hipLaunchKernelGGL(softmax_bwd_restore_kernel<1>, grid, block, 0, st, indices, vp, seg_offsets, gp, nseg, ap, op);
-    else if (n == 1024) hipLaunchKernelGGL(softmax_bwd_restore_kernel<2>, grid, block, 0, st, indices, vp, seg_offsets, gp, nseg, ap, op);
-    else if (n == 2048) hipLaunchKernelGGL(softmax_bwd_restore_kernel<4>, grid, block, 0, st, indices, vp, seg_offsets, gp, nseg, ap, op);
-    else hipLaunchKernelGGL(softmax_bwd_restore_kernel<8>, grid, block, 0, st, indices, vp, seg_offsets, gp, nseg, ap, op);
+    if (n == 512) hipLaunchKernelGGL(softmax_bwd_restore_kernel<1>, grid, block, 0, st, indices, vp, seg_offsets, gp, nseg, ap, op, out_scale);
+    else if (n == 1024) hipLaunchKernelGGL(softmax_bwd_restore_kernel<2>, grid, block, 0, st, indices, vp, seg_offsets, gp, nseg, ap, op, out_scale);
+    else if (n == 2048) hipLaunchKernelGGL(softmax_bwd_restore_kernel<4>, grid, block, 0, st, indices, vp, seg_offsets, gp, nseg, ap, op, out_scale);
+    else hipLaunchKernelGGL(softmax_bwd_restore_kernel<8>, grid, block, 0, st, indices, vp, seg_offsets, gp, nseg, ap, op, out_scale);
     return check_launch();
 }
 

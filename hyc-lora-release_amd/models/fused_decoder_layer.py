@@ -370,11 +370,11 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             # the compressed map (the reference restores, then reads the dense map twice more)
             grad_a = grad_o @ v.transpose(-2, -1)
             del v
-            a, grad_s = softmax_backward_from_compressed(S["a_idx"], S["a_val"], S["a_seg"], grad_a)
+            a, grad_s = softmax_backward_from_compressed(S["a_idx"], S["a_val"], S["a_seg"], grad_a,
+                                                         out_scale=1.0 / math.sqrt(D))
             del grad_a
             grad_v = a.transpose(-2, -1) @ grad_o
             del a, grad_o
-            grad_s = grad_s / math.sqrt(D)
             grad_k = grad_s.transpose(-2, -1) @ q
             grad_q = grad_s @ k
             del grad_s, q, k

@@ -212,7 +212,8 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
             v = hidden_to_head_shape(rebuilt("v"), H)
         grad_a = grad_o @ v.transpose(-2, -1)
         del v
-        a, grad_s = softmax_backward_from_compressed(S["a_idx"], S["a_val"], S["a_seg"], grad_a)
+        a, grad_s = softmax_backward_from_compressed(S["a_idx"], S["a_val"], S["a_seg"], grad_a,
+                                                     out_scale=1.0 / math.sqrt(D))
         del grad_a
         grad_v = a.transpose(-2, -1) @ grad_o
         del a, grad_o
@@ -220,7 +221,6 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
             q, k = deq("q", is_head=True, num_heads=H), deq("k", is_head=True, num_heads=H)
         else:
             q, k = hidden_to_head_shape(rebuilt("q"), H), hidden_to_head_shape(rebuilt("k"), H)
-        grad_s = grad_s / math.sqrt(D)
         grad_k = grad_s.transpose(-2, -1) @ q
         grad_q = grad_s @ k
         del grad_s, q, k

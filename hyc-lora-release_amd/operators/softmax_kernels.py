@@ -23,11 +23,12 @@ def softmax_backward(y: torch.Tensor, grad_y: torch.Tensor) -> torch.Tensor:
 FUSED_ROW_LENGTHS = (512, 1024, 2048, 4096)
 
 
-def softmax_backward_from_compressed(idx, val, seg_offsets, grad_y, want_map=True):
+def softmax_backward_from_compressed(idx, val, seg_offsets, grad_y, want_map=True, out_scale=1.0):
     """(restored map or None, softmax backward) straight from a compressed attention map
     (`compress_attention_map`) and the upstream gradient `grad_y` of the map's shape [..., n].
     One pass instead of restore + backward when n is 512, 1024, 2048 or 4096; other row lengths
-    take the two-kernel route."""
+    take the two-kernel route.  `out_scale` multiplies the bf16 gradient (and rounds again), which
+    is what the layers' `grad_s = grad_s / math.sqrt(head_dim)` does on the device."""
     from .compress_function import restore_attention_map
     _lib.require_gpu(idx, val, seg_offsets, grad_y)
     if grad_y.dtype != torch.bfloat16:
@@ -37,7 +38,8 @@ def softmax_backward_from_compressed(idx, val, seg_offsets, grad_y, want_map=Tru
     numel = grad_y.numel()
     if n not in FUSED_ROW_LENGTHS or numel % 4096 or numel == 0:
         a = restore_attention_map(idx, val, seg_offsets, shape)
-        return (a if want_map else None), softmax_backward(a, grad_y)
+        o = softmax_backward(a, grad_y)
+        return (a if want_map else None), (o if out_scale == 1.0 else o * out_scale)
     grad_y = grad_y.contiguous()
     idx = idx.reshape(-1).contiguous()
     val = val.reshape(-1).contiguous()
@@ -45,7 +47,7 @@ def softmax_backward_from_compressed(idx, val, seg_offsets, grad_y, want_map=Tru
     a = torch.empty(shape, device=grad_y.device, dtype=torch.bfloat16) if want_map else None
     _lib.call("hyc_softmax_bwd_restore", _lib.ptr(idx) if idx.numel() else None, _lib.ptr(val) if val.numel() else None,
               seg_offsets.data_ptr(), grad_y.data_ptr(), _lib.ptr(a), o.data_ptr(), numel // n, n,
-              _lib.stream_of(grad_y))
+              float(out_scale), _lib.stream_of(grad_y))
     return a, o
 
 

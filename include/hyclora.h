@@ -222,12 +222,15 @@ int hyc_softmax_fwd(const void *s, const void *mask, void *out, int64_t rows, in
  *   indices / values / seg_offsets  as produced by hyc_sparse_count + hyc_sparse_write for a map of
  *                                   rows*n elements;
  *   grad_y, out   bf16 [rows, n];   a_out  bf16 [rows, n] or NULL (the restored map);
+ *   out_scale     the bf16 gradient is multiplied by this and rounded again: 1.0f, or 1/sqrt(head_dim) to fold
+ *                 in the layer's grad_s = grad_s / math.sqrt(head_dim) (…full_fuse.py:436; a multiplication by
+ *                 the fp32 reciprocal in torch's device kernel);
  *   n in {512, 1024, 2048, 4096} and rows*n a multiple of 4096; other shapes: HYC_ERR_SHAPE (use
  *   hyc_sparse_restore + hyc_softmax_bwd).
  */
 int hyc_softmax_bwd_restore(const int64_t *indices, const void *values, const int64_t *seg_offsets,
                             const void *grad_y, void *a_out, void *out, int64_t rows, int64_t n,
-                            void *stream);
+                            float out_scale, void *stream);
 
 /* ---------------------------------------------------------------------------------------
  * RMSNorm forward: rstd = 1/sqrt(mean(x^2) + eps) in fp32, y = bf16(x * rstd * weight).

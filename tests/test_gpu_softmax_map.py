@@ -140,6 +140,9 @@ def test_softmax_backward_from_compressed(cf, sk, dev, shape, ratio):
     assert same_bits(a_out, dense) and same_bits(o, want)
     none, o2 = sk.softmax_backward_from_compressed(idx, val, seg, gr.to(dev), want_map=False)
     assert none is None and same_bits(o2, want)
+    # the layers' grad_s / sqrt(head_dim) folded in: the bf16 result times the fp32 reciprocal, rounded again
+    _, o3 = sk.softmax_backward_from_compressed(idx, val, seg, gr.to(dev), out_scale=1.0 / 128 ** 0.5)
+    assert same_bits(o3, (want.float() * torch.tensor(1.0 / 128 ** 0.5, dtype=torch.float32)).to(BF16))
     # against the oracle, from the oracle's own compressed form
     i_o, v_o = O.softmax_compress(a, thr.cpu())
     ref = O.softmax_bwd(O.softmax_restore(i_o, v_o, a.shape), gr)
