@@ -31,9 +31,9 @@ sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of quant_pack_kernel<4,false,false> on the benchmark tensor, measured with
-# rocprofv3 --pmc FETCH_SIZE (44 196 KiB raw, x1.9995 from the copy-kernel calibration) and
-# WRITE_SIZE (22 016 KiB, x1.0): 88 368 KiB read + 22 016 KiB written.
-MEASURED_TRAFFIC_BYTES = (88368 + 22016) * 1024
+# rocprofv3 --pmc FETCH_SIZE (44 162.3 KiB raw, x1.99948 from the copy-kernel calibration) and
+# WRITE_SIZE (22 016 KiB, x1.0): 88 301.6 KiB read + 22 016 KiB written.
+MEASURED_TRAFFIC_BYTES = int((44162.3 * 1.99948 + 22016.0) * 1024)
 
 
 def parse():
