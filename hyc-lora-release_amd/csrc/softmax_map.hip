@@ -106,12 +106,13 @@ __global__ __launch_bounds__(1024) void hist_select_kernel(const uint32_t* __res
 }
 
 // ---- ordered compaction ---------------------------------------------------------------
-// kept: a > thr and a != 0 (to_sparse drops exact zeros); NaN is never kept.  The caller
+// kept: a > thr and a != 0 (to_sparse drops exact zeros).  A NaN element is kept too: the reference
+// multiplies by the mask before to_sparse, and NaN * 0 is NaN, which is not zero.  The caller
 // passes thr already rounded to bf16: torch compares a bf16 tensor with a 0-d fp32
 // threshold in bf16.
 __device__ __forceinline__ bool keep(uint32_t bits, float thr) {
     const float v = bf_to_f((uint16_t)bits);
-    return v > thr && v != 0.0f;
+    return (v > thr || v != v) && v != 0.0f;
 }
 
 // Inclusive prefix sum over the 64 lanes with DPP moves only (no LDS traffic): a shift-and-add scan
@@ -155,9 +156,10 @@ __device__ __forceinline__ uint32_t chunk_elem(const u32x4& v, int j) {
     return (j & 1) ? d >> 16 : d & 0xffffu;
 }
 
+// cmp_mask 0xffff compares the element, 0x7fff its magnitude (|a| > thr).
 __global__ __launch_bounds__(kSegThreads) void sparse_count_kernel(const uint16_t* __restrict__ a, int64_t n,
                                                                    const float* __restrict__ thr_p, int64_t nseg,
-                                                                   uint32_t* __restrict__ counts) {
+                                                                   uint32_t* __restrict__ counts, uint32_t cmp_mask) {
     const int lane = threadIdx.x & (kWave - 1);
     const int64_t seg = blockIdx.x * (int64_t)(kSegThreads / kWave) + (threadIdx.x >> 6);
     if (seg >= nseg) return;
@@ -170,7 +172,7 @@ __global__ __launch_bounds__(kSegThreads) void sparse_count_kernel(const uint16_
             uint32_t e[8];
             load_chunk(a, c, n, e);
 #pragma unroll
-            for (int j = 0; j < 8; ++j) cnt += keep(e[j], thr) ? 1u : 0u;
+            for (int j = 0; j < 8; ++j) cnt += keep(e[j] & cmp_mask, thr) ? 1u : 0u;
         }
     }
 #pragma unroll
@@ -229,7 +231,7 @@ void sparse_write_kernel(const uint16_t* __restrict__ a, int64_t n,
                                                                    const float* __restrict__ thr_p, int64_t nseg,
                                                                    const int64_t* __restrict__ offsets,
                                                                    int64_t* __restrict__ idx_out,
-                                                                   uint16_t* __restrict__ val_out) {
+                                                                   uint16_t* __restrict__ val_out, uint32_t cmp_mask) {
     __shared__ uint32_t stage[kSegThreads / kWave][kStageEntries];
     const int lane = threadIdx.x & (kWave - 1);
     const int64_t seg = blockIdx.x * (int64_t)(kSegThreads / kWave) + (threadIdx.x >> 6);
@@ -251,7 +253,7 @@ void sparse_write_kernel(const uint16_t* __restrict__ a, int64_t n,
     for (int s = 0; s < kSegSteps; ++s) {
         mask[s] = 0;                                  // elements past n were loaded as zeros and are never kept
 #pragma unroll
-        for (int j = 0; j < 8; ++j) mask[s] |= keep(chunk_elem(e[s], j), thr) ? (1u << j) : 0u;
+        for (int j = 0; j < 8; ++j) mask[s] |= keep(chunk_elem(e[s], j) & cmp_mask, thr) ? (1u << j) : 0u;
     }
 #pragma unroll
     for (int s = 0; s < kSegSteps; ++s) {            // independent inclusive prefixes over the lanes
@@ -595,7 +597,7 @@ extern "C" int hyc_hist_select(const uint32_t* hist, int64_t kth, float* thresho
 
 extern "C" int64_t hyc_sparse_num_segments(int64_t n) { return n <= 0 ? 0 : cdiv(n, kSeg); }
 
-extern "C" int hyc_sparse_count(const void* a, int64_t n, const float* threshold, uint32_t* seg_counts,
+extern "C" int hyc_sparse_count(const void* a, int64_t n, const float* threshold, int compare_abs, uint32_t* seg_counts,
                                 int64_t* seg_offsets, void* stream) {
     if (n < 0) return HYC_ERR_SHAPE;
     if (!seg_offsets || !threshold) return HYC_ERR_NULL;
@@ -606,20 +608,21 @@ extern "C" int hyc_sparse_count(const void* a, int64_t n, const float* threshold
     hipStream_t st = (hipStream_t)stream;
     if (nseg > 0)
         hipLaunchKernelGGL(sparse_count_kernel, dim3((unsigned)cdiv(nseg, 4)), dim3(kSegThreads), 0, st,
-                           (const uint16_t*)a, n, threshold, nseg, seg_counts);
+                           (const uint16_t*)a, n, threshold, nseg, seg_counts, compare_abs ? 0x7fffu : 0xffffu);
     hipLaunchKernelGGL(seg_scan_kernel, dim3((unsigned)(nseg > 1024 ? cdiv(nseg, 1024) : 1)), dim3(1024), 0, st, seg_counts, nseg, seg_offsets);
     return check_launch();
 }
 
-extern "C" int hyc_sparse_write(const void* a, int64_t n, const float* threshold, const int64_t* seg_offsets,
-                                int64_t* indices, void* values, void* stream) {
+extern "C" int hyc_sparse_write(const void* a, int64_t n, const float* threshold, int compare_abs,
+                                const int64_t* seg_offsets, int64_t* indices, void* values, void* stream) {
     if (n < 0) return HYC_ERR_SHAPE;
     const int64_t nseg = hyc_sparse_num_segments(n);
     if (nseg == 0) return HYC_OK;
     if (!a || !threshold || !seg_offsets || !indices || !values) return HYC_ERR_NULL;
     if (!aligned16(a)) return HYC_ERR_ALIGN;
     hipLaunchKernelGGL(sparse_write_kernel, dim3((unsigned)cdiv(nseg, 4)), dim3(kSegThreads), 0, (hipStream_t)stream,
-                       (const uint16_t*)a, n, threshold, nseg, seg_offsets, indices, (uint16_t*)values);
+                       (const uint16_t*)a, n, threshold, nseg, seg_offsets, indices, (uint16_t*)values,
+                       compare_abs ? 0x7fffu : 0xffffu);
     return check_launch();
 }
 

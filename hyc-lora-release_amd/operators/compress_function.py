@@ -285,12 +285,12 @@ def _threshold_tensor(outlier, device) -> torch.Tensor:
     return torch.tensor(float(outlier), device=device, dtype=torch.float32)
 
 
-def compress_attention_map(x: torch.Tensor, outlier, seg_offsets=None):
+def compress_attention_map(x: torch.Tensor, outlier, seg_offsets=None, compare_abs=False):
     """Kept entries of the flattened map: (indices int64 [nnz] ascending, values bf16 [nnz],
     seg_offsets int64 [nseg + 1]).  An entry is kept when x > outlier (compared in bf16, as
     torch does) and x != 0.  seg_offsets lets restore_attention_map skip the index search.
     `seg_offsets` may be passed in when the producer of x already counted (softmax_forward with a
-    threshold): the counting pass is skipped."""
+    threshold): the counting pass is skipped.  compare_abs: keep by magnitude, |x| > outlier."""
     _lib.require_gpu(x)
     if x.dtype != BF16:
         x = x.to(BF16)
@@ -308,13 +308,14 @@ def compress_attention_map(x: torch.Tensor, outlier, seg_offsets=None):
     else:
         counts = torch.empty(max(nseg, 1), device=x.device, dtype=torch.int32)
         offsets = torch.empty(nseg + 1, device=x.device, dtype=torch.int64)
-        _lib.call("hyc_sparse_count", flat.data_ptr(), n, thr.data_ptr(), counts.data_ptr(), offsets.data_ptr(), st)
+        _lib.call("hyc_sparse_count", flat.data_ptr(), n, thr.data_ptr(), int(compare_abs), counts.data_ptr(),
+                  offsets.data_ptr(), st)
     nnz = int(offsets[-1].item())      # the one host sync; to_sparse() has the same one
     idx = torch.empty(nnz, device=x.device, dtype=torch.int64)
     val = torch.empty(nnz, device=x.device, dtype=BF16)
     if nnz:
-        _lib.call("hyc_sparse_write", flat.data_ptr(), n, thr.data_ptr(), offsets.data_ptr(), idx.data_ptr(),
-                  val.data_ptr(), st)
+        _lib.call("hyc_sparse_write", flat.data_ptr(), n, thr.data_ptr(), int(compare_abs), offsets.data_ptr(),
+                  idx.data_ptr(), val.data_ptr(), st)
     return idx, val, offsets
 
 
@@ -348,6 +349,78 @@ def decompression_softmax(x_sparse: torch.Tensor):
     if not x_sparse.is_coalesced():
         x_sparse = x_sparse.coalesce()
     return restore_attention_map(x_sparse.indices()[0], x_sparse.values(), None, x_sparse.shape)
+
+
+# ---------------------------------------------------------------------------------------
+# pruning forms of the reference that none of its layers call (operators/compress_function.py:39-42,
+# :320-341); kept so that the module is a complete stand-in
+# ---------------------------------------------------------------------------------------
+def get_statistics_structed_pruning(x: torch.Tensor, outlier_ratio: float):
+    """Indices of the int(N * ratio) channels with the largest norm over dim -2, per leading index
+    (x.abs().norm(dim=-2) then topk; reference :39-42).  Ties: larger norm first, then lower channel."""
+    _lib.require_gpu(x)
+    if x.dim() < 2:
+        raise ValueError("needs at least [rows, channels]")
+    xb = x.to(BF16)
+    n = xb.shape[-1]
+    k = int(n * outlier_ratio)
+    lead = xb.shape[:-2]
+    flat = xb.reshape(-1, xb.shape[-2], n)
+    out = torch.empty((flat.shape[0], k), device=x.device, dtype=torch.int64)
+    scale = torch.empty((1, n), device=x.device, dtype=BF16)
+    for b in range(flat.shape[0]):
+        stats, _ = _batch0_stats(flat[b:b + 1])
+        _lib.call("hyc_channel_select", stats.data_ptr(), n, k, 8, 0, out[b].data_ptr() if k else None,
+                  scale.data_ptr(), None, _lib.stream_of(x))
+    return out.reshape(*lead, k)
+
+
+def _unravel(flat_idx, shape):
+    idx = []
+    rem = flat_idx
+    for d in reversed(shape):
+        idx.append(rem % d)
+        rem = torch.div(rem, d, rounding_mode="floor")
+    return torch.stack(idx[::-1], dim=0)
+
+
+def compression_unstructed_pruning_coo(x: torch.Tensor, outlier):
+    """Sparse COO tensor of x's own shape holding the elements with |x| > outlier, like
+    (x * (x.abs() > outlier)).to_sparse().  Reference :320-324."""
+    idx, val, _ = compress_attention_map(x, outlier, compare_abs=True)
+    return torch.sparse_coo_tensor(_unravel(idx, tuple(x.shape)), val, tuple(x.shape), is_coalesced=True)
+
+
+def decompression_unstructed_pruning_coo(x_sparse: torch.Tensor):
+    """x_sparse.to_dense().  Reference :327-328."""
+    if not x_sparse.is_coalesced():
+        x_sparse = x_sparse.coalesce()
+    shape = tuple(x_sparse.shape)
+    flat = torch.zeros((), device=x_sparse.device, dtype=torch.int64)
+    for d, row in zip(shape, x_sparse.indices()):
+        flat = flat * d + row
+    return restore_attention_map(flat, x_sparse.values(), None, shape)
+
+
+def compression_unstructed_pruning_bitmap(x: torch.Tensor, outlier):
+    """(kept values in flat order, boolean mask |x| > outlier).  Reference :331-335: the values are
+    (x * mask)[mask], so a kept element is any with |x| > outlier (zeros cannot qualify for
+    outlier >= 0; NaN never does)."""
+    _lib.require_gpu(x)
+    thr = _threshold_tensor(outlier, x.device)
+    mask = x.to(BF16).abs() > thr.to(BF16)
+    idx, val, _ = compress_attention_map(x, outlier, compare_abs=True)
+    if idx.numel() != int(mask.sum()):                        # outlier < 0 keeps exact zeros, which the compaction drops
+        return (x.to(BF16) * mask)[mask], mask
+    return val, mask
+
+
+def decompression_unstructed_pruning_bitmap(x_sparse: torch.Tensor, mask: torch.Tensor):
+    """Dense tensor of mask's shape with x_sparse at the True positions.  Reference :338-341 (which
+    leaves the other positions uninitialised; here they are zero)."""
+    _lib.require_gpu(x_sparse, mask)
+    flat = torch.nonzero(mask.reshape(-1)).reshape(-1)
+    return restore_attention_map(flat, x_sparse, None, tuple(mask.shape))
 
 
 # ---------------------------------------------------------------------------------------
@@ -386,3 +459,16 @@ def compression_pack_softmax_base(x, o_ratio, it_num, it_num_thd, static_value):
     else:
         outlier = static_value['outlier']
     return compression_softmax(x, outlier), outlier
+
+
+def compression_pack_unstructed_pruning_coo(x, o_ratio, it_num, it_num_thd, static_value):
+    """Reference :382-388."""
+    outlier = get_statistics_outlier(x, o_ratio) if it_num < it_num_thd else static_value['outlier']
+    return compression_unstructed_pruning_coo(x, outlier), outlier
+
+
+def compression_pack_unstructed_pruning_bitmap(x, o_ratio, it_num, it_num_thd, static_value):
+    """Reference :391-397."""
+    outlier = get_statistics_outlier(x, o_ratio) if it_num < it_num_thd else static_value['outlier']
+    x_outlier, mask = compression_unstructed_pruning_bitmap(x, outlier)
+    return x_outlier, outlier, mask

@@ -159,7 +159,10 @@ int hyc_hist_select(const uint32_t *hist, int64_t kth, float *threshold, void *s
  * (:316-317; models/llama/fused_llama_layer_intra_inter_full_fuse.py:414-415).
  *
  * An element is kept when a > bf16(threshold) and a != 0 (torch compares in bf16 and
- * to_sparse drops zeros).  Output order is ascending flat index, as to_sparse gives.
+ * to_sparse drops zeros), and when it is NaN (the reference multiplies by the mask first, and
+ * NaN * 0 is not zero); with compare_abs != 0 when |a| > bf16(threshold) and a != 0, which is the
+ * unstructured-pruning form (compression_unstructed_pruning_coo / _bitmap, :320-335).  Output order
+ * is ascending flat index, as to_sparse gives.
  * The flattened tensor is processed in segments of 4096 elements;
  * hyc_sparse_num_segments(n) = ceil(n / 4096).
  *
@@ -173,10 +176,10 @@ int hyc_hist_select(const uint32_t *hist, int64_t kth, float *threshold, void *s
  *   hyc_sparse_restore out bf16 [n] (16-byte aligned): zeros, with values[i] at indices[i].
  */
 int64_t hyc_sparse_num_segments(int64_t n);
-int hyc_sparse_count(const void *a, int64_t n, const float *threshold, uint32_t *seg_counts,
+int hyc_sparse_count(const void *a, int64_t n, const float *threshold, int compare_abs, uint32_t *seg_counts,
                      int64_t *seg_offsets, void *stream);
-int hyc_sparse_write(const void *a, int64_t n, const float *threshold, const int64_t *seg_offsets,
-                     int64_t *indices, void *values, void *stream);
+int hyc_sparse_write(const void *a, int64_t n, const float *threshold, int compare_abs,
+                     const int64_t *seg_offsets, int64_t *indices, void *values, void *stream);
 int hyc_sparse_segment_offsets(const int64_t *indices, int64_t nnz, int64_t n, int64_t *seg_offsets,
                                void *stream);
 int hyc_sparse_restore(const int64_t *indices, const void *values, const int64_t *seg_offsets,

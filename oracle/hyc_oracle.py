@@ -253,12 +253,12 @@ def decompress_channel_base(p, s, x_outlier, idx, q_bit, is_head=False, num_head
 # --------------------------------------------------------------------------------------
 def softmax_compress(a: torch.Tensor, thr) -> Tuple[torch.Tensor, torch.Tensor]:
     """(a * (a > thr)).flatten().to_sparse() as (int64 indices ascending, bf16 values)
-    (compress_function.py:309-313).  to_sparse drops exact zeros, so a kept element is
-    one with a > thr and a != 0."""
+    (compress_function.py:309-313), literally: the product with the mask, then the non-zero
+    entries.  So a kept element is one with a > thr and a != 0 - or a NaN (NaN * 0 = NaN != 0)."""
     flat = a.flatten()
-    keep = (flat > thr) & (flat != 0)
-    idx = torch.nonzero(keep).flatten()
-    return idx, flat[idx]
+    prod = flat * (flat > thr)
+    idx = torch.nonzero(prod).flatten()
+    return idx, flat[idx]            # = prod[idx] as numbers; the element itself so that a NaN keeps its payload
 
 
 def softmax_restore(idx, vals, shape) -> torch.Tensor:

@@ -88,15 +88,20 @@ def test_threshold_is_compared_in_bf16_and_zeros_are_dropped(cf, dev):
     idx_ref, val_ref = O.softmax_compress(a, thr)
     idx, val, _ = cf.compress_attention_map(a.to(dev), thr.to(dev))
     assert torch.equal(idx.cpu(), idx_ref) and same_bits(val.cpu(), val_ref)
-    assert idx_ref.numel() == 16                            # only 1.015625 and 2.0
+    assert idx_ref.numel() == 24                            # 1.015625, 2.0 - and NaN: NaN * False is NaN, which to_sparse keeps
+    sp = (a * (a > thr)).flatten().to_sparse()              # the reference's own expression
+    assert torch.equal(idx_ref, sp.indices()[0])
+    assert torch.equal(val_ref.isnan(), sp.values().isnan()) and same_bits(torch.nan_to_num(val_ref), torch.nan_to_num(sp.values()))
     # negative threshold: zeros pass the comparison but to_sparse drops them
     thr = torch.tensor(-1.0)
     idx_ref, val_ref = O.softmax_compress(a, thr)
     idx, val, _ = cf.compress_attention_map(a.to(dev), -1.0)
     assert torch.equal(idx.cpu(), idx_ref) and same_bits(val.cpu(), val_ref)
-    # nothing kept / everything kept
-    idx, val, seg = cf.compress_attention_map(a.to(dev), 1e9)
+    # nothing kept (a map without NaN) / only the NaNs kept
+    idx, val, seg = cf.compress_attention_map(torch.nan_to_num(a).to(dev), 1e9)
     assert idx.numel() == 0 and (cf.restore_attention_map(idx, val, seg, a.shape) == 0).all()
+    idx, val, seg = cf.compress_attention_map(a.to(dev), 1e9)
+    assert idx.cpu().tolist() == list(range(5, 64, 8)) and bool(val.isnan().all())
 
 
 def test_pack_softmax_base_dispatch(cf, dev):
