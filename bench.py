@@ -163,6 +163,12 @@ def bench_layers(torch, dev, only_case="", arm="both"):
         if arm != "compressed":
             ms_p, saved_p = measure(lambda: run_plain(t, mask, sdpa), t)
             entry["bf16_uncompressed"] = {"fwd_bwd_ms": ms_p, "saved_activation_MB": saved_p / 1e6}
+            # the reference's own comparison arm: its default layer type, hand-written backward, nothing compressed
+            base = llama_flash_attn.FusedLlamaLayerBaseline() if maker is None else maker(cfg("baseline", 0))
+            base.set_hyclora_config(cfg("baseline", 0))
+            ms_b, saved_b = measure(lambda: run_fused(base, t, mask), t)
+            entry["baseline_layer"] = {"fwd_bwd_ms": ms_b, "saved_activation_MB": saved_b / 1e6}
+            del base
         for q in (qbits if arm != "plain" else []):
             if maker is None:
                 layer = llama_flash_attn.FusedLlamaLayerIntraInter()

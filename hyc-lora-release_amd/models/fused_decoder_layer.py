@@ -2,10 +2,14 @@
 saves *compressed* activations for backward.
 
 Restates what the reference spreads over twelve near-identical files
-(models/{llama,mistral,llama_flash_attn}/fused_*_layer_{intra,intra_inter,intra_inter_full_fuse}.py)
+(models/{llama,mistral,llama_flash_attn}/fused_*_layer_{baseline,intra,intra_inter,intra_inter_full_fuse}.py)
 as one function with three switches:
 
-  mode        'intra'                 every saved activation is quantised as is; q, k (after RoPE) and
+  mode        'baseline'              nothing is compressed: the same tensors 'intra' saves are kept
+                                      as they are and no statistics are gathered - the reference's
+                                      default layer type and the uncompressed arm of its memory /
+                                      throughput comparison          (fused_llama_layer_baseline.py:147-235)
+              'intra'                 every saved activation is quantised as is; q, k (after RoPE) and
                                       v are saved in head shape; silu(gate) and the gated product are
                                       saved too                      (fused_llama_layer_intra.py:95-310)
               'intra_inter'           only the frozen-weight outputs (x@W, "main") are quantised; the
@@ -46,13 +50,13 @@ from ..operators.compress_function import (compress_attention_map, compression_p
 from ..operators.rmsnorm_kernels import _backward as _rmsnorm_backward
 from ..operators.rmsnorm_kernels import rmsnorm_forward, rmsnorm_forward_compress
 from ..operators.silu_kernels import silu_backward, silu_hadamard
-from ..operators.softmax_kernels import softmax_backward_from_compressed, softmax_forward
+from ..operators.softmax_kernels import softmax_backward, softmax_backward_from_compressed, softmax_forward
 from ..operators.triton_fuse_lora_silu_hadamard_backward_kernels import triton_fuse_silu_backward
 from ..operators.triton_fuse_lora_silu_hadamard_forward_kernels import triton_fuse_silu_forward
 from .compute_utils import (head_to_hidden_shape, hidden_to_head_shape, lora_backward, lora_forward,
                             repeat_kv, repeat_kv_backward, rope_backward, rope_forward)
 
-MODES = ("intra", "intra_inter", "intra_inter_full_fuse")
+MODES = ("baseline", "intra", "intra_inter", "intra_inter_full_fuse")
 
 
 @dataclass(frozen=True)
@@ -69,6 +73,8 @@ class LayerSpec:
 
     def stat_slots(self):
         """(static_value key, field) of every calibration statistic the layer returns, in order."""
+        if self.mode == "baseline":
+            return []
         slots = [("x", "outlier_channel_index"), ("x", "scale"), ("x_norm_1", "scale"),
                  ("q", "scale"), ("k", "scale"), ("v", "scale")]
         if self.attention == "map":
@@ -111,22 +117,33 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
         calib = it < thd
         n_rep = num_heads // num_key_value_heads
         stats, saved = {}, {}
+        raw = spec.mode == "baseline"                   # keep activations as they are
+        whole = spec.mode in ("baseline", "intra")      # save whole activations, not the frozen-weight parts
 
         def proj(name, inp):
             w, b, qs, la, lb = W[name]
             return lora_forward(w, qs, la, lb, b, inp)
 
         def quant(name, t, key=None):
+            if raw:
+                saved[name + "_raw"] = t
+                return
             q, s = compression_pack_quant_base(t, q_bit, 'per-channel', it, thd, sv[key or name])
             stats[(key or name, "scale")] = s
             saved[name + "_q"], saved[name + "_s"] = q, s
 
         def quant_zp(name, t, key):
+            if raw:
+                saved[name + "_raw"] = t
+                return
             q, s, z = compression_pack_quant_zp_base(t, q_bit, 'per-channel', it, thd, sv[key])
             stats[(key, "scale")], stats[(key, "zero_point")] = s, z
             saved[name + "_q"], saved[name + "_s"], saved[name + "_z"] = q, s, z
 
         def channel_base(name, t):
+            if raw:
+                saved[name + "_raw"] = t
+                return
             o, q, idx, s = compression_pack_channel_base(t, layernorm_outlier_ratio, q_bit, 'per-channel', it, thd,
                                                          sv[name])
             stats[(name, "outlier_channel_index")], stats[(name, "scale")] = idx, s
@@ -138,7 +155,7 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             the output depend on the output, so the separate operators run (returns done=False and
             the caller quantises the output itself)."""
             n = t.shape[-1]
-            if calib or t.dtype != torch.bfloat16 or t.dim() != 3 or n % 32 or n > 8192:
+            if raw or calib or t.dtype != torch.bfloat16 or t.dim() != 3 or n % 32 or n > 8192:
                 y, _, rstd, _, _ = rmsnorm_forward(t, w, spec.eps)
                 channel_base(xname, t)
                 return y, rstd, False
@@ -158,7 +175,7 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
         if not norm_1_done:
             quant("x_norm_1", x_norm_1)
         del x_norm_1
-        if spec.mode != "intra":
+        if not whole:
             if spec.attention == "sdpa":
                 quant_zp("q_main", q_main, "q")
                 quant_zp("k_main", k_main, "k")
@@ -175,7 +192,7 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
         k = rope_forward(k.transpose(1, 2), cos, sin).transpose(1, 2)
         k = repeat_kv(k, n_rep)
         v = repeat_kv(v, n_rep)
-        if spec.mode == "intra":
+        if whole:
             (quant_zp if spec.attention == "sdpa" else quant)("q_rope", q, "q")
             (quant_zp if spec.attention == "sdpa" else quant)("k_rope", k, "k")
             quant("v_rep", v, "v")
@@ -192,7 +209,7 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             seg = None
             if s.dtype == torch.bfloat16 and s.shape[-1] % 8 == 0 and s.shape[-1] <= 8192 and \
                     (attention_mask is None or m is not None):
-                if calib:
+                if calib or raw:
                     a = softmax_forward(s, 1.0 / math.sqrt(head_dim), m, inplace=True)
                 else:
                     a, seg = softmax_forward(s, 1.0 / math.sqrt(head_dim), m, threshold=sv['a']['outlier'], inplace=True)
@@ -202,10 +219,12 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
                     s = s + attention_mask
                 a = torch.softmax(s, dim=-1, dtype=v.dtype)
             del s
-            thr = get_statistics_softmax(a, softmax_outlier_ratio) if calib else sv['a']['outlier']
-            stats[("a", "outlier")] = thr
-            saved["a_idx"], saved["a_val"], saved["a_seg"] = compress_attention_map(a, thr, seg)
-            ctx.a_shape = tuple(a.shape)
+            if raw:
+                saved["a_raw"] = a
+            else:
+                thr = get_statistics_softmax(a, softmax_outlier_ratio) if calib else sv['a']['outlier']
+                stats[("a", "outlier")] = thr
+                saved["a_idx"], saved["a_val"], saved["a_seg"] = compress_attention_map(a, thr, seg)
             o = a @ v
             del a, v
         else:
@@ -245,7 +264,7 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
                 quant("gate_main", gate_main, "gate")
                 quant("up_main", up_main, "up")
                 hadamard = silu_hadamard(gate, up)
-            else:
+            else:                                           # 'intra' and 'baseline'
                 fn = F.silu(gate)
                 quant("gate", gate)
                 hadamard = up * fn
@@ -258,7 +277,7 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             quant("x_norm_2", x_norm_2)
         del x_norm_2
         down, _, saved["down_lora_a"] = proj("down", hadamard)
-        if spec.mode == "intra":
+        if whole:
             quant("hadamard", hadamard)
         del hadamard
         x_out = x_medium + down
@@ -291,6 +310,8 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
         G = {}                                           # LoRA gradients
 
         def deq(name, **kw):
+            if name + "_raw" in S:
+                return S[name + "_raw"]
             if name + "_z" in S:
                 return decompression_dequantization_with_zero_point(S[name + "_q"], S[name + "_s"], S[name + "_z"],
                                                                     q_bit, **kw)
@@ -304,6 +325,12 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
 
         def lora_part(name):
             return S[name + "_lora_a"] @ W[name][4].to(S[name + "_lora_a"].dtype)
+
+        def channel_base_restored(name):
+            if name + "_raw" in S:
+                return S[name + "_raw"]
+            return outlier_addition_fuse_decompression_dequantization(
+                S[name + "_q"], S[name + "_s"], S[name + "_o"], S[name + "_idx"], q_bit)
 
         def norm_backward(dy, xin, weight, rstd, want_dw):
             return _rmsnorm_backward(dy, xin, weight, rstd, want_dw=want_dw)
@@ -342,8 +369,7 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
         grad_x2 = back("gate", x_norm_2, S["gate_lora_a"], grad_fn)
         grad_x2 = grad_x2 + back("up", x_norm_2, S["up_lora_a"], grad_h2)
         del x_norm_2, grad_fn, grad_h2
-        x_medium = outlier_addition_fuse_decompression_dequantization(
-            S["x_medium_q"], S["x_medium_s"], S["x_medium_o"], S["x_medium_idx"], q_bit)
+        x_medium = channel_base_restored("x_medium")
         grad_norm_2, grad_nw2 = norm_backward(grad_x2, x_medium, norm_weight_2, S["rstd_2"], ctx.norm_grads[1])
         del x_medium, grad_x2
         grad_medium = grad_norm_2 + grad_output
@@ -360,7 +386,7 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
                 t = rope_forward(t.transpose(1, 2), cos, sin).transpose(1, 2)
             return t
 
-        if spec.mode == "intra":
+        if spec.mode in ("baseline", "intra"):
             q, k, v = (deq(n, is_head=True, num_heads=H) for n in ("q_rope", "k_rope", "v_rep"))
         else:
             q, k, v = rebuilt("q", H), repeat_kv(rebuilt("k", KV), n_rep), repeat_kv(rebuilt("v", KV), n_rep)
@@ -370,8 +396,12 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             # the compressed map (the reference restores, then reads the dense map twice more)
             grad_a = grad_o @ v.transpose(-2, -1)
             del v
-            a, grad_s = softmax_backward_from_compressed(S["a_idx"], S["a_val"], S["a_seg"], grad_a,
-                                                         out_scale=1.0 / math.sqrt(D))
+            if "a_raw" in S:
+                a = S["a_raw"]
+                grad_s = softmax_backward(a, grad_a) / math.sqrt(D)
+            else:
+                a, grad_s = softmax_backward_from_compressed(S["a_idx"], S["a_val"], S["a_seg"], grad_a,
+                                                             out_scale=1.0 / math.sqrt(D))
             del grad_a
             grad_v = a.transpose(-2, -1) @ grad_o
             del a, grad_o
@@ -396,7 +426,7 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
         grad_x += back("k", x_norm_1, S["k_lora_a"], grad_k)
         grad_x += back("v", x_norm_1, S["v_lora_a"], grad_v)
         del x_norm_1, grad_q, grad_k, grad_v
-        x = outlier_addition_fuse_decompression_dequantization(S["x_q"], S["x_s"], S["x_o"], S["x_idx"], q_bit)
+        x = channel_base_restored("x")
         grad_norm_1, grad_nw1 = norm_backward(grad_x, x, norm_weight_1, S["rstd_1"], ctx.norm_grads[0])
         grad_input = grad_norm_1 + grad_medium
 
@@ -433,10 +463,12 @@ class FusedDecoderLayer(torch.nn.Module):
     def set_hyclora_config(self, hyclora_config):
         self.hyclora_config = hyclora_config
         self.use_hyclora = hyclora_config.use_hyclora
-        self.iteration_threshold = hyclora_config.iteration_threshold
-        self.softmax_outlier_ratio = hyclora_config.softmax_outlier_ratio
-        self.layernorm_outlier_ratio = hyclora_config.layernorm_outlier_ratio
-        self.q_bit = hyclora_config.q_bit
+        # the uncompressed layer reads none of the compression settings
+        # (fused_llama_layer_baseline.py:443-445 keeps only use_hyclora and the config itself)
+        self.iteration_threshold = getattr(hyclora_config, "iteration_threshold", 0)
+        self.softmax_outlier_ratio = getattr(hyclora_config, "softmax_outlier_ratio", 0.0)
+        self.layernorm_outlier_ratio = getattr(hyclora_config, "layernorm_outlier_ratio", 0.0)
+        self.q_bit = getattr(hyclora_config, "q_bit", 0)
 
     # The reference keeps `iteration` and `static_value` as plain attributes (…full_fuse.py:574-580),
     # so a checkpoint taken after calibration restarts calibrating.  Here they travel with

@@ -1,6 +1,10 @@
 """Llama decoder layers with compressed saved activations; class names as in the reference
-(models/llama/fused_llama_layer_{intra,intra_inter,intra_inter_full_fuse}.py)."""
+(models/llama/fused_llama_layer_{baseline,intra,intra_inter,intra_inter_full_fuse}.py)."""
 from .fused_decoder_layer import FusedDecoderLayer
+
+
+class FusedLlamaLayerBaseline(FusedDecoderLayer):
+    layer_type = "baseline"
 
 
 class FusedLlamaLayerIntra(FusedDecoderLayer):
@@ -16,6 +20,7 @@ class FusedLlamaLayerIntraInterFullFuse(FusedDecoderLayer):
 
 
 LAYER_TYPES = {
+    "baseline": FusedLlamaLayerBaseline,
     "intra": FusedLlamaLayerIntra,
     "intra_inter": FusedLlamaLayerIntraInter,
     "intra_inter_full_fuse": FusedLlamaLayerIntraInterFullFuse,

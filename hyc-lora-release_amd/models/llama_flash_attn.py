@@ -1,9 +1,14 @@
 """Long-sequence Llama layers: no attention map is materialised or saved, q/k main are quantised
 with a zero point, norm weights receive gradients
-(models/llama_flash_attn/fused_llama_layer_{intra,intra_inter}.py).  The flash-attn varlen kernels
+(models/llama_flash_attn/fused_llama_layer_{baseline,intra,intra_inter}.py).  The flash-attn varlen kernels
 of the reference are replaced by torch's scaled_dot_product_attention (its ROCm flash/CK backend);
 backward recomputes the attention instead of calling a saved-LSE backward kernel."""
 from .fused_decoder_layer import FusedDecoderLayer
+
+
+class FusedLlamaLayerBaseline(FusedDecoderLayer):
+    layer_type = "baseline"
+    attention = "sdpa"
 
 
 class FusedLlamaLayerIntra(FusedDecoderLayer):

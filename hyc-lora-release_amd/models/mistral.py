@@ -5,6 +5,10 @@ cast of lora_B (fused_mistral_layer_intra_inter_full_fuse.py:226-227), both cove
 from .fused_decoder_layer import FusedDecoderLayer
 
 
+class FusedMistralLayerBaseline(FusedDecoderLayer):
+    layer_type = "baseline"
+
+
 class FusedMistralLayerIntra(FusedDecoderLayer):
     layer_type = "intra"
 
@@ -18,6 +22,7 @@ class FusedMistralLayerIntraInterFullFuse(FusedDecoderLayer):
 
 
 LAYER_TYPES = {
+    "baseline": FusedMistralLayerBaseline,
     "intra": FusedMistralLayerIntra,
     "intra_inter": FusedMistralLayerIntraInter,
     "intra_inter_full_fuse": FusedMistralLayerIntraInterFullFuse,

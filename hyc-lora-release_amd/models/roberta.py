@@ -1,8 +1,10 @@
 """RoBERTa encoder layers (post-LayerNorm, GELU MLP) with compressed saved activations; class names,
 argument order and calibration behaviour of the reference
-(models/roberta/fused_roberta_layer_{intra,intra_inter}.py).
+(models/roberta/fused_roberta_layer_{baseline,intra,intra_inter}.py).
 
-One autograd.Function serves both layer types:
+One autograd.Function serves the layer types:
+  baseline     keeps the tensors 'intra' keeps, uncompressed, and gathers no statistics
+               (…baseline.py: the reference's default layer type);
   intra        keeps the quantised tensors the backward needs as they are (q, k, v in head shape after
                the LoRA add, up, gelu(up));
   intra_inter  keeps only the frozen-weight parts of q, k, v, up and rebuilds the rest in backward
@@ -18,10 +20,10 @@ from ..operators.compress_function import (compress_attention_map, compression_p
                                            outlier_addition_fuse_decompression_dequantization, update_dict)
 from ..operators.gelu_kernels import gelu_backward
 from ..operators.layernorm_kernels import layernorm_backward, layernorm_forward
-from ..operators.softmax_kernels import softmax_backward_from_compressed, softmax_forward
+from ..operators.softmax_kernels import softmax_backward, softmax_backward_from_compressed, softmax_forward
 from .compute_utils import head_to_hidden_shape, hidden_to_head_shape, lora_backward, lora_forward
 
-MODES = ("intra", "intra_inter")
+MODES = ("baseline", "intra", "intra_inter")
 _PROJ = ("q", "k", "v", "o", "up", "down")
 _EPS = 1e-5
 
@@ -29,6 +31,8 @@ _EPS = 1e-5
 def stat_slots(mode):
     """(static_value key, field) of every calibration statistic the layer returns, in the reference's
     order (…intra_inter.py:277-282; the intra file adds gelu(up), :296)."""
+    if mode == "baseline":
+        return []
     slots = [("x", "scale"), ("q", "scale"), ("k", "scale"), ("v", "scale"), ("a", "outlier"), ("o", "scale"),
              ("o_final", "outlier_channel_index"), ("o_final", "scale"), ("x_medium", "scale"), ("up", "scale")]
     if mode == "intra":
@@ -60,17 +64,25 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
         it, thd, sv = iteration, iteration_threshold, static_value
         calib = it < thd
         saved, stats = {}, {}
+        raw = mode == "baseline"
+        whole = mode in ("baseline", "intra")
 
         def proj(name, inp):
             w, b, qs, la, lb = W[name]
             return lora_forward(w, qs, la, lb, b, inp)
 
         def quant(name, t, key=None):
+            if raw:
+                saved[name + "_raw"] = t
+                return
             q, s = compression_pack_quant_base(t, q_bit, 'per-channel', it, thd, sv[key or name])
             stats[(key or name, "scale")] = s
             saved[name + "_q"], saved[name + "_s"] = q, s
 
         def channel_base(name, t):
+            if raw:
+                saved[name + "_raw"] = t
+                return
             o, q, idx, s = compression_pack_channel_base(t, layernorm_outlier_ratio, q_bit, 'per-channel', it, thd,
                                                          sv[name])
             stats[(name, "outlier_channel_index")], stats[(name, "scale")] = idx, s
@@ -87,7 +99,7 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
             quant("v_main", v_main, "v")
         del q_main, k_main, v_main
         q, k, v = (hidden_to_head_shape(t, num_heads) for t in (q, k, v))
-        if mode == "intra":
+        if whole:
             quant("q", q)
             quant("k", k)
         s = q @ k.transpose(-2, -1)
@@ -99,7 +111,7 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
             if m is not None and m.shape[2] == 1:                # padding mask [B,1,1,S]: one row for all queries
                 m = m.expand(m.shape[0], 1, s.shape[2], s.shape[3])
             seg = None
-            if calib:
+            if calib or raw:
                 a = softmax_forward(s, 1.0 / math.sqrt(head_dim), m, inplace=True)
             else:
                 a, seg = softmax_forward(s, 1.0 / math.sqrt(head_dim), m, threshold=sv['a']['outlier'], inplace=True)
@@ -111,12 +123,14 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
             a = torch.softmax(s, dim=-1, dtype=v.dtype)
         del s
         o = a @ v
-        thr = get_statistics_softmax(a, softmax_outlier_ratio) if calib else sv['a']['outlier']
-        stats[("a", "outlier")] = thr
-        saved["a_idx"], saved["a_val"], saved["a_seg"] = compress_attention_map(a, thr, seg)
-        ctx.a_shape = tuple(a.shape)
+        if raw:
+            saved["a_raw"] = a
+        else:
+            thr = get_statistics_softmax(a, softmax_outlier_ratio) if calib else sv['a']['outlier']
+            stats[("a", "outlier")] = thr
+            saved["a_idx"], saved["a_val"], saved["a_seg"] = compress_attention_map(a, thr, seg)
         del a
-        if mode == "intra":
+        if whole:
             quant("v", v)
         del v
         o = head_to_hidden_shape(o)
@@ -137,12 +151,12 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
             quant("up_main", up_main, "up")
         del up_main
         fn = torch.nn.functional.gelu(up)
-        if mode == "intra":
+        if whole:
             quant("up", up)
         del up
         down, _, saved["down_lora_a"] = proj("down", fn)
         down += x_medium
-        if mode == "intra":
+        if whole:
             quant("fn", fn)
         del fn, x_medium
         x_out, saved["mean_2"], saved["rstd_2"], block_size, num_warps = layernorm_forward(down, norm_weight_2, norm_bias_2, _EPS)
@@ -171,9 +185,13 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
         G = {}
 
         def deq(name, **kw):
+            if name + "_raw" in S:
+                return S[name + "_raw"]
             return decompression_dequantization(S[name + "_q"], S[name + "_s"], q_bit, **kw)
 
         def deq_cb(name):
+            if name + "_raw" in S:
+                return S[name + "_raw"]
             return outlier_addition_fuse_decompression_dequantization(S[name + "_q"], S[name + "_s"], S[name + "_o"],
                                                                       S[name + "_idx"], q_bit)
 
@@ -189,7 +207,8 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
         grad_output = grad_output.to(torch.bfloat16)
         grad_ln2, _, _ = layernorm_backward(grad_output, deq_cb("down"), nw2, nb2, S["mean_2"], S["rstd_2"], True, _EPS,
                                             ctx.num_warps, ctx.block_size)
-        if mode == "intra":
+        whole = mode in ("baseline", "intra")
+        if whole:
             fn, up = deq("fn"), deq("up")
         else:
             up = rebuilt("up")
@@ -206,18 +225,22 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
         del grad_medium
         grad_o = hidden_to_head_shape(back("o", deq("o"), S["o_lora_a"], grad_ln1), H)
 
-        if mode == "intra":
+        if whole:
             v = deq("v", is_head=True, num_heads=H)
         else:
             v = hidden_to_head_shape(rebuilt("v"), H)
         grad_a = grad_o @ v.transpose(-2, -1)
         del v
-        a, grad_s = softmax_backward_from_compressed(S["a_idx"], S["a_val"], S["a_seg"], grad_a,
-                                                     out_scale=1.0 / math.sqrt(D))
+        if "a_raw" in S:
+            a = S["a_raw"]
+            grad_s = softmax_backward(a, grad_a) / math.sqrt(D)
+        else:
+            a, grad_s = softmax_backward_from_compressed(S["a_idx"], S["a_val"], S["a_seg"], grad_a,
+                                                         out_scale=1.0 / math.sqrt(D))
         del grad_a
         grad_v = a.transpose(-2, -1) @ grad_o
         del a, grad_o
-        if mode == "intra":
+        if whole:
             q, k = deq("q", is_head=True, num_heads=H), deq("k", is_head=True, num_heads=H)
         else:
             q, k = hidden_to_head_shape(rebuilt("q"), H), hidden_to_head_shape(rebuilt("k"), H)
@@ -238,7 +261,7 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
                 *five("up"), *five("down"), None, None) + (None,) * 10
 
 
-class FusedRobertaLayer(torch.nn.Module):
+class _FusedRobertaLayerBase(torch.nn.Module):
     """Module wrapper: owns the calibration state and feeds the Function.  Same call signature as the
     reference's modules (…intra_inter.py:538-568); the state travels with state_dict()."""
 
@@ -259,10 +282,12 @@ class FusedRobertaLayer(torch.nn.Module):
     def set_hyclora_config(self, hyclora_config):
         self.hyclora_config = hyclora_config
         self.use_hyclora = hyclora_config.use_hyclora
-        self.iteration_threshold = hyclora_config.iteration_threshold
-        self.softmax_outlier_ratio = hyclora_config.softmax_outlier_ratio
-        self.layernorm_outlier_ratio = hyclora_config.layernorm_outlier_ratio
-        self.q_bit = hyclora_config.q_bit
+        # the uncompressed layer reads none of the compression settings (…baseline.py keeps only
+        # use_hyclora and the config itself)
+        self.iteration_threshold = getattr(hyclora_config, "iteration_threshold", 0)
+        self.softmax_outlier_ratio = getattr(hyclora_config, "softmax_outlier_ratio", 0.0)
+        self.layernorm_outlier_ratio = getattr(hyclora_config, "layernorm_outlier_ratio", 0.0)
+        self.q_bit = getattr(hyclora_config, "q_bit", 0)
 
     def get_extra_state(self):
         return {"iteration": int(self.iteration),
@@ -316,15 +341,24 @@ class FusedRobertaLayer(torch.nn.Module):
         return y
 
 
-class FusedRobertaLayerIntra(FusedRobertaLayer):
+class FusedRobertaLayer(_FusedRobertaLayerBase):
+    """The uncompressed layer; the reference gives it the bare name (fused_roberta_layer_baseline.py)."""
+    layer_type = "baseline"
+
+
+FusedRobertaLayerBaseline = FusedRobertaLayer
+
+
+class FusedRobertaLayerIntra(_FusedRobertaLayerBase):
     layer_type = "intra"
 
 
-class FusedRobertaLayerIntraInter(FusedRobertaLayer):
+class FusedRobertaLayerIntraInter(_FusedRobertaLayerBase):
     layer_type = "intra_inter"
 
 
-LAYER_TYPES = {"intra": FusedRobertaLayerIntra, "intra_inter": FusedRobertaLayerIntraInter}
+LAYER_TYPES = {"baseline": FusedRobertaLayer, "intra": FusedRobertaLayerIntra,
+               "intra_inter": FusedRobertaLayerIntraInter}
 
 
 def make_fused_roberta_layer(hyclora_config):

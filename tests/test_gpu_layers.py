@@ -145,6 +145,37 @@ def test_layer_matches_uncompressed_autograd(dev, layer_type, q_bit, family):
         assert cos >= COS_FLOOR[q_bit], f"{layer_type} q{q_bit} grad {name}: rel {rel:.2e} cos {cos:.5f}"
 
 
+@pytest.mark.parametrize("family", ["llama", "mistral", "llama_flash_attn"])
+def test_baseline_layer_is_the_uncompressed_layer(dev, family):
+    """layer_type 'baseline' (the reference's default, models/llama/fused_llama_layer_baseline.py)
+    keeps its activations uncompressed: its hand-written backward must agree with autograd of the
+    same bf16 graph to bf16 rounding, gradient by gradient, and it needs none of the compression
+    settings."""
+    import hyclora_amd  # noqa: F401
+    from hyclora_amd.models import llama, llama_flash_attn, mistral
+    kv = 2 if family == "mistral" else 4
+    t = make_layer_inputs(dev, seed=77, kv_heads=kv)
+    cls = {"llama": llama.FusedLlamaLayerBaseline, "mistral": mistral.FusedMistralLayerBaseline,
+           "llama_flash_attn": llama_flash_attn.FusedLlamaLayerBaseline}[family]
+    layer = cls()
+    layer.set_hyclora_config(SimpleNamespace(use_hyclora=True, layer_type="baseline"))
+    if family != "llama_flash_attn":
+        assert type(layer) is {"llama": llama, "mistral": mistral}[family].LAYER_TYPES["baseline"]
+    ref_out = reference_layer(t)
+    ref_grads = grads_of(t, ref_out)
+    out = run_fused(layer, t)
+    assert layer.iteration == 1 and layer.static_value == {}
+    rel, cos = rel_err_and_cos(out, ref_out)
+    assert rel <= 1e-2 and cos >= 0.9999, f"forward: rel {rel:.2e} cos {cos:.6f}"
+    grads = grads_of(t, out)
+    names = ["x", "norm_w1", "norm_w2"] + [f"{n}.lora_{ab}" for n in ("q", "k", "v", "o", "gate", "up", "down") for ab in "AB"]
+    for name, g, gr in zip(names, grads, ref_grads):
+        if name.startswith("norm_w") and g is None:
+            continue
+        rel, cos = rel_err_and_cos(g, gr)
+        assert rel <= 2e-2 and cos >= 0.9999, f"{family} baseline grad {name}: rel {rel:.2e} cos {cos:.6f}"
+
+
 @pytest.mark.parametrize("layer_type", ["intra", "intra_inter", "intra_inter_full_fuse"])
 @pytest.mark.parametrize("q_bit", [8, 4, 2])
 @pytest.mark.parametrize("kv_heads", [4, 2])

@@ -121,6 +121,26 @@ def test_roberta_layer_close_to_uncompressed_autograd(dev, layer_type):
         assert cos >= 0.9, f"{layer_type} grad #{i}: rel {rel:.2e} cos {cos:.5f}"    # sanity bound only: the scheme (step from batch element 0, no zero point) clips; parity is the oracle test above
 
 
+@pytest.mark.parametrize("padding", [True, False])
+def test_roberta_baseline_layer_is_the_uncompressed_layer(dev, padding):
+    """The reference's default encoder layer (models/roberta/fused_roberta_layer_baseline.py, class
+    FusedRobertaLayer) saves its activations as they are: hand-written backward == autograd of the
+    same bf16 graph to bf16 rounding."""
+    import hyclora_amd  # noqa: F401
+    from hyclora_amd.models import roberta
+    t = make_inputs(dev, seed=51, padding=padding)
+    ref_out = reference_layer(t)
+    ref_grads = grads_of(t, ref_out)
+    layer = roberta.make_fused_roberta_layer(SimpleNamespace(use_hyclora=True, layer_type="baseline"))
+    assert type(layer) is roberta.FusedRobertaLayer
+    out = run_fused(layer, t)
+    rel, cos = rel_err_and_cos(out, ref_out)
+    assert rel <= 2e-2 and cos >= 0.9999
+    for i, (got, want) in enumerate(zip(grads_of(t, out), ref_grads)):
+        rel, cos = rel_err_and_cos(got, want)
+        assert rel <= 2e-2 and cos >= 0.9999, f"baseline grad #{i}: rel {rel:.2e} cos {cos:.6f}"
+
+
 def test_roberta_calibration_freezes_and_paths_agree(dev, tmp_path):
     import hyclora_amd  # noqa: F401
     from hyclora_amd.models import roberta
