@@ -115,5 +115,6 @@ __host__ __device__ inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 
 // file, 1 if it does not.
 int tune_quant(const char* key, int value);
 int tune_fuse(const char* key, int value);
+int tune_add(const char* key, int value);
 
 }  // namespace hyc

@@ -1,0 +1,211 @@
+// LoRA add around the compressed copy of a projection's frozen part, for gfx950.
+//
+//   plain    :  y = bf16(x + bf16(xa . b))                                   (x may be y: in place)
+//   quantise :  q = pack(code(x; s [, z])),  y as above    - x is read once for both
+//   restore  :  x = DQ(q; s [, z]),          y as above    - the dense x never reaches memory
+//
+// The reference does each of these in three to four passes over [T, N]: the LoRA product
+// written out, the quantiser (or dequantiser), and the add
+// (models/utils/compute_utils.py:21-24 with fused_llama_layer_intra_inter_full_fuse.py:128-140
+// in forward, :416-417, :439-441, :447-449 in backward; compute_utils.py:34-35 for the same add
+// on the input gradient).  Here the rank-R product is an MFMA tile held in registers
+// (hyc_lora_tile.hpp) and each kernel moves its algorithmic bytes once: 4, 4 + q/8 and
+// 2 + q/8 bytes per element.
+#include "hyc_lora_tile.hpp"
+
+namespace hyc {
+
+constexpr int kAddThreads = 256;
+constexpr int kAddWaves = kAddThreads / kWave;
+static int g_add_rows_per_wave = 32;
+
+enum { kAddPlain = 0, kAddQuant = 1, kAddRestore = 2 };
+
+struct LoraAddArgs {
+    const uint16_t* xa; const uint16_t* b;
+    const uint16_t* s; const uint16_t* zp;      // steps / zero points bf16 [N] (quantise, restore)
+    const uint16_t* x;                          // dense input (plain, quantise)
+    uint8_t* q;                                 // packed codes: output of quantise, input of restore
+    uint16_t* y;
+    int64_t T;
+    int N, C, R;
+    int rows_per_wave, col_tiles;
+};
+
+template <int QBIT, int KSTEPS, int MODE, bool ZP, bool FAST>
+__device__ __forceinline__ void lora_add_rows(const LoraAddArgs& a, int64_t row_begin, int64_t row_end, int lane,
+                                              int chunk, bool active, const QuantCols<QBIT>& qc, const float (&z)[8],
+                                              const BOperand<KSTEPS>& B) {
+    const int g = lane >> 4;
+    const int col0 = chunk * 8;
+    const int row_bytes = a.N * QBIT / 8;
+    constexpr float kHalf = (float)(1 << (QBIT - 1));
+    const PackedSlot<QBIT> slot(chunk);
+    for (int64_t row0 = row_begin; row0 < row_end; row0 += kTileRows) {
+        u32x4 xv[4];
+        u32x2 w[4];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int64_t t = row0 + 4 * g + v;
+            xv[v] = u32x4{0, 0, 0, 0};
+            w[v] = u32x2{0, 0};
+            if (active && t < row_end) {
+                if constexpr (MODE == kAddRestore) w[v] = ld8(a.q + t * row_bytes + slot.offset);
+                else xv[v] = ld16_nt(a.x + t * a.N + col0);
+            }
+        }
+        uint32_t L[4][4];
+        lora_tile_bf16<KSTEPS>(a.xa, a.R, row0, row_end, lane, B, L);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int64_t t = row0 + 4 * g + v;
+            const bool live = active && t < row_end;
+            float f[8], y[8];
+            if constexpr (MODE == kAddRestore) {
+                float c[8];
+                slot.decode(w[v], c);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    if constexpr (ZP) f[j] = rbf(rbf((c[j] - kHalf) - z[j]) * qc.s[j]);
+                    else f[j] = rbf((c[j] - kHalf) * qc.s[j]);
+                }
+            } else {
+                unpack8(xv[v], f);
+            }
+            if constexpr (MODE == kAddQuant) {
+                uint32_t lo, hi;
+                // rows past the end still take part in the quad exchange; their stores are masked
+                const int64_t tq = t < row_end ? t : row_end - 1;
+                codes_to_words<QBIT, ZP, FAST>(f, qc, z, lo, hi);
+                store_packed<QBIT, true>(a.q + tq * row_bytes, chunk, live, lo, hi);
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) y[j] = f[j] + lora_elem(L[v], j);
+            if (live) st16_nt(a.y + t * a.N + col0, pack8(y));
+        }
+    }
+}
+
+template <int QBIT, int KSTEPS, int MODE, bool ZP>
+__global__ __launch_bounds__(kAddThreads) void lora_add_kernel(const LoraAddArgs a) {
+    constexpr int CT = MODE == kAddPlain ? 1 : kColTilesPerGroup<QBIT>, RS = kAddWaves / CT;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int col_tile = (blockIdx.x % a.col_tiles) * CT + wave % CT;     // a.col_tiles counts groups of CT tiles
+    const int64_t row_tile = blockIdx.x / a.col_tiles;
+    const int chunk = col_tile * (kTileCols / 8) + (lane & 15);
+    const bool active = chunk < a.C;
+    const int col0 = chunk * 8;
+
+    QuantCols<QBIT> qc;
+    float z[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    if constexpr (MODE == kAddQuant) {
+        qc.load(a.s, col0, active);
+    } else if constexpr (MODE == kAddRestore) {
+        u32x4 sv = {0, 0, 0, 0};
+        if (active) sv = ld16(a.s + col0);
+        unpack8(sv, qc.s);
+        qc.fast = false;
+    }
+    if constexpr (ZP) {
+        if (active) unpack8(ld16(a.zp + col0), z);
+    }
+    BOperand<KSTEPS> B;
+    B.load(a.b, a.N, a.R, col0, active, lane >> 4);
+
+    const int64_t row_begin = (row_tile * RS + wave / CT) * (int64_t)a.rows_per_wave;
+    int64_t row_end = row_begin + a.rows_per_wave;
+    if (row_end > a.T) row_end = a.T;
+    if (row_begin >= row_end) return;
+    if constexpr (MODE == kAddQuant && !ZP) {
+        if (__ballot(!qc.fast) == 0ull) {
+            lora_add_rows<QBIT, KSTEPS, MODE, ZP, true>(a, row_begin, row_end, lane, chunk, active, qc, z, B);
+            return;
+        }
+    }
+    lora_add_rows<QBIT, KSTEPS, MODE, ZP, false>(a, row_begin, row_end, lane, chunk, active, qc, z, B);
+}
+
+// ------------------------------------------------------------------------------------
+template <int QB, int MODE, bool ZP>
+static void add_launch_k(const LoraAddArgs& a, dim3 grid, int ksteps, hipStream_t st) {
+    const dim3 block(kAddThreads);
+    if (ksteps == 1) hipLaunchKernelGGL((lora_add_kernel<QB, 1, MODE, ZP>), grid, block, 0, st, a);
+    else if (ksteps == 2) hipLaunchKernelGGL((lora_add_kernel<QB, 2, MODE, ZP>), grid, block, 0, st, a);
+    else if (ksteps == 3) hipLaunchKernelGGL((lora_add_kernel<QB, 3, MODE, ZP>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((lora_add_kernel<QB, 4, MODE, ZP>), grid, block, 0, st, a);
+}
+
+template <int MODE>
+static int add_launch(LoraAddArgs& a, int64_t T, int64_t N, int64_t R, int q_bit, void* stream) {
+    if (MODE != kAddPlain && q_bit != 2 && q_bit != 4 && q_bit != 8) return HYC_ERR_QBIT;
+    if (T < 0 || N < 0 || N % 32 != 0 || N > (1 << 28) || T > ((int64_t)1 << 40)) return HYC_ERR_SHAPE;
+    if (R < 4 || R > 64 || R % 4 != 0) return HYC_ERR_RANK;
+    if (T * N == 0) return HYC_OK;
+    if (!a.xa || !a.b || !a.y) return HYC_ERR_NULL;
+    if (MODE != kAddRestore && !a.x) return HYC_ERR_NULL;
+    if (MODE != kAddPlain && (!a.q || !a.s)) return HYC_ERR_NULL;
+    if (!aligned16(a.b) || !aligned16(a.y) || (a.x && !aligned16(a.x)) || (a.s && !aligned16(a.s)) ||
+        (a.zp && !aligned16(a.zp)))
+        return HYC_ERR_ALIGN;
+    if ((reinterpret_cast<uintptr_t>(a.xa) & 7u) || (a.q && (reinterpret_cast<uintptr_t>(a.q) & 7u))) return HYC_ERR_ALIGN;
+    a.T = T;
+    a.N = (int)N;
+    a.C = (int)(N / 8);
+    a.R = (int)R;
+    a.rows_per_wave = g_add_rows_per_wave;
+    const int ct = MODE == kAddPlain ? 1 : 8 / q_bit;
+    a.col_tiles = (int)cdiv(cdiv(N, kTileCols), ct);
+    const int64_t row_tiles = cdiv(T, (int64_t)(kAddWaves / ct) * a.rows_per_wave);
+    if (row_tiles * a.col_tiles > INT32_MAX) return HYC_ERR_SHAPE;
+    const dim3 grid((unsigned)(row_tiles * a.col_tiles));
+    const int ksteps = (int)cdiv(R, 16);
+    hipStream_t st = (hipStream_t)stream;
+    if constexpr (MODE == kAddPlain) {
+        add_launch_k<8, MODE, false>(a, grid, ksteps, st);
+    } else {
+        const bool zp = a.zp != nullptr;
+        if (q_bit == 8) { if (zp) add_launch_k<8, MODE, true>(a, grid, ksteps, st); else add_launch_k<8, MODE, false>(a, grid, ksteps, st); }
+        else if (q_bit == 4) { if (zp) add_launch_k<4, MODE, true>(a, grid, ksteps, st); else add_launch_k<4, MODE, false>(a, grid, ksteps, st); }
+        else { if (zp) add_launch_k<2, MODE, true>(a, grid, ksteps, st); else add_launch_k<2, MODE, false>(a, grid, ksteps, st); }
+    }
+    return check_launch();
+}
+
+int tune_add(const char* key, int value) {
+    if (strcmp(key, "add_rows_per_wave") == 0) {
+        if (value < kTileRows || value > 65536 || value % kTileRows != 0) return HYC_ERR_ARG;
+        g_add_rows_per_wave = value;
+        return HYC_OK;
+    }
+    return 1;
+}
+
+}  // namespace hyc
+
+using namespace hyc;
+
+extern "C" int hyc_lora_add(const void* xa, const void* b, const void* x, void* y, int64_t T, int64_t N, int64_t R,
+                            void* stream) {
+    LoraAddArgs a{};
+    a.xa = (const uint16_t*)xa; a.b = (const uint16_t*)b; a.x = (const uint16_t*)x; a.y = (uint16_t*)y;
+    return add_launch<kAddPlain>(a, T, N, R, 8, stream);
+}
+
+extern "C" int hyc_lora_add_quant(const void* xa, const void* b, const void* x, const void* scale,
+                                  const void* zero_point, void* q, void* y, int64_t T, int64_t N, int64_t R,
+                                  int q_bit, void* stream) {
+    LoraAddArgs a{};
+    a.xa = (const uint16_t*)xa; a.b = (const uint16_t*)b; a.x = (const uint16_t*)x; a.y = (uint16_t*)y;
+    a.s = (const uint16_t*)scale; a.zp = (const uint16_t*)zero_point; a.q = (uint8_t*)q;
+    return add_launch<kAddQuant>(a, T, N, R, q_bit, stream);
+}
+
+extern "C" int hyc_lora_add_restore(const void* xa, const void* b, const void* q, const void* scale,
+                                    const void* zero_point, void* y, int64_t T, int64_t N, int64_t R, int q_bit,
+                                    void* stream) {
+    LoraAddArgs a{};
+    a.xa = (const uint16_t*)xa; a.b = (const uint16_t*)b; a.y = (uint16_t*)y;
+    a.s = (const uint16_t*)scale; a.zp = (const uint16_t*)zero_point; a.q = (uint8_t*)const_cast<void*>(q);
+    return add_launch<kAddRestore>(a, T, N, R, q_bit, stream);
+}

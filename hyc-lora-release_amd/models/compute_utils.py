@@ -4,6 +4,7 @@ torch operations in the reference as well; only what surrounds them is compresse
 in-place HIP kernel of operators/rope_kernels.py, re-exported here."""
 import torch
 
+from ..operators import lora_kernels
 from ..operators.nf4 import dequantize_nf4
 
 
@@ -27,14 +28,24 @@ def dense_weight(w: torch.Tensor, quant_state):
 
 
 def lora_forward(w, w_quant_state, w_lora_a, w_lora_b, b, x):
-    """-> (x @ W^T [+ b] + (x @ A) @ B, the frozen part alone, x @ A).  Reference :18-25."""
+    """-> (x @ W^T [+ b] + (x @ A) @ B, the frozen part alone, x @ A).  Reference :18-25.  The LoRA
+    product and the add are one MFMA kernel over the frozen part (bf16 operands); other dtypes
+    take the torch expression."""
+    x_main, x_lora_a = lora_parts(w, w_quant_state, w_lora_a, b, x)
+    w_lora_b = w_lora_b.to(x_main.dtype)
+    if lora_kernels.supported(x_main, x_lora_a, w_lora_b):
+        return lora_kernels.lora_add(x_main, x_lora_a, w_lora_b), x_main, x_lora_a
+    return x_main + x_lora_a @ w_lora_b, x_main, x_lora_a
+
+
+def lora_parts(w, w_quant_state, w_lora_a, b, x):
+    """-> (x @ W^T [+ b], x @ A): what lora_forward computes before the LoRA add."""
     wt = dense_weight(w, w_quant_state).t()
     x = x.to(wt.dtype)
     x_main = x @ wt
     if b is not None:
         x_main = x_main + b.to(wt.dtype)
-    x_lora_a = x @ w_lora_a.to(wt.dtype)
-    return x_main + x_lora_a @ w_lora_b.to(wt.dtype), x_main, x_lora_a
+    return x_main, x @ w_lora_a.to(wt.dtype)
 
 
 def lora_backward(w, w_quant_state, w_lora_a, w_lora_b, x, x_lora_a, grad_y):
@@ -47,7 +58,10 @@ def lora_backward(w, w_quant_state, w_lora_a, w_lora_b, x, x_lora_a, grad_y):
     grad_a = x.to(dt).mT @ grad_mid
     grad_b = x_lora_a.to(dt).mT @ grad_y
     grad_x = grad_y @ wd
-    grad_x += grad_mid @ w_lora_a.mT
+    if lora_kernels.supported(grad_x, grad_mid, w_lora_a.mT):
+        grad_x = lora_kernels.lora_add(grad_x, grad_mid, w_lora_a.mT, inplace=True)
+    else:
+        grad_x += grad_mid @ w_lora_a.mT
     return grad_a, grad_b, grad_x
 
 

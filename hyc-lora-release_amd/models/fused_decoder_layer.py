@@ -44,7 +44,8 @@ from ..operators.compress_function import (compress_attention_map, compression_p
                                            compression_pack_quant_base, compression_pack_quant_zp_base,
                                            decompression_dequantization,
                                            decompression_dequantization_with_zero_point,
-                                           get_statistics_only_quant, get_statistics_softmax,
+                                           get_statistics_only_quant, get_statistics_only_quant_zero_point,
+                                           get_statistics_softmax,
                                            outlier_addition_fuse_decompression_dequantization,
                                            update_dict)
 from ..operators.rmsnorm_kernels import _backward as _rmsnorm_backward
@@ -53,7 +54,8 @@ from ..operators.silu_kernels import silu_backward, silu_hadamard
 from ..operators.softmax_kernels import softmax_backward, softmax_backward_from_compressed, softmax_forward
 from ..operators.triton_fuse_lora_silu_hadamard_backward_kernels import triton_fuse_silu_backward
 from ..operators.triton_fuse_lora_silu_hadamard_forward_kernels import triton_fuse_silu_forward
-from .compute_utils import (head_to_hidden_shape, hidden_to_head_shape, lora_backward, lora_forward,
+from ..operators import lora_kernels
+from .compute_utils import (head_to_hidden_shape, hidden_to_head_shape, lora_backward, lora_forward, lora_parts,
                             repeat_kv, repeat_kv_backward, rope_backward, rope_forward)
 
 MODES = ("baseline", "intra", "intra_inter", "intra_inter_full_fuse")
@@ -124,6 +126,26 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             w, b, qs, la, lb = W[name]
             return lora_forward(w, qs, la, lb, b, inp)
 
+        def proj_quant(name, inp, zp=False):
+            """Projection `name` of inp with the frozen part quantised on the way: -> (output, x @ A).
+            One kernel reads the frozen part once, writes its codes and adds the LoRA product; the
+            reference quantises `*_main` and adds in separate passes (…full_fuse.py:105-140)."""
+            w, b, qs, la, lb = W[name]
+            main, xa = lora_parts(w, qs, la, b, inp)
+            lb = lb.to(main.dtype)
+            if not (lora_kernels.supported(main, xa, lb) and main.dim() == 3):
+                (quant_zp if zp else quant)(name + "_main", main, name)
+                return main + xa @ lb, xa
+            if zp:
+                s_, z_ = get_statistics_only_quant_zero_point(main, q_bit, 'per-channel') if calib else \
+                    (sv[name]['scale'], sv[name]['zero_point'])
+                stats[(name, "zero_point")] = saved[name + "_main_z"] = z_
+            else:
+                s_, z_ = get_statistics_only_quant(main, q_bit, 'per-channel') if calib else sv[name]['scale'], None
+            stats[(name, "scale")] = saved[name + "_main_s"] = s_
+            saved[name + "_main_q"], y = lora_kernels.lora_add_quant(main, xa, lb, s_, z_, q_bit, inplace=True)
+            return y, xa
+
         def quant(name, t, key=None):
             if raw:
                 saved[name + "_raw"] = t
@@ -169,21 +191,17 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
 
         # ---- attention block -------------------------------------------------------------------
         x_norm_1, saved["rstd_1"], norm_1_done = norm_block("x", "x_norm_1", x, norm_weight_1)
-        q, q_main, saved["q_lora_a"] = proj("q", x_norm_1)
-        k, k_main, saved["k_lora_a"] = proj("k", x_norm_1)
-        v, v_main, saved["v_lora_a"] = proj("v", x_norm_1)
+        if whole:
+            q, _, saved["q_lora_a"] = proj("q", x_norm_1)
+            k, _, saved["k_lora_a"] = proj("k", x_norm_1)
+            v, _, saved["v_lora_a"] = proj("v", x_norm_1)
+        else:
+            q, saved["q_lora_a"] = proj_quant("q", x_norm_1, zp=spec.attention == "sdpa")
+            k, saved["k_lora_a"] = proj_quant("k", x_norm_1, zp=spec.attention == "sdpa")
+            v, saved["v_lora_a"] = proj_quant("v", x_norm_1)
         if not norm_1_done:
             quant("x_norm_1", x_norm_1)
         del x_norm_1
-        if not whole:
-            if spec.attention == "sdpa":
-                quant_zp("q_main", q_main, "q")
-                quant_zp("k_main", k_main, "k")
-            else:
-                quant("q_main", q_main, "q")
-                quant("k_main", k_main, "k")
-            quant("v_main", v_main, "v")
-        del q_main, k_main, v_main
 
         q = hidden_to_head_shape(q, num_heads)
         k = hidden_to_head_shape(k, num_key_value_heads)
@@ -258,20 +276,20 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             saved.update(gate_main_q=gate_q, gate_main_s=gate_s, up_main_q=up_q, up_main_s=up_s)
             del gate_main, up_main
         else:
-            gate, gate_main, gate_lora_a = proj("gate", x_norm_2)
-            up, up_main, up_lora_a = proj("up", x_norm_2)
             if spec.mode == "intra_inter":
-                quant("gate_main", gate_main, "gate")
-                quant("up_main", up_main, "up")
+                gate, gate_lora_a = proj_quant("gate", x_norm_2)
+                up, up_lora_a = proj_quant("up", x_norm_2)
                 hadamard = silu_hadamard(gate, up)
             else:                                           # 'intra' and 'baseline'
+                gate, _, gate_lora_a = proj("gate", x_norm_2)
+                up, _, up_lora_a = proj("up", x_norm_2)
                 fn = F.silu(gate)
                 quant("gate", gate)
                 hadamard = up * fn
                 quant("up", up)
                 quant("fn", fn)
                 del fn
-            del gate, up, gate_main, up_main
+            del gate, up
         saved["gate_lora_a"], saved["up_lora_a"] = gate_lora_a, up_lora_a
         if not norm_2_done:
             quant("x_norm_2", x_norm_2)
@@ -323,8 +341,16 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             G[name] = (ga, gb)
             return gx
 
-        def lora_part(name):
-            return S[name + "_lora_a"] @ W[name][4].to(S[name + "_lora_a"].dtype)
+        def rebuilt_hidden(name):
+            """Output of projection `name` as forward produced it, from the codes of its frozen part
+            and the saved x @ A: dequantise + LoRA add in one kernel (…full_fuse.py:416-417,439-449)."""
+            xa, lb = S[name + "_lora_a"], W[name][4]
+            lb = lb.to(xa.dtype)
+            q_, s_, z_ = S[name + "_main_q"], S[name + "_main_s"], S.get(name + "_main_z")
+            if lora_kernels.supported_restore(q_, xa, lb):
+                return lora_kernels.lora_add_restore(q_, s_, xa, lb, z_, q_bit)
+            main = deq(name + "_main")
+            return main + (xa @ lb).to(main.dtype)
 
         def channel_base_restored(name):
             if name + "_raw" in S:
@@ -353,8 +379,7 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             del hadamard, grad_down
         else:
             if spec.mode == "intra_inter":
-                gate = deq("gate_main") + lora_part("gate")
-                up = deq("up_main") + lora_part("up")
+                gate, up = rebuilt_hidden("gate"), rebuilt_hidden("up")
                 fn = F.silu(gate)
                 hadamard = up * fn
             else:
@@ -380,8 +405,7 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
 
         def rebuilt(name, heads):
             """q/k/v in head shape as the forward attention saw them (before repeat_kv)."""
-            main = deq(name + "_main")
-            t = hidden_to_head_shape(main + lora_part(name).to(main.dtype), heads)
+            t = hidden_to_head_shape(rebuilt_hidden(name), heads)
             if name != "v":
                 t = rope_forward(t.transpose(1, 2), cos, sin).transpose(1, 2)
             return t

@@ -16,12 +16,13 @@ import torch
 
 from ..operators.compress_function import (compress_attention_map, compression_pack_channel_base,
                                            compression_pack_quant_base, decompression_dequantization,
-                                           get_statistics_softmax,
+                                           get_statistics_only_quant, get_statistics_softmax,
                                            outlier_addition_fuse_decompression_dequantization, update_dict)
 from ..operators.gelu_kernels import gelu_backward
 from ..operators.layernorm_kernels import layernorm_backward, layernorm_forward
 from ..operators.softmax_kernels import softmax_backward, softmax_backward_from_compressed, softmax_forward
-from .compute_utils import head_to_hidden_shape, hidden_to_head_shape, lora_backward, lora_forward
+from ..operators import lora_kernels
+from .compute_utils import head_to_hidden_shape, hidden_to_head_shape, lora_backward, lora_forward, lora_parts
 
 MODES = ("baseline", "intra", "intra_inter")
 _PROJ = ("q", "k", "v", "o", "up", "down")
@@ -71,6 +72,20 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
             w, b, qs, la, lb = W[name]
             return lora_forward(w, qs, la, lb, b, inp)
 
+        def proj_quant(name, inp):
+            """Projection with the frozen part quantised on the way, one kernel for codes + LoRA add
+            (the reference: separate passes, …intra_inter.py:90-121) -> (output, x @ A)."""
+            w, b, qs, la, lb = W[name]
+            main, xa = lora_parts(w, qs, la, b, inp)
+            lb = lb.to(main.dtype)
+            if not (lora_kernels.supported(main, xa, lb) and main.dim() == 3):
+                quant(name + "_main", main, name)
+                return main + xa @ lb, xa
+            s_ = get_statistics_only_quant(main, q_bit, 'per-channel') if calib else sv[name]['scale']
+            stats[(name, "scale")] = saved[name + "_main_s"] = s_
+            saved[name + "_main_q"], y = lora_kernels.lora_add_quant(main, xa, lb, s_, None, q_bit, inplace=True)
+            return y, xa
+
         def quant(name, t, key=None):
             if raw:
                 saved[name + "_raw"] = t
@@ -89,15 +104,15 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
             saved[name + "_o"], saved[name + "_q"], saved[name + "_s"], saved[name + "_idx"] = o, q, s, idx
 
         # ---- attention block -------------------------------------------------------------------
-        q, q_main, saved["q_lora_a"] = proj("q", x)
-        k, k_main, saved["k_lora_a"] = proj("k", x)
-        v, v_main, saved["v_lora_a"] = proj("v", x)
+        if whole:
+            q, _, saved["q_lora_a"] = proj("q", x)
+            k, _, saved["k_lora_a"] = proj("k", x)
+            v, _, saved["v_lora_a"] = proj("v", x)
+        else:
+            q, saved["q_lora_a"] = proj_quant("q", x)
+            k, saved["k_lora_a"] = proj_quant("k", x)
+            v, saved["v_lora_a"] = proj_quant("v", x)
         quant("x", x)
-        if mode == "intra_inter":
-            quant("q_main", q_main, "q")
-            quant("k_main", k_main, "k")
-            quant("v_main", v_main, "v")
-        del q_main, k_main, v_main
         q, k, v = (hidden_to_head_shape(t, num_heads) for t in (q, k, v))
         if whole:
             quant("q", q)
@@ -145,11 +160,11 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
         del o_final
 
         # ---- MLP block ---------------------------------------------------------------------------
-        up, up_main, saved["up_lora_a"] = proj("up", x_medium)
+        if whole:
+            up, _, saved["up_lora_a"] = proj("up", x_medium)
+        else:
+            up, saved["up_lora_a"] = proj_quant("up", x_medium)
         quant("x_medium", x_medium)
-        if mode == "intra_inter":
-            quant("up_main", up_main, "up")
-        del up_main
         fn = torch.nn.functional.gelu(up)
         if whole:
             quant("up", up)
@@ -201,8 +216,12 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
             return gx
 
         def rebuilt(name):
+            xa, lb = S[name + "_lora_a"], W[name][3]
+            lb = lb.to(xa.dtype)
+            if lora_kernels.supported_restore(S[name + "_main_q"], xa, lb):
+                return lora_kernels.lora_add_restore(S[name + "_main_q"], S[name + "_main_s"], xa, lb, None, q_bit)
             main = deq(name + "_main")
-            return main + S[name + "_lora_a"].to(main.dtype) @ W[name][3].to(main.dtype)
+            return main + xa.to(main.dtype) @ lb.to(main.dtype)
 
         grad_output = grad_output.to(torch.bfloat16)
         grad_ln2, _, _ = layernorm_backward(grad_output, deq_cb("down"), nw2, nb2, S["mean_2"], S["rstd_2"], True, _EPS,

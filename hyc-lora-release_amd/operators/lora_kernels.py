@@ -1,0 +1,107 @@
+"""LoRA add fused with the compression of a projection's frozen part (gfx950 MFMA kernels).
+
+No counterpart module in the reference: it computes `x_main + x_lora_a @ w_lora_b`
+(models/utils/compute_utils.py:21-24), quantises `x_main` with a separate call
+(models/llama/fused_llama_layer_intra_inter_full_fuse.py:128-140) and in backward dequantises and
+adds again (:416-417, :439-441, :447-449), each step a pass over the tensor.  The functions here give
+the same tensors, bit for bit, from one pass each."""
+import torch
+
+from .. import _lib
+from ._fuse import _prep
+
+BF16 = torch.bfloat16
+
+
+def _check(xa, b, n):
+    r = b.shape[0]
+    if xa.shape[-1] != r:
+        raise ValueError(f"LoRA rank mismatch: x@A has {xa.shape[-1]} columns, B has {r} rows")
+    if b.shape[1] != n:
+        raise ValueError(f"LoRA-B width {b.shape[1]} does not match the activation width {n}")
+    if n % 32:
+        raise ValueError(f"channel count must be a multiple of 32, got {n}")
+    if r % 4 or not 4 <= r <= 64:
+        raise ValueError(f"LoRA rank must be a multiple of 4 in 4..64, got {r}")
+    return r
+
+
+def _operands_ok(xa, b):
+    n, r = b.shape[1], b.shape[0]
+    return (xa.is_cuda and xa.dtype == BF16 and b.dtype == BF16 and xa.shape[-1] == r
+            and n % 32 == 0 and r % 4 == 0 and 4 <= r <= 64 and xa.numel() > 0)
+
+
+def supported(x_main, xa, b):
+    """Whether lora_add / lora_add_quant take these operands (bf16, rank and width within the
+    kernels' limits)."""
+    return x_main.is_cuda and x_main.dtype == BF16 and x_main.shape[-1] == b.shape[1] and _operands_ok(xa, b)
+
+
+def supported_restore(q, xa, b):
+    """The same for lora_add_restore (q: packed codes uint8 [B, M, N*bits/8])."""
+    return q.is_cuda and q.dtype == torch.uint8 and q.dim() == 3 and _operands_ok(xa, b)
+
+
+def lora_add(x_main, xa, b, inplace=False):
+    """bf16(x_main + bf16(xa @ b)); `inplace` overwrites x_main (contiguous bf16) and returns it."""
+    _lib.require_gpu(x_main, xa, b)
+    n = x_main.shape[-1]
+    r = _check(xa, b, n)
+    x = x_main if (inplace and x_main.dtype == BF16 and x_main.is_contiguous() and x_main.data_ptr() % 16 == 0) \
+        else _prep(x_main, "x_main")
+    y = x if inplace else torch.empty_like(x)
+    xa, b = _prep(xa, "xa"), _prep(b, "b")
+    _lib.call("hyc_lora_add", xa.data_ptr(), b.data_ptr(), x.data_ptr(), y.data_ptr(), x.numel() // n, n, r,
+              _lib.stream_of(x))
+    if inplace and y is not x_main:
+        x_main.copy_(y)
+        return x_main
+    return y
+
+
+def _vec(t, n, name):
+    t = t.to(BF16).reshape(-1)
+    if t.numel() != n:
+        raise ValueError(f"{name} must have {n} elements (one per channel), got {t.numel()}")
+    return _prep(t, name)
+
+
+def lora_add_quant(x_main, xa, b, scale, zero_point=None, quantize_bit=8, inplace=False):
+    """-> (q, y): q = the packed codes compression_quantization[_with_zero_point](x_main, scale[, zero_point])
+    returns, y = bf16(x_main + bf16(xa @ b)); x_main [B, M, N] is read once."""
+    if quantize_bit not in (2, 4, 8):
+        raise ValueError(f"quantize_bit must be 2, 4 or 8, got {quantize_bit}")
+    _lib.require_gpu(x_main, xa, b, scale, zero_point)
+    B, M, n = x_main.shape
+    r = _check(xa, b, n)
+    x = _prep(x_main, "x_main")
+    y = x if (inplace and x is x_main) else torch.empty_like(x)
+    xa, b = _prep(xa, "xa"), _prep(b, "b")
+    s = _vec(scale, n, "scale")
+    z = None if zero_point is None else _vec(zero_point, n, "zero point")
+    q = torch.empty((B, M, n * quantize_bit // 8), device=x.device, dtype=torch.uint8)
+    _lib.call("hyc_lora_add_quant", xa.data_ptr(), b.data_ptr(), x.data_ptr(), s.data_ptr(), _lib.ptr(z),
+              q.data_ptr(), y.data_ptr(), B * M, n, r, quantize_bit, _lib.stream_of(x))
+    return q, y
+
+
+def lora_add_restore(q, scale, xa, b, zero_point=None, quantize_bit=8):
+    """bf16(decompression_dequantization[_with_zero_point](q, scale[, zero_point]) + bf16(xa @ b)) without
+    writing the dequantised tensor."""
+    if quantize_bit not in (2, 4, 8):
+        raise ValueError(f"quantize_bit must be 2, 4 or 8, got {quantize_bit}")
+    _lib.require_gpu(q, scale, xa, b, zero_point)
+    B, M, nbytes = q.shape
+    n = scale.shape[-1]
+    if nbytes * 8 != n * quantize_bit or q.dtype != torch.uint8:
+        raise ValueError(f"packed codes must be uint8 of width {n * quantize_bit // 8}, got {q.dtype} {nbytes}")
+    r = _check(xa, b, n)
+    q = q.contiguous()
+    xa, b = _prep(xa, "xa"), _prep(b, "b")
+    s = _vec(scale, n, "scale")
+    z = None if zero_point is None else _vec(zero_point, n, "zero point")
+    y = torch.empty((B, M, n), device=q.device, dtype=BF16)
+    _lib.call("hyc_lora_add_restore", xa.data_ptr(), b.data_ptr(), q.data_ptr(), s.data_ptr(), _lib.ptr(z),
+              y.data_ptr(), B * M, n, r, quantize_bit, _lib.stream_of(q))
+    return y

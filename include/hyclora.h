@@ -381,6 +381,35 @@ int hyc_lora_silu_mul_bwd(const void *xa1, const void *b1, const void *q1, const
                           const void *grad_o, void *o, void *grad_gate, void *grad_up,
                           int64_t T, int64_t N, int64_t R, int q_bit, void *stream);
 
+/* ---------------------------------------------------------------------------------------
+ * LoRA add around the compressed copy of a projection's frozen part:
+ *     hyc_lora_add          y = bf16(x + bf16(xa . b))                     (y may be x: in place)
+ *     hyc_lora_add_quant    the same y, and q = pack(code(x; scale [, zero_point])) from the one
+ *                           read of x (code rule and layout of hyc_quant_pack)
+ *     hyc_lora_add_restore  x = value of hyc_unpack_dequant(q; scale [, zero_point]), then the
+ *                           same y; the dense x is never written
+ * bit-identical to the separate steps.
+ *
+ * Replaces the product, the add and the quantiser / dequantiser call between them:
+ * lora_forward (models/utils/compute_utils.py:21-24) with compression_pack_quant_base on the
+ * frozen part (models/llama/fused_llama_layer_intra_inter_full_fuse.py:128-140; zero-point form
+ * models/llama_flash_attn/fused_llama_layer_intra_inter.py:129-138); the rebuild of q, k, v, gate,
+ * up in backward (…full_fuse.py:416-417, :439-441, :447-449); and `grad_x += grad_medium @ A^T`
+ * of lora_backward (compute_utils.py:34-35) through the plain form.
+ *   xa bf16 [T, R] contiguous;  b bf16 [R, N] contiguous;  x, y bf16 [T, N] contiguous;
+ *   scale, zero_point bf16 [N] (zero_point NULL: symmetric codes);  q uint8 [T, N*q_bit/8].
+ *   R: multiple of 4, 4..64; N % 32 == 0; any T.
+ * Tuning key "add_rows_per_wave" (multiple of 16, default 32).
+ */
+int hyc_lora_add(const void *xa, const void *b, const void *x, void *y, int64_t T, int64_t N, int64_t R,
+                 void *stream);
+int hyc_lora_add_quant(const void *xa, const void *b, const void *x, const void *scale,
+                       const void *zero_point, void *q, void *y, int64_t T, int64_t N, int64_t R,
+                       int q_bit, void *stream);
+int hyc_lora_add_restore(const void *xa, const void *b, const void *q, const void *scale,
+                         const void *zero_point, void *y, int64_t T, int64_t N, int64_t R, int q_bit,
+                         void *stream);
+
 #ifdef __cplusplus
 }
 #endif

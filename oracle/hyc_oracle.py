@@ -395,6 +395,13 @@ def _lora_term(xa, b):
     return (xa.float() @ b.float()).to(BF16)
 
 
+def lora_add(x_main, xa, b):
+    """x_main + x_lora_a @ w_lora_b in bf16, product rounded before the add
+    (models/utils/compute_utils.py:21-24; the same expression rebuilds q, k, v in backward,
+    models/llama/fused_llama_layer_intra_inter_full_fuse.py:417,441,449)."""
+    return x_main.to(BF16) + _lora_term(xa, b)
+
+
 def fused_fwd(xa1, b1, x1, s1, xa2, b2, x2, s2, q_bit):
     """triton_fuse_silu_forward (…forward_kernels.py:104-146,152-182) -> (q1, q2, o)."""
     x1 = x1.to(BF16); x2 = x2.to(BF16)

@@ -1,0 +1,133 @@
+"""GPU parity of the LoRA-add kernels (plain, with the quantiser, from packed codes): packed codes
+bit-exact against the oracle's quantiser, the sum against the oracle's bf16 composition, and the
+three forms bit-identical among themselves and to the separate operators they replace."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import BF16, assert_close_bf16, bits
+from oracle import hyc_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def K():
+    import hyclora_amd  # noqa: F401
+    from hyclora_amd.operators import compress_function, lora_kernels
+
+    class Ns:
+        add = staticmethod(lora_kernels.lora_add)
+        add_quant = staticmethod(lora_kernels.lora_add_quant)
+        add_restore = staticmethod(lora_kernels.lora_add_restore)
+        quant = staticmethod(compress_function.compression_quantization)
+        quant_zp = staticmethod(compress_function.compression_quantization_with_zero_point)
+        dequant = staticmethod(compress_function.decompression_dequantization)
+        dequant_zp = staticmethod(compress_function.decompression_dequantization_with_zero_point)
+    return Ns
+
+
+def inputs(seed, B, M, N, R, shift=0.0):
+    g = torch.Generator().manual_seed(seed)
+    main = (torch.randn(B, M, N, generator=g) + shift).to(BF16)
+    a = torch.empty(R, 64)
+    torch.nn.init.kaiming_uniform_(a, a=math.sqrt(5), generator=g)
+    xa = (torch.randn(B, M, 64, generator=g) @ a.t()).to(BF16)
+    b = (torch.randn(R, N, generator=g) * 0.3).to(BF16)            # large enough to move the sum
+    return main, xa, b
+
+
+def mostly_same_bits(a, b, what):
+    """The rank-R dot product is accumulated in fp32 in a different order on the matrix cores than
+    in the CPU matmul, so a bf16 rounding may land on the neighbour now and then: nearly every
+    element identical, the rest within the bf16 tolerance."""
+    same = np.mean(bits(a) == bits(b))
+    assert same >= 0.998, f"{what}: only {same:.5f} of the elements bit-identical"
+    assert_close_bf16(a, b, what=what)
+
+
+DIMS = [(2, 64, 256, 16), (1, 37, 160, 16), (1, 16, 11008, 16), (2, 20, 256, 8), (1, 33, 384, 32),
+        (1, 16, 128, 64), (1, 5, 96, 4), (3, 50, 4096, 16)]
+
+
+@pytest.mark.parametrize("dims", DIMS)
+def test_plain_add_out_of_place_and_in_place(K, dev, dims):
+    B, M, N, R = dims
+    main, xa, b = inputs(N + R, B, M, N, R)
+    want = O.lora_add(main, xa, b)
+    x = main.to(dev)
+    y = K.add(x, xa.to(dev), b.to(dev))
+    assert torch.equal(x.cpu(), main), "input must be left alone"
+    mostly_same_bits(y, want, "lora_add vs oracle")
+    assert_close_bf16(y, main.float() + xa.float() @ b.float(), what="lora_add vs fp32")
+    y2 = K.add(x, xa.to(dev), b.to(dev), inplace=True)
+    assert y2.data_ptr() == x.data_ptr()
+    assert np.array_equal(bits(y2), bits(y)), "in place and out of place must agree bit for bit"
+
+
+@pytest.mark.parametrize("q_bit", [2, 4, 8])
+@pytest.mark.parametrize("zp", [False, True])
+@pytest.mark.parametrize("dims", DIMS)
+def test_add_with_quantiser_and_from_codes(K, dev, q_bit, zp, dims):
+    B, M, N, R = dims
+    main, xa, b = inputs(q_bit + N, B, M, N, R, shift=1.5 if zp else 0.0)
+    if zp:
+        s, z = O.scale_zero_point(main, q_bit)
+    else:
+        s, z = O.scale_only_quant(main, q_bit), None
+    d = lambda t: None if t is None else t.to(dev)
+    q, y = K.add_quant(d(main), d(xa), d(b), d(s), d(z), q_bit)
+    q_ref = O.compress(main, s, q_bit, z)
+    assert torch.equal(q.cpu(), q_ref), "packed codes must be bit-exact"
+    sep = K.quant_zp(d(main), d(s), d(z), q_bit) if zp else K.quant(d(main), d(s), q_bit)
+    assert torch.equal(q, sep), "same codes as the standalone quantiser"
+    mostly_same_bits(y, O.lora_add(main, xa, b), "lora_add_quant y vs oracle")
+    assert np.array_equal(bits(y), bits(K.add(d(main), d(xa), d(b)))), "same sum as the plain form"
+
+    r = K.add_restore(q, d(s), d(xa), d(b), d(z), q_bit)
+    x_hat_ref = O.decompress(q_ref, s, q_bit, z)
+    mostly_same_bits(r, O.lora_add(x_hat_ref, xa, b), "lora_add_restore vs oracle")
+    x_hat = K.dequant_zp(q, d(s), d(z), q_bit) if zp else K.dequant(q, d(s), q_bit)
+    assert np.array_equal(bits(x_hat), bits(x_hat_ref))
+    assert np.array_equal(bits(r), bits(K.add(x_hat, d(xa), d(b)))), "same as dequantise, then add"
+
+
+def test_special_values_and_degenerate_steps(K, dev):
+    """NaN / Inf inputs and steps outside the reciprocal path take the same codes as the standalone
+    quantiser; an empty tensor is a no-op."""
+    B, M, N, R = 1, 19, 128, 16
+    main, xa, b = inputs(5, B, M, N, R)
+    main[0, 3, 5] = float("nan")
+    main[0, 4, 6] = float("inf")
+    main[0, 5, 7] = -float("inf")
+    s = O.scale_only_quant(main.nan_to_num(0.0, 0.0, 0.0), 4)
+    s[0, 9] = 1e-30
+    s[0, 10] = 1e25
+    d = lambda t: t.to(dev)
+    q, y = K.add_quant(d(main), d(xa), d(b), d(s), None, 4)
+    assert torch.equal(q.cpu(), O.compress(main, s, 4))
+    assert torch.equal(q, K.quant(d(main), d(s), 4))
+    assert torch.isnan(y[0, 3, 5]) and torch.isinf(y[0, 4, 6]) and torch.isinf(y[0, 5, 7])
+    r = K.add_restore(q, d(s), d(xa), d(b), None, 4)
+    assert np.array_equal(bits(r), bits(K.add(K.dequant(q, d(s), 4), d(xa), d(b))))
+    e = torch.empty(1, 0, N, device=dev, dtype=BF16)
+    qe, ye = K.add_quant(e, torch.empty(1, 0, R, device=dev, dtype=BF16), d(b), d(s), None, 4)
+    assert qe.shape == (1, 0, N // 2) and ye.shape == (1, 0, N)
+
+
+def test_argument_checks(K, dev):
+    main, xa, b = inputs(1, 1, 4, 64, 16)
+    d = lambda t: t.to(dev)
+    s = O.scale_only_quant(main, 4)
+    with pytest.raises(ValueError):
+        K.add(d(main), d(xa)[..., :8], d(b))                       # rank mismatch
+    with pytest.raises(ValueError):
+        K.add(d(main)[..., :48], d(xa), d(b)[:, :48])              # width not a multiple of 32
+    with pytest.raises(ValueError):
+        K.add_quant(d(main), d(xa), d(b), d(s), None, 3)
+    with pytest.raises(ValueError):
+        K.add_restore(torch.zeros(1, 4, 16, device=dev, dtype=torch.uint8), d(s), d(xa), d(b), None, 4)
+    with pytest.raises(RuntimeError):
+        K.add(main, xa, b)                                          # CPU tensors: no fallback
