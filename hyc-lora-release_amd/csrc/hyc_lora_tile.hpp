@@ -24,10 +24,26 @@ template <int QBIT> constexpr int kColTilesPerGroup = 8 / QBIT;
 
 // LoRA-B operands of one 128-column tile: for each 16-deep K step and each of the 8 MFMAs, the
 // 4 bf16 values b[16*ks + 4g + kk][c0 + 8j + t], kk = 0..3, for lane (g = l/16, j = l%16).
+// b is either [R, N] row-major or, with `transposed`, [N, R] row-major - the layout nn.Linear
+// keeps lora_B.weight in, where the four k of one column are one 8-byte load.
 template <int KSTEPS>
 struct BOperand {
     s16x4 v[KSTEPS][8];
-    __device__ __forceinline__ void load(const uint16_t* b, int N, int R, int col0, bool active, int g) {
+    __device__ __forceinline__ void load(const uint16_t* b, int N, int R, int col0, bool active, int g,
+                                         bool transposed = false) {
+        if (transposed) {
+#pragma unroll
+            for (int ks = 0; ks < KSTEPS; ++ks) {
+                const int k = 16 * ks + 4 * g;
+#pragma unroll
+                for (int t = 0; t < 8; ++t) {
+                    u32x2 r = {0, 0};
+                    if (active && k < R) r = ld8(b + (int64_t)(col0 + t) * R + k);
+                    v[ks][t] = __builtin_bit_cast(s16x4, r);
+                }
+            }
+            return;
+        }
 #pragma unroll
         for (int ks = 0; ks < KSTEPS; ++ks) {
             uint32_t rows[4][4];

@@ -30,6 +30,7 @@ struct LoraAddArgs {
     int64_t T;
     int N, C, R;
     int rows_per_wave, col_tiles;
+    int b_transposed;                           // b is [N, R] instead of [R, N]
 };
 
 template <int QBIT, int KSTEPS, int MODE, bool ZP, bool FAST>
@@ -111,7 +112,7 @@ __global__ __launch_bounds__(kAddThreads) void lora_add_kernel(const LoraAddArgs
         if (active) unpack8(ld16(a.zp + col0), z);
     }
     BOperand<KSTEPS> B;
-    B.load(a.b, a.N, a.R, col0, active, lane >> 4);
+    B.load(a.b, a.N, a.R, col0, active, lane >> 4, a.b_transposed != 0);
 
     const int64_t row_begin = (row_tile * RS + wave / CT) * (int64_t)a.rows_per_wave;
     int64_t row_end = row_begin + a.rows_per_wave;
@@ -145,7 +146,7 @@ static int add_launch(LoraAddArgs& a, int64_t T, int64_t N, int64_t R, int q_bit
     if (!a.xa || !a.b || !a.y) return HYC_ERR_NULL;
     if (MODE != kAddRestore && !a.x) return HYC_ERR_NULL;
     if (MODE != kAddPlain && (!a.q || !a.s)) return HYC_ERR_NULL;
-    if (!aligned16(a.b) || !aligned16(a.y) || (a.x && !aligned16(a.x)) || (a.s && !aligned16(a.s)) ||
+    if (!(a.b_transposed ? (reinterpret_cast<uintptr_t>(a.b) & 7u) == 0 : aligned16(a.b)) || !aligned16(a.y) || (a.x && !aligned16(a.x)) || (a.s && !aligned16(a.s)) ||
         (a.zp && !aligned16(a.zp)))
         return HYC_ERR_ALIGN;
     if ((reinterpret_cast<uintptr_t>(a.xa) & 7u) || (a.q && (reinterpret_cast<uintptr_t>(a.q) & 7u))) return HYC_ERR_ALIGN;
@@ -185,26 +186,29 @@ int tune_add(const char* key, int value) {
 
 using namespace hyc;
 
-extern "C" int hyc_lora_add(const void* xa, const void* b, const void* x, void* y, int64_t T, int64_t N, int64_t R,
-                            void* stream) {
+extern "C" int hyc_lora_add(const void* xa, const void* b, int b_transposed, const void* x, void* y, int64_t T,
+                            int64_t N, int64_t R, void* stream) {
     LoraAddArgs a{};
+    a.b_transposed = b_transposed;
     a.xa = (const uint16_t*)xa; a.b = (const uint16_t*)b; a.x = (const uint16_t*)x; a.y = (uint16_t*)y;
     return add_launch<kAddPlain>(a, T, N, R, 8, stream);
 }
 
-extern "C" int hyc_lora_add_quant(const void* xa, const void* b, const void* x, const void* scale,
+extern "C" int hyc_lora_add_quant(const void* xa, const void* b, int b_transposed, const void* x, const void* scale,
                                   const void* zero_point, void* q, void* y, int64_t T, int64_t N, int64_t R,
                                   int q_bit, void* stream) {
     LoraAddArgs a{};
+    a.b_transposed = b_transposed;
     a.xa = (const uint16_t*)xa; a.b = (const uint16_t*)b; a.x = (const uint16_t*)x; a.y = (uint16_t*)y;
     a.s = (const uint16_t*)scale; a.zp = (const uint16_t*)zero_point; a.q = (uint8_t*)q;
     return add_launch<kAddQuant>(a, T, N, R, q_bit, stream);
 }
 
-extern "C" int hyc_lora_add_restore(const void* xa, const void* b, const void* q, const void* scale,
-                                    const void* zero_point, void* y, int64_t T, int64_t N, int64_t R, int q_bit,
-                                    void* stream) {
+extern "C" int hyc_lora_add_restore(const void* xa, const void* b, int b_transposed, const void* q,
+                                    const void* scale, const void* zero_point, void* y, int64_t T, int64_t N,
+                                    int64_t R, int q_bit, void* stream) {
     LoraAddArgs a{};
+    a.b_transposed = b_transposed;
     a.xa = (const uint16_t*)xa; a.b = (const uint16_t*)b; a.y = (uint16_t*)y;
     a.s = (const uint16_t*)scale; a.zp = (const uint16_t*)zero_point; a.q = (uint8_t*)const_cast<void*>(q);
     return add_launch<kAddRestore>(a, T, N, R, q_bit, stream);

@@ -38,6 +38,7 @@ struct FuseArgs {
     int64_t T;                                  // rows
     int N, C, R;                                // columns, chunks per row, LoRA rank
     int rows_per_wave, col_tiles;
+    int b_transposed;                           // b1, b2 are [N, R] instead of [R, N]
 };
 
 // ------------------------------------------------------------------------------------
@@ -113,9 +114,9 @@ HYC_FUSE_KERNEL void lora_silu_fwd_kernel(const FuseArgs a) {
     c2.load(a.s2, col0, active);
     __builtin_amdgcn_sched_barrier(0);
     BOperand<KSTEPS> B1, B2;
-    B1.load(a.b1, a.N, a.R, col0, active, lane >> 4);
+    B1.load(a.b1, a.N, a.R, col0, active, lane >> 4, a.b_transposed != 0);
     __builtin_amdgcn_sched_barrier(0);
-    B2.load(a.b2, a.N, a.R, col0, active, lane >> 4);
+    B2.load(a.b2, a.N, a.R, col0, active, lane >> 4, a.b_transposed != 0);
     __builtin_amdgcn_sched_barrier(0);
 
     const int64_t row_begin = (row_tile * RS + wave / CT) * (int64_t)a.rows_per_wave;
@@ -150,8 +151,8 @@ HYC_FUSE_KERNEL void lora_silu_bwd_kernel(const FuseArgs a) {
         unpack8(v2, s2);
     }
     BOperand<KSTEPS> B1, B2;
-    B1.load(a.b1, a.N, a.R, col0, active, g);
-    B2.load(a.b2, a.N, a.R, col0, active, g);
+    B1.load(a.b1, a.N, a.R, col0, active, g, a.b_transposed != 0);
+    B2.load(a.b2, a.N, a.R, col0, active, g, a.b_transposed != 0);
     const PackedSlot<QBIT> slot(chunk);
     const int row_bytes = a.N * QBIT / 8;
 
@@ -217,7 +218,10 @@ static int fuse_check(const FuseArgs& a, int64_t T, int64_t N, int64_t R, int q_
                           fwd ? (const void*)a.x1 : (const void*)a.g, fwd ? (const void*)a.x2 : (const void*)a.gg,
                           fwd ? (const void*)a.o : (const void*)a.gu};
     for (const void* p : need) if (!p) return HYC_ERR_NULL;
-    const void* al16[] = {a.b1, a.s1, a.b2, a.s2, a.o, fwd ? (const void*)a.x1 : (const void*)a.g,
+    if (a.b_transposed ? ((reinterpret_cast<uintptr_t>(a.b1) | reinterpret_cast<uintptr_t>(a.b2)) & 7u) != 0
+                       : !(aligned16(a.b1) && aligned16(a.b2)))
+        return HYC_ERR_ALIGN;
+    const void* al16[] = {a.s1, a.s2, a.o, fwd ? (const void*)a.x1 : (const void*)a.g,
                           fwd ? (const void*)a.x2 : (const void*)a.gg, fwd ? (const void*)a.o : (const void*)a.gu};
     for (const void* p : al16) if (!aligned16(p)) return HYC_ERR_ALIGN;
     const void* al8[] = {a.xa1, a.xa2, a.q1, a.q2};
@@ -275,8 +279,9 @@ using namespace hyc;
 extern "C" int hyc_lora_silu_mul_fwd(const void* xa1, const void* b1, const void* x1, const void* s1,
                                      const void* xa2, const void* b2, const void* x2, const void* s2,
                                      void* q1, void* q2, void* o, int64_t T, int64_t N, int64_t R, int q_bit,
-                                     void* stream) {
+                                     int b_transposed, void* stream) {
     FuseArgs a{};
+    a.b_transposed = b_transposed;
     a.xa1 = (const uint16_t*)xa1; a.b1 = (const uint16_t*)b1; a.s1 = (const uint16_t*)s1;
     a.xa2 = (const uint16_t*)xa2; a.b2 = (const uint16_t*)b2; a.s2 = (const uint16_t*)s2;
     a.x1 = (const uint16_t*)x1; a.x2 = (const uint16_t*)x2;
@@ -287,8 +292,9 @@ extern "C" int hyc_lora_silu_mul_fwd(const void* xa1, const void* b1, const void
 extern "C" int hyc_lora_silu_mul_bwd(const void* xa1, const void* b1, const void* q1, const void* s1,
                                      const void* xa2, const void* b2, const void* q2, const void* s2,
                                      const void* grad_o, void* o, void* grad_gate, void* grad_up, int64_t T,
-                                     int64_t N, int64_t R, int q_bit, void* stream) {
+                                     int64_t N, int64_t R, int q_bit, int b_transposed, void* stream) {
     FuseArgs a{};
+    a.b_transposed = b_transposed;
     a.xa1 = (const uint16_t*)xa1; a.b1 = (const uint16_t*)b1; a.s1 = (const uint16_t*)s1;
     a.xa2 = (const uint16_t*)xa2; a.b2 = (const uint16_t*)b2; a.s2 = (const uint16_t*)s2;
     a.q1 = (uint8_t*)q1; a.q2 = (uint8_t*)q2;

@@ -18,6 +18,30 @@ def head_to_hidden_shape(x: torch.Tensor):
     return x.transpose(1, 2).reshape(bsz, seq_len, -1).contiguous()
 
 
+_MAX_BATCH_LOOP = 16
+
+
+def heads_matmul(a: torch.Tensor, b: torch.Tensor, out_hidden: bool = False):
+    """a @ b for [B, H, M, K] x [B, H, K, N] operands that are *views* of hidden-layout tensors
+    ([B, S, H*D] seen as [B, H, S, D]).  torch.matmul would first copy such a view into head-major
+    memory (the reference pays that copy at every attention product); a batched GEMM over the heads
+    of one batch element reads it in place (row stride H*D, batch stride D), so this loops over the
+    batch.  out_hidden=True writes the result [B, H, M, N] into a hidden-layout buffer and returns
+    its [B, H, M, N] view, which makes the following head_to_hidden_shape free."""
+    B, H, M, _ = a.shape
+    N = b.shape[-1]
+    if B > _MAX_BATCH_LOOP or not a.is_cuda or a.dtype != b.dtype:
+        r = torch.matmul(a, b)
+        return r.transpose(1, 2).contiguous().transpose(1, 2) if out_hidden else r
+    if out_hidden:
+        out = a.new_empty(B, M, H, N).transpose(1, 2)
+    else:
+        out = a.new_empty(B, H, M, N)
+    for i in range(B):
+        torch.bmm(a[i], b[i], out=out[i])
+    return out
+
+
 def dense_weight(w: torch.Tensor, quant_state):
     """Frozen weight as a dense [out, in] matrix.  quant_state None = already dense (the benchmark
     configurations); otherwise a bitsandbytes-format NF4 weight, dequantised by the HIP kernel (the
@@ -75,8 +99,7 @@ def repeat_kv(h: torch.Tensor, n_rep: int):
 def repeat_kv_backward(g: torch.Tensor, n_rep: int):
     if n_rep == 1:
         return g
-    b, hq, s, d = g.shape
-    return g.reshape(b, hq // n_rep, n_rep, s, d).sum(dim=2)
+    return g.unflatten(1, (g.shape[1] // n_rep, n_rep)).sum(dim=2)
 
 
 from ..operators.rope_kernels import rope_backward, rope_forward  # noqa: E402,F401  (in place, HIP)

@@ -55,7 +55,7 @@ from ..operators.softmax_kernels import softmax_backward, softmax_backward_from_
 from ..operators.triton_fuse_lora_silu_hadamard_backward_kernels import triton_fuse_silu_backward
 from ..operators.triton_fuse_lora_silu_hadamard_forward_kernels import triton_fuse_silu_forward
 from ..operators import lora_kernels
-from .compute_utils import (head_to_hidden_shape, hidden_to_head_shape, lora_backward, lora_forward, lora_parts,
+from .compute_utils import (head_to_hidden_shape, heads_matmul, hidden_to_head_shape, lora_backward, lora_forward, lora_parts,
                             repeat_kv, repeat_kv_backward, rope_backward, rope_forward)
 
 MODES = ("baseline", "intra", "intra_inter", "intra_inter_full_fuse")
@@ -216,7 +216,7 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             quant("v_rep", v, "v")
 
         if spec.attention == "map":
-            s = q @ k.transpose(-2, -1)
+            s = heads_matmul(q, k.transpose(-2, -1))
             del q, k
             # scale, mask and softmax in one pass over the scores, in place; once the threshold is
             # frozen the same pass also counts the entries the compaction keeps
@@ -243,7 +243,7 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
                 thr = get_statistics_softmax(a, softmax_outlier_ratio) if calib else sv['a']['outlier']
                 stats[("a", "outlier")] = thr
                 saved["a_idx"], saved["a_val"], saved["a_seg"] = compress_attention_map(a, thr, seg)
-            o = a @ v
+            o = heads_matmul(a, v, out_hidden=True)
             del a, v
         else:
             o = F.scaled_dot_product_attention(q, k, v, attn_mask=attention_mask, is_causal=attention_mask is None)
@@ -311,11 +311,14 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
         ctx.norm_grads = (norm_weight_1.requires_grad, norm_weight_2.requires_grad)
         out_stats = tuple(stats[slot] for slot in spec.stat_slots())
         ctx.mark_non_differentiable(*[t for t in out_stats if torch.is_tensor(t)])
+        ctx.set_materialize_grads(False)         # no zero-filled gradients for the statistics outputs
         return (x_out,) + out_stats
 
     @staticmethod
     def backward(ctx, grad_output, *_unused):
         spec, q_bit = ctx.spec, ctx.q_bit
+        if grad_output is None:
+            return (None,) * 53
         tensors = list(ctx.saved_tensors)
         ns = len(ctx.names)
         S = dict(zip(ctx.names, tensors[:ns]))
@@ -371,7 +374,10 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             grad_b_down = S["down_lora_a"].to(wd.dtype).mT @ g
             grad_down = g @ wd
             grad_mid = g @ lb.mT
-            grad_down += grad_mid @ la.mT
+            if lora_kernels.supported(grad_down, grad_mid, la.mT):
+                grad_down = lora_kernels.lora_add(grad_down, grad_mid, la.mT, inplace=True)
+            else:
+                grad_down += grad_mid @ la.mT
             hadamard, grad_fn, grad_h2 = triton_fuse_silu_backward(
                 S["gate_lora_a"], W["gate"][4], S["gate_main_q"], S["gate_main_s"],
                 S["up_lora_a"], W["up"][4], S["up_main_q"], S["up_main_s"], grad_down, q_bit)
@@ -418,7 +424,7 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
         if spec.attention == "map":
             # grad_a first, then the restored map and the softmax backward come out of one pass over
             # the compressed map (the reference restores, then reads the dense map twice more)
-            grad_a = grad_o @ v.transpose(-2, -1)
+            grad_a = heads_matmul(grad_o, v.transpose(-2, -1))
             del v
             if "a_raw" in S:
                 a = S["a_raw"]
@@ -427,10 +433,10 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
                 a, grad_s = softmax_backward_from_compressed(S["a_idx"], S["a_val"], S["a_seg"], grad_a,
                                                              out_scale=1.0 / math.sqrt(D))
             del grad_a
-            grad_v = a.transpose(-2, -1) @ grad_o
+            grad_v = heads_matmul(a.transpose(-2, -1), grad_o, out_hidden=True)
             del a, grad_o
-            grad_k = grad_s.transpose(-2, -1) @ q
-            grad_q = grad_s @ k
+            grad_k = heads_matmul(grad_s.transpose(-2, -1), q, out_hidden=True)
+            grad_q = heads_matmul(grad_s, k, out_hidden=True)
             del grad_s, q, k
         else:
             with torch.enable_grad():

@@ -22,7 +22,8 @@ from ..operators.gelu_kernels import gelu_backward
 from ..operators.layernorm_kernels import layernorm_backward, layernorm_forward
 from ..operators.softmax_kernels import softmax_backward, softmax_backward_from_compressed, softmax_forward
 from ..operators import lora_kernels
-from .compute_utils import head_to_hidden_shape, hidden_to_head_shape, lora_backward, lora_forward, lora_parts
+from .compute_utils import (head_to_hidden_shape, heads_matmul, hidden_to_head_shape, lora_backward, lora_forward,
+                            lora_parts)
 
 MODES = ("baseline", "intra", "intra_inter")
 _PROJ = ("q", "k", "v", "o", "up", "down")
@@ -117,7 +118,7 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
         if whole:
             quant("q", q)
             quant("k", k)
-        s = q @ k.transpose(-2, -1)
+        s = heads_matmul(q, k.transpose(-2, -1))
         del q, k
         m = attention_mask
         fits = m is None or (m.dim() == 4 and m.shape[1] == 1 and m.shape[0] in (1, s.shape[0]) and
@@ -137,7 +138,7 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
                 s = s + attention_mask
             a = torch.softmax(s, dim=-1, dtype=v.dtype)
         del s
-        o = a @ v
+        o = heads_matmul(a, v, out_hidden=True)
         if raw:
             saved["a_raw"] = a
         else:
@@ -186,6 +187,7 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
         ctx.block_size, ctx.num_warps = block_size, num_warps
         out_stats = tuple(stats[slot] for slot in stat_slots(mode))
         ctx.mark_non_differentiable(*[t for t in out_stats if torch.is_tensor(t)])
+        ctx.set_materialize_grads(False)         # no zero-filled gradients for the statistics outputs
         return (x_out,) + out_stats
 
     @staticmethod
@@ -223,6 +225,8 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
             main = deq(name + "_main")
             return main + xa.to(main.dtype) @ lb.to(main.dtype)
 
+        if grad_output is None:
+            return (None,) * 45
         grad_output = grad_output.to(torch.bfloat16)
         grad_ln2, _, _ = layernorm_backward(grad_output, deq_cb("down"), nw2, nb2, S["mean_2"], S["rstd_2"], True, _EPS,
                                             ctx.num_warps, ctx.block_size)
@@ -248,7 +252,7 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
             v = deq("v", is_head=True, num_heads=H)
         else:
             v = hidden_to_head_shape(rebuilt("v"), H)
-        grad_a = grad_o @ v.transpose(-2, -1)
+        grad_a = heads_matmul(grad_o, v.transpose(-2, -1))
         del v
         if "a_raw" in S:
             a = S["a_raw"]
@@ -257,14 +261,14 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
             a, grad_s = softmax_backward_from_compressed(S["a_idx"], S["a_val"], S["a_seg"], grad_a,
                                                          out_scale=1.0 / math.sqrt(D))
         del grad_a
-        grad_v = a.transpose(-2, -1) @ grad_o
+        grad_v = heads_matmul(a.transpose(-2, -1), grad_o, out_hidden=True)
         del a, grad_o
         if whole:
             q, k = deq("q", is_head=True, num_heads=H), deq("k", is_head=True, num_heads=H)
         else:
             q, k = hidden_to_head_shape(rebuilt("q"), H), hidden_to_head_shape(rebuilt("k"), H)
-        grad_k = grad_s.transpose(-2, -1) @ q
-        grad_q = grad_s @ k
+        grad_k = heads_matmul(grad_s.transpose(-2, -1), q, out_hidden=True)
+        grad_q = heads_matmul(grad_s, k, out_hidden=True)
         del grad_s, q, k
         grad_q, grad_k, grad_v = (head_to_hidden_shape(t) for t in (grad_q, grad_k, grad_v))
 

@@ -25,15 +25,20 @@ def _common(xa1, b1, s1, xa2, b2, s2, quantize_bit, n):
         raise ValueError("LoRA-B width does not match the activation width")
     if n % 32:
         raise ValueError(f"channel count must be a multiple of 32, got {n}")
-    return (_prep(xa1, "xa1"), _prep(b1, "b1"), _prep(s1.reshape(-1), "s1"),
-            _prep(xa2, "xa2"), _prep(b2, "b2"), _prep(s2.reshape(-1), "s2"), r)
+    # [R, N] views of [N, R] contiguous weights (lora_B.weight.T) are read as they lie in memory
+    bt = int(all(b.dtype == BF16 and not b.is_contiguous() and b.mT.is_contiguous() and b.data_ptr() % 8 == 0
+                 for b in (b1, b2)))
+    if not bt:
+        b1, b2 = _prep(b1, "b1"), _prep(b2, "b2")
+    return (_prep(xa1, "xa1"), b1, _prep(s1.reshape(-1), "s1"),
+            _prep(xa2, "xa2"), b2, _prep(s2.reshape(-1), "s2"), r, bt)
 
 
 def fuse_forward(xa1, b1, x1, s1, xa2, b2, x2, s2, quantize_bit=8):
     _lib.require_gpu(xa1, b1, x1, s1, xa2, b2, x2, s2)
     B, M, N = x1.shape
     assert x2.shape == x1.shape
-    xa1, b1, s1, xa2, b2, s2, R = _common(xa1, b1, s1, xa2, b2, s2, quantize_bit, N)
+    xa1, b1, s1, xa2, b2, s2, R, bt = _common(xa1, b1, s1, xa2, b2, s2, quantize_bit, N)
     x1 = _prep(x1, "x1")
     x2 = _prep(x2, "x2")
     epp = 8 // quantize_bit
@@ -42,14 +47,14 @@ def fuse_forward(xa1, b1, x1, s1, xa2, b2, x2, s2, quantize_bit=8):
     o = torch.empty((B, M, N), device=x1.device, dtype=BF16)
     _lib.call("hyc_lora_silu_mul_fwd", xa1.data_ptr(), b1.data_ptr(), x1.data_ptr(), s1.data_ptr(),
               xa2.data_ptr(), b2.data_ptr(), x2.data_ptr(), s2.data_ptr(), q1.data_ptr(), q2.data_ptr(),
-              o.data_ptr(), B * M, N, R, quantize_bit, _lib.stream_of(x1))
+              o.data_ptr(), B * M, N, R, quantize_bit, bt, _lib.stream_of(x1))
     return q1, q2, o
 
 
 def fuse_backward(xa1, b1, q1, s1, xa2, b2, q2, s2, grad_o, quantize_bit=8):
     _lib.require_gpu(xa1, b1, q1, s1, xa2, b2, q2, s2, grad_o)
     B, M, N = grad_o.shape
-    xa1, b1, s1, xa2, b2, s2, R = _common(xa1, b1, s1, xa2, b2, s2, quantize_bit, N)
+    xa1, b1, s1, xa2, b2, s2, R, bt = _common(xa1, b1, s1, xa2, b2, s2, quantize_bit, N)
     grad_o = _prep(grad_o, "grad_o")
     q1 = q1.contiguous()
     q2 = q2.contiguous()
@@ -61,5 +66,5 @@ def fuse_backward(xa1, b1, q1, s1, xa2, b2, q2, s2, grad_o, quantize_bit=8):
     gu = torch.empty_like(o)
     _lib.call("hyc_lora_silu_mul_bwd", xa1.data_ptr(), b1.data_ptr(), q1.data_ptr(), s1.data_ptr(),
               xa2.data_ptr(), b2.data_ptr(), q2.data_ptr(), s2.data_ptr(), grad_o.data_ptr(), o.data_ptr(),
-              gg.data_ptr(), gu.data_ptr(), B * M, N, R, quantize_bit, _lib.stream_of(grad_o))
+              gg.data_ptr(), gu.data_ptr(), B * M, N, R, quantize_bit, bt, _lib.stream_of(grad_o))
     return o, gg, gu

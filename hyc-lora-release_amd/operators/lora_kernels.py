@@ -43,6 +43,14 @@ def supported_restore(q, xa, b):
     return q.is_cuda and q.dtype == torch.uint8 and q.dim() == 3 and _operands_ok(xa, b)
 
 
+def _lora_b(b):
+    """-> (tensor to pass, b_transposed flag).  A [R, N] view of an [N, R] contiguous weight (what
+    `lora_B.weight.T` is) is handed over as it lies in memory."""
+    if b.dtype == BF16 and not b.is_contiguous() and b.mT.is_contiguous() and b.data_ptr() % 8 == 0:
+        return b, 1
+    return _prep(b, "b"), 0
+
+
 def lora_add(x_main, xa, b, inplace=False):
     """bf16(x_main + bf16(xa @ b)); `inplace` overwrites x_main (contiguous bf16) and returns it."""
     _lib.require_gpu(x_main, xa, b)
@@ -51,8 +59,8 @@ def lora_add(x_main, xa, b, inplace=False):
     x = x_main if (inplace and x_main.dtype == BF16 and x_main.is_contiguous() and x_main.data_ptr() % 16 == 0) \
         else _prep(x_main, "x_main")
     y = x if inplace else torch.empty_like(x)
-    xa, b = _prep(xa, "xa"), _prep(b, "b")
-    _lib.call("hyc_lora_add", xa.data_ptr(), b.data_ptr(), x.data_ptr(), y.data_ptr(), x.numel() // n, n, r,
+    xa, (b, bt) = _prep(xa, "xa"), _lora_b(b)
+    _lib.call("hyc_lora_add", xa.data_ptr(), b.data_ptr(), bt, x.data_ptr(), y.data_ptr(), x.numel() // n, n, r,
               _lib.stream_of(x))
     if inplace and y is not x_main:
         x_main.copy_(y)
@@ -77,11 +85,11 @@ def lora_add_quant(x_main, xa, b, scale, zero_point=None, quantize_bit=8, inplac
     r = _check(xa, b, n)
     x = _prep(x_main, "x_main")
     y = x if (inplace and x is x_main) else torch.empty_like(x)
-    xa, b = _prep(xa, "xa"), _prep(b, "b")
+    xa, (b, bt) = _prep(xa, "xa"), _lora_b(b)
     s = _vec(scale, n, "scale")
     z = None if zero_point is None else _vec(zero_point, n, "zero point")
     q = torch.empty((B, M, n * quantize_bit // 8), device=x.device, dtype=torch.uint8)
-    _lib.call("hyc_lora_add_quant", xa.data_ptr(), b.data_ptr(), x.data_ptr(), s.data_ptr(), _lib.ptr(z),
+    _lib.call("hyc_lora_add_quant", xa.data_ptr(), b.data_ptr(), bt, x.data_ptr(), s.data_ptr(), _lib.ptr(z),
               q.data_ptr(), y.data_ptr(), B * M, n, r, quantize_bit, _lib.stream_of(x))
     return q, y
 
@@ -98,10 +106,10 @@ def lora_add_restore(q, scale, xa, b, zero_point=None, quantize_bit=8):
         raise ValueError(f"packed codes must be uint8 of width {n * quantize_bit // 8}, got {q.dtype} {nbytes}")
     r = _check(xa, b, n)
     q = q.contiguous()
-    xa, b = _prep(xa, "xa"), _prep(b, "b")
+    xa, (b, bt) = _prep(xa, "xa"), _lora_b(b)
     s = _vec(scale, n, "scale")
     z = None if zero_point is None else _vec(zero_point, n, "zero point")
     y = torch.empty((B, M, n), device=q.device, dtype=BF16)
-    _lib.call("hyc_lora_add_restore", xa.data_ptr(), b.data_ptr(), q.data_ptr(), s.data_ptr(), _lib.ptr(z),
+    _lib.call("hyc_lora_add_restore", xa.data_ptr(), b.data_ptr(), bt, q.data_ptr(), s.data_ptr(), _lib.ptr(z),
               y.data_ptr(), B * M, n, r, quantize_bit, _lib.stream_of(q))
     return y

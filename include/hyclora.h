@@ -357,7 +357,9 @@ int hyc_gelu_bwd(const void *x, const void *g, void *out, int64_t n, void *strea
  *
  * Replaces triton_fuse_silu_forward_kernel
  * (operators/triton_fuse_lora_silu_hadamard_forward_kernels.py:28-149).
- *   xa1, xa2 bf16 [T, R] contiguous (x @ lora_A);   b1, b2 bf16 [R, N] contiguous (lora_B);
+ *   xa1, xa2 bf16 [T, R] contiguous (x @ lora_A);   b1, b2 bf16 [R, N] contiguous (lora_B), or with
+ *   b_transposed = 1 both [N, R] contiguous, the layout torch.nn.Linear keeps lora_B.weight in (the
+ *   reference copies them to [R, N] first, …forward_kernels.py:166-167);
  *   x1, x2   bf16 [T, N] contiguous;                s1, s2 bf16 [N];
  *   q1, q2   uint8 [T, N*q_bit/8];                  o      bf16 [T, N].
  *   R: multiple of 4, 4..64 (the reference needs a power of two >= 16); N % 32 == 0; any T.
@@ -365,7 +367,7 @@ int hyc_gelu_bwd(const void *x, const void *g, void *out, int64_t n, void *strea
 int hyc_lora_silu_mul_fwd(const void *xa1, const void *b1, const void *x1, const void *s1,
                           const void *xa2, const void *b2, const void *x2, const void *s2,
                           void *q1, void *q2, void *o, int64_t T, int64_t N, int64_t R, int q_bit,
-                          void *stream);
+                          int b_transposed, void *stream);
 
 /* ---------------------------------------------------------------------------------------
  * Fused LoRA-SiLU-Hadamard backward: dequantises q1, q2, recomputes y1, y2 and the gated
@@ -379,7 +381,7 @@ int hyc_lora_silu_mul_fwd(const void *xa1, const void *b1, const void *x1, const
 int hyc_lora_silu_mul_bwd(const void *xa1, const void *b1, const void *q1, const void *s1,
                           const void *xa2, const void *b2, const void *q2, const void *s2,
                           const void *grad_o, void *o, void *grad_gate, void *grad_up,
-                          int64_t T, int64_t N, int64_t R, int q_bit, void *stream);
+                          int64_t T, int64_t N, int64_t R, int q_bit, int b_transposed, void *stream);
 
 /* ---------------------------------------------------------------------------------------
  * LoRA add around the compressed copy of a projection's frozen part:
@@ -396,19 +398,21 @@ int hyc_lora_silu_mul_bwd(const void *xa1, const void *b1, const void *q1, const
  * models/llama_flash_attn/fused_llama_layer_intra_inter.py:129-138); the rebuild of q, k, v, gate,
  * up in backward (…full_fuse.py:416-417, :439-441, :447-449); and `grad_x += grad_medium @ A^T`
  * of lora_backward (compute_utils.py:34-35) through the plain form.
- *   xa bf16 [T, R] contiguous;  b bf16 [R, N] contiguous;  x, y bf16 [T, N] contiguous;
+ *   xa bf16 [T, R] contiguous;  x, y bf16 [T, N] contiguous;
+ *   b bf16 [R, N] contiguous (b_transposed 0) or [N, R] contiguous (b_transposed 1: the layout
+ *   torch.nn.Linear keeps lora_B.weight in, so no copy of the adapter is needed);
  *   scale, zero_point bf16 [N] (zero_point NULL: symmetric codes);  q uint8 [T, N*q_bit/8].
  *   R: multiple of 4, 4..64; N % 32 == 0; any T.
  * Tuning key "add_rows_per_wave" (multiple of 16, default 32).
  */
-int hyc_lora_add(const void *xa, const void *b, const void *x, void *y, int64_t T, int64_t N, int64_t R,
-                 void *stream);
-int hyc_lora_add_quant(const void *xa, const void *b, const void *x, const void *scale,
+int hyc_lora_add(const void *xa, const void *b, int b_transposed, const void *x, void *y, int64_t T,
+                 int64_t N, int64_t R, void *stream);
+int hyc_lora_add_quant(const void *xa, const void *b, int b_transposed, const void *x, const void *scale,
                        const void *zero_point, void *q, void *y, int64_t T, int64_t N, int64_t R,
                        int q_bit, void *stream);
-int hyc_lora_add_restore(const void *xa, const void *b, const void *q, const void *scale,
-                         const void *zero_point, void *y, int64_t T, int64_t N, int64_t R, int q_bit,
-                         void *stream);
+int hyc_lora_add_restore(const void *xa, const void *b, int b_transposed, const void *q,
+                         const void *scale, const void *zero_point, void *y, int64_t T, int64_t N,
+                         int64_t R, int q_bit, void *stream);
 
 #ifdef __cplusplus
 }

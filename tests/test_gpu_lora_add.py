@@ -94,6 +94,35 @@ def test_add_with_quantiser_and_from_codes(K, dev, q_bit, zp, dims):
     assert np.array_equal(bits(r), bits(K.add(x_hat, d(xa), d(b)))), "same as dequantise, then add"
 
 
+@pytest.mark.parametrize("R", [4, 16, 32, 64])
+def test_lora_b_in_linear_layout(K, dev, R):
+    """A [R, N] view of an [N, R] contiguous weight - what `lora_B.weight.T` is - is read where it
+    lies: same bits as with a contiguous [R, N] copy, in all three forms and in the fused kernels."""
+    import hyclora_amd  # noqa: F401
+    from hyclora_amd.operators.triton_fuse_lora_silu_hadamard_backward_kernels import triton_fuse_silu_backward
+    from hyclora_amd.operators.triton_fuse_lora_silu_hadamard_forward_kernels import triton_fuse_silu_forward
+    B, M, N = 2, 40, 384
+    main, xa, b = inputs(R, B, M, N, R)
+    s = O.scale_only_quant(main, 4)
+    d = lambda t: t.to(dev)
+    w = d(b).t().contiguous()                  # [N, R], the nn.Linear layout
+    bt = w.t()                                 # [R, N] view
+    assert not bt.is_contiguous()
+    assert np.array_equal(bits(K.add(d(main), d(xa), bt)), bits(K.add(d(main), d(xa), d(b))))
+    q1, y1 = K.add_quant(d(main), d(xa), bt, d(s), None, 4)
+    q2, y2 = K.add_quant(d(main), d(xa), d(b), d(s), None, 4)
+    assert torch.equal(q1, q2) and np.array_equal(bits(y1), bits(y2))
+    assert np.array_equal(bits(K.add_restore(q1, d(s), d(xa), bt, None, 4)),
+                          bits(K.add_restore(q1, d(s), d(xa), d(b), None, 4)))
+    fa = triton_fuse_silu_forward(d(xa), bt, d(main), d(s), d(xa), bt, d(main), d(s), 4)
+    fb = triton_fuse_silu_forward(d(xa), d(b), d(main), d(s), d(xa), d(b), d(main), d(s), 4)
+    assert all(np.array_equal(u.cpu().view(torch.uint8).numpy(), v.cpu().view(torch.uint8).numpy()) for u, v in zip(fa, fb))
+    g = torch.randn(B, M, N, generator=torch.Generator().manual_seed(3)).to(BF16).to(dev)
+    ba = triton_fuse_silu_backward(d(xa), bt, fa[0], d(s), d(xa), bt, fa[1], d(s), g, 4)
+    bb = triton_fuse_silu_backward(d(xa), d(b), fa[0], d(s), d(xa), d(b), fa[1], d(s), g, 4)
+    assert all(np.array_equal(bits(u), bits(v)) for u, v in zip(ba, bb))
+
+
 def test_special_values_and_degenerate_steps(K, dev):
     """NaN / Inf inputs and steps outside the reciprocal path take the same codes as the standalone
     quantiser; an empty tensor is a no-op."""
