@@ -72,15 +72,39 @@ def lora_parts(w, w_quant_state, w_lora_a, b, x):
     return x_main, x @ w_lora_a.to(wt.dtype)
 
 
-def lora_backward(w, w_quant_state, w_lora_a, w_lora_b, x, x_lora_a, grad_y):
-    """-> (grad lora_A, grad lora_B, grad x).  Reference :28-36."""
+def lora_backward(w, w_quant_state, w_lora_a, w_lora_b, x, x_lora_a, grad_y, x_codes=None):
+    """-> (grad lora_A, grad lora_B, grad x).  Reference :28-36.
+
+    With bf16 operands the rank-R products stream their wide operand once on the matrix cores:
+    grad_y gives `grad_y @ B^T` and `xa^T @ grad_y` in one pass, and `x^T @ grad_medium` is taken
+    from x - or straight from its packed codes `x_codes = (q, scale, zero_point or None, q_bit)`,
+    in which case x may be None and is never dequantised.  Those results are summed over the batch in
+    fp32 and have the parameters' shapes; the torch expressions below return one gradient per batch
+    element, as the reference does, and leave the sum to autograd."""
     wd = dense_weight(w, w_quant_state)          # [out, in]
     dt = wd.dtype
     grad_y = grad_y.to(dt)
     w_lora_a, w_lora_b = w_lora_a.to(dt), w_lora_b.to(dt)
-    grad_mid = grad_y @ w_lora_b.mT
-    grad_a = x.to(dt).mT @ grad_mid
-    grad_b = x_lora_a.to(dt).mT @ grad_y
+    r = w_lora_b.shape[0]
+    if lora_kernels.contract_supported(grad_y, grad_y.shape[-1], r) and x_lora_a.dtype == dt:
+        grad_b, grad_mid = lora_kernels.lora_products(grad_y, u=x_lora_a, v=w_lora_b)
+    else:
+        grad_mid = grad_y @ w_lora_b.mT
+        grad_b = x_lora_a.to(dt).mT @ grad_y
+    if x_codes is not None and lora_kernels.contract_supported(grad_mid, w_lora_a.shape[0], r):
+        q, scale, zero_point, q_bit = x_codes
+        grad_a = lora_kernels.lora_product_from_codes(q, scale, grad_mid, zero_point, q_bit).t()
+    else:
+        if x is None:
+            from ..operators.compress_function import (decompression_dequantization,
+                                                       decompression_dequantization_with_zero_point)
+            q, scale, zero_point, q_bit = x_codes
+            x = decompression_dequantization(q, scale, q_bit) if zero_point is None else \
+                decompression_dequantization_with_zero_point(q, scale, zero_point, q_bit)
+        if lora_kernels.contract_supported(x, x.shape[-1], r) and grad_mid.dtype == x.dtype:
+            grad_a = lora_kernels.lora_products(x, u=grad_mid)[0].t()
+        else:
+            grad_a = x.to(dt).mT @ grad_mid
     grad_x = grad_y @ wd
     if lora_kernels.supported(grad_x, grad_mid, w_lora_a.mT):
         grad_x = lora_kernels.lora_add(grad_x, grad_mid, w_lora_a.mT, inplace=True)

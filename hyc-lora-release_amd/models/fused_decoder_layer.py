@@ -339,8 +339,16 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             return decompression_dequantization(S[name + "_q"], S[name + "_s"], q_bit, **kw)
 
         def back(name, inp, inp_lora_a, grad_y):
+            """Backward of projection `name`.  `inp` is its input, or the name under which the layer
+            saved that input: a compressed one is then read from its codes, not dequantised."""
             w, _, qs, la, lb = W[name]
-            ga, gb, gx = lora_backward(w, qs, la, lb, inp, inp_lora_a, grad_y)
+            codes = None
+            if isinstance(inp, str):
+                if inp + "_raw" in S:
+                    inp = S[inp + "_raw"]
+                else:
+                    codes, inp = (S[inp + "_q"], S[inp + "_s"], S.get(inp + "_z"), q_bit), None
+            ga, gb, gx = lora_backward(w, qs, la, lb, inp, inp_lora_a, grad_y, x_codes=codes)
             G[name] = (ga, gb)
             return gx
 
@@ -371,9 +379,14 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             wd = dense_weight(w, qs)
             la, lb = la.to(wd.dtype), lb.to(wd.dtype)
             g = grad_output.to(wd.dtype)
-            grad_b_down = S["down_lora_a"].to(wd.dtype).mT @ g
+            r = lb.shape[0]
+            fast = lora_kernels.contract_supported(g, g.shape[-1], r) and S["down_lora_a"].dtype == g.dtype
+            if fast:                      # both rank-R products of grad_output from one pass over it
+                grad_b_down, grad_mid = lora_kernels.lora_products(g, u=S["down_lora_a"], v=lb)
+            else:
+                grad_b_down = S["down_lora_a"].to(wd.dtype).mT @ g
+                grad_mid = g @ lb.mT
             grad_down = g @ wd
-            grad_mid = g @ lb.mT
             if lora_kernels.supported(grad_down, grad_mid, la.mT):
                 grad_down = lora_kernels.lora_add(grad_down, grad_mid, la.mT, inplace=True)
             else:
@@ -381,7 +394,10 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             hadamard, grad_fn, grad_h2 = triton_fuse_silu_backward(
                 S["gate_lora_a"], W["gate"][4], S["gate_main_q"], S["gate_main_s"],
                 S["up_lora_a"], W["up"][4], S["up_main_q"], S["up_main_s"], grad_down, q_bit)
-            G["down"] = (hadamard.to(wd.dtype).mT @ grad_mid, grad_b_down)
+            if fast and lora_kernels.contract_supported(hadamard, hadamard.shape[-1], r):
+                G["down"] = (lora_kernels.lora_products(hadamard, u=grad_mid)[0].t(), grad_b_down)
+            else:
+                G["down"] = (hadamard.to(wd.dtype).mT @ grad_mid, grad_b_down)
             del hadamard, grad_down
         else:
             if spec.mode == "intra_inter":
@@ -396,17 +412,16 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             grad_h2 = grad_down * fn
             grad_fn = silu_backward(gate, grad_h1)
             del grad_down, up, fn, gate, grad_h1
-        x_norm_2 = deq("x_norm_2")
-        grad_x2 = back("gate", x_norm_2, S["gate_lora_a"], grad_fn)
-        grad_x2 = grad_x2 + back("up", x_norm_2, S["up_lora_a"], grad_h2)
-        del x_norm_2, grad_fn, grad_h2
+        grad_x2 = back("gate", "x_norm_2", S["gate_lora_a"], grad_fn)
+        grad_x2 = grad_x2 + back("up", "x_norm_2", S["up_lora_a"], grad_h2)
+        del grad_fn, grad_h2
         x_medium = channel_base_restored("x_medium")
         grad_norm_2, grad_nw2 = norm_backward(grad_x2, x_medium, norm_weight_2, S["rstd_2"], ctx.norm_grads[1])
         del x_medium, grad_x2
         grad_medium = grad_norm_2 + grad_output
 
         # ---- attention block -------------------------------------------------------------------
-        grad_o = back("o", deq("o"), S["o_lora_a"], grad_medium)
+        grad_o = back("o", "o", S["o_lora_a"], grad_medium)
         grad_o = hidden_to_head_shape(grad_o, H)
 
         def rebuilt(name, heads):
@@ -451,11 +466,10 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
         grad_k = rope_backward(grad_k.transpose(1, 2), cos, sin).transpose(1, 2)
         grad_q, grad_k, grad_v = (head_to_hidden_shape(t) for t in (grad_q, grad_k, grad_v))
 
-        x_norm_1 = deq("x_norm_1")
-        grad_x = back("q", x_norm_1, S["q_lora_a"], grad_q)
-        grad_x += back("k", x_norm_1, S["k_lora_a"], grad_k)
-        grad_x += back("v", x_norm_1, S["v_lora_a"], grad_v)
-        del x_norm_1, grad_q, grad_k, grad_v
+        grad_x = back("q", "x_norm_1", S["q_lora_a"], grad_q)
+        grad_x += back("k", "x_norm_1", S["k_lora_a"], grad_k)
+        grad_x += back("v", "x_norm_1", S["v_lora_a"], grad_v)
+        del grad_q, grad_k, grad_v
         x = channel_base_restored("x")
         grad_norm_1, grad_nw1 = norm_backward(grad_x, x, norm_weight_1, S["rstd_1"], ctx.norm_grads[0])
         grad_input = grad_norm_1 + grad_medium

@@ -213,8 +213,16 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
                                                                       S[name + "_idx"], q_bit)
 
         def back(name, inp, inp_lora_a, grad_y):
+            """Backward of projection `name`; `inp` is its input or the name the layer saved it under
+            (a compressed input is then read from its codes, not dequantised)."""
             w, qs, la, lb = W[name]
-            G[name + "_a"], G[name + "_b"], gx = lora_backward(w, qs, la, lb, inp, inp_lora_a, grad_y)
+            codes = None
+            if isinstance(inp, str):
+                if inp + "_raw" in S:
+                    inp = S[inp + "_raw"]
+                else:
+                    codes, inp = (S[inp + "_q"], S[inp + "_s"], None, q_bit), None
+            G[name + "_a"], G[name + "_b"], gx = lora_backward(w, qs, la, lb, inp, inp_lora_a, grad_y, x_codes=codes)
             return gx
 
         def rebuilt(name):
@@ -240,13 +248,13 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
         del fn
         grad_fn = gelu_backward(up, grad_down)
         del up, grad_down
-        grad_up = back("up", deq("x_medium"), S["up_lora_a"], grad_fn)
+        grad_up = back("up", "x_medium", S["up_lora_a"], grad_fn)
         grad_medium = grad_ln2 + grad_up
         del grad_ln2, grad_up, grad_fn
         grad_ln1, _, _ = layernorm_backward(grad_medium, deq_cb("o_final"), nw1, nb1, S["mean_1"], S["rstd_1"], True, _EPS,
                                             ctx.num_warps, ctx.block_size)
         del grad_medium
-        grad_o = hidden_to_head_shape(back("o", deq("o"), S["o_lora_a"], grad_ln1), H)
+        grad_o = hidden_to_head_shape(back("o", "o", S["o_lora_a"], grad_ln1), H)
 
         if whole:
             v = deq("v", is_head=True, num_heads=H)
@@ -272,10 +280,9 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
         del grad_s, q, k
         grad_q, grad_k, grad_v = (head_to_hidden_shape(t) for t in (grad_q, grad_k, grad_v))
 
-        x = deq("x")
-        grad_x = back("q", x, S["q_lora_a"], grad_q)
-        grad_x += back("k", x, S["k_lora_a"], grad_k)
-        grad_x += back("v", x, S["v_lora_a"], grad_v)
+        grad_x = back("q", "x", S["q_lora_a"], grad_q)
+        grad_x += back("k", "x", S["k_lora_a"], grad_k)
+        grad_x += back("v", "x", S["v_lora_a"], grad_v)
         grad_input = grad_x + grad_ln1
 
         def five(n):

@@ -4,7 +4,10 @@ No counterpart module in the reference: it computes `x_main + x_lora_a @ w_lora_
 (models/utils/compute_utils.py:21-24), quantises `x_main` with a separate call
 (models/llama/fused_llama_layer_intra_inter_full_fuse.py:128-140) and in backward dequantises and
 adds again (:416-417, :439-441, :447-449), each step a pass over the tensor.  The functions here give
-the same tensors, bit for bit, from one pass each."""
+the same tensors, bit for bit, from one pass each.
+
+`lora_products` / `lora_product_from_codes` are the rank-R GEMMs of lora_forward / lora_backward
+(compute_utils.py:22, :30-33) as one streaming pass over the wide operand."""
 import torch
 
 from .. import _lib
@@ -113,3 +116,66 @@ def lora_add_restore(q, scale, xa, b, zero_point=None, quantize_bit=8):
     _lib.call("hyc_lora_add_restore", xa.data_ptr(), b.data_ptr(), bt, q.data_ptr(), s.data_ptr(), _lib.ptr(z),
               y.data_ptr(), B * M, n, r, quantize_bit, _lib.stream_of(q))
     return y
+
+
+def contract_supported(x, n, r):
+    """Whether lora_products takes a wide operand of this dtype / width and this rank."""
+    return x.is_cuda and x.dtype == BF16 and n % 32 == 0 and 2 <= r <= 64 and r % 2 == 0 and x.numel() > 0
+
+
+def _contract(x, codes, u, v, T, n, r, dev):
+    want1, want2 = u is not None, v is not None
+    vt = 0
+    if want1:
+        u = _prep(u, "u")
+        if u.shape[-1] != r or u.numel() != T * r:
+            raise ValueError(f"u must be [T, {r}] with T = {T}, got {tuple(u.shape)}")
+    if want2:
+        if tuple(v.shape) != (r, n):
+            raise ValueError(f"v must be [{r}, {n}], got {tuple(v.shape)}")
+        v, vt = _lora_b(v)
+    nbytes = _lib.lib().hyc_lora_contract_workspace(T, n, r, int(want1), int(want2))
+    ws = torch.empty(max(nbytes, 16), device=dev, dtype=torch.uint8)
+    p1 = torch.empty((r, n), device=dev, dtype=BF16) if want1 else None
+    p2 = torch.empty((T, r), device=dev, dtype=BF16) if want2 else None
+    q, s, z, bits = codes if codes is not None else (None, None, None, 0)
+    _lib.call("hyc_lora_contract", _lib.ptr(x), _lib.ptr(q), _lib.ptr(s), _lib.ptr(z), bits, _lib.ptr(u), _lib.ptr(v), vt,
+              _lib.ptr(p1), _lib.ptr(p2), ws.data_ptr(), ws.numel(), T, n, r, _lib.stream_of(ws))
+    return p1, p2
+
+
+def lora_products(x, u=None, v=None):
+    """x [..., N] bf16 read once -> (u^T x as [R, N] or None, x v^T as [..., R] or None), u [..., R], v [R, N]
+    (a `weight.T` view of an [N, R] weight is read in place).  fp32 accumulation over the whole
+    contraction, one bf16 rounding."""
+    _lib.require_gpu(x, u, v)
+    if u is None and v is None:
+        raise ValueError("nothing to compute: pass u, v or both")
+    n = x.shape[-1]
+    r = u.shape[-1] if u is not None else v.shape[0]
+    if n % 32 or r % 2 or not 2 <= r <= 64:
+        raise ValueError(f"width must be a multiple of 32 and the rank even within 2..64, got {n}, {r}")
+    lead = tuple(x.shape[:-1])
+    x = _prep(x, "x")
+    T = x.numel() // n
+    p1, p2 = _contract(x, None, u, v, T, n, r, x.device)
+    return p1, (p2.reshape(*lead, r) if p2 is not None else None)
+
+
+def lora_product_from_codes(q, scale, u, zero_point=None, quantize_bit=8):
+    """u^T . DQ(q) as [R, N] straight from packed codes q [B, M, N*bits/8] (what
+    decompression_dequantization[_with_zero_point](q, scale[, zero_point]) would expand first)."""
+    if quantize_bit not in (2, 4, 8):
+        raise ValueError(f"quantize_bit must be 2, 4 or 8, got {quantize_bit}")
+    _lib.require_gpu(q, scale, u, zero_point)
+    B, M, nbytes = q.shape
+    n = scale.shape[-1]
+    if nbytes * 8 != n * quantize_bit or q.dtype != torch.uint8:
+        raise ValueError(f"packed codes must be uint8 of width {n * quantize_bit // 8}, got {q.dtype} {nbytes}")
+    r = u.shape[-1]
+    if n % 32 or r % 2 or not 2 <= r <= 64:
+        raise ValueError(f"width must be a multiple of 32 and the rank even within 2..64, got {n}, {r}")
+    s = _vec(scale, n, "scale")
+    z = None if zero_point is None else _vec(zero_point, n, "zero point")
+    p1, _ = _contract(None, (q.contiguous(), s, z, quantize_bit), u, None, B * M, n, r, q.device)
+    return p1

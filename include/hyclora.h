@@ -414,6 +414,32 @@ int hyc_lora_add_restore(const void *xa, const void *b, int b_transposed, const 
                          const void *scale, const void *zero_point, void *y, int64_t T, int64_t N,
                          int64_t R, int q_bit, void *stream);
 
+/* ---------------------------------------------------------------------------------------
+ * The skinny LoRA products that stream a whole [T, N] tensor X for a rank-R result, from one read
+ * of X and with fp32 accumulation over the whole contraction:
+ *     p1 = bf16( U^T . X )   [R, N]      U bf16 [T, R]
+ *     p2 = bf16( X . V^T )   [T, R]      V bf16 [R, N] (v_transposed 0) or [N, R] (v_transposed 1)
+ * X is dense bf16 [T, N] (x), or - p1 only - the packed codes of hyc_quant_pack (q, scale,
+ * optional zero_point, q_bit; x NULL), dequantised in registers to the value hyc_unpack_dequant
+ * gives.  Pass p1 or p2 as NULL to skip that product.
+ *
+ * Replaces the rank-R GEMMs of lora_forward / lora_backward (models/utils/compute_utils.py:22,
+ * :30-33): x @ A (p2, V = lora_A.weight), grad_y @ B^T with xa^T @ grad_y (p2 and p1 of X = grad_y),
+ * x^T @ grad_medium (p1), the last one without the decompression_dequantization call in front of it
+ * (models/llama/fused_llama_layer_intra_inter_full_fuse.py:375-383, :469-481).  The reference
+ * rounds per batch element and sums the batch in bf16; here the sum over all T rows is one fp32
+ * accumulation rounded once.
+ *   R even, 2..64; N % 32 == 0; any T.
+ *   workspace: device scratch of hyc_lora_contract_workspace(T, N, R, p1 != NULL, p2 != NULL) bytes,
+ *   16-byte aligned, contents undefined on entry and exit; partial sums are combined in a fixed
+ *   order (no atomics), so results are reproducible.
+ */
+int64_t hyc_lora_contract_workspace(int64_t T, int64_t N, int64_t R, int want_p1, int want_p2);
+int hyc_lora_contract(const void *x, const void *q, const void *scale, const void *zero_point, int q_bit,
+                      const void *u, const void *v, int v_transposed, void *p1, void *p2,
+                      void *workspace, int64_t workspace_bytes, int64_t T, int64_t N, int64_t R,
+                      void *stream);
+
 #ifdef __cplusplus
 }
 #endif

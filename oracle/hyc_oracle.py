@@ -402,6 +402,16 @@ def lora_add(x_main, xa, b):
     return x_main.to(BF16) + _lora_term(xa, b)
 
 
+def lora_products(x, u=None, v=None):
+    """The rank-R products of lora_forward / lora_backward over a wide operand x [T, N]
+    (models/utils/compute_utils.py:22, :30-33), accumulated in float64 and rounded once:
+    u^T x [R, N] (xa^T @ grad_y, x^T @ grad_medium) and x v^T [T, R] (x @ A, grad_y @ B^T)."""
+    x2 = x.reshape(-1, x.shape[-1]).double()
+    p1 = None if u is None else (u.reshape(-1, u.shape[-1]).double().t() @ x2).to(BF16)
+    p2 = None if v is None else (x2 @ v.double().t()).to(BF16).reshape(*x.shape[:-1], v.shape[0])
+    return p1, p2
+
+
 def fused_fwd(xa1, b1, x1, s1, xa2, b2, x2, s2, q_bit):
     """triton_fuse_silu_forward (…forward_kernels.py:104-146,152-182) -> (q1, q2, o)."""
     x1 = x1.to(BF16); x2 = x2.to(BF16)
