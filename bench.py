@@ -43,7 +43,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=1000,
                     help="untimed steps; ~50 ms of work lets the GPU reach its steady clocks (20 steps do not)")
     ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU-oracle timing (for profiler runs)")
-    ap.add_argument("--only", choices=["all", "roundtrip", "quant", "fused", "copy", "layers", "stack"], default="all",
+    ap.add_argument("--only", choices=["all", "roundtrip", "quant", "fused", "lora", "copy", "layers", "stack"], default="all",
                     help="restrict the run to one part (for profiler runs)")
     ap.add_argument("--layer-case", default="", help="with --only layers: run only the cases whose name contains this")
     ap.add_argument("--layer-arm", choices=["both", "plain", "compressed"], default="both",
@@ -523,6 +523,87 @@ def main():
                  "note": "the fused kernels also produce/consume the 4-bit saved activations; the torch arm keeps bf16"}
         del sets, saved
 
+    lora = None
+    if args.only in ("all", "lora"):
+        # The LoRA kernels around a projection's frozen part, at the two widths of the layer (hidden
+        # 4096, intermediate 11008), beside the torch / library calls they replace.  All arms are
+        # timed as HIP-graph replays (the kernels run 5-40 us, less than an eager launch costs).
+        lora = {}
+        Kl = 40
+        for wname, Nw in (("n4096", H), ("n11008", N)):
+            NBl = 4
+            x_l = [randn(B, M, Nw) for _ in range(NBl)]
+            y_l = [torch.empty(B, M, Nw, device=dev, dtype=BF16) for _ in range(NBl)]
+            q_l = [torch.empty(B, M, Nw * QB // 8, device=dev, dtype=torch.uint8) for _ in range(NBl)]
+            xa = randn(B, M, R)
+            w_b = randn(Nw, R, scale=0.05)                     # lora_B.weight as nn.Linear keeps it: [N, R]
+            b_view = w_b.t()                                   # the [R, N] view the layers pass around
+            s_l = cf.get_statistics_only_quant(x_l[0], QB, 'per-channel').reshape(-1).contiguous()
+            p1 = torch.empty(R, Nw, device=dev, dtype=BF16)
+            p2 = torch.empty(B * M, R, device=dev, dtype=BF16)
+            ws_bytes = L.hyc_lora_contract_workspace(T, Nw, R, 1, 1)
+            ws = torch.empty(ws_bytes, device=dev, dtype=torch.uint8)
+            El = T * Nw
+
+            def c_add(i, st):
+                j = i % NBl
+                assert L.hyc_lora_add(xa.data_ptr(), w_b.data_ptr(), 1, x_l[j].data_ptr(), y_l[j].data_ptr(), T, Nw, R, st) == 0
+
+            def c_add_quant(i, st):
+                j = i % NBl
+                assert L.hyc_lora_add_quant(xa.data_ptr(), w_b.data_ptr(), 1, x_l[j].data_ptr(), s_l.data_ptr(), None,
+                                            q_l[j].data_ptr(), y_l[j].data_ptr(), T, Nw, R, QB, st) == 0
+
+            def c_add_restore(i, st):
+                j = i % NBl
+                assert L.hyc_lora_add_restore(xa.data_ptr(), w_b.data_ptr(), 1, q_l[j].data_ptr(), s_l.data_ptr(), None,
+                                              y_l[j].data_ptr(), T, Nw, R, QB, st) == 0
+
+            def c_both(i, st):
+                j = i % NBl
+                assert L.hyc_lora_contract(x_l[j].data_ptr(), None, None, None, 0, xa.data_ptr(), w_b.data_ptr(), 1,
+                                           p1.data_ptr(), p2.data_ptr(), ws.data_ptr(), ws_bytes, T, Nw, R, st) == 0
+
+            def c_codes(i, st):
+                j = i % NBl
+                assert L.hyc_lora_contract(None, q_l[j].data_ptr(), s_l.data_ptr(), None, QB, xa.data_ptr(), None, 0,
+                                           p1.data_ptr(), None, ws.data_ptr(), ws_bytes, T, Nw, R, st) == 0
+
+            def on(st, fn):
+                with torch.cuda.stream(torch.cuda.ExternalStream(st)):
+                    fn()
+
+            def t_add(i, st):
+                on(st, lambda: torch.add(x_l[i % NBl], xa @ b_view, out=y_l[i % NBl]))
+
+            def t_quant(i, st):
+                on(st, lambda: cf.compression_quantization(x_l[i % NBl], s_l, QB))
+
+            def t_dequant(i, st):
+                on(st, lambda: cf.decompression_dequantization(q_l[i % NBl], s_l, QB))
+
+            def t_both(i, st):
+                on(st, lambda: (x_l[i % NBl] @ b_view.mT, (xa.mT @ x_l[i % NBl]).sum(0)))
+
+            def t_xt(i, st):
+                on(st, lambda: (x_l[i % NBl].mT @ xa).sum(0))
+
+            e = {}
+            for key, fn, nbytes in (("lora_add", c_add, 4 * El), ("lora_add_quant", c_add_quant, (4 + QB / 8) * El),
+                                    ("lora_add_restore", c_add_restore, (2 + QB / 8) * El),
+                                    ("contract_both_products", c_both, 2 * El), ("contract_from_codes", c_codes, QB / 8 * El)):
+                fn(0, stream)                                   # once eagerly: nothing may initialise during capture
+                torch.cuda.synchronize()
+                ms, _ = timed_graph(fn, Kl, 200)
+                e[key] = {"ms": ms, "GBps": nbytes / ms / 1e6}
+            for key, fn in (("torch_add_after_lora_gemm", t_add), ("quantiser_alone", t_quant), ("dequantiser_alone", t_dequant),
+                            ("torch_both_products", t_both), ("torch_xT_grad_medium", t_xt)):
+                fn(0, stream)
+                torch.cuda.synchronize()
+                e[key] = {"ms": timed_graph(fn, Kl, 200)[0]}
+            lora[wname] = e
+            del x_l, y_l, q_l, ws
+
     if args.only == "all":
         Kx, Wx = max(K // 4, 10), max(W // 4, 3)
         x_h = [randn(B, M, H) for _ in range(4)]
@@ -633,6 +714,7 @@ def main():
         "roofline": roofline,
         "cpu_baseline": cpu,
         "fused": fused,
+        "lora": lora,
         "kernels": kernels,
         "layers": layers,
         "stack": stack,
