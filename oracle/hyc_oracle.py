@@ -33,6 +33,9 @@ Pinning status (what independent evidence holds each function in place):
   * rope: pinned against the textbook rotate-half form x*cos + rotate_half(x)*sin with
     full-width tables, against an explicit complex-number rotation in float64, and by
     norm preservation / forward-then-backward identity (tests/test_oracle_rope.py).
+  * lora_add / lora_products: a library matmul of the operands (float32 rounded to bf16 before
+    the add, as lora_forward does; float64 for the products) - they reduce to library routines,
+    and the CPU tests check them against explicit loops on small inputs (tests/test_oracle_lora.py).
 The reference ships no tests, golden vectors or CPU implementation of its Triton
 kernels, so there is nothing of its own to check against.
 """
