@@ -547,7 +547,7 @@ def main():
 
             def c_add(i, st):
                 j = i % NBl
-                assert L.hyc_lora_add(xa.data_ptr(), w_b.data_ptr(), 1, x_l[j].data_ptr(), y_l[j].data_ptr(), T, Nw, R, st) == 0
+                assert L.hyc_lora_add(xa.data_ptr(), w_b.data_ptr(), 1, x_l[j].data_ptr(), None, y_l[j].data_ptr(), T, Nw, R, st) == 0
 
             def c_add_quant(i, st):
                 j = i % NBl

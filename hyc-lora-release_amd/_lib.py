@@ -61,7 +61,7 @@ _SIGNATURES = {
     "hyc_lora_silu_mul_bwd": (_I, [_P] * 12 + [_L, _L, _L, _I, _I, _P]),
     "hyc_lora_contract_workspace": (_L, [_L, _L, _L, _I, _I]),
     "hyc_lora_contract": (_I, [_P, _P, _P, _P, _I, _P, _P, _I, _P, _P, _P, _L, _L, _L, _L, _P]),
-    "hyc_lora_add": (_I, [_P, _P, _I, _P, _P, _L, _L, _L, _P]),
+    "hyc_lora_add": (_I, [_P, _P, _I, _P, _P, _P, _L, _L, _L, _P]),
     "hyc_lora_add_quant": (_I, [_P, _P, _I] + [_P] * 5 + [_L, _L, _L, _I, _P]),
     "hyc_lora_add_restore": (_I, [_P, _P, _I] + [_P] * 4 + [_L, _L, _L, _I, _P]),
 }

@@ -1,6 +1,6 @@
 // LoRA add around the compressed copy of a projection's frozen part, for gfx950.
 //
-//   plain    :  y = bf16(x + bf16(xa . b))                                   (x may be y: in place)
+//   plain    :  y = bf16(x + bf16(xa . b))  [ then y = bf16(residual + y) ]   (x may be y: in place)
 //   quantise :  q = pack(code(x; s [, z])),  y as above    - x is read once for both
 //   restore  :  x = DQ(q; s [, z]),          y as above    - the dense x never reaches memory
 //
@@ -25,6 +25,7 @@ struct LoraAddArgs {
     const uint16_t* xa; const uint16_t* b;
     const uint16_t* s; const uint16_t* zp;      // steps / zero points bf16 [N] (quantise, restore)
     const uint16_t* x;                          // dense input (plain, quantise)
+    const uint16_t* res;                        // optional residual added to the sum (plain)
     uint8_t* q;                                 // packed codes: output of quantise, input of restore
     uint16_t* y;
     int64_t T;
@@ -33,7 +34,7 @@ struct LoraAddArgs {
     int b_transposed;                           // b is [N, R] instead of [R, N]
 };
 
-template <int QBIT, int KSTEPS, int MODE, bool ZP, bool FAST>
+template <int QBIT, int KSTEPS, int MODE, bool ZP, bool FAST, bool RES = false>
 __device__ __forceinline__ void lora_add_rows(const LoraAddArgs& a, int64_t row_begin, int64_t row_end, int lane,
                                               int chunk, bool active, const QuantCols<QBIT>& qc, const float (&z)[8],
                                               const BOperand<KSTEPS>& B) {
@@ -43,16 +44,18 @@ __device__ __forceinline__ void lora_add_rows(const LoraAddArgs& a, int64_t row_
     constexpr float kHalf = (float)(1 << (QBIT - 1));
     const PackedSlot<QBIT> slot(chunk);
     for (int64_t row0 = row_begin; row0 < row_end; row0 += kTileRows) {
-        u32x4 xv[4];
+        u32x4 xv[4], rv[RES ? 4 : 1];
         u32x2 w[4];
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
             const int64_t t = row0 + 4 * g + v;
             xv[v] = u32x4{0, 0, 0, 0};
             w[v] = u32x2{0, 0};
+            if constexpr (RES) rv[v] = u32x4{0, 0, 0, 0};
             if (active && t < row_end) {
                 if constexpr (MODE == kAddRestore) w[v] = ld8(a.q + t * row_bytes + slot.offset);
                 else xv[v] = ld16_nt(a.x + t * a.N + col0);
+                if constexpr (RES) rv[v] = ld16_nt(a.res + t * a.N + col0);
             }
         }
         uint32_t L[4][4];
@@ -80,8 +83,15 @@ __device__ __forceinline__ void lora_add_rows(const LoraAddArgs& a, int64_t row_
                 codes_to_words<QBIT, ZP, FAST>(f, qc, z, lo, hi);
                 store_packed<QBIT, true>(a.q + tq * row_bytes, chunk, live, lo, hi);
             }
+            if constexpr (RES) {
+                float r[8];
+                unpack8(rv[v], r);
 #pragma unroll
-            for (int j = 0; j < 8; ++j) y[j] = f[j] + lora_elem(L[v], j);
+                for (int j = 0; j < 8; ++j) y[j] = r[j] + rbf(f[j] + lora_elem(L[v], j));
+            } else {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) y[j] = f[j] + lora_elem(L[v], j);
+            }
             if (live) st16_nt(a.y + t * a.N + col0, pack8(y));
         }
     }
@@ -124,6 +134,12 @@ __global__ __launch_bounds__(kAddThreads) void lora_add_kernel(const LoraAddArgs
             return;
         }
     }
+    if constexpr (MODE == kAddPlain) {
+        if (a.res) {
+            lora_add_rows<QBIT, KSTEPS, MODE, ZP, false, true>(a, row_begin, row_end, lane, chunk, active, qc, z, B);
+            return;
+        }
+    }
     lora_add_rows<QBIT, KSTEPS, MODE, ZP, false>(a, row_begin, row_end, lane, chunk, active, qc, z, B);
 }
 
@@ -146,6 +162,7 @@ static int add_launch(LoraAddArgs& a, int64_t T, int64_t N, int64_t R, int q_bit
     if (!a.xa || !a.b || !a.y) return HYC_ERR_NULL;
     if (MODE != kAddRestore && !a.x) return HYC_ERR_NULL;
     if (MODE != kAddPlain && (!a.q || !a.s)) return HYC_ERR_NULL;
+    if (a.res && !aligned16(a.res)) return HYC_ERR_ALIGN;
     if (!(a.b_transposed ? (reinterpret_cast<uintptr_t>(a.b) & 7u) == 0 : aligned16(a.b)) || !aligned16(a.y) || (a.x && !aligned16(a.x)) || (a.s && !aligned16(a.s)) ||
         (a.zp && !aligned16(a.zp)))
         return HYC_ERR_ALIGN;
@@ -186,11 +203,12 @@ int tune_add(const char* key, int value) {
 
 using namespace hyc;
 
-extern "C" int hyc_lora_add(const void* xa, const void* b, int b_transposed, const void* x, void* y, int64_t T,
-                            int64_t N, int64_t R, void* stream) {
+extern "C" int hyc_lora_add(const void* xa, const void* b, int b_transposed, const void* x, const void* residual,
+                            void* y, int64_t T, int64_t N, int64_t R, void* stream) {
     LoraAddArgs a{};
     a.b_transposed = b_transposed;
     a.xa = (const uint16_t*)xa; a.b = (const uint16_t*)b; a.x = (const uint16_t*)x; a.y = (uint16_t*)y;
+    a.res = (const uint16_t*)residual;
     return add_launch<kAddPlain>(a, T, N, R, 8, stream);
 }
 

@@ -295,42 +295,48 @@ __global__ __launch_bounds__(kCtThreads) void lora_contract_kernel(const Contrac
 }
 
 // out[i][c] = bf16( sum_k part[k][i][c] ), i < rows_out, c < cols_out, partial planes of
-// [rows_part][cols_part] floats; two such reductions per launch (the second may be empty).
+// [rows_part][cols_part] floats; two such reductions per launch (either may be empty).
 struct ReduceJob {
     const float* part; uint16_t* out;
     int64_t rows_out, rows_part;
     int cols_out, cols_part, planes;
     int64_t blocks;
 };
+// A thread owns W neighbouring outputs of one row (cols_out % W == 0) and reads one W-wide vector
+// per plane; planes are added in index order.
+template <int W>
 __global__ __launch_bounds__(256) void contract_reduce_kernel(const ReduceJob j0, const ReduceJob j1) {
+    typedef float fvec __attribute__((ext_vector_type(W)));
     const bool second = (int64_t)blockIdx.x >= j0.blocks;
     const ReduceJob& jb = second ? j1 : j0;
     const int64_t blk = second ? blockIdx.x - j0.blocks : blockIdx.x;
     const int64_t n_out = jb.rows_out * jb.cols_out;
-    const int64_t idx = (blk * 256 + threadIdx.x) * 2;            // two neighbouring outputs per thread
+    const int64_t idx = (blk * 256 + threadIdx.x) * W;
     if (idx >= n_out) return;
     const int64_t plane = jb.rows_part * (int64_t)jb.cols_part;
-    // planes are added in index order; loads are issued eight planes at a time
-    const int64_t i0 = idx / jb.cols_out, i1 = (idx + 1) / jb.cols_out;
-    const float* p0 = jb.part + i0 * jb.cols_part + (idx - i0 * jb.cols_out);
-    const float* p1 = idx + 1 < n_out ? jb.part + i1 * jb.cols_part + (idx + 1 - i1 * jb.cols_out) : p0;
-    float sum[2] = {0.0f, 0.0f};
+    const int64_t i = idx / jb.cols_out;
+    const float* p = jb.part + i * jb.cols_part + (idx - i * jb.cols_out);
+    float sum[W];
+#pragma unroll
+    for (int e = 0; e < W; ++e) sum[e] = 0.0f;
     int k = 0;
-    for (; k + 8 <= jb.planes; k += 8) {
-        float v0[8], v1[8];
+    for (; k + 4 <= jb.planes; k += 4) {                    // four planes in flight
+        fvec v[4];
 #pragma unroll
-        for (int e = 0; e < 8; ++e) { v0[e] = p0[(k + e) * plane]; v1[e] = p1[(k + e) * plane]; }
+        for (int u = 0; u < 4; ++u) v[u] = *reinterpret_cast<const fvec*>(p + (k + u) * plane);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) { sum[0] += v0[e]; sum[1] += v1[e]; }
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int e = 0; e < W; ++e) sum[e] += v[u][e];
     }
-    for (; k < jb.planes; ++k) { sum[0] += p0[k * plane]; sum[1] += p1[k * plane]; }
-    const uint32_t pk = pk_bf16(sum[0], sum[1]);
-    if (idx + 1 < n_out && (idx & 1) == 0 && (reinterpret_cast<uintptr_t>(jb.out + idx) & 3u) == 0) {
-        *reinterpret_cast<uint32_t*>(jb.out + idx) = pk;
-    } else {
-        jb.out[idx] = (uint16_t)(pk & 0xffffu);
-        if (idx + 1 < n_out) jb.out[idx + 1] = (uint16_t)(pk >> 16);
+    for (; k < jb.planes; ++k) {
+        const fvec v = *reinterpret_cast<const fvec*>(p + k * plane);
+#pragma unroll
+        for (int e = 0; e < W; ++e) sum[e] += v[e];
     }
+    uint32_t* out = reinterpret_cast<uint32_t*>(jb.out + idx);
+#pragma unroll
+    for (int e = 0; e < W; e += 2) out[e / 2] = pk_bf16(sum[e], sum[e + 1]);
 }
 
 // ------------------------------------------------------------------------------------
@@ -422,17 +428,20 @@ extern "C" int hyc_lora_contract(const void* x, const void* q, const void* scale
     }
     if (hipGetLastError() != hipSuccess) return HYC_ERR_LAUNCH;
     ReduceJob j1{}, j2{};
+    const int w = (want2 && R % 4 != 0) ? 2 : 4;             // N % 32 == 0; R is even
     if (want1) {
         j1.part = a.part1; j1.out = (uint16_t*)p1; j1.rows_out = R; j1.rows_part = 16 * nb;
         j1.cols_out = (int)N; j1.cols_part = (int)N; j1.planes = (int)strips;
-        j1.blocks = cdiv(R * N, 512);
+        j1.blocks = cdiv(R * N, 256 * w);
     }
     if (want2) {
         j2.part = a.part2; j2.out = (uint16_t*)p2; j2.rows_out = T; j2.rows_part = T;
         j2.cols_out = (int)R; j2.cols_part = 16 * nb; j2.planes = a.groups;
-        j2.blocks = cdiv(T * R, 512);
+        j2.blocks = cdiv(T * R, 256 * w);
     }
     if (j1.blocks + j2.blocks > INT32_MAX) return HYC_ERR_SHAPE;
-    hipLaunchKernelGGL(contract_reduce_kernel, dim3((unsigned)(j1.blocks + j2.blocks)), dim3(256), 0, st, j1, j2);
+    const dim3 rgrid((unsigned)(j1.blocks + j2.blocks));
+    if (w == 4) hipLaunchKernelGGL(contract_reduce_kernel<4>, rgrid, dim3(256), 0, st, j1, j2);
+    else hipLaunchKernelGGL(contract_reduce_kernel<2>, rgrid, dim3(256), 0, st, j1, j2);
     return check_launch();
 }

@@ -51,15 +51,17 @@ def dense_weight(w: torch.Tensor, quant_state):
     return dequantize_nf4(w, quant_state)
 
 
-def lora_forward(w, w_quant_state, w_lora_a, w_lora_b, b, x):
+def lora_forward(w, w_quant_state, w_lora_a, w_lora_b, b, x, residual=None):
     """-> (x @ W^T [+ b] + (x @ A) @ B, the frozen part alone, x @ A).  Reference :18-25.  The LoRA
     product and the add are one MFMA kernel over the frozen part (bf16 operands); other dtypes
-    take the torch expression."""
+    take the torch expression.  `residual` (not in the reference's signature) is added to the first
+    result in the same pass - the `x + o_final` that follows the projection in the layers."""
     x_main, x_lora_a = lora_parts(w, w_quant_state, w_lora_a, b, x)
     w_lora_b = w_lora_b.to(x_main.dtype)
-    if lora_kernels.supported(x_main, x_lora_a, w_lora_b):
-        return lora_kernels.lora_add(x_main, x_lora_a, w_lora_b), x_main, x_lora_a
-    return x_main + x_lora_a @ w_lora_b, x_main, x_lora_a
+    if lora_kernels.supported(x_main, x_lora_a, w_lora_b) and (residual is None or residual.dtype == x_main.dtype):
+        return lora_kernels.lora_add(x_main, x_lora_a, w_lora_b, residual=residual), x_main, x_lora_a
+    y = x_main + x_lora_a @ w_lora_b
+    return (y if residual is None else residual + y), x_main, x_lora_a
 
 
 def lora_parts(w, w_quant_state, w_lora_a, b, x):
@@ -72,7 +74,7 @@ def lora_parts(w, w_quant_state, w_lora_a, b, x):
     return x_main, x @ w_lora_a.to(wt.dtype)
 
 
-def lora_backward(w, w_quant_state, w_lora_a, w_lora_b, x, x_lora_a, grad_y, x_codes=None):
+def lora_backward(w, w_quant_state, w_lora_a, w_lora_b, x, x_lora_a, grad_y, x_codes=None, accumulate=None):
     """-> (grad lora_A, grad lora_B, grad x).  Reference :28-36.
 
     With bf16 operands the rank-R products stream their wide operand once on the matrix cores:
@@ -80,7 +82,9 @@ def lora_backward(w, w_quant_state, w_lora_a, w_lora_b, x, x_lora_a, grad_y, x_c
     from x - or straight from its packed codes `x_codes = (q, scale, zero_point or None, q_bit)`,
     in which case x may be None and is never dequantised.  Those results are summed over the batch in
     fp32 and have the parameters' shapes; the torch expressions below return one gradient per batch
-    element, as the reference does, and leave the sum to autograd."""
+    element, as the reference does, and leave the sum to autograd.  `accumulate`, a running sum of
+    input gradients, is added to grad x in the pass that adds its LoRA part (`grad_x += grad_x_temp`
+    in the layers) and may be overwritten."""
     wd = dense_weight(w, w_quant_state)          # [out, in]
     dt = wd.dtype
     grad_y = grad_y.to(dt)
@@ -106,10 +110,12 @@ def lora_backward(w, w_quant_state, w_lora_a, w_lora_b, x, x_lora_a, grad_y, x_c
         else:
             grad_a = x.to(dt).mT @ grad_mid
     grad_x = grad_y @ wd
-    if lora_kernels.supported(grad_x, grad_mid, w_lora_a.mT):
-        grad_x = lora_kernels.lora_add(grad_x, grad_mid, w_lora_a.mT, inplace=True)
+    if lora_kernels.supported(grad_x, grad_mid, w_lora_a.mT) and (accumulate is None or accumulate.dtype == dt):
+        grad_x = lora_kernels.lora_add(grad_x, grad_mid, w_lora_a.mT, inplace=True, residual=accumulate)
     else:
         grad_x += grad_mid @ w_lora_a.mT
+        if accumulate is not None:
+            grad_x = accumulate + grad_x
     return grad_a, grad_b, grad_x
 
 

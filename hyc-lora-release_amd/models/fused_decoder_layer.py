@@ -122,9 +122,9 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
         raw = spec.mode == "baseline"                   # keep activations as they are
         whole = spec.mode in ("baseline", "intra")      # save whole activations, not the frozen-weight parts
 
-        def proj(name, inp):
+        def proj(name, inp, residual=None):
             w, b, qs, la, lb = W[name]
-            return lora_forward(w, qs, la, lb, b, inp)
+            return lora_forward(w, qs, la, lb, b, inp, residual=residual)
 
         def proj_quant(name, inp, zp=False):
             """Projection `name` of inp with the frozen part quantised on the way: -> (output, x @ A).
@@ -249,11 +249,9 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             o = F.scaled_dot_product_attention(q, k, v, attn_mask=attention_mask, is_causal=attention_mask is None)
             del q, k, v
         o = head_to_hidden_shape(o)
-        o_final, _, saved["o_lora_a"] = proj("o", o)
+        x_medium, _, saved["o_lora_a"] = proj("o", o, residual=x)       # x + o_proj(o) in the projection's add pass
         quant("o", o)
         del o
-        x_medium = x + o_final
-        del o_final
 
         # ---- MLP block ---------------------------------------------------------------------------
         x_norm_2, saved["rstd_2"], norm_2_done = norm_block("x_medium", "x_norm_2", x_medium, norm_weight_2)
@@ -294,11 +292,10 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
         if not norm_2_done:
             quant("x_norm_2", x_norm_2)
         del x_norm_2
-        down, _, saved["down_lora_a"] = proj("down", hadamard)
+        x_out, _, saved["down_lora_a"] = proj("down", hadamard, residual=x_medium)
         if whole:
             quant("hadamard", hadamard)
         del hadamard
-        x_out = x_medium + down
 
         ctx.names = list(saved.keys())
         ctx.save_for_backward(*saved.values(), cos, sin, norm_weight_1, norm_weight_2,
@@ -338,7 +335,7 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
                                                                     q_bit, **kw)
             return decompression_dequantization(S[name + "_q"], S[name + "_s"], q_bit, **kw)
 
-        def back(name, inp, inp_lora_a, grad_y):
+        def back(name, inp, inp_lora_a, grad_y, accumulate=None):
             """Backward of projection `name`.  `inp` is its input, or the name under which the layer
             saved that input: a compressed one is then read from its codes, not dequantised."""
             w, _, qs, la, lb = W[name]
@@ -348,7 +345,7 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
                     inp = S[inp + "_raw"]
                 else:
                     codes, inp = (S[inp + "_q"], S[inp + "_s"], S.get(inp + "_z"), q_bit), None
-            ga, gb, gx = lora_backward(w, qs, la, lb, inp, inp_lora_a, grad_y, x_codes=codes)
+            ga, gb, gx = lora_backward(w, qs, la, lb, inp, inp_lora_a, grad_y, x_codes=codes, accumulate=accumulate)
             G[name] = (ga, gb)
             return gx
 
@@ -413,7 +410,7 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             grad_fn = silu_backward(gate, grad_h1)
             del grad_down, up, fn, gate, grad_h1
         grad_x2 = back("gate", "x_norm_2", S["gate_lora_a"], grad_fn)
-        grad_x2 = grad_x2 + back("up", "x_norm_2", S["up_lora_a"], grad_h2)
+        grad_x2 = back("up", "x_norm_2", S["up_lora_a"], grad_h2, accumulate=grad_x2)
         del grad_fn, grad_h2
         x_medium = channel_base_restored("x_medium")
         grad_norm_2, grad_nw2 = norm_backward(grad_x2, x_medium, norm_weight_2, S["rstd_2"], ctx.norm_grads[1])
@@ -467,8 +464,8 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
         grad_q, grad_k, grad_v = (head_to_hidden_shape(t) for t in (grad_q, grad_k, grad_v))
 
         grad_x = back("q", "x_norm_1", S["q_lora_a"], grad_q)
-        grad_x += back("k", "x_norm_1", S["k_lora_a"], grad_k)
-        grad_x += back("v", "x_norm_1", S["v_lora_a"], grad_v)
+        grad_x = back("k", "x_norm_1", S["k_lora_a"], grad_k, accumulate=grad_x)
+        grad_x = back("v", "x_norm_1", S["v_lora_a"], grad_v, accumulate=grad_x)
         del grad_q, grad_k, grad_v
         x = channel_base_restored("x")
         grad_norm_1, grad_nw1 = norm_backward(grad_x, x, norm_weight_1, S["rstd_1"], ctx.norm_grads[0])

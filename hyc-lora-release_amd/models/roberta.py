@@ -69,9 +69,9 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
         raw = mode == "baseline"
         whole = mode in ("baseline", "intra")
 
-        def proj(name, inp):
+        def proj(name, inp, residual=None):
             w, b, qs, la, lb = W[name]
-            return lora_forward(w, qs, la, lb, b, inp)
+            return lora_forward(w, qs, la, lb, b, inp, residual=residual)
 
         def proj_quant(name, inp):
             """Projection with the frozen part quantised on the way, one kernel for codes + LoRA add
@@ -150,12 +150,11 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
             quant("v", v)
         del v
         o = head_to_hidden_shape(o)
-        o_final, _, saved["o_lora_a"] = proj("o", o)
+        o_final, _, saved["o_lora_a"] = proj("o", o, residual=x)        # o_proj(o) + x in the projection's add pass
         quant("o", o)
         del o
 
         # ---- first LayerNorm (post-norm: on the residual sum) ----------------------------------
-        o_final += x
         x_medium, saved["mean_1"], saved["rstd_1"], _, _ = layernorm_forward(o_final, norm_weight_1, norm_bias_1, _EPS)
         channel_base("o_final", o_final)
         del o_final
@@ -170,8 +169,7 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
         if whole:
             quant("up", up)
         del up
-        down, _, saved["down_lora_a"] = proj("down", fn)
-        down += x_medium
+        down, _, saved["down_lora_a"] = proj("down", fn, residual=x_medium)
         if whole:
             quant("fn", fn)
         del fn, x_medium
@@ -212,7 +210,7 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
             return outlier_addition_fuse_decompression_dequantization(S[name + "_q"], S[name + "_s"], S[name + "_o"],
                                                                       S[name + "_idx"], q_bit)
 
-        def back(name, inp, inp_lora_a, grad_y):
+        def back(name, inp, inp_lora_a, grad_y, accumulate=None):
             """Backward of projection `name`; `inp` is its input or the name the layer saved it under
             (a compressed input is then read from its codes, not dequantised)."""
             w, qs, la, lb = W[name]
@@ -222,7 +220,8 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
                     inp = S[inp + "_raw"]
                 else:
                     codes, inp = (S[inp + "_q"], S[inp + "_s"], None, q_bit), None
-            G[name + "_a"], G[name + "_b"], gx = lora_backward(w, qs, la, lb, inp, inp_lora_a, grad_y, x_codes=codes)
+            G[name + "_a"], G[name + "_b"], gx = lora_backward(w, qs, la, lb, inp, inp_lora_a, grad_y, x_codes=codes,
+                                                                 accumulate=accumulate)
             return gx
 
         def rebuilt(name):
@@ -281,8 +280,8 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
         grad_q, grad_k, grad_v = (head_to_hidden_shape(t) for t in (grad_q, grad_k, grad_v))
 
         grad_x = back("q", "x", S["q_lora_a"], grad_q)
-        grad_x += back("k", "x", S["k_lora_a"], grad_k)
-        grad_x += back("v", "x", S["v_lora_a"], grad_v)
+        grad_x = back("k", "x", S["k_lora_a"], grad_k, accumulate=grad_x)
+        grad_x = back("v", "x", S["v_lora_a"], grad_v, accumulate=grad_x)
         grad_input = grad_x + grad_ln1
 
         def five(n):

@@ -54,17 +54,22 @@ def _lora_b(b):
     return _prep(b, "b"), 0
 
 
-def lora_add(x_main, xa, b, inplace=False):
-    """bf16(x_main + bf16(xa @ b)); `inplace` overwrites x_main (contiguous bf16) and returns it."""
-    _lib.require_gpu(x_main, xa, b)
+def lora_add(x_main, xa, b, inplace=False, residual=None):
+    """bf16(x_main + bf16(xa @ b)), then - with a residual of x_main's shape - bf16(residual + that);
+    `inplace` overwrites x_main (contiguous bf16) and returns it."""
+    _lib.require_gpu(x_main, xa, b, residual)
     n = x_main.shape[-1]
     r = _check(xa, b, n)
     x = x_main if (inplace and x_main.dtype == BF16 and x_main.is_contiguous() and x_main.data_ptr() % 16 == 0) \
         else _prep(x_main, "x_main")
     y = x if inplace else torch.empty_like(x)
     xa, (b, bt) = _prep(xa, "xa"), _lora_b(b)
-    _lib.call("hyc_lora_add", xa.data_ptr(), b.data_ptr(), bt, x.data_ptr(), y.data_ptr(), x.numel() // n, n, r,
-              _lib.stream_of(x))
+    if residual is not None:
+        if residual.shape != x_main.shape:
+            raise ValueError(f"residual must have the shape of x_main {tuple(x_main.shape)}, got {tuple(residual.shape)}")
+        residual = _prep(residual, "residual")
+    _lib.call("hyc_lora_add", xa.data_ptr(), b.data_ptr(), bt, x.data_ptr(), _lib.ptr(residual), y.data_ptr(),
+              x.numel() // n, n, r, _lib.stream_of(x))
     if inplace and y is not x_main:
         x_main.copy_(y)
         return x_main

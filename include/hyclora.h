@@ -385,7 +385,8 @@ int hyc_lora_silu_mul_bwd(const void *xa1, const void *b1, const void *q1, const
 
 /* ---------------------------------------------------------------------------------------
  * LoRA add around the compressed copy of a projection's frozen part:
- *     hyc_lora_add          y = bf16(x + bf16(xa . b))                     (y may be x: in place)
+ *     hyc_lora_add          y = bf16(x + bf16(xa . b)), and with a residual (bf16 [T, N], or NULL)
+ *                           y = bf16(residual + bf16(x + bf16(xa . b)))    (y may be x or residual: in place)
  *     hyc_lora_add_quant    the same y, and q = pack(code(x; scale [, zero_point])) from the one
  *                           read of x (code rule and layout of hyc_quant_pack)
  *     hyc_lora_add_restore  x = value of hyc_unpack_dequant(q; scale [, zero_point]), then the
@@ -397,7 +398,9 @@ int hyc_lora_silu_mul_bwd(const void *xa1, const void *b1, const void *q1, const
  * frozen part (models/llama/fused_llama_layer_intra_inter_full_fuse.py:128-140; zero-point form
  * models/llama_flash_attn/fused_llama_layer_intra_inter.py:129-138); the rebuild of q, k, v, gate,
  * up in backward (…full_fuse.py:416-417, :439-441, :447-449); and `grad_x += grad_medium @ A^T`
- * of lora_backward (compute_utils.py:34-35) through the plain form.
+ * of lora_backward (compute_utils.py:34-35) through the plain form; the residual covers the add that
+ * follows a projection (`x + o_final`, `x_medium + down`, …full_fuse.py:198,250) and the running sum of
+ * input gradients (`grad_x += grad_x_temp`, :477,481).
  *   xa bf16 [T, R] contiguous;  x, y bf16 [T, N] contiguous;
  *   b bf16 [R, N] contiguous (b_transposed 0) or [N, R] contiguous (b_transposed 1: the layout
  *   torch.nn.Linear keeps lora_B.weight in, so no copy of the adapter is needed);
@@ -405,8 +408,8 @@ int hyc_lora_silu_mul_bwd(const void *xa1, const void *b1, const void *q1, const
  *   R: multiple of 4, 4..64; N % 32 == 0; any T.
  * Tuning key "add_rows_per_wave" (multiple of 16, default 32).
  */
-int hyc_lora_add(const void *xa, const void *b, int b_transposed, const void *x, void *y, int64_t T,
-                 int64_t N, int64_t R, void *stream);
+int hyc_lora_add(const void *xa, const void *b, int b_transposed, const void *x, const void *residual,
+                 void *y, int64_t T, int64_t N, int64_t R, void *stream);
 int hyc_lora_add_quant(const void *xa, const void *b, int b_transposed, const void *x, const void *scale,
                        const void *zero_point, void *q, void *y, int64_t T, int64_t N, int64_t R,
                        int q_bit, void *stream);

@@ -94,6 +94,25 @@ def test_add_with_quantiser_and_from_codes(K, dev, q_bit, zp, dims):
     assert np.array_equal(bits(r), bits(K.add(x_hat, d(xa), d(b)))), "same as dequantise, then add"
 
 
+@pytest.mark.parametrize("dims", [(2, 64, 256, 16), (1, 37, 160, 16), (3, 50, 4096, 16), (1, 5, 96, 4)])
+def test_plain_add_with_residual(K, dev, dims):
+    """y = residual + (x + xa.b), each sum rounded to bf16: bit-identical to the plain form followed
+    by torch's add, out of place and in place."""
+    B, M, N, R = dims
+    main, xa, b = inputs(N + 3 * R, B, M, N, R)
+    res = torch.randn(B, M, N, generator=torch.Generator().manual_seed(7)).to(BF16)
+    d = lambda t: t.to(dev)
+    two_steps = d(res) + K.add(d(main), d(xa), d(b))
+    y = K.add(d(main), d(xa), d(b), residual=d(res))
+    assert np.array_equal(bits(y), bits(two_steps))
+    mostly_same_bits(y, res + O.lora_add(main, xa, b), "residual + lora_add vs oracle")
+    x = d(main)
+    y2 = K.add(x, d(xa), d(b), inplace=True, residual=d(res))
+    assert y2.data_ptr() == x.data_ptr() and np.array_equal(bits(y2), bits(two_steps))
+    with pytest.raises(ValueError):
+        K.add(d(main), d(xa), d(b), residual=d(res)[:, :1])
+
+
 @pytest.mark.parametrize("R", [4, 16, 32, 64])
 def test_lora_b_in_linear_layout(K, dev, R):
     """A [R, N] view of an [N, R] contiguous weight - what `lora_B.weight.T` is - is read where it
