@@ -19,9 +19,11 @@ as one function with three switches:
                                       product in one fused kernel each way
                                                       (fused_llama_layer_intra_inter_full_fuse.py:218-235,359-371)
   attention   'map'   softmax map is materialised, thresholded and saved sparse (:159-176,414-432)
-              'sdpa'  no map is saved; attention is recomputed in backward; q/k main use a zero point
-                      (llama_flash_attn/fused_llama_layer_intra_inter.py:118-180 - the flash-attn
-                      kernels themselves are replaced by torch's scaled_dot_product_attention)
+              'sdpa'  no map is saved; the flash kernel's log-sum-exps are, and its backward gets the
+                      dequantised attention output; q/k main use a zero point
+                      (llama_flash_attn/fused_llama_layer_intra_inter.py:118-180, :450-468 - the
+                      flash-attn kernels themselves are replaced by the ones behind torch's
+                      scaled_dot_product_attention)
   norm weights receive gradients when they require grad (rmsnorm_updatable_kernels.py:173-220).
 
 Deliberate differences from the reference:
@@ -59,6 +61,14 @@ from .compute_utils import (head_to_hidden_shape, heads_matmul, hidden_to_head_s
                             repeat_kv, repeat_kv_backward, rope_backward, rope_forward)
 
 MODES = ("baseline", "intra", "intra_inter", "intra_inter_full_fuse")
+# Map-free attention keeps the flash kernel's row log-sum-exps for backward, whose kernel is then
+# handed the *dequantised* attention output - the reference's scheme
+# (llama_flash_attn/fused_llama_layer_intra_inter.py:450-468).  False recomputes the attention in
+# backward instead: one more attention forward per step, gradients free of that output's
+# quantisation error (q/k LoRA gradients: cosine 0.99 -> 1.0 against the uncompressed layer at 8
+# bits).  Recomputation is also what happens with an explicit mask, or where the flash kernel does not
+# take the operands.
+KEEP_ATTENTION_LSE = True
 
 
 @dataclass(frozen=True)
@@ -246,7 +256,21 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             o = heads_matmul(a, v, out_hidden=True)
             del a, v
         else:
-            o = F.scaled_dot_product_attention(q, k, v, attn_mask=attention_mask, is_causal=attention_mask is None)
+            # causal attention without a map: the flash kernel behind torch's SDPA, called through its
+            # aten entry point so that the row log-sum-exps come back and backward needs no second
+            # forward (the reference keeps flash-attn's softmax_lse the same way,
+            # llama_flash_attn/fused_llama_layer_intra_inter.py:169-180, :459-468)
+            ctx.flash = None
+            if KEEP_ATTENTION_LSE and attention_mask is None and q.is_cuda:
+                try:
+                    res = torch.ops.aten._scaled_dot_product_flash_attention(q, k, v, 0.0, True, False)
+                    o, saved["sdpa_lse"] = res[0], res[1]
+                    saved["sdpa_rng"], saved["sdpa_unused"] = res[6], res[7]
+                    ctx.flash = tuple(res[2:6])
+                except RuntimeError:
+                    ctx.flash = None
+            if ctx.flash is None:
+                o = F.scaled_dot_product_attention(q, k, v, attn_mask=attention_mask, is_causal=attention_mask is None)
             del q, k, v
         o = head_to_hidden_shape(o)
         x_medium, _, saved["o_lora_a"] = proj("o", o, residual=x)       # x + o_proj(o) in the projection's add pass
@@ -450,6 +474,15 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             grad_k = heads_matmul(grad_s.transpose(-2, -1), q, out_hidden=True)
             grad_q = heads_matmul(grad_s, k, out_hidden=True)
             del grad_s, q, k
+        elif ctx.flash is not None:
+            # the attention output handed to the backward kernel is the dequantised one, as in the
+            # reference (…intra_inter.py:450-461)
+            out = hidden_to_head_shape(deq("o"), H)
+            cum_q, cum_k, max_q, max_k = ctx.flash
+            grad_q, grad_k, grad_v = torch.ops.aten._scaled_dot_product_flash_attention_backward(
+                grad_o, q, k, v, out, S["sdpa_lse"], cum_q, cum_k, max_q, max_k, 0.0, True,
+                S["sdpa_rng"], S["sdpa_unused"])
+            del q, k, v, out, grad_o
         else:
             with torch.enable_grad():
                 q_, k_, v_ = (t.detach().requires_grad_() for t in (q, k, v))

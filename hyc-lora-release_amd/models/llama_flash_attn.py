@@ -1,8 +1,9 @@
 """Long-sequence Llama layers: no attention map is materialised or saved, q/k main are quantised
 with a zero point, norm weights receive gradients
 (models/llama_flash_attn/fused_llama_layer_{baseline,intra,intra_inter}.py).  The flash-attn varlen kernels
-of the reference are replaced by torch's scaled_dot_product_attention (its ROCm flash/CK backend);
-backward recomputes the attention instead of calling a saved-LSE backward kernel."""
+of the reference are replaced by the flash kernels behind torch's scaled_dot_product_attention, called
+through their aten entry points: forward returns the log-sum-exps, backward takes them and the
+dequantised attention output, as the reference's call does (…intra_inter.py:450-468)."""
 from .fused_decoder_layer import FusedDecoderLayer
 
 

@@ -231,6 +231,32 @@ def test_sdpa_variant_and_norm_weight_grads(dev):
         assert layer.static_value['q']['zero_point'] is not None and 'a' not in layer.static_value
 
 
+def test_map_free_backward_from_saved_lse_equals_recomputation(dev, monkeypatch):
+    """The map-free layers keep the flash kernel's log-sum-exps and call its backward directly; with
+    uncompressed activations (layer type 'baseline') that must give the gradients of recomputing the
+    attention under autograd, and with compressed ones stay within the layer's tolerance of them."""
+    import hyclora_amd  # noqa: F401
+    from hyclora_amd.models import fused_decoder_layer as fdl
+    from hyclora_amd.models import llama_flash_attn as lf
+    t = make_layer_inputs(dev, seed=5, kv_heads=2)
+    for cls, q_bit, floor in ((lf.FusedLlamaLayerBaseline, 8, 0.9999), (lf.FusedLlamaLayerIntraInter, 8, 0.97)):
+        got = {}
+        for keep in (True, False):
+            monkeypatch.setattr(fdl, "KEEP_ATTENTION_LSE", keep)
+            layer = cls()
+            layer.set_hyclora_config(config(layer.layer_type, q_bit))
+            out = run_fused(layer, t, use_mask=False)
+            got[keep] = (out, grads_of(t, out))
+        assert torch.equal(got[True][0], got[False][0])
+        for i, (g1, g0) in enumerate(zip(got[True][1], got[False][1])):
+            if g1 is None and g0 is None:
+                continue
+            rel, cos = rel_err_and_cos(g1, g0)
+            # compressed: the backward kernel is handed the dequantised attention output, as in the
+            # reference, so its row term  sum(dO * O)  carries the codes' error - direction only
+            assert cos >= floor and (floor < 0.999 or rel <= 2e-2), f"{cls.__name__} grad #{i}: rel {rel:.2e} cos {cos:.6f}"
+
+
 def test_calibration_state_machine(dev):
     import hyclora_amd  # noqa: F401
     from hyclora_amd.models import FusedLlamaLayerIntraInterFullFuse
