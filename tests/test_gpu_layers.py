@@ -211,6 +211,45 @@ def test_layer_matches_oracle_layer(dev, layer_type, q_bit, kv_heads):
         assert rel <= rel_tol and cos >= 0.999, f"{layer_type} q{q_bit} kv{kv_heads} grad {name}: rel {rel:.2e} cos {cos:.5f}"
 
 
+@pytest.mark.parametrize("layer_type", ["baseline", "intra", "intra_inter", "intra_inter_full_fuse"])
+@pytest.mark.parametrize("dims", [dict(B=3, S=40, hidden=192, heads=6, kv_heads=3, inter=320, rank=8),
+                                  dict(B=1, S=17, hidden=128, heads=2, kv_heads=2, inter=96, rank=4),
+                                  dict(B=2, S=264, hidden=256, heads=4, kv_heads=1, inter=512, rank=32)])
+def test_layer_on_ragged_shapes(dev, layer_type, dims):
+    """Shapes that fill none of the kernels' tiles evenly (rows not a multiple of 16 or 256, widths
+    not a multiple of 128, a sequence length the fused softmax does not take, ranks 4 / 8 / 32):
+    every layer type against the oracle layer (baseline: against autograd of the same graph)."""
+    import hyclora_amd  # noqa: F401
+    from hyclora_amd.models import llama
+    from oracle import layer_oracle
+    t = make_layer_inputs(dev, seed=23, **dims)
+    layer = llama.make_fused_llama_layer(config(layer_type, 4, sm_ratio=0.05, ln_ratio=0.02))
+    out = run_fused(layer, t)
+    grads = grads_of(t, out)
+    names = ["x", "norm_w1", "norm_w2"] + [f"{n}.lora_{ab}" for n in ("q", "k", "v", "o", "gate", "up", "down") for ab in "AB"]
+    if layer_type == "baseline":
+        ref_out = reference_layer(t)
+        expect = grads_of(t, ref_out)
+        expect[1] = expect[2] = None
+    else:
+        weights = {n: tuple(m.weight.detach() for m in t.P[n]) for n in t.P}
+        with torch.no_grad():
+            ref_out, G = layer_oracle.layer_forward_backward(
+                t.x.detach(), t.nw1.detach(), t.nw2.detach(), t.cos, t.sin, weights, t.mask, t.heads, t.kv_heads,
+                t.grad, mode=layer_type, q_bit=4, softmax_ratio=0.05, layernorm_ratio=0.02)
+        expect = [G["x"], None, None]
+        for n in ("q", "k", "v", "o", "gate", "up", "down"):
+            expect += [G[(n, "A")].sum(0).t(), G[(n, "B")].sum(0).t()]
+    rel, cos = rel_err_and_cos(out, ref_out)
+    assert rel <= 1e-2 and cos >= 0.9999
+    for name, got, want in zip(names, grads, expect):
+        if want is None:
+            continue
+        assert got.shape == want.shape, name
+        rel, cos = rel_err_and_cos(got, want)
+        assert rel <= 3e-2 and cos >= 0.999, f"{layer_type} {dims} grad {name}: rel {rel:.2e} cos {cos:.5f}"
+
+
 def test_sdpa_variant_and_norm_weight_grads(dev):
     import hyclora_amd  # noqa: F401
     from hyclora_amd.models import llama_flash_attn as lf
