@@ -4,6 +4,8 @@
 parameters of the reference's Triton kernels and are carried only so that callers can hand
 them back to `rmsnorm_backward` unchanged.  `mean` is an uninitialised placeholder there as
 well."""
+import weakref
+
 import torch
 
 from .. import _lib
@@ -75,10 +77,22 @@ def rmsnorm_backward(dy, x, w, m, v, needs_inputs_grad, eps, num_warps, BLOCK_SI
     return dx, None
 
 
-def outlier_table(outlier_idx, n):
-    """uint16 [n] lookup for rmsnorm_forward_compress: 1 + list position for an outlier channel, else
-    0.  Worth caching while the channel list is frozen."""
+_TABLES = {}          # id(channel-list tensor) -> (weak reference to it, its version, n, table)
+
+
+def outlier_table(outlier_idx, n, cached=False):
+    """uint16 [n] lookup for the fused norm kernels: 1 + list position for an outlier channel, else 0.
+    cached=True keeps the table with the channel-list tensor (weakly, and only while the tensor is
+    not modified in place): a frozen list is the same tensor object step after step."""
     _lib.require_gpu(outlier_idx)
+    if cached:
+        key = id(outlier_idx)
+        hit = _TABLES.get(key)
+        if hit is not None and hit[0]() is outlier_idx and hit[1] == outlier_idx._version and hit[2] == n:
+            return hit[3]
+        table = outlier_table(outlier_idx, n)
+        _TABLES[key] = (weakref.ref(outlier_idx, lambda _r, k=key: _TABLES.pop(k, None)), outlier_idx._version, n, table)
+        return table
     idx = outlier_idx.reshape(-1).to(torch.int64).contiguous()
     table = torch.empty((n,), dtype=torch.int16, device=idx.device)
     _lib.call("hyc_outlier_table", idx.data_ptr() if idx.numel() else None, idx.numel(), n, table.data_ptr(),
@@ -125,7 +139,7 @@ def rmsnorm_forward_compress(x, weight, eps, q_bit, scale_y=None, scale_x=None, 
         k = 0 if outlier_idx is None else outlier_idx.numel()
         x_out = torch.empty((b, m, k), dtype=torch.bfloat16, device=dev)
         if k and table is None:
-            table = outlier_table(outlier_idx, n)
+            table = outlier_table(outlier_idx, n, cached=True)
     _lib.call("hyc_rmsnorm_fwd_compress", x.data_ptr(), w.data_ptr(), w32, y.data_ptr(), rstd.data_ptr(), rows, n,
               float(eps), q_bit, _lib.ptr(scale_y), _lib.ptr(q_y), _lib.ptr(scale_x), _lib.ptr(q_x),
               _lib.ptr(table) if k else None, k, _lib.ptr(x_out) if k else None, _lib.stream_of(x))
