@@ -17,7 +17,7 @@ namespace hyc {
 
 constexpr int kAddThreads = 256;
 constexpr int kAddWaves = kAddThreads / kWave;
-static int g_add_rows_per_wave = 32;
+static int g_add_rows_per_wave[3] = {32, 48, 48};   // plain, quantise, restore; see hyc_set_tuning
 
 enum { kAddPlain = 0, kAddQuant = 1, kAddRestore = 2 };
 
@@ -171,7 +171,7 @@ static int add_launch(LoraAddArgs& a, int64_t T, int64_t N, int64_t R, int q_bit
     a.N = (int)N;
     a.C = (int)(N / 8);
     a.R = (int)R;
-    a.rows_per_wave = g_add_rows_per_wave;
+    a.rows_per_wave = g_add_rows_per_wave[MODE];
     const int ct = MODE == kAddPlain ? 1 : 8 / q_bit;
     a.col_tiles = (int)cdiv(cdiv(N, kTileCols), ct);
     const int64_t row_tiles = cdiv(T, (int64_t)(kAddWaves / ct) * a.rows_per_wave);
@@ -191,10 +191,13 @@ static int add_launch(LoraAddArgs& a, int64_t T, int64_t N, int64_t R, int q_bit
 }
 
 int tune_add(const char* key, int value) {
-    if (strcmp(key, "add_rows_per_wave") == 0) {
-        if (value < kTileRows || value > 65536 || value % kTileRows != 0) return HYC_ERR_ARG;
-        g_add_rows_per_wave = value;
-        return HYC_OK;
+    static const char* keys[3] = {"add_rows_per_wave", "add_quant_rows_per_wave", "add_restore_rows_per_wave"};
+    for (int m = 0; m < 3; ++m) {
+        if (strcmp(key, keys[m]) == 0) {
+            if (value < kTileRows || value > 65536 || value % kTileRows != 0) return HYC_ERR_ARG;
+            g_add_rows_per_wave[m] = value;
+            return HYC_OK;
+        }
     }
     return 1;
 }
