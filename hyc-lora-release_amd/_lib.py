@@ -26,6 +26,7 @@ class HycError(RuntimeError):
 
 
 # name -> (restype, argtypes)
+ABI_VERSION = 2          # hyc_abi_version() of the library these signatures describe
 _P, _I, _L = c_void_p, c_int, c_int64
 _SIGNATURES = {
     "hyc_error_string": (c_char_p, [_I]),
@@ -80,6 +81,12 @@ def lib() -> ctypes.CDLL:
                 f"{LIB_PATH} not found: build it with `python {(_HERE / 'build.py')}` "
                 "(hipcc, gfx950). There is no fallback implementation.")
         handle = ctypes.CDLL(str(LIB_PATH))
+        handle.hyc_abi_version.restype = ctypes.c_int
+        have = handle.hyc_abi_version()
+        if have != ABI_VERSION:
+            # calling through signatures of another revision would hand kernels misplaced arguments
+            raise RuntimeError(f"{LIB_PATH} has ABI revision {have}, these bindings are written for {ABI_VERSION}: "
+                               f"rebuild it with `python {(_HERE / 'build.py')}`")
         for name, (res, args) in _SIGNATURES.items():
             fn = getattr(handle, name)
             fn.restype = res
