@@ -49,6 +49,7 @@ struct ContractArgs {
     int64_t T;
     int N, C, R;
     int tiles_per_group, groups, v_transposed;
+    int64_t n_blocks;                    // strips * groups
 };
 
 __device__ __forceinline__ s16x4 pick_column(const u32x4 (&xv)[4], int u8) {
@@ -68,8 +69,20 @@ __global__ __launch_bounds__(kCtThreads) void lora_contract_kernel(const Contrac
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int j = lane & 15, g = lane >> 4;
-    const int group = blockIdx.x % a.groups;
-    const int64_t strip = blockIdx.x / a.groups;
+    // Workgroups go round-robin over the 8 XCDs, each with its own L2.  A 128-column tile of packed
+    // codes is 16*q bytes per row, so 8/q neighbouring tiles share every 128-byte line: the block
+    // index is permuted so that those tiles run on one XCD and the line is fetched from HBM once
+    // (measured before: 2.1x the algorithmic bytes at q = 4).
+    constexpr int kShare = QBIT ? 8 / QBIT : 1;
+    int64_t logical = blockIdx.x;
+    if constexpr (kShare > 1) {
+        const int64_t super = logical / (8 * kShare);
+        const int local = (int)(logical % (8 * kShare));
+        logical = super * (8 * kShare) + (local % 8) * kShare + local / 8;
+    }
+    if (logical >= a.n_blocks) return;                          // padding of the permuted grid (uniform)
+    const int group = (int)(logical % a.groups);
+    const int64_t strip = logical / a.groups;
     const int64_t row_base = strip * kCtStrip + (int64_t)wave * (kCtSteps * 16);
     constexpr int QB = QBIT ? QBIT : 8;
     constexpr float kHalf = (float)(1 << (QB - 1));
@@ -405,8 +418,10 @@ extern "C" int hyc_lora_contract(const void* x, const void* q, const void* scale
     if (workspace_bytes < bytes1 + bytes2) return HYC_ERR_ARG;
     a.part1 = (float*)workspace;
     a.part2 = (float*)((char*)workspace + bytes1);
-    if (strips * a.groups > INT32_MAX) return HYC_ERR_SHAPE;
-    const dim3 grid((unsigned)(strips * a.groups));
+    a.n_blocks = strips * a.groups;
+    const int64_t pad = codes ? 8 * (8 / q_bit) : 1;            // see the block-index permutation in the kernel
+    if (cdiv(a.n_blocks, pad) * pad > INT32_MAX) return HYC_ERR_SHAPE;
+    const dim3 grid((unsigned)(cdiv(a.n_blocks, pad) * pad));
     hipStream_t st = (hipStream_t)stream;
     if (codes) {
         const bool zp = zero_point != nullptr;
