@@ -65,6 +65,8 @@ _SIGNATURES = {
     "hyc_lora_add": (_I, [_P, _P, _I, _P, _P, _P, _L, _L, _L, _P]),
     "hyc_lora_add_quant": (_I, [_P, _P, _I] + [_P] * 5 + [_L, _L, _L, _I, _P]),
     "hyc_lora_add_restore": (_I, [_P, _P, _I] + [_P] * 4 + [_L, _L, _L, _I, _P]),
+    "hyc_lora_add_quant_rope": (_I, [_P, _P, _I] + [_P] * 7 + [_I, _L, _L, _L, _L, _L, _L, _I, _P]),
+    "hyc_lora_add_restore_rope": (_I, [_P, _P, _I] + [_P] * 6 + [_I, _L, _L, _L, _L, _L, _L, _I, _P]),
 }
 
 

@@ -11,6 +11,14 @@
 // on the input gradient).  Here the rank-R product is an MFMA tile held in registers
 // (hyc_lora_tile.hpp) and each kernel moves its algorithmic bytes once: 4, 4 + q/8 and
 // 2 + q/8 bytes per element.
+//
+// For q and k the sum is rotated next (rope_forward, operators/rope_kernels.py:36-109; in the
+// layers fused_llama_layer_intra_inter_full_fuse.py:151-152 and again after the rebuild in
+// backward, :444, :452).  With head_dim 128 a column tile is exactly one head: the two halves of
+// a head sit 8 lanes apart in the 16-lane row group, one DPP row rotate away, so the quantise and
+// restore forms can apply the rotation before the store (same arithmetic as rope.hip).
+#include <type_traits>
+
 #include "hyc_lora_tile.hpp"
 
 namespace hyc {
@@ -26,6 +34,9 @@ struct LoraAddArgs {
     const uint16_t* s; const uint16_t* zp;      // steps / zero points bf16 [N] (quantise, restore)
     const uint16_t* x;                          // dense input (plain, quantise)
     const uint16_t* res;                        // optional residual added to the sum (plain)
+    const void* cos_t; const void* sin_t;       // optional rotation of the sum (quantise, restore); row s = t % S
+    int64_t stride_cos, stride_sin;
+    int S, rope_f32;
     uint8_t* q;                                 // packed codes: output of quantise, input of restore
     uint16_t* y;
     int64_t T;
@@ -34,7 +45,37 @@ struct LoraAddArgs {
     int b_transposed;                           // b is [N, R] instead of [R, N]
 };
 
-template <int QBIT, int KSTEPS, int MODE, bool ZP, bool FAST, bool RES = false>
+// lane <- the lane 8 further round its row of 16 (the other half of the head)
+__device__ __forceinline__ uint32_t other_half(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x128 /* row_ror:8 */, 0xF, 0xF, false);
+}
+
+// Rotates the 8 dims a lane holds of row t: y <- y*cos + partner*(+-sin), first half of the head
+// (lanes 0-7 of the row group) with -sin, second half with +sin.  yv is the bf16-rounded sum.
+template <bool F32>
+__device__ __forceinline__ u32x4 rope_chunk(const LoraAddArgs& a, u32x4 yv, int64_t t, int j) {
+    const u32x4 pv = {other_half(yv.x), other_half(yv.y), other_half(yv.z), other_half(yv.w)};
+    const int s = (int)(t % a.S);
+    const int c = (j & 7) * 8;
+    const float sgn = j < 8 ? -1.0f : 1.0f;
+    float y[8], p[8], cf[8], sf[8], o[8];
+    unpack8(yv, y);
+    unpack8(pv, p);
+    if constexpr (F32) {
+        const float* cp = (const float*)a.cos_t + s * a.stride_cos + c;
+        const float* sp = (const float*)a.sin_t + s * a.stride_sin + c;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = y[e] * cp[e] + p[e] * (sp[e] * sgn);
+    } else {
+        unpack8(ld16((const uint16_t*)a.cos_t + s * a.stride_cos + c), cf);
+        unpack8(ld16((const uint16_t*)a.sin_t + s * a.stride_sin + c), sf);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = rbf(y[e] * cf[e]) + rbf(p[e] * (sf[e] * sgn));
+    }
+    return pack8(o);
+}
+
+template <int QBIT, int KSTEPS, int MODE, bool ZP, bool FAST, bool RES = false, int ROPE = 0>
 __device__ __forceinline__ void lora_add_rows(const LoraAddArgs& a, int64_t row_begin, int64_t row_end, int lane,
                                               int chunk, bool active, const QuantCols<QBIT>& qc, const float (&z)[8],
                                               const BOperand<KSTEPS>& B) {
@@ -92,7 +133,12 @@ __device__ __forceinline__ void lora_add_rows(const LoraAddArgs& a, int64_t row_
 #pragma unroll
                 for (int j = 0; j < 8; ++j) y[j] = f[j] + lora_elem(L[v], j);
             }
-            if (live) st16_nt(a.y + t * a.N + col0, pack8(y));
+            u32x4 yv = pack8(y);
+            if constexpr (ROPE != 0) {
+                // every lane of the row group takes part in the exchange; rows past the end hold zeros
+                yv = rope_chunk<ROPE == 2>(a, yv, t < row_end ? t : row_end - 1, lane & 15);
+            }
+            if (live) st16_nt(a.y + t * a.N + col0, yv);
         }
     }
 }
@@ -128,8 +174,24 @@ __global__ __launch_bounds__(kAddThreads) void lora_add_kernel(const LoraAddArgs
     int64_t row_end = row_begin + a.rows_per_wave;
     if (row_end > a.T) row_end = a.T;
     if (row_begin >= row_end) return;
+    bool fast = false;
+    if constexpr (MODE == kAddQuant && !ZP) fast = __ballot(!qc.fast) == 0ull;
+    if constexpr (MODE != kAddPlain) {
+        if (a.cos_t) {                                          // uniform over the grid
+            auto run = [&](auto fast_tag) {
+                constexpr bool F = decltype(fast_tag)::value;
+                if (a.rope_f32) lora_add_rows<QBIT, KSTEPS, MODE, ZP, F, false, 2>(a, row_begin, row_end, lane, chunk, active, qc, z, B);
+                else lora_add_rows<QBIT, KSTEPS, MODE, ZP, F, false, 1>(a, row_begin, row_end, lane, chunk, active, qc, z, B);
+            };
+            if constexpr (MODE == kAddQuant && !ZP) {
+                if (fast) { run(std::true_type{}); return; }
+            }
+            run(std::false_type{});
+            return;
+        }
+    }
     if constexpr (MODE == kAddQuant && !ZP) {
-        if (__ballot(!qc.fast) == 0ull) {
+        if (fast) {
             lora_add_rows<QBIT, KSTEPS, MODE, ZP, true>(a, row_begin, row_end, lane, chunk, active, qc, z, B);
             return;
         }
@@ -163,6 +225,14 @@ static int add_launch(LoraAddArgs& a, int64_t T, int64_t N, int64_t R, int q_bit
     if (MODE != kAddRestore && !a.x) return HYC_ERR_NULL;
     if (MODE != kAddPlain && (!a.q || !a.s)) return HYC_ERR_NULL;
     if (a.res && !aligned16(a.res)) return HYC_ERR_ALIGN;
+    if (a.cos_t) {
+        // the rotation pairs dims 64 apart inside one 128-column tile: heads of 128 dims, whole tiles only
+        if (MODE == kAddPlain || !a.sin_t || N % kTileCols != 0 || a.S <= 0) return HYC_ERR_ARG;
+        const int talign = a.rope_f32 ? 4 : 8;
+        if (!aligned16(a.cos_t) || !aligned16(a.sin_t) || a.stride_cos % talign || a.stride_sin % talign ||
+            a.stride_cos < kTileCols / 2 || a.stride_sin < kTileCols / 2)
+            return HYC_ERR_ALIGN;
+    }
     if (!(a.b_transposed ? (reinterpret_cast<uintptr_t>(a.b) & 7u) == 0 : aligned16(a.b)) || !aligned16(a.y) || (a.x && !aligned16(a.x)) || (a.s && !aligned16(a.s)) ||
         (a.zp && !aligned16(a.zp)))
         return HYC_ERR_ALIGN;
@@ -232,5 +302,36 @@ extern "C" int hyc_lora_add_restore(const void* xa, const void* b, int b_transpo
     a.b_transposed = b_transposed;
     a.xa = (const uint16_t*)xa; a.b = (const uint16_t*)b; a.y = (uint16_t*)y;
     a.s = (const uint16_t*)scale; a.zp = (const uint16_t*)zero_point; a.q = (uint8_t*)const_cast<void*>(q);
+    return add_launch<kAddRestore>(a, T, N, R, q_bit, stream);
+}
+
+extern "C" int hyc_lora_add_quant_rope(const void* xa, const void* b, int b_transposed, const void* x, const void* scale,
+                                       const void* zero_point, void* q, void* y, const void* cos_t, const void* sin_t,
+                                       int table_is_fp32, int64_t seq_len, int64_t stride_cos, int64_t stride_sin,
+                                       int64_t T, int64_t N, int64_t R, int q_bit, void* stream) {
+    if (!cos_t || !sin_t) return HYC_ERR_NULL;
+    if (seq_len <= 0 || seq_len > INT32_MAX) return HYC_ERR_SHAPE;
+    LoraAddArgs a{};
+    a.b_transposed = b_transposed;
+    a.xa = (const uint16_t*)xa; a.b = (const uint16_t*)b; a.x = (const uint16_t*)x; a.y = (uint16_t*)y;
+    a.s = (const uint16_t*)scale; a.zp = (const uint16_t*)zero_point; a.q = (uint8_t*)q;
+    a.cos_t = cos_t; a.sin_t = sin_t; a.rope_f32 = table_is_fp32; a.S = (int)seq_len;
+    a.stride_cos = stride_cos; a.stride_sin = stride_sin;
+    return add_launch<kAddQuant>(a, T, N, R, q_bit, stream);
+}
+
+extern "C" int hyc_lora_add_restore_rope(const void* xa, const void* b, int b_transposed, const void* q,
+                                         const void* scale, const void* zero_point, void* y, const void* cos_t,
+                                         const void* sin_t, int table_is_fp32, int64_t seq_len, int64_t stride_cos,
+                                         int64_t stride_sin, int64_t T, int64_t N, int64_t R, int q_bit,
+                                         void* stream) {
+    if (!cos_t || !sin_t) return HYC_ERR_NULL;
+    if (seq_len <= 0 || seq_len > INT32_MAX) return HYC_ERR_SHAPE;
+    LoraAddArgs a{};
+    a.b_transposed = b_transposed;
+    a.xa = (const uint16_t*)xa; a.b = (const uint16_t*)b; a.y = (uint16_t*)y;
+    a.s = (const uint16_t*)scale; a.zp = (const uint16_t*)zero_point; a.q = (uint8_t*)const_cast<void*>(q);
+    a.cos_t = cos_t; a.sin_t = sin_t; a.rope_f32 = table_is_fp32; a.S = (int)seq_len;
+    a.stride_cos = stride_cos; a.stride_sin = stride_sin;
     return add_launch<kAddRestore>(a, T, N, R, q_bit, stream);
 }

@@ -136,16 +136,19 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             w, b, qs, la, lb = W[name]
             return lora_forward(w, qs, la, lb, b, inp, residual=residual)
 
-        def proj_quant(name, inp, zp=False):
-            """Projection `name` of inp with the frozen part quantised on the way: -> (output, x @ A).
-            One kernel reads the frozen part once, writes its codes and adds the LoRA product; the
-            reference quantises `*_main` and adds in separate passes (…full_fuse.py:105-140)."""
+        def proj_quant(name, inp, zp=False, rotate=False):
+            """Projection `name` of inp with the frozen part quantised on the way: -> (output, x @ A,
+            whether the output is already rotated).  One kernel reads the frozen part once, writes its
+            codes, adds the LoRA product and - for q and k with heads of 128 dims - applies the rotary
+            embedding; the reference quantises `*_main`, adds and rotates in separate passes
+            (…full_fuse.py:105-152)."""
             w, b, qs, la, lb = W[name]
             main, xa = lora_parts(w, qs, la, b, inp)
             lb = lb.to(main.dtype)
             if not (lora_kernels.supported(main, xa, lb) and main.dim() == 3):
                 (quant_zp if zp else quant)(name + "_main", main, name)
-                return main + xa @ lb, xa
+                return main + xa @ lb, xa, False
+            rope = (cos, sin) if rotate and head_dim == lora_kernels.ROPE_HEAD_DIM else None
             if zp:
                 s_, z_ = get_statistics_only_quant_zero_point(main, q_bit, 'per-channel') if calib else \
                     (sv[name]['scale'], sv[name]['zero_point'])
@@ -153,8 +156,8 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             else:
                 s_, z_ = get_statistics_only_quant(main, q_bit, 'per-channel') if calib else sv[name]['scale'], None
             stats[(name, "scale")] = saved[name + "_main_s"] = s_
-            saved[name + "_main_q"], y = lora_kernels.lora_add_quant(main, xa, lb, s_, z_, q_bit, inplace=True)
-            return y, xa
+            saved[name + "_main_q"], y = lora_kernels.lora_add_quant(main, xa, lb, s_, z_, q_bit, inplace=True, rope=rope)
+            return y, xa, rope is not None
 
         def quant(name, t, key=None):
             if raw:
@@ -201,14 +204,15 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
 
         # ---- attention block -------------------------------------------------------------------
         x_norm_1, saved["rstd_1"], norm_1_done = norm_block("x", "x_norm_1", x, norm_weight_1)
+        q_rotated = k_rotated = False
         if whole:
             q, _, saved["q_lora_a"] = proj("q", x_norm_1)
             k, _, saved["k_lora_a"] = proj("k", x_norm_1)
             v, _, saved["v_lora_a"] = proj("v", x_norm_1)
         else:
-            q, saved["q_lora_a"] = proj_quant("q", x_norm_1, zp=spec.attention == "sdpa")
-            k, saved["k_lora_a"] = proj_quant("k", x_norm_1, zp=spec.attention == "sdpa")
-            v, saved["v_lora_a"] = proj_quant("v", x_norm_1)
+            q, saved["q_lora_a"], q_rotated = proj_quant("q", x_norm_1, zp=spec.attention == "sdpa", rotate=True)
+            k, saved["k_lora_a"], k_rotated = proj_quant("k", x_norm_1, zp=spec.attention == "sdpa", rotate=True)
+            v, saved["v_lora_a"], _ = proj_quant("v", x_norm_1)
         if not norm_1_done:
             quant("x_norm_1", x_norm_1)
         del x_norm_1
@@ -216,8 +220,10 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
         q = hidden_to_head_shape(q, num_heads)
         k = hidden_to_head_shape(k, num_key_value_heads)
         v = hidden_to_head_shape(v, num_key_value_heads)
-        q = rope_forward(q.transpose(1, 2), cos, sin).transpose(1, 2)
-        k = rope_forward(k.transpose(1, 2), cos, sin).transpose(1, 2)
+        if not q_rotated:
+            q = rope_forward(q.transpose(1, 2), cos, sin).transpose(1, 2)
+        if not k_rotated:
+            k = rope_forward(k.transpose(1, 2), cos, sin).transpose(1, 2)
         k = repeat_kv(k, n_rep)
         v = repeat_kv(v, n_rep)
         if whole:
@@ -299,8 +305,8 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             del gate_main, up_main
         else:
             if spec.mode == "intra_inter":
-                gate, gate_lora_a = proj_quant("gate", x_norm_2)
-                up, up_lora_a = proj_quant("up", x_norm_2)
+                gate, gate_lora_a, _ = proj_quant("gate", x_norm_2)
+                up, up_lora_a, _ = proj_quant("up", x_norm_2)
                 hadamard = silu_hadamard(gate, up)
             else:                                           # 'intra' and 'baseline'
                 gate, _, gate_lora_a = proj("gate", x_norm_2)
@@ -373,16 +379,18 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             G[name] = (ga, gb)
             return gx
 
-        def rebuilt_hidden(name):
+        def rebuilt_hidden(name, rotate=False):
             """Output of projection `name` as forward produced it, from the codes of its frozen part
-            and the saved x @ A: dequantise + LoRA add in one kernel (…full_fuse.py:416-417,439-449)."""
+            and the saved x @ A: dequantise + LoRA add (+ the rotary embedding for q and k with heads
+            of 128 dims) in one kernel (…full_fuse.py:416-417,439-452).  -> (tensor, rotated or not)."""
             xa, lb = S[name + "_lora_a"], W[name][4]
             lb = lb.to(xa.dtype)
             q_, s_, z_ = S[name + "_main_q"], S[name + "_main_s"], S.get(name + "_main_z")
             if lora_kernels.supported_restore(q_, xa, lb):
-                return lora_kernels.lora_add_restore(q_, s_, xa, lb, z_, q_bit)
+                rope = (cos, sin) if rotate and D == lora_kernels.ROPE_HEAD_DIM else None
+                return lora_kernels.lora_add_restore(q_, s_, xa, lb, z_, q_bit, rope=rope), rope is not None
             main = deq(name + "_main")
-            return main + (xa @ lb).to(main.dtype)
+            return main + (xa @ lb).to(main.dtype), False
 
         def channel_base_restored(name):
             if name + "_raw" in S:
@@ -422,7 +430,7 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             del hadamard, grad_down
         else:
             if spec.mode == "intra_inter":
-                gate, up = rebuilt_hidden("gate"), rebuilt_hidden("up")
+                gate, up = rebuilt_hidden("gate")[0], rebuilt_hidden("up")[0]
                 fn = F.silu(gate)
                 hadamard = up * fn
             else:
@@ -447,8 +455,9 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
 
         def rebuilt(name, heads):
             """q/k/v in head shape as the forward attention saw them (before repeat_kv)."""
-            t = hidden_to_head_shape(rebuilt_hidden(name), heads)
-            if name != "v":
+            t, rotated = rebuilt_hidden(name, rotate=name != "v")
+            t = hidden_to_head_shape(t, heads)
+            if name != "v" and not rotated:
                 t = rope_forward(t.transpose(1, 2), cos, sin).transpose(1, 2)
             return t
 

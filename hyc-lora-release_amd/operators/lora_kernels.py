@@ -83,9 +83,22 @@ def _vec(t, n, name):
     return _prep(t, name)
 
 
-def lora_add_quant(x_main, xa, b, scale, zero_point=None, quantize_bit=8, inplace=False):
+ROPE_HEAD_DIM = 128          # the fused rotation needs heads as wide as a column tile
+
+
+def _rope_tables(rope, seq_len):
+    from .rope_kernels import _table
+    cos, sin = rope
+    cos, sin = _table(cos, seq_len, ROPE_HEAD_DIM // 2), _table(sin, seq_len, ROPE_HEAD_DIM // 2)
+    if cos.dtype != sin.dtype or cos.dtype not in (BF16, torch.float32):
+        raise NotImplementedError("cos/sin tables must both be bfloat16 or both float32")
+    return cos, sin
+
+
+def lora_add_quant(x_main, xa, b, scale, zero_point=None, quantize_bit=8, inplace=False, rope=None):
     """-> (q, y): q = the packed codes compression_quantization[_with_zero_point](x_main, scale[, zero_point])
-    returns, y = bf16(x_main + bf16(xa @ b)); x_main [B, M, N] is read once."""
+    returns, y = bf16(x_main + bf16(xa @ b)); x_main [B, M, N] is read once.  rope=(cos, sin) also
+    rotates y as rope_forward would on its [B, M, N / 128, 128] view (heads of 128 dims only)."""
     if quantize_bit not in (2, 4, 8):
         raise ValueError(f"quantize_bit must be 2, 4 or 8, got {quantize_bit}")
     _lib.require_gpu(x_main, xa, b, scale, zero_point)
@@ -97,14 +110,22 @@ def lora_add_quant(x_main, xa, b, scale, zero_point=None, quantize_bit=8, inplac
     s = _vec(scale, n, "scale")
     z = None if zero_point is None else _vec(zero_point, n, "zero point")
     q = torch.empty((B, M, n * quantize_bit // 8), device=x.device, dtype=torch.uint8)
+    if rope is not None:
+        if n % ROPE_HEAD_DIM:
+            raise ValueError(f"the fused rotation needs a width that is a multiple of {ROPE_HEAD_DIM}, got {n}")
+        cos, sin = _rope_tables(rope, M)
+        _lib.call("hyc_lora_add_quant_rope", xa.data_ptr(), b.data_ptr(), bt, x.data_ptr(), s.data_ptr(), _lib.ptr(z),
+                  q.data_ptr(), y.data_ptr(), cos.data_ptr(), sin.data_ptr(), int(cos.dtype == torch.float32), M,
+                  cos.stride(0), sin.stride(0), B * M, n, r, quantize_bit, _lib.stream_of(x))
+        return q, y
     _lib.call("hyc_lora_add_quant", xa.data_ptr(), b.data_ptr(), bt, x.data_ptr(), s.data_ptr(), _lib.ptr(z),
               q.data_ptr(), y.data_ptr(), B * M, n, r, quantize_bit, _lib.stream_of(x))
     return q, y
 
 
-def lora_add_restore(q, scale, xa, b, zero_point=None, quantize_bit=8):
+def lora_add_restore(q, scale, xa, b, zero_point=None, quantize_bit=8, rope=None):
     """bf16(decompression_dequantization[_with_zero_point](q, scale[, zero_point]) + bf16(xa @ b)) without
-    writing the dequantised tensor."""
+    writing the dequantised tensor; rope=(cos, sin) rotates the result like lora_add_quant's."""
     if quantize_bit not in (2, 4, 8):
         raise ValueError(f"quantize_bit must be 2, 4 or 8, got {quantize_bit}")
     _lib.require_gpu(q, scale, xa, b, zero_point)
@@ -118,6 +139,14 @@ def lora_add_restore(q, scale, xa, b, zero_point=None, quantize_bit=8):
     s = _vec(scale, n, "scale")
     z = None if zero_point is None else _vec(zero_point, n, "zero point")
     y = torch.empty((B, M, n), device=q.device, dtype=BF16)
+    if rope is not None:
+        if n % ROPE_HEAD_DIM:
+            raise ValueError(f"the fused rotation needs a width that is a multiple of {ROPE_HEAD_DIM}, got {n}")
+        cos, sin = _rope_tables(rope, M)
+        _lib.call("hyc_lora_add_restore_rope", xa.data_ptr(), b.data_ptr(), bt, q.data_ptr(), s.data_ptr(), _lib.ptr(z),
+                  y.data_ptr(), cos.data_ptr(), sin.data_ptr(), int(cos.dtype == torch.float32), M,
+                  cos.stride(0), sin.stride(0), B * M, n, r, quantize_bit, _lib.stream_of(q))
+        return y
     _lib.call("hyc_lora_add_restore", xa.data_ptr(), b.data_ptr(), bt, q.data_ptr(), s.data_ptr(), _lib.ptr(z),
               y.data_ptr(), B * M, n, r, quantize_bit, _lib.stream_of(q))
     return y

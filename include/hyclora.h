@@ -418,6 +418,22 @@ int hyc_lora_add_restore(const void *xa, const void *b, int b_transposed, const 
                          const void *scale, const void *zero_point, void *y, int64_t T, int64_t N,
                          int64_t R, int q_bit, void *stream);
 
+/* hyc_lora_add_quant / hyc_lora_add_restore with the rotary position embedding applied to the sum
+ * before it is stored: y = rope(bf16(x + bf16(xa . b))), the codes still those of x.  Same value as
+ * the plain entry point followed by hyc_rope on y viewed as [T / seq_len, seq_len, N / 128, 128]
+ * (row t takes table row t % seq_len), bit for bit.  Heads of 128 dims only (a column tile is one head):
+ * N % 128 == 0.  cos, sin, table_is_fp32, stride_cos, stride_sin as in hyc_rope.
+ * Replaces rope_forward on q and k after the projection and after their rebuild in backward
+ * (models/llama/fused_llama_layer_intra_inter_full_fuse.py:151-152, :444, :452). */
+int hyc_lora_add_quant_rope(const void *xa, const void *b, int b_transposed, const void *x, const void *scale,
+                            const void *zero_point, void *q, void *y, const void *cos, const void *sin,
+                            int table_is_fp32, int64_t seq_len, int64_t stride_cos, int64_t stride_sin,
+                            int64_t T, int64_t N, int64_t R, int q_bit, void *stream);
+int hyc_lora_add_restore_rope(const void *xa, const void *b, int b_transposed, const void *q,
+                              const void *scale, const void *zero_point, void *y, const void *cos,
+                              const void *sin, int table_is_fp32, int64_t seq_len, int64_t stride_cos,
+                              int64_t stride_sin, int64_t T, int64_t N, int64_t R, int q_bit, void *stream);
+
 /* ---------------------------------------------------------------------------------------
  * The skinny LoRA products that stream a whole [T, N] tensor X for a rank-R result, from one read
  * of X and with fp32 accumulation over the whole contraction:

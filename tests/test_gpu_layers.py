@@ -214,7 +214,8 @@ def test_layer_matches_oracle_layer(dev, layer_type, q_bit, kv_heads):
 @pytest.mark.parametrize("layer_type", ["baseline", "intra", "intra_inter", "intra_inter_full_fuse"])
 @pytest.mark.parametrize("dims", [dict(B=3, S=40, hidden=192, heads=6, kv_heads=3, inter=320, rank=8),
                                   dict(B=1, S=17, hidden=128, heads=2, kv_heads=2, inter=96, rank=4),
-                                  dict(B=2, S=264, hidden=256, heads=4, kv_heads=1, inter=512, rank=32)])
+                                  dict(B=2, S=264, hidden=256, heads=4, kv_heads=1, inter=512, rank=32),
+                                  dict(B=2, S=48, hidden=256, heads=2, kv_heads=1, inter=256, rank=16)])   # heads of 128 dims: rotation fused into the LoRA add
 def test_layer_on_ragged_shapes(dev, layer_type, dims):
     """Shapes that fill none of the kernels' tiles evenly (rows not a multiple of 16 or 256, widths
     not a multiple of 128, a sequence length the fused softmax does not take, ranks 4 / 8 / 32):

@@ -142,6 +142,46 @@ def test_lora_b_in_linear_layout(K, dev, R):
     assert all(np.array_equal(bits(u), bits(v)) for u, v in zip(ba, bb))
 
 
+@pytest.mark.parametrize("q_bit", [2, 4, 8])
+@pytest.mark.parametrize("zp", [False, True])
+@pytest.mark.parametrize("table", [BF16, torch.float32])
+@pytest.mark.parametrize("dims", [(2, 40, 256, 16), (1, 17, 128, 8), (3, 64, 1024, 16)])
+def test_rotation_fused_into_the_add(K, dev, q_bit, zp, table, dims):
+    """rope=(cos, sin): the sum leaves the kernel already rotated - bit-identical to the plain entry
+    point followed by rope_forward on the [B, M, N/128, 128] view; the codes are those of the
+    unrotated frozen part."""
+    import hyclora_amd  # noqa: F401
+    from hyclora_amd.operators.rope_kernels import rope_forward
+    B, M, N, R = dims
+    main, xa, b = inputs(q_bit + N + 1, B, M, N, R, shift=1.5 if zp else 0.0)
+    s, z = O.scale_zero_point(main, q_bit) if zp else (O.scale_only_quant(main, q_bit), None)
+    pos = torch.arange(M + 3, dtype=torch.float32)                 # a table longer than the sequence
+    inv = 1.0 / (10000 ** (torch.arange(0, 128, 2, dtype=torch.float32) / 128))
+    ang = torch.cat([pos[:, None] * inv[None, :]] * 2, dim=-1)
+    cos, sin = ang.cos().to(table).to(dev)[None], ang.sin().to(table).to(dev)[None]
+    d = lambda t: None if t is None else t.to(dev)
+    q0, y0 = K.add_quant(d(main), d(xa), d(b), d(s), d(z), q_bit)
+    want = rope_forward(y0.clone().view(B, M, N // 128, 128), cos, sin).view(B, M, N)
+    q1, y1 = K.add_quant(d(main), d(xa), d(b), d(s), d(z), q_bit, rope=(cos, sin))
+    assert torch.equal(q1, q0), "codes are taken before the rotation"
+    assert np.array_equal(bits(y1), bits(want)), "fused rotation == rope_forward afterwards"
+    r0 = K.add_restore(q0, d(s), d(xa), d(b), d(z), q_bit)
+    r_want = rope_forward(r0.clone().view(B, M, N // 128, 128), cos, sin).view(B, M, N)
+    r1 = K.add_restore(q0, d(s), d(xa), d(b), d(z), q_bit, rope=(cos, sin))
+    assert np.array_equal(bits(r1), bits(r_want))
+    assert_close_bf16(y1, O.rope(O.lora_add(main, xa, b).view(B, M, N // 128, 128), cos.cpu(), sin.cpu()).reshape(B, M, N),
+                      what="rotated sum vs oracle")
+
+
+def test_rotation_needs_whole_heads_of_128(K, dev):
+    main, xa, b = inputs(2, 1, 8, 192, 16)
+    s = O.scale_only_quant(main, 4)
+    cos = torch.ones(1, 8, 128, device=dev, dtype=BF16)
+    d = lambda t: t.to(dev)
+    with pytest.raises(ValueError):
+        K.add_quant(d(main), d(xa), d(b), d(s), None, 4, rope=(cos, cos))
+
+
 def test_special_values_and_degenerate_steps(K, dev):
     """NaN / Inf inputs and steps outside the reciprocal path take the same codes as the standalone
     quantiser; an empty tensor is a no-op."""
