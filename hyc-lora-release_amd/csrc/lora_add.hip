@@ -52,23 +52,24 @@ __device__ __forceinline__ uint32_t other_half(uint32_t v) {
 
 // Rotates the 8 dims a lane holds of row t: y <- y*cos + partner*(+-sin), first half of the head
 // (lanes 0-7 of the row group) with -sin, second half with +sin.  yv is the bf16-rounded sum.
+// (cv, sv: the lane's 8 cos / sin values of the row, bf16 tables only - loaded with the tile)
 template <bool F32>
-__device__ __forceinline__ u32x4 rope_chunk(const LoraAddArgs& a, u32x4 yv, int64_t t, int j) {
+__device__ __forceinline__ u32x4 rope_chunk(const LoraAddArgs& a, u32x4 yv, int64_t t, int j, u32x4 cv, u32x4 sv) {
     const u32x4 pv = {other_half(yv.x), other_half(yv.y), other_half(yv.z), other_half(yv.w)};
-    const int s = (int)(t % a.S);
-    const int c = (j & 7) * 8;
     const float sgn = j < 8 ? -1.0f : 1.0f;
     float y[8], p[8], cf[8], sf[8], o[8];
     unpack8(yv, y);
     unpack8(pv, p);
     if constexpr (F32) {
+        const int s = (int)(t % a.S);
+        const int c = (j & 7) * 8;
         const float* cp = (const float*)a.cos_t + s * a.stride_cos + c;
         const float* sp = (const float*)a.sin_t + s * a.stride_sin + c;
 #pragma unroll
         for (int e = 0; e < 8; ++e) o[e] = y[e] * cp[e] + p[e] * (sp[e] * sgn);
     } else {
-        unpack8(ld16((const uint16_t*)a.cos_t + s * a.stride_cos + c), cf);
-        unpack8(ld16((const uint16_t*)a.sin_t + s * a.stride_sin + c), sf);
+        unpack8(cv, cf);
+        unpack8(sv, sf);
 #pragma unroll
         for (int e = 0; e < 8; ++e) o[e] = rbf(y[e] * cf[e]) + rbf(p[e] * (sf[e] * sgn));
     }
@@ -85,7 +86,7 @@ __device__ __forceinline__ void lora_add_rows(const LoraAddArgs& a, int64_t row_
     constexpr float kHalf = (float)(1 << (QBIT - 1));
     const PackedSlot<QBIT> slot(chunk);
     for (int64_t row0 = row_begin; row0 < row_end; row0 += kTileRows) {
-        u32x4 xv[4], rv[RES ? 4 : 1];
+        u32x4 xv[4], rv[RES ? 4 : 1], cv[ROPE == 1 ? 4 : 1], sv[ROPE == 1 ? 4 : 1];
         u32x2 w[4];
 #pragma unroll
         for (int v = 0; v < 4; ++v) {
@@ -97,6 +98,13 @@ __device__ __forceinline__ void lora_add_rows(const LoraAddArgs& a, int64_t row_
                 if constexpr (MODE == kAddRestore) w[v] = ld8(a.q + t * row_bytes + slot.offset);
                 else xv[v] = ld16_nt(a.x + t * a.N + col0);
                 if constexpr (RES) rv[v] = ld16_nt(a.res + t * a.N + col0);
+            }
+            if constexpr (ROPE == 1) {
+                // table row of this position with the tile's other loads (rows past the end: the last row's)
+                const int sp = (int)((t < row_end ? t : row_end - 1) % a.S);
+                const int c = (lane & 7) * 8;
+                cv[v] = ld16((const uint16_t*)a.cos_t + sp * a.stride_cos + c);
+                sv[v] = ld16((const uint16_t*)a.sin_t + sp * a.stride_sin + c);
             }
         }
         uint32_t L[4][4];
@@ -136,7 +144,8 @@ __device__ __forceinline__ void lora_add_rows(const LoraAddArgs& a, int64_t row_
             u32x4 yv = pack8(y);
             if constexpr (ROPE != 0) {
                 // every lane of the row group takes part in the exchange; rows past the end hold zeros
-                yv = rope_chunk<ROPE == 2>(a, yv, t < row_end ? t : row_end - 1, lane & 15);
+                yv = rope_chunk<ROPE == 2>(a, yv, t < row_end ? t : row_end - 1, lane & 15, cv[ROPE == 1 ? v : 0],
+                                           sv[ROPE == 1 ? v : 0]);
             }
             if (live) st16_nt(a.y + t * a.N + col0, yv);
         }
