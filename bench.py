@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-Workload: BASELINE configuration 2 — the activations of a Llama-2-7B-shaped MLP layer,
+Workload: benchmark configuration 2 — the activations of a Llama-2-7B-shaped MLP layer,
 T = 4 x 1024 tokens, intermediate size 11008, LoRA rank 16, q_bit = 4, synthetic N(0,1) data.
 
 A step = one compress (quantise + pack) followed by one decompress (unpack + dequantise) of
@@ -658,7 +658,7 @@ def main():
         kernels["softmax_restore_bwd_one_pass"] = {"ms": ms, "GBps": (6 * Ea + 10 * nnz) / ms / 1e6}
         del a, g_a, idx_a, val_a
 
-    # ---- whole decoder layers (BASELINE configurations 2, 4, 5): fwd+bwd ms and saved bytes ----
+    # ---- whole decoder layers (benchmark configurations 2, 4, 5): fwd+bwd ms and saved bytes ----
     layers = None
     want_cpu = args.only == "all" and not args.skip_cpu
     if want_cpu:

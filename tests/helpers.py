@@ -24,7 +24,7 @@ def same_bits(a: torch.Tensor, b: torch.Tensor) -> bool:
 
 
 def activation_with_outlier_channels(seed, shape=(2, 512, 4096), frac=0.005, gain=50.0):
-    """BASELINE configuration 1: N(0,1) values, a fixed random 0.5 % of channels scaled x50.
+    """benchmark configuration 1: N(0,1) values, a fixed random 0.5 % of channels scaled x50.
     Returns (x bf16, planted channel indices sorted)."""
     g = torch.Generator().manual_seed(seed)
     x = torch.randn(*shape, generator=g)

@@ -27,7 +27,7 @@ def fz():
 
 
 def mlp_inputs(seed, B, M, H, I, R):
-    """BASELINE configuration 2 in the given size: x ~ N(0,1), frozen W ~ N(0,0.02), LoRA A
+    """benchmark configuration 2 in the given size: x ~ N(0,1), frozen W ~ N(0,0.02), LoRA A
     kaiming-uniform(a=sqrt(5)) as PEFT initialises it, LoRA B ~ N(0,1e-3) (scaled up here so
     that the LoRA term is visible in the outputs)."""
     g = torch.Generator().manual_seed(seed)
@@ -109,7 +109,7 @@ def test_fused_errors(fz, dev):
 
 @pytest.mark.parametrize("q_bit", [4])
 def test_fused_full_size_config2(fz, dev, q_bit):
-    # BASELINE configuration 2: T = 4x1024, N = 11008, R = 16.  Codes against the standalone
+    # benchmark configuration 2: T = 4x1024, N = 11008, R = 16.  Codes against the standalone
     # quantiser (already pinned bit-exact), o against the unfused torch composition on the GPU.
     from hyclora_amd.operators import compress_function as cf
     g = torch.Generator(device=dev).manual_seed(0)

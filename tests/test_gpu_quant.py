@@ -92,7 +92,7 @@ def test_zero_point_path(cf, dev, q_bit):
 
 @pytest.mark.parametrize("q_bit", QBITS)
 def test_config1_outlier_channels_round_trip(cf, dev, q_bit):
-    # BASELINE configuration 1 at full size: bf16 [2,512,4096], 0.5 % channels x50
+    # benchmark configuration 1 at full size: bf16 [2,512,4096], 0.5 % channels x50
     x, planted = activation_with_outlier_channels(seed=1234)
     idx, s = O.channel_stats(x, 0.005, q_bit)
     assert torch.equal(torch.sort(idx).values, planted)
@@ -164,7 +164,7 @@ def test_empty_and_bad_arguments(cf, dev):
 
 @pytest.mark.parametrize("q_bit", QBITS)
 def test_full_size_properties_config2_shape(cf, dev, q_bit):
-    # [4,1024,11008] (BASELINE configuration 2's activation shape): properties that need no CPU pass
+    # [4,1024,11008] (benchmark configuration 2's activation shape): properties that need no CPU pass
     g = torch.Generator(device=dev).manual_seed(q_bit)
     x = torch.randn(4, 1024, 11008, generator=g, device=dev, dtype=torch.float32).to(BF16)
     hi = x[0].max(dim=0, keepdim=True).values

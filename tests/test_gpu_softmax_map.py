@@ -24,7 +24,7 @@ def sk():
 
 
 def attention_map(seed, shape=(2, 4, 128, 128), causal=True):
-    """BASELINE configuration 3 in small: softmax of N(0,1)*8/sqrt(128) logits with a causal mask."""
+    """benchmark configuration 3 in small: softmax of N(0,1)*8/sqrt(128) logits with a causal mask."""
     g = torch.Generator().manual_seed(seed)
     b, h, n, _ = shape
     s = torch.randn(*shape, generator=g) * 8 / 128 ** 0.5
@@ -213,7 +213,7 @@ def test_softmax_forward_counts_for_the_compaction(cf, sk, dev, shape):
 
 
 def test_full_size_config3_properties(cf, sk, dev):
-    # BASELINE configuration 3 at full size: [4,32,1024,1024], ratio 0.05
+    # benchmark configuration 3 at full size: [4,32,1024,1024], ratio 0.05
     g = torch.Generator(device=dev).manual_seed(1)
     s = torch.randn(4, 32, 1024, 1024, generator=g, device=dev, dtype=torch.float32) * (8 / 128 ** 0.5)
     s += torch.full((1024, 1024), float("-inf"), device=dev).triu(1)

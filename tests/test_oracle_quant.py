@@ -98,7 +98,7 @@ def test_against_scalar_c(q_bit, with_zp):
 
 @pytest.mark.parametrize("q_bit", QBITS)
 def test_error_bound_and_outlier_columns_config1(q_bit):
-    # BASELINE configuration 1 (reduced in rows for CPU time): off-clamp error <= s/2,
+    # benchmark configuration 1 (reduced in rows for CPU time): off-clamp error <= s/2,
     # outlier columns carry code 2^(q-1) and decode to exactly 0 before the scatter
     x, planted = activation_with_outlier_channels(seed=7, shape=(2, 64, 4096))
     idx, s = O.channel_stats(x, 0.005, q_bit)
