@@ -12,7 +12,8 @@ Pinning status (what independent evidence holds each function in place):
   * quant_codes / pack_codes / unpack_codes / dequant: pinned by the scalar C
     restatement in oracle/scalar_ref.c (an independent loop-level implementation),
     by hand-computed known answers, by round trips, by |x - x^| <= s/2, and by the
-    q=8 identity layout (tests/test_oracle_quant.py).
+    q=8 identity layout (tests/test_oracle_quant.py), and by the committed known-answer vectors
+    of tests/golden/kat.json (scalar numpy arithmetic, tests/test_golden.py).
   * scale_* / outlier_channels: reduce to torch.max/min/norm plus two bf16 scalar
     operations; pinned by closed forms and planted outlier channels.
   * softmax_threshold / softmax_compress / softmax_restore: pinned against
