@@ -8,6 +8,7 @@ the rules the reference's kernels implement:
   value = bf16( (code - 2^(q-1) [- z]) * s )                                    (:193-206, :382-388)
   keep  : entries of the flattened map strictly above the threshold, ascending index
                                                    (operators/compress_function.py:309-313)
+  steps, zero points and outlier channels of the calibration statistics (:45-105), see main()
 
 bf16 values are stored as their 16-bit patterns.  Run:  python tests/golden/make_golden.py
 The vectors pin both the CPU oracle (tests/test_golden.py, CPU) and the kernels (GPU part of it)."""
@@ -123,7 +124,51 @@ def main():
     keep = [i for i, v in enumerate(vals) if (v > thr or v != v) and v != 0]
     softmax = {"shape": [2, 3, 8], "map_bits": [bf16_bits(v) for v in vals], "threshold": thr,
                "indices": keep, "value_bits": [bf16_bits(vals[i]) for i in keep]}
-    out = {"quant": cases, "compaction": softmax}
+    # calibration statistics from batch element 0 (operators/compress_function.py:45-105), bf16 after
+    # every tensor operation: d = bf16(max - min), s = bf16(fp32(d) / (2^q - 1)); zero point
+    # z = int8(bf16(-rne(bf16(min / s)) - 2^(q-1))); channel base: the k = int(N*ratio) channels of
+    # largest bf16 norm (ties: lower channel first) are zeroed first, a zero step becomes bf16(0 + 1e-3)
+    nb, rows, n = 2, 6, 64
+    xs = rng.normal(size=(nb, rows, n))
+    xs[:, :, 9] *= 40.0
+    xs[:, :, 33] *= 25.0
+    xs[:, :, 50] *= 60.0
+    xs[:, :, 20] = 0.5                                       # a constant channel: zero step
+    xs[1] *= 3.0                                             # batch element 1 must not matter
+    xb = [[[bf16_bits(v) for v in row] for row in bt] for bt in xs]
+    x0 = [[bf16_val(b) for b in row] for row in xb[0]]
+    bf = lambda v: bf16_val(bf16_bits(v))
+    stats = {"x_bits": xb, "ratio": 0.05, "only_quant": {}, "zero_point": {}, "channel_base": {}}
+    col = lambda c: [x0[r][c] for r in range(rows)]
+    for q in (2, 4, 8):
+        levels = float((1 << q) - 1)
+        half = float(1 << (q - 1))
+        sc, zs = [], []
+        for c in range(n):
+            lo, hi = min(col(c)), max(col(c))
+            d = bf(hi - lo)
+            sv = bf(float(np.float32(d) / np.float32(levels)))
+            sc.append(bf16_bits(sv))
+            if sv != 0.0:
+                t = bf(float(np.float32(lo) / np.float32(sv)))
+                r = float(np.round(np.float32(t)))            # numpy rounds half to even
+                zs.append(int(bf(bf(-r) - half)))
+            else:
+                zs.append(None)                               # 0 / 0: not defined, not compared
+        stats["only_quant"][str(q)] = sc
+        stats["zero_point"][str(q)] = zs
+        norms = [bf(math.sqrt(float(sum(np.float32(v) * np.float32(v) for v in col(c))))) for c in range(n)]
+        k = int(n * 0.05)
+        idx = sorted(range(n), key=lambda c: (-norms[c], c))[:k]
+        sb = []
+        for c in range(n):
+            vals = [0.0] * rows if c in idx else col(c)
+            sv = bf(float(np.float32(bf(max(vals) - min(vals))) / np.float32(levels)))
+            if sv == 0.0:
+                sv = bf(float(np.float32(sv) + np.float32(1e-3)))
+            sb.append(bf16_bits(sv))
+        stats["channel_base"][str(q)] = {"outlier_channel_index": idx, "scale_bits": sb}
+    out = {"quant": cases, "compaction": softmax, "statistics": stats}
     path = Path(__file__).with_name("kat.json")
     path.write_text(json.dumps(out, separators=(",", ":")))
     print("wrote", path, path.stat().st_size, "bytes")

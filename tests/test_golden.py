@@ -77,3 +77,39 @@ def test_kernels_reproduce_the_compaction_vector(dev):
     keep = np.zeros(a.numel(), dtype=bool)
     keep[c["indices"]] = True
     assert np.array_equal(bits(dense).reshape(-1)[~keep], np.zeros((~keep).sum(), dtype=np.uint16))
+
+
+def _stat_input():
+    st = KAT["statistics"]
+    return st, from_bits(np.array(st["x_bits"], dtype=np.uint16))
+
+
+def _check_stats(st, q, scale, zp_pair, cb_pair):
+    assert np.array_equal(bits(scale).reshape(-1), np.array(st["only_quant"][str(q)], dtype=np.uint16))
+    s_zp, z = zp_pair
+    want_z = st["zero_point"][str(q)]
+    defined = np.array([v is not None for v in want_z])
+    assert np.array_equal(bits(s_zp).reshape(-1), np.array(st["only_quant"][str(q)], dtype=np.uint16))
+    assert np.array_equal(z.reshape(-1).cpu().numpy()[defined], np.array([v for v in want_z if v is not None], dtype=np.int8))
+    idx, s_cb = cb_pair
+    want = st["channel_base"][str(q)]
+    assert idx.reshape(-1).tolist() == want["outlier_channel_index"]
+    assert np.array_equal(bits(s_cb).reshape(-1), np.array(want["scale_bits"], dtype=np.uint16))
+
+
+@pytest.mark.parametrize("q", [2, 4, 8])
+def test_oracle_reproduces_the_statistics_vectors(q):
+    st, x = _stat_input()
+    _check_stats(st, q, O.scale_only_quant(x, q), O.scale_zero_point(x, q), O.channel_stats(x, st["ratio"], q))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("q", [2, 4, 8])
+def test_kernels_reproduce_the_statistics_vectors(dev, q):
+    import hyclora_amd  # noqa: F401
+    from hyclora_amd.operators import compress_function as cf
+    st, x = _stat_input()
+    x = x.to(dev)
+    _check_stats(st, q, cf.get_statistics_only_quant(x, q, 'per-channel'),
+                 cf.get_statistics_only_quant_zero_point(x, q, 'per-channel'),
+                 cf.get_statistics_channel_base(x, st["ratio"], q, 'per-channel'))
