@@ -116,5 +116,6 @@ __host__ __device__ inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 
 int tune_quant(const char* key, int value);
 int tune_fuse(const char* key, int value);
 int tune_add(const char* key, int value);
+int tune_contract(const char* key, int value);
 
 }  // namespace hyc

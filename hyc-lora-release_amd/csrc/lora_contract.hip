@@ -36,7 +36,7 @@ constexpr int kCtSteps = 4;                               // 16-row steps per wa
 constexpr int kCtStrip = kCtWaves * kCtSteps * 16;        // 256 rows per workgroup
 constexpr int kCtTile = 128;                              // columns per tile
 constexpr int kCtPitch = kCtTile + 8;                     // LDS row pitch of a transposed tile (bf16 elements)
-constexpr int kCtMaxGroups = 128;                         // column groups (bounds the P2 partials)
+static int g_ct_max_groups = 32;                          // column groups (bounds the P2 partials); see hyc_set_tuning
 
 struct ContractArgs {
     const uint16_t* x;                   // dense X [T, N]
@@ -365,11 +365,20 @@ static void contract_launch_nb(const ContractArgs& a, dim3 grid, int nb, hipStre
 static int64_t contract_geometry(int64_t T, int64_t N, int64_t R, int* tiles_per_group, int* groups, int64_t* strips,
                                  int* nb) {
     const int64_t tiles = cdiv(N, kCtTile);
-    *tiles_per_group = (int)cdiv(tiles, kCtMaxGroups);
+    *tiles_per_group = (int)cdiv(tiles, g_ct_max_groups);
     *groups = (int)cdiv(tiles, *tiles_per_group);
     *strips = cdiv(T, kCtStrip);
     *nb = (int)cdiv(R, 16);
     return 0;
+}
+
+int tune_contract(const char* key, int value) {
+    if (strcmp(key, "contract_max_groups") == 0) {
+        if (value < 1 || value > 65536) return HYC_ERR_ARG;
+        g_ct_max_groups = value;
+        return HYC_OK;
+    }
+    return 1;
 }
 
 }  // namespace hyc

@@ -452,7 +452,8 @@ int hyc_lora_add_restore_rope(const void *xa, const void *b, int b_transposed, c
  *   R even, 2..64; N % 32 == 0; any T.
  *   workspace: device scratch of hyc_lora_contract_workspace(T, N, R, p1 != NULL, p2 != NULL) bytes,
  *   16-byte aligned, contents undefined on entry and exit; partial sums are combined in a fixed
- *   order (no atomics), so results are reproducible.
+ *   order (no atomics), so results are reproducible.  Tuning key "contract_max_groups" (default 32):
+ *   upper bound on the column groups a row strip is split into (each adds a plane of p2 partials).
  */
 int64_t hyc_lora_contract_workspace(int64_t T, int64_t N, int64_t R, int want_p1, int want_p2);
 int hyc_lora_contract(const void *x, const void *q, const void *scale, const void *zero_point, int q_bit,
