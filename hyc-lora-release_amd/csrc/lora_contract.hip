@@ -32,7 +32,10 @@ namespace hyc {
 
 constexpr int kCtThreads = 256;
 constexpr int kCtWaves = kCtThreads / kWave;
-constexpr int kCtSteps = 4;                               // 16-row steps per wave
+#ifndef HYC_CT_STEPS
+#define HYC_CT_STEPS 4
+#endif
+constexpr int kCtSteps = HYC_CT_STEPS;                    // 16-row steps per wave
 constexpr int kCtStrip = kCtWaves * kCtSteps * 16;        // 256 rows per workgroup
 constexpr int kCtTile = 128;                              // columns per tile
 constexpr int kCtPitch = kCtTile + 8;                     // LDS row pitch of a transposed tile (bf16 elements)
