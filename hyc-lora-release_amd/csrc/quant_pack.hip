@@ -48,6 +48,8 @@ constexpr int kDeqUnroll = HYC_D_UNROLL;       // dequantiser: rows per group
 
 static int g_quant_rows_per_wave = 8;     // strip heights; see hyc_set_tuning
 static int g_dequant_rows_per_wave = 2;
+static int g_quant_outlier_rows_per_wave = 8;     // the same two with an outlier list
+static int g_dequant_outlier_rows_per_wave = 8;
 
 struct QuantArgs {
     uint16_t* x;            // bf16 activations (input of quantise / output of dequantise)
@@ -162,13 +164,15 @@ __device__ __forceinline__ void load_rows(const QuantArgs& a, RowCursor& cur, in
 // s_waitcnt vmcnt(<stores in flight>) instead of vmcnt(0) at the top of the loop.
 template <int QBIT, bool ZP, bool OUTL, bool FAST, bool FULL>
 __device__ __forceinline__ void quant_rows(const QuantArgs& a, int64_t row0, int64_t row1, bool active, int chunk,
-                                           int64_t coff, const QuantCols<QBIT>& qc, const float (&z)[8],
-                                           const OutlierLane& ol) {
+                                           int64_t coff, const QuantCols<QBIT>& qc, const float (&z)[8]) {
     const int row_bytes = a.N * QBIT / 8;
     if (row0 >= row1) return;
     RowCursor cur(row0, a.M, a.stride_b, a.stride_m);
     u32x4 v[kRowUnroll];
     load_rows<FULL>(a, cur, row0, row1, active, coff, v);
+    // the first rows are already on their way while the wave looks up its outlier columns
+    OutlierLane ol;
+    if constexpr (OUTL) ol = find_outliers(a.oidx, a.k, (chunk & ~(kWave - 1)) * 8, chunk * 8, chunk & (kWave - 1));
     auto compute = [&](u32x4 (&v)[kRowUnroll], int64_t t0, uint32_t (&lo)[kRowUnroll], uint32_t (&hi)[kRowUnroll]) {
 #pragma unroll
         for (int u = 0; u < kRowUnroll; ++u) {
@@ -242,9 +246,6 @@ void quant_pack_kernel(const QuantArgs a) {
     if constexpr (ZP) {
         if (active) unpack8(ld16(a.zp + col0), z);
     }
-    OutlierLane ol;
-    if constexpr (OUTL) ol = find_outliers(a.oidx, a.k, col_tile * kWave * 8, col0, lane);
-
     const int64_t coff = active ? chunk_offset(col0, a.head_dim, a.stride_h) : 0;
     const int64_t row0 = (row_tile * kQuantWaves + wave) * (int64_t)a.rows_per_wave;
     int64_t row1 = row0 + a.rows_per_wave;
@@ -254,11 +255,11 @@ void quant_pack_kernel(const QuantArgs a) {
                       a.rows_per_wave % kRowUnroll == 0;      // uniform across the wave
     // one slow column anywhere in the wave sends the whole wave down the IEEE-division path
     if (ZP || __ballot(!qc.fast) != 0ull)
-        quant_rows<QBIT, ZP, OUTL, false, false>(a, row0, row1, active, chunk, coff, qc, z, ol);
+        quant_rows<QBIT, ZP, OUTL, false, false>(a, row0, row1, active, chunk, coff, qc, z);
     else if (full)
-        quant_rows<QBIT, ZP, OUTL, true, true>(a, row0, row1, active, chunk, coff, qc, z, ol);
+        quant_rows<QBIT, ZP, OUTL, true, true>(a, row0, row1, active, chunk, coff, qc, z);
     else
-        quant_rows<QBIT, ZP, OUTL, true, false>(a, row0, row1, active, chunk, coff, qc, z, ol);
+        quant_rows<QBIT, ZP, OUTL, true, false>(a, row0, row1, active, chunk, coff, qc, z);
 }
 
 // ------------------------------------------------------------------------------------
@@ -287,7 +288,6 @@ __global__ __launch_bounds__(kQuantThreads) void unpack_dequant_kernel(const Qua
         }
     }
     OutlierLane ol;
-    if constexpr (OUTL) ol = find_outliers(a.oidx, a.k, col_tile * kWave * 8, col0, lane);
 
     const int64_t coff = active ? chunk_offset(col0, a.head_dim, a.stride_h) : 0;
     const int64_t row0 = (row_tile * kQuantWaves + wave) * (int64_t)a.rows_per_wave;
@@ -312,6 +312,24 @@ __global__ __launch_bounds__(kQuantThreads) void unpack_dequant_kernel(const Qua
                 } else {
                     w[u] = u32x2{0, 0};
                     if (active && t0 + u < row1) w[u] = ld8(a.q + (t0 + u) * row_bytes + slot.offset);
+                }
+            }
+        };
+        // Outlier values travel with the codes of their row, one load per flagged column, so
+        // that the row's store waits for one round of memory latency and not for two.
+        uint32_t ov[OUTL ? kDeqUnroll : 1][8];
+        auto load_outliers = [&](int64_t t0) {
+            if constexpr (OUTL) {
+                if (ol.mask) {
+#pragma unroll
+                    for (int u = 0; u < kDeqUnroll; ++u) {
+                        const int64_t t = t0 + u;
+                        if (FULL || (active && t < row1)) {
+#pragma unroll
+                            for (int j = 0; j < 8; ++j)
+                                if (ol.mask & (1u << j)) ov[u][j] = a.xo[t * a.k + outlier_pos(ol, j)];
+                        }
+                    }
                 }
             }
         };
@@ -344,8 +362,7 @@ __global__ __launch_bounds__(kQuantThreads) void unpack_dequant_kernel(const Qua
                         for (int j = 0; j < 8; ++j) {
                             if (ol.mask & (1u << j)) {
                                 const uint32_t sh = 16 * (j & 1);
-                                const uint32_t val = a.xo[t * a.k + outlier_pos(ol, j)];
-                                d[j >> 1] = (d[j >> 1] & ~(0xffffu << sh)) | (val << sh);
+                                d[j >> 1] = (d[j >> 1] & ~(0xffffu << sh)) | (ov[u][j] << sh);
                             }
                         }
                         o[u] = u32x4{d[0], d[1], d[2], d[3]};
@@ -360,14 +377,19 @@ __global__ __launch_bounds__(kQuantThreads) void unpack_dequant_kernel(const Qua
         };
         // next group's loads go out before this group's stores (see quant_rows)
         load_codes(row0);
+        // the first codes are already on their way while the wave looks up its outlier columns
+        if constexpr (OUTL) ol = find_outliers(a.oidx, a.k, col_tile * kWave * 8, col0, lane);
+        load_outliers(row0);
         int64_t t0 = row0;
         compute(t0);                              // first group peeled, as in quant_rows
         if (t0 + kDeqUnroll < row1) {
             load_codes(t0 + kDeqUnroll);
+            load_outliers(t0 + kDeqUnroll);
             store(t0);
             for (t0 += kDeqUnroll; t0 + kDeqUnroll < row1; t0 += kDeqUnroll) {
                 compute(t0);
                 load_codes(t0 + kDeqUnroll);
+                load_outliers(t0 + kDeqUnroll);
                 store(t0);
             }
             compute(t0);
@@ -451,7 +473,7 @@ extern "C" int hyc_quant_pack(const void* x, const void* scale, const void* zero
     if (zero_point && !aligned16(zero_point)) return HYC_ERR_ALIGN;
     const void* zp = zero_point;
     QuantArgs a = make_args(x, scale, zp, q, outlier_idx, k, x_outlier, zero_input, B, M, N, stride_b, stride_m,
-                            head_dim, stride_h, g_quant_rows_per_wave);
+                            head_dim, stride_h, (outlier_idx && k) ? g_quant_outlier_rows_per_wave : g_quant_rows_per_wave);
     const int64_t row_tiles = cdiv(a.T, (int64_t)kQuantWaves * a.rows_per_wave);
     if (row_tiles * a.col_tiles > INT32_MAX) return HYC_ERR_SHAPE;
     const dim3 grid((unsigned)(row_tiles * a.col_tiles)), block(kQuantThreads);
@@ -471,7 +493,7 @@ extern "C" int hyc_unpack_dequant(const void* q, const void* scale, const void* 
     if (!((reinterpret_cast<uintptr_t>(q) & 7u) == 0)) return HYC_ERR_ALIGN;
     const void* zp = zero_point;
     QuantArgs a = make_args(x, scale, zp, q, outlier_idx, k, x_outlier, 0, B, M, N, stride_b, stride_m, head_dim,
-                            stride_h, g_dequant_rows_per_wave);
+                            stride_h, (outlier_idx && k) ? g_dequant_outlier_rows_per_wave : g_dequant_rows_per_wave);
     const int64_t row_tiles = cdiv(a.T, (int64_t)kQuantWaves * a.rows_per_wave);
     if (row_tiles * a.col_tiles > INT32_MAX) return HYC_ERR_SHAPE;
     const dim3 grid((unsigned)(row_tiles * a.col_tiles)), block(kQuantThreads);
@@ -481,10 +503,14 @@ extern "C" int hyc_unpack_dequant(const void* q, const void* scale, const void* 
 }
 
 int hyc::tune_quant(const char* key, int value) {
-    const bool q = strcmp(key, "quant_rows_per_wave") == 0, d = strcmp(key, "dequant_rows_per_wave") == 0;
-    if (q || d) {
+    int* const knobs[4] = {&g_quant_rows_per_wave, &g_dequant_rows_per_wave, &g_quant_outlier_rows_per_wave,
+                           &g_dequant_outlier_rows_per_wave};
+    const char* const names[4] = {"quant_rows_per_wave", "dequant_rows_per_wave", "quant_outlier_rows_per_wave",
+                                  "dequant_outlier_rows_per_wave"};
+    for (int i = 0; i < 4; ++i) {
+        if (strcmp(key, names[i]) != 0) continue;
         if (value < 1 || value > 4096) return HYC_ERR_ARG;
-        (q ? g_quant_rows_per_wave : g_dequant_rows_per_wave) = value;
+        *knobs[i] = value;
         return HYC_OK;
     }
     return 1;  // not one of this file's keys

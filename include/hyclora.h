@@ -42,6 +42,8 @@ int hyc_abi_version(void);
 /* Launch-shape knobs for benchmarking (process-wide, not thread-safe against concurrent
  * launches).  Keys: "quant_rows_per_wave" (rows each wave walks in hyc_quant_pack,
  * default 8), "dequant_rows_per_wave" (same for hyc_unpack_dequant, default 2),
+ * "quant_outlier_rows_per_wave" / "dequant_outlier_rows_per_wave" (the same two when called with
+ * an outlier list; default 8 each: a wave first has to find its outlier columns in the list),
  * "fuse_rows_per_wave" (same for both fused LoRA-SiLU kernels, multiple of 16; defaults 48 forward,
  * 32 backward).  Unknown key or bad value: HYC_ERR_ARG.  No
  * counterpart in the reference (its launch shapes come from triton.autotune). */
