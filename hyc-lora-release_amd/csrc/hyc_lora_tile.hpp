@@ -101,6 +101,25 @@ __device__ __forceinline__ void lora_tile_bf16(const uint16_t* xa, int R, int64_
 #pragma unroll
         for (int p = 0; p < 4; ++p) L[v][p] = pk_bf16(acc_elem(acc[2 * p], v), acc_elem(acc[2 * p + 1], v));
 }
+// The same with the LoRA-A operand already in registers (A[ks] = the four bf16
+// xa[row0 + l%16][16*ks + 4*(l/16) .. +3] of lane l), for callers that load a tile ahead of its use.
+template <int KSTEPS>
+__device__ __forceinline__ void lora_tile_bf16_regs(const u32x2 (&A)[KSTEPS], const BOperand<KSTEPS>& B,
+                                                    uint32_t (&L)[4][4]) {
+    f32x4 acc[8];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) acc[t] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+        const s16x4 Av = __builtin_bit_cast(s16x4, A[ks]);
+#pragma unroll
+        for (int t = 0; t < 8; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(Av, B.v[ks][t], acc[t], 0, 0, 0);
+    }
+#pragma unroll
+    for (int v = 0; v < 4; ++v)
+#pragma unroll
+        for (int p = 0; p < 4; ++p) L[v][p] = pk_bf16(acc_elem(acc[2 * p], v), acc_elem(acc[2 * p + 1], v));
+}
 __device__ __forceinline__ float lora_elem(const uint32_t (&Lv)[4], int j) {
     return (j & 1) ? bf_hi(Lv[j >> 1]) : bf_lo(Lv[j >> 1]);
 }

@@ -14,6 +14,8 @@
 // down a strip of rows 16 at a time; the rank-R contraction runs on the matrix cores in the
 // "one lane = one 16-byte chunk" ownership (hyc_lora_tile.hpp).
 // The LoRA-B operand registers are built once per wave and reused for the whole strip.
+#include <type_traits>
+
 #include "hyc_lora_tile.hpp"
 
 namespace hyc {
@@ -26,7 +28,7 @@ constexpr int kFuseThreads = 256;                  // 4 waves
 #define HYC_FUSE_KERNEL __global__ __launch_bounds__(kFuseThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
 constexpr int kFuseWaves = kFuseThreads / kWave;
 
-static int g_fuse_rows_per_wave[2] = {32, 48};   // backward, forward; see hyc_set_tuning
+static int g_fuse_rows_per_wave[2] = {32, 32};   // backward, forward; see hyc_set_tuning
 
 struct FuseArgs {
     const uint16_t* xa1; const uint16_t* b1; const uint16_t* s1;
@@ -96,6 +98,95 @@ __device__ __forceinline__ void fuse_fwd_rows(const FuseArgs& a, int64_t row_beg
     }
 }
 
+// Interior strips (every lane inside the tensor, whole 16-row tiles): no predicate guards a memory
+// operation, so the compiler can count the outstanding ones exactly, and the strip is walked as a
+// rolling prefetch that needs no second set of registers: as soon as a row of the current tile
+// has been unpacked, the same registers are requested again for that row of the NEXT tile (the
+// LoRA-A operands likewise, right after the matrix instructions that read them).  Every wait is
+// then for data requested a whole tile earlier, and the stores of the rows in between stay in
+// flight (loads and stores retire through one in-order counter).  The first tile is peeled so
+// that the loop is entered in the state its back edge carries; the last one requests nothing.
+template <int KSTEPS>
+__device__ __forceinline__ void request_lora_a(const uint16_t* xa, int R, int64_t row, int g, u32x2 (&A)[KSTEPS]) {
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+        const int k = 16 * ks + 4 * g;
+        A[ks] = ld8(xa + row * R + (k < R ? k : 0));         // past the rank: any valid address, see below
+    }
+}
+// Zeroes the operands past the rank (a rank that is not a multiple of 16).  Done when the operand
+// is used, not when it is requested: touching the value would wait for the load.
+template <int KSTEPS>
+__device__ __forceinline__ void mask_lora_a(int R, int g, const u32x2 (&A)[KSTEPS], u32x2 (&M)[KSTEPS]) {
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+        const bool ok = 16 * ks + 4 * g < R;
+        M[ks] = u32x2{ok ? A[ks].x : 0u, ok ? A[ks].y : 0u};
+    }
+}
+
+template <int QBIT, int KSTEPS>
+__device__ __forceinline__ void fuse_fwd_rows_full(const FuseArgs& a, int64_t row_begin, int64_t row_end, int lane,
+                                                   int chunk, const QuantCols<QBIT>& c1, const QuantCols<QBIT>& c2,
+                                                   const BOperand<KSTEPS>& B1, const BOperand<KSTEPS>& B2) {
+    const int g = lane >> 4, i = lane & 15;
+    const int row_bytes = a.N * QBIT / 8;
+    const float zero8[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    u32x4 xv1[4], xv2[4];
+    u32x2 A1[KSTEPS], A2[KSTEPS];
+    auto request_a = [&](int64_t row0) {
+        request_lora_a<KSTEPS>(a.xa1, a.R, row0 + i, g, A1);
+        request_lora_a<KSTEPS>(a.xa2, a.R, row0 + i, g, A2);
+    };
+    auto request_row = [&](int64_t row0, int v) {
+        const int64_t off = (row0 + 4 * g + v) * a.N + chunk * 8;
+        xv1[v] = ld16_nt(a.x1 + off);
+        xv2[v] = ld16_nt(a.x2 + off);
+    };
+    auto work = [&](int64_t row0, auto ahead_tag) {
+        constexpr bool AHEAD = decltype(ahead_tag)::value;
+        uint32_t L1[4][4], L2[4][4];
+        u32x2 M1[KSTEPS], M2[KSTEPS];
+        mask_lora_a<KSTEPS>(a.R, g, A1, M1);
+        mask_lora_a<KSTEPS>(a.R, g, A2, M2);
+        lora_tile_bf16_regs<KSTEPS>(M1, B1, L1);
+        lora_tile_bf16_regs<KSTEPS>(M2, B2, L2);
+        if constexpr (AHEAD) request_a(row0 + kTileRows);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int64_t r = row0 + 4 * g + v;
+            float f1[8], f2[8], of[8];
+            unpack8(xv1[v], f1);
+            unpack8(xv2[v], f2);
+            if constexpr (AHEAD) request_row(row0 + kTileRows, v);
+            uint32_t lo, hi;
+            codes_to_words<QBIT, false, true>(f1, c1, zero8, lo, hi);
+            store_packed<QBIT, true>(a.q1 + r * row_bytes, chunk, true, lo, hi);
+            codes_to_words<QBIT, false, true>(f2, c2, zero8, lo, hi);
+            store_packed<QBIT, true>(a.q2 + r * row_bytes, chunk, true, lo, hi);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                float y1 = rbf(f1[j] + lora_elem(L1[v], j));
+                y1 = rbf(y1 * rbf(sigmoidf_(y1)));
+                const float y2 = rbf(f2[j] + lora_elem(L2[v], j));
+                of[j] = y1 * y2;
+            }
+            st16_nt(a.o + r * a.N + chunk * 8, pack8(of));
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    request_a(row_begin);
+#pragma unroll
+    for (int v = 0; v < 4; ++v) request_row(row_begin, v);
+    int64_t row0 = row_begin;
+    if (row0 + kTileRows < row_end) {
+        work(row0, std::true_type{});
+        for (row0 += kTileRows; row0 + kTileRows < row_end; row0 += kTileRows) work(row0, std::true_type{});
+    }
+    work(row0, std::false_type{});
+}
+
 template <int QBIT, int KSTEPS>
 HYC_FUSE_KERNEL void lora_silu_fwd_kernel(const FuseArgs a) {
     constexpr int CT = kColTilesPerGroup<QBIT>, RS = kFuseWaves / CT;
@@ -123,8 +214,11 @@ HYC_FUSE_KERNEL void lora_silu_fwd_kernel(const FuseArgs a) {
     int64_t row_end = row_begin + a.rows_per_wave;
     if (row_end > a.T) row_end = a.T;
     if (row_begin >= row_end) return;
+    const bool full = (col_tile + 1) * (kTileCols / 8) <= a.C && (row_end - row_begin) % kTileRows == 0;   // uniform
     if (__ballot(!(c1.fast && c2.fast)) != 0ull)
         fuse_fwd_rows<QBIT, KSTEPS, false>(a, row_begin, row_end, lane, chunk, active, c1, c2, B1, B2);
+    else if (KSTEPS == 1 && full)                  // deeper ranks have no registers to spare for it
+        fuse_fwd_rows_full<QBIT, KSTEPS>(a, row_begin, row_end, lane, chunk, c1, c2, B1, B2);
     else
         fuse_fwd_rows<QBIT, KSTEPS, true>(a, row_begin, row_end, lane, chunk, active, c1, c2, B1, B2);
 }
@@ -160,6 +254,80 @@ HYC_FUSE_KERNEL void lora_silu_bwd_kernel(const FuseArgs a) {
     int64_t row_end = row_begin + a.rows_per_wave;
     if (row_end > a.T) row_end = a.T;
 
+    // one row of 8 element pairs: codes + upstream gradient -> hadamard, grad_gate, grad_up
+    auto row_math = [&](const float (&cd1)[8], const float (&cd2)[8], const float (&gf)[8], const uint32_t (&La)[4],
+                        const uint32_t (&Lb)[4], int64_t t) {
+        float of[8], gg[8], gu[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const float x1 = rbf((cd1[j] - kHalf) * s1[j]);
+            const float x2 = rbf((cd2[j] - kHalf) * s2[j]);
+            const float y1 = rbf(x1 + lora_elem(La, j));
+            const float y2 = rbf(x2 + lora_elem(Lb, j));
+            const float sig = rbf(sigmoidf_(y1));
+            const float sil = rbf(y1 * sig);
+            of[j] = sil * y2;
+            const float gh1 = rbf(gf[j] * y2);
+            gu[j] = gf[j] * sil;
+            const float dsilu = rbf(sig * rbf(1.0f + rbf(y1 * rbf(1.0f - sig))));
+            gg[j] = gh1 * dsilu;
+        }
+        st16_nt(a.o + t * a.N + col0, pack8(of));
+        st16_nt(a.gg + t * a.N + col0, pack8(gg));
+        st16_nt(a.gu + t * a.N + col0, pack8(gu));
+    };
+
+    // Interior strips at rank 16: the rolling prefetch of fuse_fwd_rows_full - a row's registers
+    // are requested again for the next tile as soon as the row has been taken out of them.
+    const bool full = KSTEPS == 1 && (col_tile + 1) * (kTileCols / 8) <= a.C && row_begin < row_end &&
+                      (row_end - row_begin) % kTileRows == 0;      // uniform across the wave
+    if (full) {
+        const int i = lane & 15;
+        u32x2 w1[4], w2[4], A1[KSTEPS], A2[KSTEPS];
+        u32x4 gv[4];
+        auto request_a = [&](int64_t row0) {
+            request_lora_a<KSTEPS>(a.xa1, a.R, row0 + i, g, A1);
+            request_lora_a<KSTEPS>(a.xa2, a.R, row0 + i, g, A2);
+        };
+        auto request_row = [&](int64_t row0, int v) {
+            const int64_t t = row0 + 4 * g + v;
+            w1[v] = ld8(a.q1 + t * row_bytes + slot.offset);
+            w2[v] = ld8(a.q2 + t * row_bytes + slot.offset);
+            gv[v] = ld16_nt(a.g + t * a.N + col0);
+        };
+        auto work = [&](int64_t row0, auto ahead_tag) {
+            constexpr bool AHEAD = decltype(ahead_tag)::value;
+            uint32_t L1[4][4], L2[4][4];
+            u32x2 M1[KSTEPS], M2[KSTEPS];
+            mask_lora_a<KSTEPS>(a.R, g, A1, M1);
+            mask_lora_a<KSTEPS>(a.R, g, A2, M2);
+            lora_tile_bf16_regs<KSTEPS>(M1, B1, L1);
+            lora_tile_bf16_regs<KSTEPS>(M2, B2, L2);
+            if constexpr (AHEAD) request_a(row0 + kTileRows);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                float cd1[8], cd2[8], gf[8];
+                slot.decode(w1[v], cd1);
+                slot.decode(w2[v], cd2);
+                unpack8(gv[v], gf);
+                if constexpr (AHEAD) request_row(row0 + kTileRows, v);
+                row_math(cd1, cd2, gf, L1[v], L2[v], row0 + 4 * g + v);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+        request_a(row_begin);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) request_row(row_begin, v);
+        int64_t row0 = row_begin;
+        if (row0 + kTileRows < row_end) {
+            work(row0, std::true_type{});
+            for (row0 += kTileRows; row0 + kTileRows < row_end; row0 += kTileRows) work(row0, std::true_type{});
+        }
+        work(row0, std::false_type{});
+        return;
+    }
+
     for (int64_t row0 = row_begin; row0 < row_end; row0 += kTileRows) {
         u32x2 w1[4], w2[4];
         u32x4 gv[4];
@@ -182,27 +350,11 @@ HYC_FUSE_KERNEL void lora_silu_bwd_kernel(const FuseArgs a) {
         for (int v = 0; v < 4; ++v) {
             const int64_t t = row0 + 4 * g + v;
             if (!(active && t < row_end)) continue;
-            float cd1[8], cd2[8], gf[8], of[8], gg[8], gu[8];
+            float cd1[8], cd2[8], gf[8];
             slot.decode(w1[v], cd1);
             slot.decode(w2[v], cd2);
             unpack8(gv[v], gf);
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const float x1 = rbf((cd1[j] - kHalf) * s1[j]);
-                const float x2 = rbf((cd2[j] - kHalf) * s2[j]);
-                const float y1 = rbf(x1 + lora_elem(L1[v], j));
-                const float y2 = rbf(x2 + lora_elem(L2[v], j));
-                const float sig = rbf(sigmoidf_(y1));
-                const float sil = rbf(y1 * sig);
-                of[j] = sil * y2;
-                const float gh1 = rbf(gf[j] * y2);
-                gu[j] = gf[j] * sil;
-                const float dsilu = rbf(sig * rbf(1.0f + rbf(y1 * rbf(1.0f - sig))));
-                gg[j] = gh1 * dsilu;
-            }
-            st16_nt(a.o + t * a.N + col0, pack8(of));
-            st16_nt(a.gg + t * a.N + col0, pack8(gg));
-            st16_nt(a.gu + t * a.N + col0, pack8(gu));
+            row_math(cd1, cd2, gf, L1[v], L2[v], t);
             __builtin_amdgcn_sched_barrier(0);
         }
     }
@@ -264,9 +416,13 @@ static int fuse_launch(FuseArgs& a, int64_t T, int64_t N, int64_t R, int q_bit, 
 }
 
 int tune_fuse(const char* key, int value) {
-    if (strcmp(key, "fuse_rows_per_wave") == 0) {
+    const bool both = strcmp(key, "fuse_rows_per_wave") == 0;
+    const bool fwd = both || strcmp(key, "fuse_fwd_rows_per_wave") == 0;
+    const bool bwd = both || strcmp(key, "fuse_bwd_rows_per_wave") == 0;
+    if (fwd || bwd) {
         if (value < kTileRows || value > 65536 || value % kTileRows != 0) return HYC_ERR_ARG;
-        g_fuse_rows_per_wave[0] = g_fuse_rows_per_wave[1] = value;
+        if (bwd) g_fuse_rows_per_wave[0] = value;
+        if (fwd) g_fuse_rows_per_wave[1] = value;
         return HYC_OK;
     }
     return 1;

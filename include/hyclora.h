@@ -44,8 +44,8 @@ int hyc_abi_version(void);
  * default 8), "dequant_rows_per_wave" (same for hyc_unpack_dequant, default 2),
  * "quant_outlier_rows_per_wave" / "dequant_outlier_rows_per_wave" (the same two when called with
  * an outlier list; default 8 each: a wave first has to find its outlier columns in the list),
- * "fuse_rows_per_wave" (same for both fused LoRA-SiLU kernels, multiple of 16; defaults 48 forward,
- * 32 backward).  Unknown key or bad value: HYC_ERR_ARG.  No
+ * "fuse_rows_per_wave" (same for both fused LoRA-SiLU kernels, multiple of 16, default 32;
+ * "fuse_fwd_rows_per_wave" / "fuse_bwd_rows_per_wave" set one of them).  Unknown key or bad value: HYC_ERR_ARG.  No
  * counterpart in the reference (its launch shapes come from triton.autotune). */
 int hyc_set_tuning(const char *key, int value);
 

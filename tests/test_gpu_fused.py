@@ -79,6 +79,41 @@ def test_fused_forward_and_backward(fz, dev, q_bit, dims):
     assert_close_bf16(gu, up.grad, what="grad_up vs autograd")
 
 
+@pytest.mark.parametrize("q_bit", QBITS)
+@pytest.mark.parametrize("R", [16, 8])
+def test_fused_results_do_not_depend_on_the_strip_height(fz, dev, q_bit, R):
+    # Interior strips are walked with the next tile requested ahead: one tile per strip takes only
+    # the closing step of that walk, two tiles the opening and the closing one, more the loop in
+    # between.  All of them, and the guarded path of the ragged last strip, must agree bit for bit.
+    from hyclora_amd import _lib
+    B, M, H, I = 1, 200, 64, 384                     # 200 rows: whole strips and a ragged remainder
+    t = mlp_inputs(7 + q_bit, B, M, H, I, R)
+    xa1, b1, x1 = t["gate"]
+    xa2, b2, x2 = t["up"]
+    s1 = O.scale_only_quant(x1, q_bit)
+    s2 = O.scale_only_quant(x2, q_bit)
+    g = torch.randn(B, M, I, generator=torch.Generator().manual_seed(2)).to(BF16)
+    d = lambda *ts: [v.to(dev) for v in ts]
+    outs = []
+    try:
+        for rows in (16, 32, 48, 96, 208):
+            _lib.set_tuning("fuse_rows_per_wave", rows)
+            q1, q2, o = fz.fwd(*d(xa1, b1, x1, s1, xa2, b2, x2, s2), q_bit)
+            ob, gg, gu = fz.bwd(*d(xa1, b1), q1, s1.to(dev), *d(xa2, b2), q2, s2.to(dev), g.to(dev), q_bit)
+            outs.append((q1, q2, o, ob, gg, gu))
+    finally:
+        _lib.set_tuning("fuse_rows_per_wave", 32)
+    for other in outs[1:]:
+        for a, b in zip(outs[0], other):
+            assert torch.equal(a, b)
+    q1_ref, q2_ref, o_ref = O.fused_fwd(xa1, b1, x1, s1, xa2, b2, x2, s2, q_bit)
+    assert torch.equal(outs[0][0].cpu(), q1_ref) and torch.equal(outs[0][1].cpu(), q2_ref)
+    assert_close_bf16(outs[0][2], o_ref, what="fused forward o vs oracle")
+    ob_ref, gg_ref, gu_ref = O.fused_bwd(xa1, b1, q1_ref, s1, xa2, b2, q2_ref, s2, g, q_bit)
+    assert_close_bf16(outs[0][4], gg_ref, what="grad_gate vs oracle")
+    assert_close_bf16(outs[0][5], gu_ref, what="grad_up vs oracle")
+
+
 def test_fused_lora_term_is_applied_per_row_and_column(fz, dev):
     # x1 = x2 = 0 and a one-hot xa isolates the MFMA operand mapping: y = b[r, :] for row r
     R, N, M = 16, 256, 32
