@@ -120,6 +120,26 @@ __device__ __forceinline__ void lora_tile_bf16_regs(const u32x2 (&A)[KSTEPS], co
 #pragma unroll
         for (int p = 0; p < 4; ++p) L[v][p] = pk_bf16(acc_elem(acc[2 * p], v), acc_elem(acc[2 * p + 1], v));
 }
+// Requests the LoRA-A operand of one tile row (row = row0 + l%16) without touching it.
+template <int KSTEPS>
+__device__ __forceinline__ void request_lora_a(const uint16_t* xa, int R, int64_t row, int g, u32x2 (&A)[KSTEPS]) {
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+        const int k = 16 * ks + 4 * g;
+        A[ks] = ld8(xa + row * R + (k < R ? k : 0));         // past the rank: any valid address, see below
+    }
+}
+// Zeroes the operands past the rank (a rank that is not a multiple of 16).  Done when the operand
+// is used, not when it is requested: touching the value would wait for the load.
+template <int KSTEPS>
+__device__ __forceinline__ void mask_lora_a(int R, int g, const u32x2 (&A)[KSTEPS], u32x2 (&M)[KSTEPS]) {
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+        const bool ok = 16 * ks + 4 * g < R;
+        M[ks] = u32x2{ok ? A[ks].x : 0u, ok ? A[ks].y : 0u};
+    }
+}
+
 __device__ __forceinline__ float lora_elem(const uint32_t (&Lv)[4], int j) {
     return (j & 1) ? bf_hi(Lv[j >> 1]) : bf_lo(Lv[j >> 1]);
 }

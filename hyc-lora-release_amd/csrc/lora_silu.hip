@@ -106,25 +106,6 @@ __device__ __forceinline__ void fuse_fwd_rows(const FuseArgs& a, int64_t row_beg
 // then for data requested a whole tile earlier, and the stores of the rows in between stay in
 // flight (loads and stores retire through one in-order counter).  The first tile is peeled so
 // that the loop is entered in the state its back edge carries; the last one requests nothing.
-template <int KSTEPS>
-__device__ __forceinline__ void request_lora_a(const uint16_t* xa, int R, int64_t row, int g, u32x2 (&A)[KSTEPS]) {
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) {
-        const int k = 16 * ks + 4 * g;
-        A[ks] = ld8(xa + row * R + (k < R ? k : 0));         // past the rank: any valid address, see below
-    }
-}
-// Zeroes the operands past the rank (a rank that is not a multiple of 16).  Done when the operand
-// is used, not when it is requested: touching the value would wait for the load.
-template <int KSTEPS>
-__device__ __forceinline__ void mask_lora_a(int R, int g, const u32x2 (&A)[KSTEPS], u32x2 (&M)[KSTEPS]) {
-#pragma unroll
-    for (int ks = 0; ks < KSTEPS; ++ks) {
-        const bool ok = 16 * ks + 4 * g < R;
-        M[ks] = u32x2{ok ? A[ks].x : 0u, ok ? A[ks].y : 0u};
-    }
-}
-
 template <int QBIT, int KSTEPS>
 __device__ __forceinline__ void fuse_fwd_rows_full(const FuseArgs& a, int64_t row_begin, int64_t row_end, int lane,
                                                    int chunk, const QuantCols<QBIT>& c1, const QuantCols<QBIT>& c2,
