@@ -531,7 +531,7 @@ def main():
         lora = {}
         Kl = 40
         for wname, Nw in (("n4096", H), ("n11008", N)):
-            NBl = 4
+            NBl = -(-600_000_000 // (T * Nw * 2))        # the rotating inputs alone exceed the 256 MiB last-level cache
             x_l = [randn(B, M, Nw) for _ in range(NBl)]
             y_l = [torch.empty(B, M, Nw, device=dev, dtype=BF16) for _ in range(NBl)]
             q_l = [torch.empty(B, M, Nw * QB // 8, device=dev, dtype=torch.uint8) for _ in range(NBl)]
@@ -606,29 +606,30 @@ def main():
 
     if args.only == "all":
         Kx, Wx = max(K // 4, 10), max(W // 4, 3)
-        x_h = [randn(B, M, H) for _ in range(4)]
+        NH = 16                                   # 16 x 33.5 MB: past the 256 MiB last-level cache
+        x_h = [randn(B, M, H) for _ in range(NH)]
         w_h = torch.ones(H, device=dev, dtype=BF16)
-        ms, _ = timed(lambda i: rmsnorm_kernels.rmsnorm_forward(x_h[i % 4], w_h, 1e-5), Kx, Wx)
+        ms, _ = timed(lambda i: rmsnorm_kernels.rmsnorm_forward(x_h[i % NH], w_h, 1e-5), Kx, Wx)
         kernels["rmsnorm_fwd_4096"] = {"ms": ms, "GBps": T * H * 4 / ms / 1e6}
         y, mean, rstd, bs, nw = rmsnorm_kernels.rmsnorm_forward(x_h[0], w_h, 1e-5)
-        ms, _ = timed(lambda i: rmsnorm_kernels.rmsnorm_backward(x_h[(i + 1) % 4], x_h[i % 4], w_h, mean, rstd, True, 1e-5, nw, bs), Kx, Wx)
+        ms, _ = timed(lambda i: rmsnorm_kernels.rmsnorm_backward(x_h[(i + 1) % NH], x_h[i % NH], w_h, mean, rstd, True, 1e-5, nw, bs), Kx, Wx)
         kernels["rmsnorm_bwd_4096"] = {"ms": ms, "GBps": T * H * 6 / ms / 1e6}
         ms, _ = timed(lambda i: silu_kernels.silu_backward(xs[i % NB], xs[(i + 1) % NB]), Kx, Wx)
         kernels["silu_bwd"] = {"ms": ms, "GBps": E * 6 / ms / 1e6}
         idx = torch.randperm(H, device=dev)[:20].contiguous()
         _, sc = cf.get_statistics_channel_base(x_h[0], 0.005, QB, 'per-channel')
-        ms, _ = timed(lambda i: cf.outlier_subtraction_fuse_compression_quantization(x_h[i % 4], sc, idx, QB), Kx, Wx)
+        ms, _ = timed(lambda i: cf.outlier_subtraction_fuse_compression_quantization(x_h[i % NH], sc, idx, QB), Kx, Wx)
         kernels["quant_pack_q4_outlier_4096"] = {"ms": ms, "GBps": T * H * 2.5 / ms / 1e6}
         sy = cf.get_statistics_only_quant(y, QB, 'per-channel')
         tbl = rmsnorm_kernels.outlier_table(idx, H)
-        ms, _ = timed(lambda i: rmsnorm_kernels.rmsnorm_forward_compress(x_h[i % 4], w_h, 1e-5, QB, scale_y=sy, scale_x=sc,
+        ms, _ = timed(lambda i: rmsnorm_kernels.rmsnorm_forward_compress(x_h[i % NH], w_h, 1e-5, QB, scale_y=sy, scale_x=sc,
                                                                          outlier_idx=idx, table=tbl), Kx, Wx)
-        ms3, _ = timed(lambda i: (rmsnorm_kernels.rmsnorm_forward(x_h[i % 4], w_h, 1e-5),
-                                  cf.outlier_subtraction_fuse_compression_quantization(x_h[i % 4], sc, idx, QB),
-                                  cf.compression_quantization(x_h[(i + 1) % 4], sy, QB)), Kx, Wx)
+        ms3, _ = timed(lambda i: (rmsnorm_kernels.rmsnorm_forward(x_h[i % NH], w_h, 1e-5),
+                                  cf.outlier_subtraction_fuse_compression_quantization(x_h[i % NH], sc, idx, QB),
+                                  cf.compression_quantization(x_h[(i + 1) % NH], sy, QB)), Kx, Wx)
         kernels["rmsnorm_fwd_compress_4096"] = {"ms": ms, "GBps": T * H * (4 + 2 * QB / 8) / ms / 1e6,
                                                 "three_separate_kernels_ms": ms3}
-        ms, _ = timed(lambda i: cf.get_statistics_channel_base(x_h[i % 4], 0.005, QB, 'per-channel'), Kx, Wx)
+        ms, _ = timed(lambda i: cf.get_statistics_channel_base(x_h[i % NH], 0.005, QB, 'per-channel'), Kx, Wx)
         kernels["calibration_stats_4096"] = {"ms": ms}
         # attention map (configuration 3 shape): compaction, restore, softmax backward
         a = torch.softmax(torch.randn(4, 32, 1024, 1024, generator=gen, device=dev) * 0.707

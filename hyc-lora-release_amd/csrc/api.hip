@@ -28,5 +28,7 @@ extern "C" int hyc_set_tuning(const char* key, int value) {
     if (rc != 1) return rc;
     rc = hyc::tune_contract(key, value);
     if (rc != 1) return rc;
+    rc = hyc::tune_norm_compress(key, value);
+    if (rc != 1) return rc;
     return HYC_ERR_ARG;
 }

@@ -85,6 +85,13 @@ __device__ __forceinline__ float wave_sum(float v) {
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
     return v;
 }
+// sum of the squares of one 8-element chunk: a fused-multiply-add chain from zero
+__device__ __forceinline__ float chunk_sumsq(const float (&f)[8]) {
+    float p = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) p = fmaf(f[j], f[j], p);
+    return p;
+}
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
@@ -117,5 +124,6 @@ int tune_quant(const char* key, int value);
 int tune_fuse(const char* key, int value);
 int tune_add(const char* key, int value);
 int tune_contract(const char* key, int value);
+int tune_norm_compress(const char* key, int value);
 
 }  // namespace hyc

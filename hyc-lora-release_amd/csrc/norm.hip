@@ -45,12 +45,14 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_fwd_kernel(const uint16_
         xv[c] = u32x4{0, 0, 0, 0};
         if (col < N) xv[c] = ld16_nt(xr + col);
     }
+    // Summation order (shared with the fused norm + compress kernels, whose results must be the
+    // same bits): the 8 squares of a chunk as one fused-multiply-add chain from zero, a lane's
+    // chunks added in column order, then the butterfly over the lanes.
 #pragma unroll
     for (int c = 0; c < CH; ++c) {
         float f[8];
         unpack8(xv[c], f);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) ss = fmaf(f[j], f[j], ss);
+        ss += chunk_sumsq(f);
     }
     ss = wave_sum(ss);
     const float rstd = 1.0f / sqrtf(ss / (float)N + eps);

@@ -8,13 +8,18 @@
 //     y      = bf16(x * rstd * w), rstd = 1/sqrt(mean(x^2) + eps)        (rmsnorm_kernels.py:34-54)
 //     q_y    = Q(y; scale_y)                                              packed codes
 //     x_out  = x[:, outlier channels];  q_x = Q(x with those channels zeroed; scale_x)
-// One wave owns one row, each lane CH 16-byte chunks of it, as in the plain forward kernel; the
+// Two kernels: the general one below, and a column-slab form further down for rows that are a
+// whole number of 512-column slabs.
+// General form: one wave owns one row, each lane CH 16-byte chunks of it, as in the plain forward kernel; the
 // per-column steps are re-read per row (L2 hits, like the norm weight).  The row is parked in LDS
 // after the sum of squares (each lane reads back only what it wrote, so no barrier is involved)
 // and the second phase walks the chunks in a rolled loop: one copy of the quantiser code and a
 // few dozen live registers instead of CH unrolled copies, which is what keeps enough waves
 // resident to hide the latency of the per-chunk constant loads.
 // Only frozen (calibrated) steps can be used here: during calibration the steps of y depend on y.
+#include <cstring>
+#include <type_traits>
+
 #include "hyc_pack.hpp"
 
 namespace hyc {
@@ -68,8 +73,7 @@ void rmsnorm_fwd_compress_kernel(const NormCompressArgs a) {
         for (int c = 0; c < CH; ++c) {
             float f[8];
             unpack8(xv[c], f);
-#pragma unroll
-            for (int j = 0; j < 8; ++j) ss = fmaf(f[j], f[j], ss);
+            ss += chunk_sumsq(f);                       // the plain forward kernel's order
             park[c * kWave + lane] = xv[c];
         }
     }
@@ -128,6 +132,160 @@ void rmsnorm_fwd_compress_kernel(const NormCompressArgs a) {
     }
 }
 
+// ------------------------------------------------------------------------------------
+// Column-slab form for rows that are a whole number of 512-column slabs (hidden sizes 4096, 5120,
+// 8192 ...) and even row counts.
+//
+// In the row-per-wave kernel above every wave re-reads the per-column constants of all its chunks
+// (norm weight, two steps with their reciprocals, the outlier table) for a single row, and all
+// waves of the launch move through "load, reduce, store" together.  Here a workgroup has one wave
+// per slab and walks a strip of rows: a lane keeps ONE chunk of columns, so its constants live in
+// registers for the whole strip, and the strip is streamed two rows at a time with the next two
+// requested as soon as the current ones are unpacked (the rolling prefetch of the fused LoRA
+// kernels).  The price is a workgroup-wide sum per row: each wave leaves its lanes' chunk sums in
+// LDS, one barrier per two rows, and every wave then adds the slabs of each lane in column order
+// and runs the butterfly over the lanes - the plain forward kernel's summation order, so rstd, y
+// and all codes are the same bits as from the kernel above.  The partial sums are double-buffered:
+// a wave can be at most one step ahead of the slowest one.
+constexpr int kSlabRows = 2;                        // rows per step; row counts must be a multiple of it
+static int g_slab_rows_per_group = 0;               // strip height per workgroup; 0 = from the row count
+static int g_slab_enabled = 1;
+
+// Compute units of the current device (asked once; 256 if the query fails).
+static int compute_units() {
+    static int n = 0;
+    if (n == 0) {
+        int dev = 0, v = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && v > 0)
+            n = v;
+        else
+            n = 256;
+    }
+    return n;
+}
+
+// MAXW: the most waves a workgroup may have (8: rows up to 4096 columns, 16: up to 8192).  Four
+// waves per SIMD either way: two workgroups of 8 waves or one of 16 on a compute unit.
+template <int QBIT, bool W32, int MAXW>
+__global__ __launch_bounds__(MAXW * kWave) __attribute__((amdgpu_waves_per_eu(4)))
+void rmsnorm_fwd_compress_slab_kernel(const NormCompressArgs a, int rows_per_group) {
+    constexpr int G = kSlabRows;
+    extern __shared__ float slab_part[];                // [2][G][waves][64]
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int nw = blockDim.x >> 6;
+    const int chunk = wave * kWave + lane;
+    const int col = chunk * 8;
+    const int N = a.N;
+    const int row_bytes = N * QBIT / 8;
+    const int64_t r0 = (int64_t)blockIdx.x * rows_per_group;
+    int64_t r1 = r0 + rows_per_group;
+    if (r1 > a.rows) r1 = a.rows;
+    if (r0 >= r1) return;                               // whole workgroups leave together
+
+    // per-column constants, once per strip
+    float wf[8];
+    if constexpr (W32) {
+        const f32x4 w0 = *reinterpret_cast<const f32x4*>((const float*)a.w + col);
+        const f32x4 w1 = *reinterpret_cast<const f32x4*>((const float*)a.w + col + 4);
+        wf[0] = w0.x; wf[1] = w0.y; wf[2] = w0.z; wf[3] = w0.w;
+        wf[4] = w1.x; wf[5] = w1.y; wf[6] = w1.z; wf[7] = w1.w;
+    } else {
+        unpack8(ld16((const uint16_t*)a.w + col), wf);
+    }
+    QuantCols<QBIT> qy, qx;
+    qy.load(a.q_y ? a.scale_y : a.scale_x, col, a.q_y != nullptr);      // an unused set reads as steps of 1
+    qx.load(a.q_x ? a.scale_x : a.scale_y, col, a.q_x != nullptr);
+    u32x4 tv = {0, 0, 0, 0};
+    if (a.q_x && a.k > 0) tv = ld16(a.otable + col);
+    const uint32_t td[4] = {tv.x, tv.y, tv.z, tv.w};
+    const bool has_outlier = (tv.x | tv.y | tv.z | tv.w) != 0u;
+    const bool fast = __ballot(!(qy.fast && qx.fast)) == 0ull;          // uniform across the wave
+    const float zero8[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+
+    u32x4 xv[G];
+    auto request = [&](int64_t r) __attribute__((always_inline)) {
+#pragma unroll
+        for (int g = 0; g < G; ++g) xv[g] = ld16_nt(a.x + (r + g) * N + col);
+    };
+    auto step = [&](int64_t r, int buf, auto ahead_tag, auto fast_tag) __attribute__((always_inline)) {
+        constexpr bool AHEAD = decltype(ahead_tag)::value;
+        constexpr bool FAST = decltype(fast_tag)::value;
+        float f[G][8];
+        float* mine = slab_part + ((buf * G) * nw + wave) * kWave + lane;
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            unpack8(xv[g], f[g]);
+            mine[g * nw * kWave] = chunk_sumsq(f[g]);
+        }
+        if constexpr (AHEAD) request(r + G);
+        // A barrier that orders LDS only: __syncthreads() would also wait for every global access in
+        // flight - the rows just requested and the previous step's stores.
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+        float rstd[G];
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            const float* all = slab_part + ((buf * G + g) * nw) * kWave + lane;
+            float t = 0.0f;
+#pragma unroll 4
+            for (int w = 0; w < nw; ++w) t += all[w * kWave];            // slabs in column order
+            t = wave_sum(t);
+            rstd[g] = 1.0f / sqrtf(t / (float)N + a.eps);
+        }
+        if (wave == 0 && lane == 0) {
+#pragma unroll
+            for (int g = 0; g < G; ++g) a.rstd[r + g] = rstd[g];
+        }
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            const int64_t row = r + g;
+            float o[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) o[j] = (f[g][j] * rstd[g]) * wf[j];
+            const u32x4 yv = pack8(o);
+            st16_nt(a.y + row * N + col, yv);
+            uint32_t lo, hi;
+            if (a.q_y) {
+                float fy[8];
+                unpack8(yv, fy);
+                codes_to_words<QBIT, false, FAST>(fy, qy, zero8, lo, hi);
+                store_packed<QBIT, true>(a.q_y + row * row_bytes, chunk, true, lo, hi);
+            }
+            if (a.q_x) {
+                if (has_outlier) {
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) {
+                        const uint32_t p = (td[j >> 1] >> (16 * (j & 1))) & 0xffffu;
+                        if (p) {
+                            a.xo[row * a.k + (p - 1)] = (uint16_t)(__float_as_uint(f[g][j]) >> 16);
+                            f[g][j] = 0.0f;
+                        }
+                    }
+                }
+                codes_to_words<QBIT, false, FAST>(f[g], qx, zero8, lo, hi);
+                store_packed<QBIT, true>(a.q_x + row * row_bytes, chunk, true, lo, hi);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    auto run = [&](auto fast_tag) __attribute__((always_inline)) {
+        request(r0);
+        int64_t r = r0;
+        int buf = 0;
+        if (r + G < r1) {
+            step(r, buf, std::true_type{}, fast_tag);
+            for (r += G, buf ^= 1; r + G < r1; r += G, buf ^= 1) step(r, buf, std::true_type{}, fast_tag);
+        }
+        step(r, buf, std::false_type{}, fast_tag);
+    };
+    // every wave of the workgroup makes the same number of steps whichever branch it takes
+    if (fast) run(std::true_type{});
+    else run(std::false_type{});
+}
+
 // otable[c] = 1 + i for c = oidx[i], everything else 0 (table cleared by the first kernel)
 __global__ void otable_fill_kernel(uint16_t* __restrict__ table, int n) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -143,6 +301,26 @@ __global__ void otable_mark_kernel(const int64_t* __restrict__ oidx, int k, int 
 
 template <int QBIT, bool W32>
 static int launch_nc(const NormCompressArgs& a, hipStream_t st) {
+    if (g_slab_enabled && a.N % (kWave * 8) == 0 && a.N / (kWave * 8) <= 16 && a.rows % kSlabRows == 0) {
+        const int waves = a.N / (kWave * 8);
+        // Strip height: all workgroups resident at once (16 waves per compute unit), each walking as
+        // long a strip as that allows - the per-column constants are set up once per strip.
+        int rows_per_group = g_slab_rows_per_group;
+        if (rows_per_group == 0) {
+            const int64_t resident = (int64_t)compute_units() * (16 / (waves <= 8 ? waves : 16));
+            rows_per_group = (int)(cdiv(cdiv(a.rows, resident), (int64_t)kSlabRows) * kSlabRows);
+        }
+        const int64_t groups = cdiv(a.rows, (int64_t)rows_per_group);
+        if (groups > INT32_MAX) return HYC_ERR_SHAPE;
+        const size_t lds = 2 * kSlabRows * waves * kWave * sizeof(float);
+        if (waves <= 8)
+            hipLaunchKernelGGL((rmsnorm_fwd_compress_slab_kernel<QBIT, W32, 8>), dim3((unsigned)groups), dim3(waves * kWave), lds,
+                               st, a, rows_per_group);
+        else
+            hipLaunchKernelGGL((rmsnorm_fwd_compress_slab_kernel<QBIT, W32, 16>), dim3((unsigned)groups), dim3(waves * kWave), lds,
+                               st, a, rows_per_group);
+        return check_launch();
+    }
     const dim3 grid((unsigned)cdiv(a.rows, (int64_t)kNcWaves)), block(kNcThreads);
 #define HYC_NC(CH) \
     hipLaunchKernelGGL((rmsnorm_fwd_compress_kernel<CH, QBIT, W32>), grid, block, kNcWaves * CH * kWave * 16, st, a)
@@ -153,6 +331,20 @@ static int launch_nc(const NormCompressArgs& a, hipStream_t st) {
     else HYC_NC(16);
 #undef HYC_NC
     return check_launch();
+}
+
+int tune_norm_compress(const char* key, int value) {
+    if (strcmp(key, "norm_compress_slab") == 0) {
+        if (value != 0 && value != 1) return HYC_ERR_ARG;
+        g_slab_enabled = value;
+        return HYC_OK;
+    }
+    if (strcmp(key, "norm_compress_rows_per_group") == 0) {
+        if (value < 0 || value > 65536 || value % kSlabRows != 0) return HYC_ERR_ARG;   // 0: choose from the row count
+        g_slab_rows_per_group = value;
+        return HYC_OK;
+    }
+    return 1;
 }
 
 }  // namespace hyc

@@ -44,6 +44,9 @@ int hyc_abi_version(void);
  * default 8), "dequant_rows_per_wave" (same for hyc_unpack_dequant, default 2),
  * "quant_outlier_rows_per_wave" / "dequant_outlier_rows_per_wave" (the same two when called with
  * an outlier list; default 8 each: a wave first has to find its outlier columns in the list),
+ * "norm_compress_slab" (0 / 1: whether hyc_rmsnorm_fwd_compress may use its column-slab kernel, default 1)
+ * and "norm_compress_rows_per_group" (rows a workgroup of that kernel walks, even; 0 = chosen from the
+ * row count, the default),
  * "fuse_rows_per_wave" (same for both fused LoRA-SiLU kernels, multiple of 16, default 32;
  * "fuse_fwd_rows_per_wave" / "fuse_bwd_rows_per_wave" set one of them).  Unknown key or bad value: HYC_ERR_ARG.  No
  * counterpart in the reference (its launch shapes come from triton.autotune). */

@@ -22,7 +22,10 @@ def ops():
 
 
 @pytest.mark.parametrize("q_bit", [2, 4, 8])
-@pytest.mark.parametrize("shape", [(2, 37, 4096), (1, 5, 512), (3, 4, 96), (1, 9, 8192), (2, 3, 1024 + 32)])
+@pytest.mark.parametrize("shape", [(2, 37, 4096), (1, 5, 512), (3, 4, 96), (1, 9, 8192), (2, 3, 1024 + 32),
+                                   # whole 512-column slabs and an even row count: the
+                                   # column-slab kernel (1, 2, 8, 10 and 16 waves per workgroup)
+                                   (2, 34, 4096), (1, 8, 512), (4, 1, 1024), (1, 20, 5120), (1, 12, 8192)])
 @pytest.mark.parametrize("wdtype", [BF16, torch.float32])
 def test_fused_equals_separate_operators(ops, dev, q_bit, shape, wdtype):
     x, planted = activation_with_outlier_channels(seed=shape[-1] + q_bit, shape=shape, frac=0.01)
@@ -51,6 +54,33 @@ def test_fused_equals_separate_operators(ops, dev, q_bit, shape, wdtype):
     y3, _, q_y3, q_x3, xo3 = ops.norm.rmsnorm_forward_compress(xd, wd, 1e-5, q_bit, scale_x=s_x)   # no outlier channels
     assert q_y3 is None and xo3.shape[-1] == 0
     assert torch.equal(q_x3, ops.cf.compression_quantization(xd, s_x, q_bit))
+
+
+@pytest.mark.parametrize("q_bit", [2, 4, 8])
+@pytest.mark.parametrize("shape", [(1, 72, 4096), (1, 40, 8192), (2, 10, 1536)])
+def test_both_kernel_forms_give_the_same_bits(ops, dev, q_bit, shape):
+    # the row-per-wave kernel and the column-slab kernel, the latter at several strip heights
+    # (one step per strip, two, several, a short last strip)
+    from hyclora_amd import _lib
+    x, _ = activation_with_outlier_channels(seed=3 + q_bit, shape=shape, frac=0.01)
+    w = (1 + 0.1 * torch.randn(shape[-1], generator=torch.Generator().manual_seed(2))).to(BF16)
+    xd, wd = x.to(dev), w.to(dev)
+    idx, s_x = ops.cf.get_statistics_channel_base(xd, 0.01, q_bit, 'per-channel')
+    y_ref = ops.norm.rmsnorm_forward(xd, wd, 1e-5)[0]
+    s_y = ops.cf.get_statistics_only_quant(y_ref, q_bit, 'per-channel')
+    run = lambda: ops.norm.rmsnorm_forward_compress(xd, wd, 1e-5, q_bit, scale_y=s_y, scale_x=s_x, outlier_idx=idx)
+    try:
+        _lib.set_tuning("norm_compress_slab", 0)
+        base = run()
+        _lib.set_tuning("norm_compress_slab", 1)
+        for rows in (0, 2, 4, 6, 16, 128):             # 0: the library's own choice
+            _lib.set_tuning("norm_compress_rows_per_group", rows)
+            for got, want in zip(run(), base):
+                assert torch.equal(got.view(torch.uint8) if got.dtype == BF16 else got,
+                                   want.view(torch.uint8) if want.dtype == BF16 else want), f"strip height {rows}"
+    finally:
+        _lib.set_tuning("norm_compress_slab", 1)
+        _lib.set_tuning("norm_compress_rows_per_group", 0)
 
 
 def test_outlier_table_and_errors(ops, dev):
