@@ -47,7 +47,8 @@ int hyc_abi_version(void);
  * "norm_compress_slab" (0 / 1: whether hyc_rmsnorm_fwd_compress may use its column-slab kernel, default 1)
  * and "norm_compress_rows_per_group" (rows a workgroup of that kernel walks, even; 0 = chosen from the
  * row count, the default),
- * "fuse_rows_per_wave" (same for both fused LoRA-SiLU kernels, multiple of 16, default 32;
+ * "fuse_rows_per_wave" (same for both fused LoRA-SiLU kernels, multiple of 16; defaults: backward 32,
+ * forward 0 = 96 for tensors of 2^24 elements and more, else 32;
  * "fuse_fwd_rows_per_wave" / "fuse_bwd_rows_per_wave" set one of them).  Unknown key or bad value: HYC_ERR_ARG.  No
  * counterpart in the reference (its launch shapes come from triton.autotune). */
 int hyc_set_tuning(const char *key, int value);

@@ -102,7 +102,8 @@ def test_fused_results_do_not_depend_on_the_strip_height(fz, dev, q_bit, R):
             ob, gg, gu = fz.bwd(*d(xa1, b1), q1, s1.to(dev), *d(xa2, b2), q2, s2.to(dev), g.to(dev), q_bit)
             outs.append((q1, q2, o, ob, gg, gu))
     finally:
-        _lib.set_tuning("fuse_rows_per_wave", 32)
+        _lib.set_tuning("fuse_bwd_rows_per_wave", 32)      # the library's defaults
+        _lib.set_tuning("fuse_fwd_rows_per_wave", 0)
     for other in outs[1:]:
         for a, b in zip(outs[0], other):
             assert torch.equal(a, b)
