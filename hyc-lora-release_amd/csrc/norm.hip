@@ -103,9 +103,14 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_fwd_long_kernel(const ui
 // dx = (w*dy - (x^*c1 + c2)) * rstd,  c1 = mean(x^ * w*dy),  c2 = mean(w*dy),  x^ = x*rstd.
 // The c2 term belongs to LayerNorm; the reference keeps it for RMSNorm
 // (operators/rmsnorm_kernels.py:92-100) and so does this kernel.
-template <int CH, bool W32, bool DW>
+// RES: dx = bf16(bf16(that) + residual) - the gradient arriving over the residual connection,
+// which the layers add right after this call (`grad_norm + grad_output`,
+// models/llama/fused_llama_layer_intra_inter_full_fuse.py:393, :493): the same two roundings as the
+// separate add, without its pass over three tensors.
+template <int CH, bool W32, bool DW, bool RES>
 __global__ __launch_bounds__(kNormThreads) void rmsnorm_bwd_kernel(const uint16_t* __restrict__ dy, const uint16_t* __restrict__ x,
                                                                    const void* __restrict__ w, const float* __restrict__ rstd_in,
+                                                                   const uint16_t* __restrict__ res,
                                                                    uint16_t* __restrict__ dx, float* __restrict__ dw_partial,
                                                                    int64_t rows, int N) {
     const int lane = threadIdx.x & (kWave - 1);
@@ -122,15 +127,17 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_bwd_kernel(const uint16_
     const float inv_n = 1.0f / (float)N;
     for (int64_t row = (int64_t)blockIdx.x * kNormWaves + wave; row < rows; row += (int64_t)gridDim.x * kNormWaves) {
         const float rstd = rstd_in[row];
-        u32x4 xv[CH], gv[CH];
+        u32x4 xv[CH], gv[CH], rv[RES ? CH : 1];
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
             const int col = (c * kWave + lane) * 8;
             xv[c] = u32x4{0, 0, 0, 0};
             gv[c] = u32x4{0, 0, 0, 0};
+            if constexpr (RES) rv[c] = u32x4{0, 0, 0, 0};
             if (col < N) {
                 xv[c] = ld16_nt(x + row * N + col);
                 gv[c] = ld16_nt(dy + row * N + col);
+                if constexpr (RES) rv[c] = ld16_nt(res + row * N + col);
             }
         }
         float s1 = 0.0f, s2 = 0.0f;
@@ -162,6 +169,12 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_bwd_kernel(const uint16_
                 for (int j = 0; j < 8; ++j) {
                     const float xh = xf[j] * rstd, wdy = wf[j] * gf[j];
                     o[j] = (wdy - (xh * c1 + c2)) * rstd;
+                }
+                if constexpr (RES) {
+                    float rf[8];
+                    unpack8(rv[c], rf);
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) o[j] = rbf(o[j]) + rf[j];
                 }
                 st16_nt(dx + row * N + col, pack8(o));
             }
@@ -222,11 +235,11 @@ static int launch_fwd(const uint16_t* x, const void* w, uint16_t* y, float* rstd
     return check_launch();
 }
 
-template <bool W32, bool DW>
-static int launch_bwd(const uint16_t* dy, const uint16_t* x, const void* w, const float* rstd, uint16_t* dx,
-                      float* partial, int64_t rows, int N, int blocks, hipStream_t st) {
+template <bool W32, bool DW, bool RES>
+static int launch_bwd_r(const uint16_t* dy, const uint16_t* x, const void* w, const float* rstd, const uint16_t* res,
+                        uint16_t* dx, float* partial, int64_t rows, int N, int blocks, hipStream_t st) {
     const dim3 grid((unsigned)blocks), block(kNormThreads);
-#define HYC_BWD(CH) hipLaunchKernelGGL((rmsnorm_bwd_kernel<CH, W32, DW>), grid, block, 0, st, dy, x, w, rstd, dx, partial, rows, N)
+#define HYC_BWD(CH) hipLaunchKernelGGL((rmsnorm_bwd_kernel<CH, W32, DW, RES>), grid, block, 0, st, dy, x, w, rstd, res, dx, partial, rows, N)
     if (N <= 512) HYC_BWD(1);
     else if (N <= 1024) HYC_BWD(2);
     else if (N <= 2048) HYC_BWD(4);
@@ -234,6 +247,12 @@ static int launch_bwd(const uint16_t* dy, const uint16_t* x, const void* w, cons
     else HYC_BWD(16);
 #undef HYC_BWD
     return check_launch();
+}
+template <bool W32, bool DW>
+static int launch_bwd(const uint16_t* dy, const uint16_t* x, const void* w, const float* rstd, const uint16_t* res,
+                      uint16_t* dx, float* partial, int64_t rows, int N, int blocks, hipStream_t st) {
+    return res ? launch_bwd_r<W32, DW, true>(dy, x, w, rstd, res, dx, partial, rows, N, blocks, st)
+               : launch_bwd_r<W32, DW, false>(dy, x, w, rstd, res, dx, partial, rows, N, blocks, st);
 }
 
 }  // namespace hyc
@@ -257,13 +276,14 @@ extern "C" int64_t hyc_rmsnorm_bwd_workspace(int64_t rows, int64_t N) {
     return (int64_t)bwd_blocks(rows) * N * (int64_t)sizeof(float);
 }
 
-extern "C" int hyc_rmsnorm_bwd(const void* dy, const void* x, const void* weight, int weight_is_fp32,
-                               const float* rstd, void* dx, void* dw, void* workspace, int64_t workspace_bytes,
-                               int64_t rows, int64_t N, void* stream) {
+static int rmsnorm_bwd_any(const void* dy, const void* x, const void* weight, int weight_is_fp32, const float* rstd,
+                           const void* residual, void* dx, void* dw, void* workspace, int64_t workspace_bytes,
+                           int64_t rows, int64_t N, void* stream) {
     if (rows < 0 || N < 0 || N % 8 != 0 || N > 8192) return HYC_ERR_SHAPE;
     if (rows == 0 || N == 0) return HYC_OK;
     if (!dy || !x || !weight || !rstd || !dx) return HYC_ERR_NULL;
-    if (!aligned16(dy) || !aligned16(x) || !aligned16(weight) || !aligned16(dx)) return HYC_ERR_ALIGN;
+    if (!aligned16(dy) || !aligned16(x) || !aligned16(weight) || !aligned16(dx) || !aligned16(residual)) return HYC_ERR_ALIGN;
+    const uint16_t* res = (const uint16_t*)residual;
     hipStream_t st = (hipStream_t)stream;
     const int blocks = bwd_blocks(rows);
     int rc;
@@ -271,8 +291,8 @@ extern "C" int hyc_rmsnorm_bwd(const void* dy, const void* x, const void* weight
         if (!workspace) return HYC_ERR_NULL;
         if (workspace_bytes < hyc_rmsnorm_bwd_workspace(rows, N)) return HYC_ERR_WORKSPACE;
         rc = weight_is_fp32
-                 ? launch_bwd<true, true>((const uint16_t*)dy, (const uint16_t*)x, weight, rstd, (uint16_t*)dx, (float*)workspace, rows, (int)N, blocks, st)
-                 : launch_bwd<false, true>((const uint16_t*)dy, (const uint16_t*)x, weight, rstd, (uint16_t*)dx, (float*)workspace, rows, (int)N, blocks, st);
+                 ? launch_bwd<true, true>((const uint16_t*)dy, (const uint16_t*)x, weight, rstd, res, (uint16_t*)dx, (float*)workspace, rows, (int)N, blocks, st)
+                 : launch_bwd<false, true>((const uint16_t*)dy, (const uint16_t*)x, weight, rstd, res, (uint16_t*)dx, (float*)workspace, rows, (int)N, blocks, st);
         if (rc != HYC_OK) return rc;
         const dim3 grid((unsigned)cdiv(N, 256)), block(256);
         if (weight_is_fp32) hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel<true>, grid, block, 0, st, (const float*)workspace, blocks, (int)N, dw);
@@ -281,6 +301,19 @@ extern "C" int hyc_rmsnorm_bwd(const void* dy, const void* x, const void* weight
     }
     // without dw the grid need not be capped, but the same persistent loop is used
     return weight_is_fp32
-               ? launch_bwd<true, false>((const uint16_t*)dy, (const uint16_t*)x, weight, rstd, (uint16_t*)dx, nullptr, rows, (int)N, (int)(cdiv(rows, kNormWaves) > 65535 * 16 ? 65535 * 16 : cdiv(rows, kNormWaves)), st)
-               : launch_bwd<false, false>((const uint16_t*)dy, (const uint16_t*)x, weight, rstd, (uint16_t*)dx, nullptr, rows, (int)N, (int)(cdiv(rows, kNormWaves) > 65535 * 16 ? 65535 * 16 : cdiv(rows, kNormWaves)), st);
+               ? launch_bwd<true, false>((const uint16_t*)dy, (const uint16_t*)x, weight, rstd, res, (uint16_t*)dx, nullptr, rows, (int)N, (int)(cdiv(rows, kNormWaves) > 65535 * 16 ? 65535 * 16 : cdiv(rows, kNormWaves)), st)
+               : launch_bwd<false, false>((const uint16_t*)dy, (const uint16_t*)x, weight, rstd, res, (uint16_t*)dx, nullptr, rows, (int)N, (int)(cdiv(rows, kNormWaves) > 65535 * 16 ? 65535 * 16 : cdiv(rows, kNormWaves)), st);
+}
+
+extern "C" int hyc_rmsnorm_bwd(const void* dy, const void* x, const void* weight, int weight_is_fp32,
+                               const float* rstd, void* dx, void* dw, void* workspace, int64_t workspace_bytes,
+                               int64_t rows, int64_t N, void* stream) {
+    return rmsnorm_bwd_any(dy, x, weight, weight_is_fp32, rstd, nullptr, dx, dw, workspace, workspace_bytes, rows, N, stream);
+}
+
+extern "C" int hyc_rmsnorm_bwd_add(const void* dy, const void* x, const void* weight, int weight_is_fp32,
+                                   const float* rstd, const void* residual, void* dx, void* dw, void* workspace,
+                                   int64_t workspace_bytes, int64_t rows, int64_t N, void* stream) {
+    if (!residual && rows > 0 && N > 0) return HYC_ERR_NULL;
+    return rmsnorm_bwd_any(dy, x, weight, weight_is_fp32, rstd, residual, dx, dw, workspace, workspace_bytes, rows, N, stream);
 }

@@ -398,8 +398,13 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             return outlier_addition_fuse_decompression_dequantization(
                 S[name + "_q"], S[name + "_s"], S[name + "_o"], S[name + "_idx"], q_bit)
 
-        def norm_backward(dy, xin, weight, rstd, want_dw):
-            return _rmsnorm_backward(dy, xin, weight, rstd, want_dw=want_dw)
+        def norm_backward(dy, xin, weight, rstd, want_dw, residual):
+            """Norm backward plus the gradient of the residual connection (`grad_norm + residual` in
+            the reference, …full_fuse.py:391-393,491-493), added inside the kernel where it can be."""
+            if residual.dtype == dy.dtype == torch.bfloat16 and residual.shape == dy.shape:
+                return _rmsnorm_backward(dy, xin, weight, rstd, want_dw=want_dw, residual=residual)
+            dx, dw = _rmsnorm_backward(dy, xin, weight, rstd, want_dw=want_dw)
+            return dx + residual, dw
 
         # ---- MLP block ---------------------------------------------------------------------------
         if spec.mode == "intra_inter_full_fuse":
@@ -445,9 +450,8 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
         grad_x2 = back("up", "x_norm_2", S["up_lora_a"], grad_h2, accumulate=grad_x2)
         del grad_fn, grad_h2
         x_medium = channel_base_restored("x_medium")
-        grad_norm_2, grad_nw2 = norm_backward(grad_x2, x_medium, norm_weight_2, S["rstd_2"], ctx.norm_grads[1])
+        grad_medium, grad_nw2 = norm_backward(grad_x2, x_medium, norm_weight_2, S["rstd_2"], ctx.norm_grads[1], grad_output)
         del x_medium, grad_x2
-        grad_medium = grad_norm_2 + grad_output
 
         # ---- attention block -------------------------------------------------------------------
         grad_o = back("o", "o", S["o_lora_a"], grad_medium)
@@ -510,8 +514,7 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
         grad_x = back("v", "x_norm_1", S["v_lora_a"], grad_v, accumulate=grad_x)
         del grad_q, grad_k, grad_v
         x = channel_base_restored("x")
-        grad_norm_1, grad_nw1 = norm_backward(grad_x, x, norm_weight_1, S["rstd_1"], ctx.norm_grads[0])
-        grad_input = grad_norm_1 + grad_medium
+        grad_input, grad_nw1 = norm_backward(grad_x, x, norm_weight_1, S["rstd_1"], ctx.norm_grads[0], grad_medium)
 
         def lora_grads(name):
             return (None, None, None) + G[name]

@@ -43,8 +43,10 @@ def rmsnorm_forward(x, weight, eps):
     return y, mean, rstd, block_size, num_warps
 
 
-def _backward(dy, x, w, rstd, want_dw):
-    _lib.require_gpu(dy, x, w, rstd)
+def _backward(dy, x, w, rstd, want_dw, residual=None):
+    """-> (dx, dw or None).  With `residual` (bf16, dy's shape) dx is bf16(dx + residual): the
+    gradient of the residual connection added in the same pass, same bits as adding it afterwards."""
+    _lib.require_gpu(dy, x, w, rstd, residual)
     if dy.dtype != torch.bfloat16 or x.dtype != torch.bfloat16:
         raise NotImplementedError("rmsnorm_backward computes on bfloat16 activations")
     n = x.shape[-1]
@@ -61,19 +63,27 @@ def _backward(dy, x, w, rstd, want_dw):
         dw = torch.empty((n,), dtype=wt.dtype, device=x.device)
         ws_bytes = _lib.lib().hyc_rmsnorm_bwd_workspace(rows, n)
         ws = torch.empty((max(ws_bytes, 4) // 4,), dtype=torch.float32, device=x.device)
-    _lib.call("hyc_rmsnorm_bwd", dy.data_ptr(), x.data_ptr(), wt.data_ptr(), w32,
-              rstd.to(torch.float32).contiguous().data_ptr(), dx.data_ptr(), _lib.ptr(dw), _lib.ptr(ws), ws_bytes,
-              rows, n, _lib.stream_of(x))
+    rstd = rstd.to(torch.float32).contiguous()
+    if residual is None:
+        _lib.call("hyc_rmsnorm_bwd", dy.data_ptr(), x.data_ptr(), wt.data_ptr(), w32, rstd.data_ptr(), dx.data_ptr(),
+                  _lib.ptr(dw), _lib.ptr(ws), ws_bytes, rows, n, _lib.stream_of(x))
+    else:
+        if residual.shape != dy.shape or residual.dtype != torch.bfloat16:
+            raise ValueError(f"residual must be bfloat16 of shape {tuple(dy.shape)}")
+        residual = residual.contiguous()
+        _lib.call("hyc_rmsnorm_bwd_add", dy.data_ptr(), x.data_ptr(), wt.data_ptr(), w32, rstd.data_ptr(),
+                  residual.data_ptr(), dx.data_ptr(), _lib.ptr(dw), _lib.ptr(ws), ws_bytes, rows, n, _lib.stream_of(x))
     if want_dw and dw.dtype != w.dtype:
         dw = dw.to(w.dtype)
     return dx, dw
 
 
-def rmsnorm_backward(dy, x, w, m, v, needs_inputs_grad, eps, num_warps, BLOCK_SIZE):
-    """-> (dx, None); `v` is the rstd returned by rmsnorm_forward.  Reference :149-185."""
+def rmsnorm_backward(dy, x, w, m, v, needs_inputs_grad, eps, num_warps, BLOCK_SIZE, residual=None):
+    """-> (dx, None); `v` is the rstd returned by rmsnorm_forward.  Reference :149-185.
+    `residual` (not in the reference's signature): a tensor added to dx in the same pass."""
     if not needs_inputs_grad:
         return None, None
-    dx, _ = _backward(dy, x, w, v, want_dw=False)
+    dx, _ = _backward(dy, x, w, v, want_dw=False, residual=residual)
     return dx, None
 
 

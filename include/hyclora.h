@@ -36,7 +36,7 @@ extern "C" {
 /* Text for a HYC_ERR_* code (static storage). */
 const char *hyc_error_string(int code);
 
-/* ABI revision; bumped when a signature changes. */
+/* ABI revision; bumped when a signature changes or an entry point is added. */
 int hyc_abi_version(void);
 
 /* Launch-shape knobs for benchmarking (process-wide, not thread-safe against concurrent
@@ -267,6 +267,16 @@ int64_t hyc_rmsnorm_bwd_workspace(int64_t rows, int64_t N);
 int hyc_rmsnorm_bwd(const void *dy, const void *x, const void *weight, int weight_is_fp32,
                     const float *rstd, void *dx, void *dw, void *workspace, int64_t workspace_bytes,
                     int64_t rows, int64_t N, void *stream);
+
+/* The same with the gradient that arrives over the residual connection added in the same pass:
+ * dx = bf16(bf16(dx of hyc_rmsnorm_bwd) + residual), i.e. the bits of that call followed by a bf16
+ * add.  Replaces `grad_norm_2 + grad_output` / `grad_norm_1 + grad_medium` after the norm backward
+ * in the layers (models/llama/fused_llama_layer_intra_inter_full_fuse.py:391-393, :491-493).
+ *   residual   bf16 [rows, N] contiguous, 16-byte aligned; must not overlap dx.
+ */
+int hyc_rmsnorm_bwd_add(const void *dy, const void *x, const void *weight, int weight_is_fp32,
+                        const float *rstd, const void *residual, void *dx, void *dw, void *workspace,
+                        int64_t workspace_bytes, int64_t rows, int64_t N, void *stream);
 
 /* ---------------------------------------------------------------------------------------
  * NF4 block-wise weight dequantisation to bf16, bitsandbytes 0.43.2 layout (the version the

@@ -108,6 +108,14 @@ def test_rmsnorm_backward(ops, dev, n, rows):
     assert dw.dtype == w.dtype and dw.shape == (n,)
     assert_close_bf16(dw, dw_ref, what="rmsnorm_backward dw vs oracle")
     assert ops.norm.rmsnorm_backward(dyg, xg, wg, mean, rstd, False, 1e-5, warps, block) == (None, None)
+    # the residual connection's gradient added in the same pass: the bits of dx + residual
+    res = torch.randn(*rows, n, generator=g).to(BF16).to(dev)
+    dx3, _ = ops.norm.rmsnorm_backward(dyg, xg, wg, mean, rstd, True, 1e-5, warps, block, residual=res)
+    assert torch.equal(dx3, dx + res)
+    dx4, dw4 = ops.norm._backward(dyg, xg, wg, rstd, want_dw=True, residual=res)
+    assert torch.equal(dx4, dx3) and torch.equal(dw4, dw)
+    with pytest.raises(ValueError):
+        ops.norm.rmsnorm_backward(dyg, xg, wg, mean, rstd, True, 1e-5, warps, block, residual=res[..., :8])
     # independent check of dw and of dx's x^-dependent part: autograd of true RMSNorm, to
     # which the reference formula adds only the -mean(w*dy)*rstd term
     xf = x.double().requires_grad_()
