@@ -56,6 +56,7 @@ _SIGNATURES = {
     "hyc_rmsnorm_bwd_workspace": (_L, [_L, _L]),
     "hyc_rmsnorm_bwd": (_I, [_P, _P, _P, _I, _P, _P, _P, _P, _L, _L, _L, _P]),
     "hyc_rmsnorm_bwd_add": (_I, [_P, _P, _P, _I, _P, _P, _P, _P, _P, _L, _L, _L, _P]),
+    "hyc_rmsnorm_bwd_codes": (_I, [_P, _P, _P, _P, _L, _P, _I, _P, _I, _P, _P, _P, _L, _L, _P]),
     "hyc_silu_bwd": (_I, [_P, _P, _P, _L, _P]),
     "hyc_silu_mul": (_I, [_P, _P, _P, _L, _P]),
     "hyc_gelu_bwd": (_I, [_P, _P, _P, _L, _P]),

@@ -140,6 +140,9 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_bwd_kernel(const uint16_
                 if constexpr (RES) rv[c] = ld16_nt(res + row * N + col);
             }
         }
+        // Summation order (shared with the form that reads x from its codes, whose results must
+        // be the same bits): each chunk's two sums as chains from zero, a lane's chunks added in
+        // column order, then the butterfly over the lanes.
         float s1 = 0.0f, s2 = 0.0f;
 #pragma unroll
         for (int c = 0; c < CH; ++c) {
@@ -148,13 +151,16 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_bwd_kernel(const uint16_
             unpack8(xv[c], xf);
             unpack8(gv[c], gf);
             if (col < N) load_w8<W32>(w, col, wf);
+            float p1 = 0.0f, p2 = 0.0f;
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 const float xh = xf[j] * rstd, wdy = wf[j] * gf[j];
-                s1 = fmaf(xh, wdy, s1);
-                s2 += wdy;
+                p1 = fmaf(xh, wdy, p1);
+                p2 += wdy;
                 if constexpr (DW) dwacc[c][j] = fmaf(gf[j], xh, dwacc[c][j]);
             }
+            s1 += p1;
+            s2 += p2;
         }
         const float c1 = wave_sum(s1) * inv_n, c2 = wave_sum(s2) * inv_n;
 #pragma unroll

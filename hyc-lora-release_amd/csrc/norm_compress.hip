@@ -286,6 +286,192 @@ void rmsnorm_fwd_compress_slab_kernel(const NormCompressArgs a, int rows_per_gro
     else run(std::false_type{});
 }
 
+// ------------------------------------------------------------------------------------
+// RMSNorm backward that reads its input from the channel-base compressed copy the forward kernels
+// above leave behind (codes, steps, outlier values), in the same column-slab decomposition: the
+// layers otherwise restore x to a dense tensor first
+// (outlier_addition_fuse_decompression_dequantization, then rmsnorm_backward:
+// models/llama/fused_llama_layer_intra_inter_full_fuse.py:386-393, :486-493).  A lane's per-column
+// constants (norm weight, step, outlier positions) stay in registers for a strip of rows; a row's
+// two sums (x^ . w dy and w dy) go through LDS like the forward kernel's sum of squares, in the
+// dense backward kernel's summation order, so dx is the same bits as from dequantise + backward.
+// Optionally adds the residual connection's gradient, like hyc_rmsnorm_bwd_add.
+struct NormBwdCodesArgs {
+    const uint16_t* dy; const uint8_t* q_x; const uint16_t* scale_x;
+    const uint16_t* otable; const uint16_t* xo;
+    const void* w; const float* rstd; const uint16_t* res; uint16_t* dx;
+    int64_t rows;
+    int N, k;
+};
+
+template <int QBIT, bool W32, int MAXW, bool RES>
+__global__ __launch_bounds__(MAXW * kWave) __attribute__((amdgpu_waves_per_eu(4)))
+void rmsnorm_bwd_codes_slab_kernel(const NormBwdCodesArgs a, int rows_per_group) {
+    constexpr int G = kSlabRows;
+    extern __shared__ float slab_part[];                // [2][G][2][waves][64]
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int nw = blockDim.x >> 6;
+    const int chunk = wave * kWave + lane;
+    const int col = chunk * 8;
+    const int N = a.N;
+    const int row_bytes = N * QBIT / 8;
+    constexpr float kHalf = (float)(1 << (QBIT - 1));
+    const int64_t r0 = (int64_t)blockIdx.x * rows_per_group;
+    int64_t r1 = r0 + rows_per_group;
+    if (r1 > a.rows) r1 = a.rows;
+    if (r0 >= r1) return;                               // whole workgroups leave together
+
+    // Per-column constants, kept packed where they are bf16 (registers are what limits this kernel
+    // to four waves per SIMD): norm weight, steps, and the lane's outlier columns.
+    float wf[W32 ? 8 : 1];
+    u32x4 wp = {0, 0, 0, 0};
+    if constexpr (W32) {
+        const f32x4 w0 = *reinterpret_cast<const f32x4*>((const float*)a.w + col);
+        const f32x4 w1 = *reinterpret_cast<const f32x4*>((const float*)a.w + col + 4);
+        wf[0] = w0.x; wf[1] = w0.y; wf[2] = w0.z; wf[3] = w0.w;
+        wf[4] = w1.x; wf[5] = w1.y; wf[6] = w1.z; wf[7] = w1.w;
+    } else {
+        wp = ld16((const uint16_t*)a.w + col);
+    }
+    auto weight8 = [&](float (&out)[8]) __attribute__((always_inline)) {
+        if constexpr (W32) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) out[j] = wf[j];
+        } else {
+            unpack8(wp, out);
+        }
+    };
+    const u32x4 sp = ld16(a.scale_x + col);
+    // Outlier columns of this lane: the first two are fetched ahead with the row (slots 1 and 2 of
+    // `oslot`, two bits a column), any further one when it is used (slot 3).  Few lanes have any.
+    u32x4 tv = {0, 0, 0, 0};
+    if (a.k > 0) tv = ld16(a.otable + col);
+    const uint32_t td[4] = {tv.x, tv.y, tv.z, tv.w};
+    uint32_t oslot = 0, opos0 = 0, opos1 = 0;
+    {
+        int cnt = 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const uint32_t p = (td[j >> 1] >> (16 * (j & 1))) & 0xffffu;
+            if (p) {
+                oslot |= (uint32_t)(cnt < 2 ? cnt + 1 : 3) << (2 * j);
+                if (cnt == 0) opos0 = p - 1;
+                if (cnt == 1) opos1 = p - 1;
+                ++cnt;
+            }
+        }
+    }
+    const PackedSlot<QBIT> slot(chunk);
+    const float inv_n = 1.0f / (float)N;
+
+    u32x2 cw[G];
+    u32x4 gv[G];
+    float rs[G];
+    uint32_t ov[G][2];
+    auto request = [&](int64_t r) __attribute__((always_inline)) {
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            const int64_t row = r + g;
+            cw[g] = ld8(a.q_x + row * row_bytes + slot.offset);
+            gv[g] = ld16_nt(a.dy + row * N + col);
+            rs[g] = a.rstd[row];
+            if (oslot) {
+                ov[g][0] = a.xo[row * a.k + opos0];
+                if (oslot & 0xaaaau) ov[g][1] = a.xo[row * a.k + opos1];        // a second outlier column
+            }
+        }
+    };
+    auto step = [&](int64_t r, int buf, auto ahead_tag) __attribute__((always_inline)) {
+        constexpr bool AHEAD = decltype(ahead_tag)::value;
+        // What a row needs after the barrier is kept packed (x is a bf16 value by construction) and
+        // unpacked again there: 12 registers a row instead of 24.
+        u32x4 xp[G], gp[G];
+        float rstd[G];
+        float* mine = slab_part + ((buf * G) * 2 * nw + wave) * kWave + lane;
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            float c[8], gf[8], x[8], sf[8], w8[8];
+            slot.decode(cw[g], c);
+            unpack8(gv[g], gf);
+            unpack8(sp, sf);
+            weight8(w8);
+            gp[g] = gv[g];
+            rstd[g] = rs[g];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) x[j] = (c[j] - kHalf) * sf[j];  // the dequantiser's arithmetic ...
+            if (oslot) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const uint32_t code = (oslot >> (2 * j)) & 3u;
+                    if (code == 1) x[j] = __uint_as_float(ov[g][0] << 16);
+                    else if (code == 2) x[j] = __uint_as_float(ov[g][1] << 16);
+                    else if (code == 3) {
+                        const uint32_t p = (td[j >> 1] >> (16 * (j & 1))) & 0xffffu;
+                        x[j] = __uint_as_float((uint32_t)a.xo[(r + g) * a.k + (p - 1)] << 16);
+                    }
+                }
+            }
+            xp[g] = pack8(x);                                           // ... and its rounding to bf16
+            unpack8(xp[g], x);
+            float p1 = 0.0f, p2 = 0.0f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float xh = x[j] * rstd[g], wdy = w8[j] * gf[j];
+                p1 = fmaf(xh, wdy, p1);
+                p2 += wdy;
+            }
+            mine[(g * 2 + 0) * nw * kWave] = p1;
+            mine[(g * 2 + 1) * nw * kWave] = p2;
+            __builtin_amdgcn_sched_barrier(0);          // one row at a time: fewer live temporaries
+        }
+        // The residual is asked for only now, for the rows of THIS step (the barrier and the sums
+        // below cover most of its latency): fetched a step ahead like the rest it would need
+        // registers this kernel does not have at four waves per SIMD.
+        u32x4 rv[RES ? G : 1];
+        if constexpr (RES) {
+#pragma unroll
+            for (int g = 0; g < G; ++g) rv[g] = ld16_nt(a.res + (r + g) * N + col);
+        }
+        if constexpr (AHEAD) request(r + G);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");   // LDS-only barrier, see above
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            const float* all = slab_part + ((buf * G + g) * 2 * nw) * kWave + lane;
+            float t1 = 0.0f, t2 = 0.0f;
+#pragma unroll 4
+            for (int w = 0; w < nw; ++w) {
+                t1 += all[w * kWave];
+                t2 += all[(nw + w) * kWave];
+            }
+            const float c1 = wave_sum(t1) * inv_n, c2 = wave_sum(t2) * inv_n;
+            float x[8], gf[8], rf[8], w8[8], o[8];
+            unpack8(xp[g], x);
+            unpack8(gp[g], gf);
+            weight8(w8);
+            if constexpr (RES) unpack8(rv[g], rf);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float xh = x[j] * rstd[g], wdy = w8[j] * gf[j];
+                o[j] = (wdy - (xh * c1 + c2)) * rstd[g];
+                if constexpr (RES) o[j] = rbf(o[j]) + rf[j];
+            }
+            st16_nt(a.dx + (r + g) * N + col, pack8(o));
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    request(r0);
+    int64_t r = r0;
+    int buf = 0;
+    if (r + G < r1) {
+        step(r, buf, std::true_type{});
+        for (r += G, buf ^= 1; r + G < r1; r += G, buf ^= 1) step(r, buf, std::true_type{});
+    }
+    step(r, buf, std::false_type{});
+}
+
 // otable[c] = 1 + i for c = oidx[i], everything else 0 (table cleared by the first kernel)
 __global__ void otable_fill_kernel(uint16_t* __restrict__ table, int n) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -390,4 +576,49 @@ extern "C" int hyc_rmsnorm_fwd_compress(const void* x, const void* weight, int w
     if (q_bit == 4) return HYC_NC_Q(4);
     return HYC_NC_Q(2);
 #undef HYC_NC_Q
+}
+
+extern "C" int hyc_rmsnorm_bwd_codes(const void* dy, const void* q_x, const void* scale_x, const uint16_t* outlier_table,
+                                     int64_t k, const void* x_outlier, int q_bit, const void* weight, int weight_is_fp32,
+                                     const float* rstd, const void* residual, void* dx, int64_t rows, int64_t N,
+                                     void* stream) {
+    if (q_bit != 2 && q_bit != 4 && q_bit != 8) return HYC_ERR_QBIT;
+    if (rows < 0 || N < 0 || k < 0 || k > 65535) return HYC_ERR_SHAPE;
+    if (N % (kWave * 8) != 0 || N / (kWave * 8) > 16 || rows % kSlabRows != 0) return HYC_ERR_SHAPE;
+    if (rows == 0 || N == 0) return HYC_OK;
+    if (!dy || !q_x || !scale_x || !weight || !rstd || !dx || (k > 0 && (!outlier_table || !x_outlier))) return HYC_ERR_NULL;
+    if (!aligned16(dy) || !aligned16(scale_x) || !aligned16(weight) || !aligned16(dx) || !aligned16(residual) ||
+        (outlier_table && !aligned16(outlier_table)) || (reinterpret_cast<uintptr_t>(q_x) & 7u))
+        return HYC_ERR_ALIGN;
+    NormBwdCodesArgs a;
+    a.dy = (const uint16_t*)dy; a.q_x = (const uint8_t*)q_x; a.scale_x = (const uint16_t*)scale_x;
+    a.otable = outlier_table; a.xo = (const uint16_t*)x_outlier; a.w = weight; a.rstd = rstd;
+    a.res = (const uint16_t*)residual; a.dx = (uint16_t*)dx; a.rows = rows; a.N = (int)N; a.k = (int)k;
+    const int waves = a.N / (kWave * 8);
+    int rows_per_group = g_slab_rows_per_group;
+    if (rows_per_group == 0) {
+        const int64_t resident = (int64_t)compute_units() * (16 / (waves <= 8 ? waves : 16));
+        rows_per_group = (int)(cdiv(cdiv(rows, resident), (int64_t)kSlabRows) * kSlabRows);
+    }
+    const int64_t groups = cdiv(rows, (int64_t)rows_per_group);
+    if (groups > INT32_MAX) return HYC_ERR_SHAPE;
+    const size_t lds = 2 * kSlabRows * 2 * waves * kWave * sizeof(float);
+    const dim3 grid((unsigned)groups), block(waves * kWave);
+    hipStream_t st = (hipStream_t)stream;
+#define HYC_NBC(QB, W32, MAXW)                                                                                          \
+    do {                                                                                                                \
+        if (a.res) hipLaunchKernelGGL((rmsnorm_bwd_codes_slab_kernel<QB, W32, MAXW, true>), grid, block, lds, st, a, rows_per_group); \
+        else hipLaunchKernelGGL((rmsnorm_bwd_codes_slab_kernel<QB, W32, MAXW, false>), grid, block, lds, st, a, rows_per_group);      \
+    } while (0)
+#define HYC_NBC_W(QB)                                                      \
+    do {                                                                   \
+        if (weight_is_fp32) { if (waves <= 8) HYC_NBC(QB, true, 8); else HYC_NBC(QB, true, 16); }   \
+        else { if (waves <= 8) HYC_NBC(QB, false, 8); else HYC_NBC(QB, false, 16); }                \
+    } while (0)
+    if (q_bit == 8) HYC_NBC_W(8);
+    else if (q_bit == 4) HYC_NBC_W(4);
+    else HYC_NBC_W(2);
+#undef HYC_NBC_W
+#undef HYC_NBC
+    return check_launch();
 }

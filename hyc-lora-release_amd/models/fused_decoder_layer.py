@@ -51,7 +51,8 @@ from ..operators.compress_function import (compress_attention_map, compression_p
                                            outlier_addition_fuse_decompression_dequantization,
                                            update_dict)
 from ..operators.rmsnorm_kernels import _backward as _rmsnorm_backward
-from ..operators.rmsnorm_kernels import rmsnorm_forward, rmsnorm_forward_compress
+from ..operators.rmsnorm_kernels import (backward_from_codes_supported, rmsnorm_backward_from_codes, rmsnorm_forward,
+                                         rmsnorm_forward_compress)
 from ..operators.silu_kernels import silu_backward, silu_hadamard
 from ..operators.softmax_kernels import softmax_backward, softmax_backward_from_compressed, softmax_forward
 from ..operators.triton_fuse_lora_silu_hadamard_backward_kernels import triton_fuse_silu_backward
@@ -398,10 +399,18 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             return outlier_addition_fuse_decompression_dequantization(
                 S[name + "_q"], S[name + "_s"], S[name + "_o"], S[name + "_idx"], q_bit)
 
-        def norm_backward(dy, xin, weight, rstd, want_dw, residual):
-            """Norm backward plus the gradient of the residual connection (`grad_norm + residual` in
-            the reference, …full_fuse.py:391-393,491-493), added inside the kernel where it can be."""
-            if residual.dtype == dy.dtype == torch.bfloat16 and residual.shape == dy.shape:
+        def norm_backward(dy, name, weight, rstd, want_dw, residual):
+            """Backward of the norm whose input the layer saved under `name`, plus the gradient of the
+            residual connection (`grad_norm + residual` in the reference, …full_fuse.py:386-393,486-493).
+            A compressed input is read from its codes where the kernel takes the shape; otherwise it
+            is restored first.  The residual is added inside the kernel where it can be."""
+            fused_add = residual.dtype == dy.dtype == torch.bfloat16 and residual.shape == dy.shape
+            if name + "_raw" not in S and fused_add and backward_from_codes_supported(dy, dy.shape[-1], want_dw):
+                dx = rmsnorm_backward_from_codes(dy, S[name + "_q"], S[name + "_s"], S[name + "_o"], S[name + "_idx"],
+                                                 q_bit, weight, rstd, residual=residual)
+                return dx, None
+            xin = channel_base_restored(name)
+            if fused_add:
                 return _rmsnorm_backward(dy, xin, weight, rstd, want_dw=want_dw, residual=residual)
             dx, dw = _rmsnorm_backward(dy, xin, weight, rstd, want_dw=want_dw)
             return dx + residual, dw
@@ -449,9 +458,8 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
         grad_x2 = back("gate", "x_norm_2", S["gate_lora_a"], grad_fn)
         grad_x2 = back("up", "x_norm_2", S["up_lora_a"], grad_h2, accumulate=grad_x2)
         del grad_fn, grad_h2
-        x_medium = channel_base_restored("x_medium")
-        grad_medium, grad_nw2 = norm_backward(grad_x2, x_medium, norm_weight_2, S["rstd_2"], ctx.norm_grads[1], grad_output)
-        del x_medium, grad_x2
+        grad_medium, grad_nw2 = norm_backward(grad_x2, "x_medium", norm_weight_2, S["rstd_2"], ctx.norm_grads[1], grad_output)
+        del grad_x2
 
         # ---- attention block -------------------------------------------------------------------
         grad_o = back("o", "o", S["o_lora_a"], grad_medium)
@@ -513,8 +521,7 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
         grad_x = back("k", "x_norm_1", S["k_lora_a"], grad_k, accumulate=grad_x)
         grad_x = back("v", "x_norm_1", S["v_lora_a"], grad_v, accumulate=grad_x)
         del grad_q, grad_k, grad_v
-        x = channel_base_restored("x")
-        grad_input, grad_nw1 = norm_backward(grad_x, x, norm_weight_1, S["rstd_1"], ctx.norm_grads[0], grad_medium)
+        grad_input, grad_nw1 = norm_backward(grad_x, "x", norm_weight_1, S["rstd_1"], ctx.norm_grads[0], grad_medium)
 
         def lora_grads(name):
             return (None, None, None) + G[name]

@@ -78,6 +78,49 @@ def _backward(dy, x, w, rstd, want_dw, residual=None):
     return dx, dw
 
 
+def backward_from_codes_supported(dy, n, want_dw):
+    """Whether rmsnorm_backward_from_codes takes this case (whole 512-column slabs, an even number of
+    rows, bf16 gradient, no weight gradient)."""
+    return (not want_dw and dy.is_cuda and dy.dtype == torch.bfloat16 and n % 512 == 0 and 0 < n <= 8192
+            and dy.numel() > 0 and (dy.numel() // n) % 2 == 0)
+
+
+def rmsnorm_backward_from_codes(dy, q_x, scale_x, x_outlier, outlier_idx, q_bit, w, rstd, residual=None, table=None):
+    """dx of rmsnorm_backward with the norm's input given as its channel-base compressed copy
+    (q_x, scale_x, x_outlier, outlier_idx) - the same bits as
+    outlier_addition_fuse_decompression_dequantization followed by rmsnorm_backward
+    (fused_llama_layer_intra_inter_full_fuse.py:386-393), with `residual` added like there."""
+    _lib.require_gpu(dy, q_x, scale_x, w, rstd, residual)
+    n = dy.shape[-1]
+    if not backward_from_codes_supported(dy, n, False):
+        raise NotImplementedError("rmsnorm_backward_from_codes: bfloat16 gradient, N a multiple of 512 up to 8192, even row count")
+    dy = dy.contiguous()
+    rows = dy.numel() // n
+    k = 0 if outlier_idx is None else int(outlier_idx.numel())
+    if k and table is None:
+        table = outlier_table(outlier_idx, n, cached=True)
+    if q_x.dtype != torch.uint8 or q_x.numel() != rows * n * q_bit // 8:
+        raise ValueError("q_x does not hold the packed codes of a tensor of dy's shape")
+    q_x = q_x.contiguous()
+    sx = scale_x.to(torch.bfloat16).reshape(-1).contiguous()
+    xo = None
+    if k:
+        xo = x_outlier.to(torch.bfloat16).contiguous()
+        if xo.numel() != rows * k:
+            raise ValueError("x_outlier does not match the outlier list")
+    wt, w32 = _weight(w)
+    rstd = rstd.to(torch.float32).contiguous()
+    if residual is not None:
+        if residual.shape != dy.shape or residual.dtype != torch.bfloat16:
+            raise ValueError(f"residual must be bfloat16 of shape {tuple(dy.shape)}")
+        residual = residual.contiguous()
+    dx = torch.empty_like(dy)
+    _lib.call("hyc_rmsnorm_bwd_codes", dy.data_ptr(), q_x.data_ptr(), sx.data_ptr(), _lib.ptr(table) if k else None, k,
+              _lib.ptr(xo), q_bit, wt.data_ptr(), w32, rstd.data_ptr(), _lib.ptr(residual), dx.data_ptr(), rows, n,
+              _lib.stream_of(dy))
+    return dx
+
+
 def rmsnorm_backward(dy, x, w, m, v, needs_inputs_grad, eps, num_warps, BLOCK_SIZE, residual=None):
     """-> (dx, None); `v` is the rstd returned by rmsnorm_forward.  Reference :149-185.
     `residual` (not in the reference's signature): a tensor added to dx in the same pass."""

@@ -278,6 +278,22 @@ int hyc_rmsnorm_bwd_add(const void *dy, const void *x, const void *weight, int w
                         const float *rstd, const void *residual, void *dx, void *dw, void *workspace,
                         int64_t workspace_bytes, int64_t rows, int64_t N, void *stream);
 
+/* RMSNorm backward that reads its input from the channel-base compressed copy (what
+ * hyc_rmsnorm_fwd_compress or hyc_quant_pack with an outlier list left: codes, steps, outlier
+ * values) instead of a dense tensor; dx is the same bits as hyc_unpack_dequant followed by
+ * hyc_rmsnorm_bwd (or _add, with a residual).  Replaces
+ * outlier_addition_fuse_decompression_dequantization + rmsnorm_backward (+ the add) in the layers'
+ * backward (models/llama/fused_llama_layer_intra_inter_full_fuse.py:386-393, :486-493).
+ *   q_x, scale_x, outlier_table, k, x_outlier   as in hyc_rmsnorm_fwd_compress (k may be 0).
+ *   residual   bf16 [rows, N] or NULL.   No dw.
+ * Only for rows that are a whole number of 512-column slabs (N % 512 == 0, N <= 8192) and an even
+ * number of rows: HYC_ERR_SHAPE otherwise (callers then dequantise and use hyc_rmsnorm_bwd).
+ */
+int hyc_rmsnorm_bwd_codes(const void *dy, const void *q_x, const void *scale_x, const uint16_t *outlier_table,
+                          int64_t k, const void *x_outlier, int q_bit, const void *weight, int weight_is_fp32,
+                          const float *rstd, const void *residual, void *dx, int64_t rows, int64_t N,
+                          void *stream);
+
 /* ---------------------------------------------------------------------------------------
  * NF4 block-wise weight dequantisation to bf16, bitsandbytes 0.43.2 layout (the version the
  * reference pins in requirements.txt:3).

@@ -83,6 +83,65 @@ def test_both_kernel_forms_give_the_same_bits(ops, dev, q_bit, shape):
         _lib.set_tuning("norm_compress_rows_per_group", 0)
 
 
+@pytest.mark.parametrize("q_bit", [2, 4, 8])
+@pytest.mark.parametrize("shape", [(2, 34, 4096), (1, 8, 512), (4, 1, 1024), (1, 20, 5120), (1, 12, 8192)])
+@pytest.mark.parametrize("wdtype", [BF16, torch.float32])
+def test_backward_from_codes_equals_restore_then_backward(ops, dev, q_bit, shape, wdtype):
+    from hyclora_amd import _lib
+    x, _ = activation_with_outlier_channels(seed=11 + q_bit, shape=shape, frac=0.01)
+    g = torch.Generator().manual_seed(5)
+    w = (1 + 0.1 * torch.randn(shape[-1], generator=g)).to(wdtype).to(dev)
+    dy = torch.randn(*shape, generator=g).to(BF16).to(dev)
+    res = torch.randn(*shape, generator=g).to(BF16).to(dev)
+    xd = x.to(dev)
+    idx, s_x = ops.cf.get_statistics_channel_base(xd, 0.01, q_bit, 'per-channel')
+    rstd = ops.norm.rmsnorm_forward(xd, w, 1e-5)[2]
+    xo, q_x = ops.cf.outlier_subtraction_fuse_compression_quantization(xd.clone(), s_x, idx, q_bit)
+    restored = ops.cf.outlier_addition_fuse_decompression_dequantization(q_x, s_x, xo, idx, q_bit)
+    want = ops.norm._backward(dy, restored, w, rstd, want_dw=False)[0]
+    want_res = ops.norm._backward(dy, restored, w, rstd, want_dw=False, residual=res)[0]
+    try:
+        for rows in (0, 2, 6, 64):
+            _lib.set_tuning("norm_compress_rows_per_group", rows)
+            got = ops.norm.rmsnorm_backward_from_codes(dy, q_x, s_x, xo, idx, q_bit, w, rstd)
+            got_res = ops.norm.rmsnorm_backward_from_codes(dy, q_x, s_x, xo, idx, q_bit, w, rstd, residual=res)
+            assert same_bits(got, want) and same_bits(got_res, want_res), f"strip height {rows}"
+    finally:
+        _lib.set_tuning("norm_compress_rows_per_group", 0)
+    # against the oracle's formula on the oracle's restored input
+    x_o = O.decompress_channel_base(q_x.cpu(), s_x.cpu(), xo.cpu(), idx.cpu(), q_bit)
+    dx_o, _ = O.rmsnorm_bwd(dy.cpu(), x_o, w.cpu(), rstd.cpu())
+    assert_close_bf16(got, dx_o, what="backward from codes vs oracle")
+    # no outlier channels at all
+    q_plain = ops.cf.compression_quantization(xd, s_x, q_bit)
+    plain = ops.cf.decompression_dequantization(q_plain, s_x, q_bit)
+    got0 = ops.norm.rmsnorm_backward_from_codes(dy, q_plain, s_x, None, None, q_bit, w, rstd, residual=res)
+    assert same_bits(got0, ops.norm._backward(dy, plain, w, rstd, want_dw=False, residual=res)[0])
+
+
+def test_backward_from_codes_many_outliers_in_one_chunk_and_errors(ops, dev):
+    # more than two outlier columns inside one lane's 8 columns: the third and later ones are read
+    # when they are used instead of with the row
+    shape, q_bit = (1, 6, 512), 4
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn(*shape, generator=g).to(BF16).to(dev)
+    idx = torch.tensor([16, 17, 19, 22, 23, 300, 8], device=dev)
+    s_x = ops.cf.get_statistics_only_quant(x, q_bit, 'per-channel')
+    w = torch.ones(512, dtype=BF16, device=dev)
+    dy = torch.randn(*shape, generator=g).to(BF16).to(dev)
+    rstd = ops.norm.rmsnorm_forward(x, w, 1e-5)[2]
+    xo, q_x = ops.cf.outlier_subtraction_fuse_compression_quantization(x.clone(), s_x, idx, q_bit)
+    restored = ops.cf.outlier_addition_fuse_decompression_dequantization(q_x, s_x, xo, idx, q_bit)
+    got = ops.norm.rmsnorm_backward_from_codes(dy, q_x, s_x, xo, idx, q_bit, w, rstd)
+    assert same_bits(got, ops.norm._backward(dy, restored, w, rstd, want_dw=False)[0])
+    with pytest.raises(NotImplementedError):      # odd row count
+        ops.norm.rmsnorm_backward_from_codes(dy[:, :5], q_x[:, :5], s_x, xo[:, :5], idx, q_bit, w, rstd[:5])
+    with pytest.raises(ValueError):               # codes of another shape
+        ops.norm.rmsnorm_backward_from_codes(dy, q_x[:, :4], s_x, xo, idx, q_bit, w, rstd)
+    assert not ops.norm.backward_from_codes_supported(dy, 512, True)
+    assert not ops.norm.backward_from_codes_supported(dy[..., :96], 96, False)
+
+
 def test_outlier_table_and_errors(ops, dev):
     idx = torch.tensor([5, 0, 31, 7], device=dev)
     t = ops.norm.outlier_table(idx, 32).cpu().tolist()
