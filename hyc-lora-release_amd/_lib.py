@@ -59,6 +59,7 @@ _SIGNATURES = {
     "hyc_rmsnorm_bwd_codes": (_I, [_P, _P, _P, _P, _L, _P, _I, _P, _I, _P, _P, _P, _L, _L, _P]),
     "hyc_silu_bwd": (_I, [_P, _P, _P, _L, _P]),
     "hyc_silu_mul": (_I, [_P, _P, _P, _L, _P]),
+    "hyc_silu_mul_bwd": (_I, [_P, _P, _P, _P, _P, _L, _P]),
     "hyc_gelu_bwd": (_I, [_P, _P, _P, _L, _P]),
     "hyc_lora_silu_mul_fwd": (_I, [_P] * 11 + [_L, _L, _L, _I, _I, _P]),
     "hyc_lora_silu_mul_bwd": (_I, [_P] * 12 + [_L, _L, _L, _I, _I, _P]),

@@ -67,6 +67,54 @@ __global__ __launch_bounds__(kEwThreads) void binary_kernel(const uint16_t* __re
     }
 }
 
+// Backward of o = silu(x) * u in one pass: grad_x = silu_backward(x, bf16(g * u)) and
+// grad_u = g * silu(x), with silu(x) = bf16(bf16(sig(x)) * x) as SiluMul forms it.  The layers that do
+// not use the fused LoRA kernels compute this with F.silu, two products and silu_backward
+// (models/llama/fused_llama_layer_intra_inter.py:361-381, whose comment asks for this kernel).
+__global__ __launch_bounds__(kEwThreads) void silu_mul_bwd_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ u,
+                                                                  const uint16_t* __restrict__ g, uint16_t* __restrict__ gx,
+                                                                  uint16_t* __restrict__ gu, int64_t n) {
+    const SiluBwd dsilu;
+    auto one = [&](float xf, float uf, float gf, float& ox, float& ou) {
+        ox = dsilu(xf, rbf(gf * uf));
+        ou = gf * rbf(rbf(sigmoidf_(xf)) * xf);
+    };
+    const int64_t chunks = n / 8;
+    constexpr int kUnroll = 2;
+    const int64_t c0 = (int64_t)blockIdx.x * (kEwThreads * kUnroll) + threadIdx.x;
+    u32x4 xv[kUnroll], uv[kUnroll], gv[kUnroll];
+#pragma unroll
+    for (int k = 0; k < kUnroll; ++k) {
+        const int64_t c = c0 + k * kEwThreads;
+        if (c < chunks) {
+            xv[k] = ld16_nt(x + c * 8);
+            uv[k] = ld16_nt(u + c * 8);
+            gv[k] = ld16_nt(g + c * 8);
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < kUnroll; ++k) {
+        const int64_t c = c0 + k * kEwThreads;
+        if (c < chunks) {
+            float xf[8], uf[8], gf[8], ox[8], ou[8];
+            unpack8(xv[k], xf);
+            unpack8(uv[k], uf);
+            unpack8(gv[k], gf);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) one(xf[j], uf[j], gf[j], ox[j], ou[j]);
+            st16_nt(gx + c * 8, pack8(ox));
+            st16_nt(gu + c * 8, pack8(ou));
+        }
+    }
+    if (blockIdx.x == 0 && threadIdx.x < (n & 7)) {       // ragged tail
+        const int64_t i = chunks * 8 + threadIdx.x;
+        float ox, ou;
+        one(bf_to_f(x[i]), bf_to_f(u[i]), bf_to_f(g[i]), ox, ou);
+        gx[i] = f_to_bf(ox);
+        gu[i] = f_to_bf(ou);
+    }
+}
+
 template <class Op>
 static int launch_binary(const void* a, const void* b, void* o, int64_t n, void* stream) {
     if (n < 0) return HYC_ERR_SHAPE;
@@ -92,4 +140,16 @@ extern "C" int hyc_silu_mul(const void* x1, const void* x2, void* out, int64_t n
 }
 extern "C" int hyc_gelu_bwd(const void* x, const void* g, void* out, int64_t n, void* stream) {
     return launch_binary<GeluBwd>(x, g, out, n, stream);
+}
+extern "C" int hyc_silu_mul_bwd(const void* x, const void* u, const void* g, void* grad_x, void* grad_u, int64_t n,
+                                void* stream) {
+    if (n < 0) return HYC_ERR_SHAPE;
+    if (n == 0) return HYC_OK;
+    if (!x || !u || !g || !grad_x || !grad_u) return HYC_ERR_NULL;
+    if (!aligned16(x) || !aligned16(u) || !aligned16(g) || !aligned16(grad_x) || !aligned16(grad_u)) return HYC_ERR_ALIGN;
+    const int64_t blocks = cdiv(cdiv(n, 8), kEwThreads * 2);
+    if (blocks > INT32_MAX) return HYC_ERR_SHAPE;
+    hipLaunchKernelGGL(silu_mul_bwd_kernel, dim3((unsigned)(blocks < 1 ? 1 : blocks)), dim3(kEwThreads), 0, (hipStream_t)stream,
+                       (const uint16_t*)x, (const uint16_t*)u, (const uint16_t*)g, (uint16_t*)grad_x, (uint16_t*)grad_u, n);
+    return check_launch();
 }

@@ -53,7 +53,7 @@ from ..operators.compress_function import (compress_attention_map, compression_p
 from ..operators.rmsnorm_kernels import _backward as _rmsnorm_backward
 from ..operators.rmsnorm_kernels import (backward_from_codes_supported, rmsnorm_backward_from_codes, rmsnorm_forward,
                                          rmsnorm_forward_compress)
-from ..operators.silu_kernels import silu_backward, silu_hadamard
+from ..operators.silu_kernels import silu_backward, silu_hadamard, silu_hadamard_backward
 from ..operators.softmax_kernels import softmax_backward, softmax_backward_from_compressed, softmax_forward
 from ..operators.triton_fuse_lora_silu_hadamard_backward_kernels import triton_fuse_silu_backward
 from ..operators.triton_fuse_lora_silu_hadamard_forward_kernels import triton_fuse_silu_forward
@@ -443,18 +443,25 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
                 G["down"] = (hadamard.to(wd.dtype).mT @ grad_mid, grad_b_down)
             del hadamard, grad_down
         else:
+            fn = None
             if spec.mode == "intra_inter":
                 gate, up = rebuilt_hidden("gate")[0], rebuilt_hidden("up")[0]
-                fn = F.silu(gate)
-                hadamard = up * fn
+                hadamard = silu_hadamard(gate, up)            # as forward formed it
             else:
                 hadamard, up, fn, gate = deq("hadamard"), deq("up"), deq("fn"), deq("gate")
             grad_down = back("down", hadamard, S["down_lora_a"], grad_output)
             del hadamard
-            grad_h1 = grad_down * up
-            grad_h2 = grad_down * fn
-            grad_fn = silu_backward(gate, grad_h1)
-            del grad_down, up, fn, gate, grad_h1
+            if fn is None and grad_down.dtype == gate.dtype == torch.bfloat16:
+                # grad_down * up, silu_backward of it, and grad_down * silu(gate): one pass
+                grad_fn, grad_h2 = silu_hadamard_backward(gate, up, grad_down)
+            else:
+                if fn is None:
+                    fn = F.silu(gate)
+                grad_h1 = grad_down * up
+                grad_h2 = grad_down * fn
+                grad_fn = silu_backward(gate, grad_h1)
+                del grad_h1
+            del grad_down, up, fn, gate
         grad_x2 = back("gate", "x_norm_2", S["gate_lora_a"], grad_fn)
         grad_x2 = back("up", "x_norm_2", S["up_lora_a"], grad_h2, accumulate=grad_x2)
         del grad_fn, grad_h2

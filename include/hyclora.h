@@ -378,6 +378,11 @@ int hyc_rope(void *x, const void *cos, const void *sin, int table_is_fp32, int64
  */
 int hyc_silu_bwd(const void *x, const void *g, void *out, int64_t n, void *stream);
 int hyc_silu_mul(const void *x1, const void *x2, void *out, int64_t n, void *stream);
+/* Backward of o = silu(x) * u in one pass: grad_x = hyc_silu_bwd(x, bf16(g * u)), grad_u = g * silu(x) with
+ * silu(x) as hyc_silu_mul forms it.  Replaces F.silu + two products + silu_backward in the layers that
+ * do not use the fused LoRA kernels (models/llama/fused_llama_layer_intra_inter.py:361-381). */
+int hyc_silu_mul_bwd(const void *x, const void *u, const void *g, void *grad_x, void *grad_u, int64_t n,
+                     void *stream);
 int hyc_gelu_bwd(const void *x, const void *g, void *out, int64_t n, void *stream);
 
 /* ---------------------------------------------------------------------------------------

@@ -374,6 +374,14 @@ def silu_mul(x1, x2):
     return (_sig_bf16(x1) * x1) * x2
 
 
+def silu_mul_bwd(x, u, g):
+    """Backward of silu_mul(x, u): (silu_bwd(x, g*u), g * (sig(x)*x)), every product rounded to bf16 -
+    the composition the layers write out (fused_llama_layer_intra_inter.py:361-381) with silu(x) as
+    silu_mul forms it."""
+    x = x.to(BF16); u = u.to(BF16); g = g.to(BF16)
+    return silu_bwd(x, g * u), g * (_sig_bf16(x) * x)
+
+
 GELU_GAMMA = 0.7978845608028654
 GELU_KAPPA = 0.044715
 

@@ -52,6 +52,24 @@ def test_silu_hadamard(ops, dev, shape):
 
 
 @pytest.mark.parametrize("shape", SHAPES)
+def test_silu_hadamard_backward(ops, dev, shape):
+    x, u = _pair(shape, 4)
+    g = _pair(shape, 5)[0]
+    gx, gu = ops.silu.silu_hadamard_backward(x.to(dev), u.to(dev), g.to(dev))
+    # the composition it stands for, from the operators already checked: bit for bit
+    gd, ud, xd = g.to(dev), u.to(dev), x.to(dev)
+    assert torch.equal(gx, ops.silu.silu_backward(xd, gd * ud))
+    assert torch.equal(gu, gd * ops.silu.silu_hadamard(xd, torch.ones_like(xd)))
+    gx_o, gu_o = O.silu_mul_bwd(x, u, g)
+    assert_close_bf16(gx, gx_o, what="grad_x vs oracle")
+    assert_close_bf16(gu, gu_o, what="grad_u vs oracle")
+    xf, uf = x.float().requires_grad_(), u.float().requires_grad_()
+    (F.silu(xf) * uf).backward(g.float())
+    assert_close_bf16(gx, xf.grad, rel_tol=2e-2, what="grad_x vs autograd")
+    assert_close_bf16(gu, uf.grad, what="grad_u vs autograd")
+
+
+@pytest.mark.parametrize("shape", SHAPES)
 def test_gelu_backward(ops, dev, shape):
     x, g = _pair(shape, 3)
     o = ops.gelu.gelu_backward(x.to(dev), g.to(dev))
