@@ -631,6 +631,18 @@ def main():
                                                 "three_separate_kernels_ms": ms3}
         ms, _ = timed(lambda i: cf.get_statistics_channel_base(x_h[i % NH], 0.005, QB, 'per-channel'), Kx, Wx)
         kernels["calibration_stats_4096"] = {"ms": ms}
+        # norm backward straight from the channel-base compressed input, residual gradient added, against
+        # restore + backward with the same add
+        xo_h, qx_h = cf.outlier_subtraction_fuse_compression_quantization(x_h[0].clone(), sc, idx, QB)
+        ms, _ = timed(lambda i: rmsnorm_kernels.rmsnorm_backward_from_codes(x_h[i % NH], qx_h, sc, xo_h, idx, QB, w_h, rstd,
+                                                                            residual=x_h[(i + 1) % NH], table=tbl), Kx, Wx)
+        ms2, _ = timed(lambda i: rmsnorm_kernels._backward(
+            x_h[i % NH], cf.outlier_addition_fuse_decompression_dequantization(qx_h, sc, xo_h, idx, QB), w_h, rstd,
+            want_dw=False, residual=x_h[(i + 1) % NH]), Kx, Wx)
+        kernels["rmsnorm_bwd_from_codes_4096"] = {"ms": ms, "GBps": T * H * (6 + QB / 8) / ms / 1e6,
+                                                  "restore_then_backward_ms": ms2}
+        ms, _ = timed(lambda i: silu_kernels.silu_hadamard_backward(xs[i % NB], xs[(i + 1) % NB], xs[(i + 2) % NB]), Kx, Wx)
+        kernels["silu_mul_bwd"] = {"ms": ms, "GBps": E * 10 / ms / 1e6}
         # attention map (configuration 3 shape): compaction, restore, softmax backward
         a = torch.softmax(torch.randn(4, 32, 1024, 1024, generator=gen, device=dev) * 0.707
                           + torch.full((1024, 1024), float("-inf"), device=dev).triu(1), dim=-1).to(BF16)
