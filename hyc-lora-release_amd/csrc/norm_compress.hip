@@ -307,7 +307,7 @@ struct NormBwdCodesArgs {
 template <int QBIT, bool W32, int MAXW, bool RES>
 __global__ __launch_bounds__(MAXW * kWave) __attribute__((amdgpu_waves_per_eu(4)))
 void rmsnorm_bwd_codes_slab_kernel(const NormBwdCodesArgs a, int rows_per_group) {
-    constexpr int G = kSlabRows;
+    constexpr int G = RES ? 1 : kSlabRows;              // with a residual: one row per step, or registers spill
     extern __shared__ float slab_part[];                // [2][G][2][waves][64]
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
