@@ -130,7 +130,7 @@ __device__ __forceinline__ void lora_add_rows(const LoraAddArgs& a, int64_t row_
                 // rows past the end still take part in the quad exchange; their stores are masked
                 const int64_t tq = t < row_end ? t : row_end - 1;
                 codes_to_words<QBIT, ZP, FAST>(f, qc, z, lo, hi);
-                store_packed<QBIT, true>(a.q + tq * row_bytes, chunk, live, lo, hi);
+                store_packed<QBIT, false>(a.q + tq * row_bytes, chunk, live, lo, hi);
             }
             if constexpr (RES) {
                 float r[8];

@@ -84,9 +84,9 @@ __device__ __forceinline__ void fuse_fwd_rows(const FuseArgs& a, int64_t row_beg
             // rows past the end still take part in the quad exchange; their stores are masked
             const int64_t tq = t < row_end ? t : row_end - 1;
             codes_to_words<QBIT, false, FAST>(f1, c1, zero8, lo, hi);
-            store_packed<QBIT, true>(a.q1 + tq * row_bytes, chunk, live, lo, hi);
+            store_packed<QBIT, false>(a.q1 + tq * row_bytes, chunk, live, lo, hi);
             codes_to_words<QBIT, false, FAST>(f2, c2, zero8, lo, hi);
-            store_packed<QBIT, true>(a.q2 + tq * row_bytes, chunk, live, lo, hi);
+            store_packed<QBIT, false>(a.q2 + tq * row_bytes, chunk, live, lo, hi);
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 float y1 = rbf(f1[j] + lora_elem(L1[v], j));
@@ -147,9 +147,9 @@ __device__ __forceinline__ void fuse_fwd_rows_full(const FuseArgs& a, int64_t ro
             if constexpr (AHEAD) request_row(row0 + kTileRows, v);
             uint32_t lo, hi;
             codes_to_words<QBIT, false, true>(f1, c1, zero8, lo, hi);
-            store_packed<QBIT, true>(a.q1 + r * row_bytes, chunk, true, lo, hi);
+            store_packed<QBIT, false>(a.q1 + r * row_bytes, chunk, true, lo, hi);
             codes_to_words<QBIT, false, true>(f2, c2, zero8, lo, hi);
-            store_packed<QBIT, true>(a.q2 + r * row_bytes, chunk, true, lo, hi);
+            store_packed<QBIT, false>(a.q2 + r * row_bytes, chunk, true, lo, hi);
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 float y1 = rbf(f1[j] + lora_elem(L1[v], j));
