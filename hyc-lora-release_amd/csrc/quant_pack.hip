@@ -205,7 +205,7 @@ __device__ __forceinline__ void quant_rows(const QuantArgs& a, int64_t row0, int
 #pragma unroll
         for (int u = 0; u < kRowUnroll; ++u) {
             const int64_t t = t0 + u;
-            store_merged<QBIT, true>(a.q + t * row_bytes, chunk, FULL || (active && t < row1), lo[u], hi[u]);
+            store_merged<QBIT, false>(a.q + t * row_bytes, chunk, FULL || (active && t < row1), lo[u], hi[u]);
         }
     };
     // The first group is peeled so that the loop is always entered with "4 loads, then 4 stores"
