@@ -1,6 +1,8 @@
 // Element-wise backward operators for gfx950: SiLU backward, SiLU*x2 (forward of the gated
 // MLP product) and tanh-GELU backward.  Pure streaming kernels: one 128-bit load per
-// operand per lane, four independent chunks in flight per lane.
+// operand per lane, four independent chunks in flight per lane.  The two-operand kernels write
+// with ordinary stores (measured 5-10 % faster than non-temporal ones on [4096 x 11008] and
+// [8192 x 11008]); the three-operand backward keeps non-temporal ones (faster at 8192 rows).
 //
 // The SiLU kernels round to bf16 after every arithmetic operation, as the reference's bf16
 // Triton expressions do (operators/silu_kernels.py:42-43, :103-104); the sigmoid itself is
@@ -58,7 +60,7 @@ __global__ __launch_bounds__(kEwThreads) void binary_kernel(const uint16_t* __re
             unpack8(bv[u], bf);
 #pragma unroll
             for (int j = 0; j < 8; ++j) of[j] = op(af[j], bf[j]);
-            st16_nt(o + c * 8, pack8(of));
+            st16(o + c * 8, pack8(of));
         }
     }
     if (blockIdx.x == 0 && threadIdx.x < (n & 7)) {       // ragged tail
