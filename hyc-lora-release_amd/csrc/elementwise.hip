@@ -1,8 +1,9 @@
 // Element-wise backward operators for gfx950: SiLU backward, SiLU*x2 (forward of the gated
 // MLP product) and tanh-GELU backward.  Pure streaming kernels: one 128-bit load per
-// operand per lane, four independent chunks in flight per lane.  The two-operand kernels write
-// with ordinary stores (measured 5-10 % faster than non-temporal ones on [4096 x 11008] and
-// [8192 x 11008]); the three-operand backward keeps non-temporal ones (faster at 8192 rows).
+// operand per lane, four independent chunks in flight per lane.  Loads are ordinary loads (the
+// operands were usually written by the kernel before: 5 % faster than non-temporal loads); the
+// two-operand kernels also write with ordinary stores (another 5-10 % on [4096 x 11008] and
+// [8192 x 11008]), the three-operand backward keeps non-temporal stores (faster at 8192 rows).
 //
 // The SiLU kernels round to bf16 after every arithmetic operation, as the reference's bf16
 // Triton expressions do (operators/silu_kernels.py:42-43, :103-104); the sigmoid itself is
@@ -47,8 +48,8 @@ __global__ __launch_bounds__(kEwThreads) void binary_kernel(const uint16_t* __re
     for (int u = 0; u < kEwUnroll; ++u) {
         const int64_t c = c0 + u * kEwThreads;
         if (c < chunks) {
-            av[u] = ld16_nt(a + c * 8);
-            bv[u] = ld16_nt(b + c * 8);
+            av[u] = ld16(a + c * 8);
+            bv[u] = ld16(b + c * 8);
         }
     }
 #pragma unroll
@@ -89,9 +90,9 @@ __global__ __launch_bounds__(kEwThreads) void silu_mul_bwd_kernel(const uint16_t
     for (int k = 0; k < kUnroll; ++k) {
         const int64_t c = c0 + k * kEwThreads;
         if (c < chunks) {
-            xv[k] = ld16_nt(x + c * 8);
-            uv[k] = ld16_nt(u + c * 8);
-            gv[k] = ld16_nt(g + c * 8);
+            xv[k] = ld16(x + c * 8);
+            uv[k] = ld16(u + c * 8);
+            gv[k] = ld16(g + c * 8);
         }
     }
 #pragma unroll

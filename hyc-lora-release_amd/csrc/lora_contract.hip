@@ -186,7 +186,7 @@ __global__ __launch_bounds__(kCtThreads) void lora_contract_kernel(const Contrac
                     xv[st][vv] = u32x4{0, 0, 0, 0};
                     if (active && t < a.T) {
                         if constexpr (QBIT == 0) {
-                            xv[st][vv] = ld16_nt(a.x + t * a.N + chunk * 8);
+                            xv[st][vv] = ld16(a.x + t * a.N + chunk * 8);
                         } else {
                             const u32x2 w = ld8(a.q + t * row_bytes + slot.offset);
                             xv[st][vv].x = w.x;
