@@ -110,6 +110,8 @@ def rmsnorm_backward_from_codes(dy, q_x, scale_x, x_outlier, outlier_idx, q_bit,
             raise ValueError("x_outlier does not match the outlier list")
     wt, w32 = _weight(w)
     rstd = rstd.to(torch.float32).contiguous()
+    if sx.numel() != n or wt.numel() != n or rstd.numel() != rows:
+        raise ValueError(f"steps and weight must have {n} entries and rstd {rows}, got {sx.numel()}, {wt.numel()}, {rstd.numel()}")
     if residual is not None:
         if residual.shape != dy.shape or residual.dtype != torch.bfloat16:
             raise ValueError(f"residual must be bfloat16 of shape {tuple(dy.shape)}")
