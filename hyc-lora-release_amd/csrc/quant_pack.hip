@@ -21,8 +21,9 @@
 // Cache policy (measured on MI355X, [4096, 11008] bf16): the activation is touched once, so
 // its loads (quantise) and stores (dequantise) are non-temporal — that alone is worth ~25 %
 // on the dequantiser, whose stores otherwise evict useful lines.  The packed codes are stored
-// non-temporally but LOADED normally: neighbouring lanes read the same 8 bytes and rely on
-// the cache to merge those requests.
+// and loaded with ordinary cache policy: the kernel that reads the codes next waits behind
+// non-temporal stores on their way to memory, and neighbouring lanes of the dequantiser read
+// the same 8 bytes and rely on the cache to merge those requests.
 #include <type_traits>
 
 #include "hyc_pack.hpp"

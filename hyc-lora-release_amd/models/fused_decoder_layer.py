@@ -49,7 +49,7 @@ from ..operators.compress_function import (compress_attention_map, compression_p
                                            get_statistics_only_quant, get_statistics_only_quant_zero_point,
                                            get_statistics_softmax,
                                            outlier_addition_fuse_decompression_dequantization,
-                                           update_dict)
+                                           update_dict, validate_channel_list)
 from ..operators.rmsnorm_kernels import _backward as _rmsnorm_backward
 from ..operators.rmsnorm_kernels import (backward_from_codes_supported, rmsnorm_backward_from_codes, rmsnorm_forward,
                                          rmsnorm_forward_compress)
@@ -587,6 +587,10 @@ class FusedDecoderLayer(torch.nn.Module):
         if set(got) != set(want) or any(set(got[k]) != set(want[k]) for k in want):
             raise ValueError(f"calibration state of another layer type: has {sorted(got)}, "
                              f"{self.spec.mode}/{self.spec.attention} needs {sorted(want)}")
+        for key, fields in got.items():
+            channel, scale = fields.get("outlier_channel_index"), fields.get("scale")
+            if torch.is_tensor(channel) and torch.is_tensor(scale):
+                validate_channel_list(channel, scale.numel())
         self.iteration = int(state["iteration"])
         self.static_value = {key: {f: (v.detach().clone() if torch.is_tensor(v) else v) for f, v in fields.items()}
                              for key, fields in got.items()}

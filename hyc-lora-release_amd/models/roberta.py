@@ -17,7 +17,8 @@ import torch
 from ..operators.compress_function import (compress_attention_map, compression_pack_channel_base,
                                            compression_pack_quant_base, decompression_dequantization,
                                            get_statistics_only_quant, get_statistics_softmax,
-                                           outlier_addition_fuse_decompression_dequantization, update_dict)
+                                           outlier_addition_fuse_decompression_dequantization, update_dict,
+                                           validate_channel_list)
 from ..operators.gelu_kernels import gelu_backward
 from ..operators.layernorm_kernels import layernorm_backward, layernorm_forward
 from ..operators.softmax_kernels import softmax_backward, softmax_backward_from_compressed, softmax_forward
@@ -329,6 +330,10 @@ class _FusedRobertaLayerBase(torch.nn.Module):
         want, got = self._empty(), state["static_value"]
         if set(got) != set(want) or any(set(got[k]) != set(want[k]) for k in want):
             raise ValueError(f"calibration state of another layer type: has {sorted(got)}, needs {sorted(want)}")
+        for fields in got.values():
+            channel, scale = fields.get("outlier_channel_index"), fields.get("scale")
+            if torch.is_tensor(channel) and torch.is_tensor(scale):
+                validate_channel_list(channel, scale.numel())
         self.iteration = int(state["iteration"])
         self.static_value = {key: {f: (v.detach().clone() if torch.is_tensor(v) else v) for f, v in fields.items()}
                              for key, fields in got.items()}

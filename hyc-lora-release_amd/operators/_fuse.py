@@ -15,16 +15,34 @@ def _prep(t, name):
     return t
 
 
-def _common(xa1, b1, s1, xa2, b2, s2, quantize_bit, n):
+def _validate(xa1, b1, s1, xa2, b2, s2, quantize_bit, rows, n):
+    """Everything the kernels take on trust: they read xa[row, 0..R) for each of `rows` rows,
+    B[0..R, 0..N) and s[0..N), so a short operand would be read out of bounds on the device."""
     if quantize_bit not in (2, 4, 8):
         raise ValueError(f"quantize_bit must be 2, 4 or 8, got {quantize_bit}")
+    if b1.dim() != 2 or b2.dim() != 2:
+        raise ValueError("LoRA-B operands must be matrices [R, N]")
     r = b1.shape[0]
     if b2.shape[0] != r or xa1.shape[-1] != r or xa2.shape[-1] != r:
         raise ValueError("LoRA rank mismatch between xa1/b1/xa2/b2")
+    if r % 4 or not 4 <= r <= 64:
+        raise ValueError(f"LoRA rank must be a multiple of 4 in 4..64, got {r}")
     if b1.shape[1] != n or b2.shape[1] != n:
         raise ValueError("LoRA-B width does not match the activation width")
     if n % 32:
         raise ValueError(f"channel count must be a multiple of 32, got {n}")
+    for xa, name in ((xa1, "xa1"), (xa2, "xa2")):
+        if xa.numel() != rows * r:
+            raise ValueError(f"{name} must hold one row of {r} values per activation row ({rows} rows), "
+                             f"got shape {tuple(xa.shape)}")
+    for s, name in ((s1, "s1"), (s2, "s2")):
+        if s.numel() != n:
+            raise ValueError(f"{name} must have {n} elements (one per channel), got {s.numel()}")
+    return r
+
+
+def _common(xa1, b1, s1, xa2, b2, s2, quantize_bit, n):
+    r = b1.shape[0]
     # [R, N] views of [N, R] contiguous weights (lora_B.weight.T) are read as they lie in memory
     bt = int(all(b.dtype == BF16 and not b.is_contiguous() and b.mT.is_contiguous() and b.data_ptr() % 8 == 0
                  for b in (b1, b2)))
@@ -35,9 +53,11 @@ def _common(xa1, b1, s1, xa2, b2, s2, quantize_bit, n):
 
 
 def fuse_forward(xa1, b1, x1, s1, xa2, b2, x2, s2, quantize_bit=8):
-    _lib.require_gpu(xa1, b1, x1, s1, xa2, b2, x2, s2)
+    if x1.dim() != 3 or x2.shape != x1.shape:
+        raise ValueError(f"x1 and x2 must be [B, M, N] of one shape, got {tuple(x1.shape)} and {tuple(x2.shape)}")
     B, M, N = x1.shape
-    assert x2.shape == x1.shape
+    _validate(xa1, b1, s1, xa2, b2, s2, quantize_bit, B * M, N)
+    _lib.require_gpu(xa1, b1, x1, s1, xa2, b2, x2, s2)
     xa1, b1, s1, xa2, b2, s2, R, bt = _common(xa1, b1, s1, xa2, b2, s2, quantize_bit, N)
     x1 = _prep(x1, "x1")
     x2 = _prep(x2, "x2")
@@ -52,15 +72,18 @@ def fuse_forward(xa1, b1, x1, s1, xa2, b2, x2, s2, quantize_bit=8):
 
 
 def fuse_backward(xa1, b1, q1, s1, xa2, b2, q2, s2, grad_o, quantize_bit=8):
-    _lib.require_gpu(xa1, b1, q1, s1, xa2, b2, q2, s2, grad_o)
+    if grad_o.dim() != 3:
+        raise ValueError(f"grad_o must be [B, M, N], got shape {tuple(grad_o.shape)}")
     B, M, N = grad_o.shape
+    _validate(xa1, b1, s1, xa2, b2, s2, quantize_bit, B * M, N)
+    want = (B, M, N * quantize_bit // 8)
+    if tuple(q1.shape) != want or tuple(q2.shape) != want or q1.dtype != torch.uint8 or q2.dtype != torch.uint8:
+        raise ValueError(f"packed codes must be uint8 of shape {want}")
+    _lib.require_gpu(xa1, b1, q1, s1, xa2, b2, q2, s2, grad_o)
     xa1, b1, s1, xa2, b2, s2, R, bt = _common(xa1, b1, s1, xa2, b2, s2, quantize_bit, N)
     grad_o = _prep(grad_o, "grad_o")
     q1 = q1.contiguous()
     q2 = q2.contiguous()
-    want = (B, M, N * quantize_bit // 8)
-    if tuple(q1.shape) != want or tuple(q2.shape) != want or q1.dtype != torch.uint8 or q2.dtype != torch.uint8:
-        raise ValueError(f"packed codes must be uint8 of shape {want}")
     o = torch.empty((B, M, N), device=grad_o.device, dtype=BF16)
     gg = torch.empty_like(o)
     gu = torch.empty_like(o)

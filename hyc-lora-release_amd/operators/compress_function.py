@@ -5,7 +5,8 @@ Function names, argument order and return values follow the reference so that th
 decoder layers can call either implementation.  Differences, all deliberate:
   * `outlier_subtraction_fuse_compression_quantization` does not modify its input
     unless `zero_input=True` is passed (the reference zeroes the outlier columns of `x`
-    in place, which is why its callers hand it a clone);
+    in place, which is why its callers hand it a clone); `zero_input=True` needs a bf16 tensor
+    the kernels can address in place and raises otherwise;
   * 4-D `[B, H, S, D]` inputs are read in place through their strides instead of being
     transposed into a temporary `[B, S, H*D]` copy;
   * outlier channels are chosen with a defined tie rule (norm descending, then channel
@@ -179,6 +180,21 @@ def get_statistics_channel_base(x: torch.Tensor, outlier_ratio: float, q_bit: in
     return idx, scale
 
 
+def validate_channel_list(channel: torch.Tensor, n: int) -> None:
+    """An outlier channel list must name distinct channels inside [0, n): the kernels skip an index
+    outside the tensor and keep one position of a repeated one, where `x[:, :, channel]` of the
+    reference (:125) raises / gathers.  Reads the list back to the host, so it is meant for the
+    places where a list enters from outside (a checkpoint), not for the per-step path."""
+    if channel is None or channel.numel() == 0:
+        return
+    c = channel.detach().reshape(-1).to("cpu", torch.int64)
+    if int(c.min()) < 0 or int(c.max()) >= n:
+        raise ValueError(f"outlier channel index out of range for {n} channels: "
+                         f"[{int(c.min())}, {int(c.max())}]")
+    if torch.unique(c).numel() != c.numel():
+        raise ValueError("outlier channel list names a channel twice")
+
+
 def _check_bits(quantize_bit: int) -> int:
     if quantize_bit not in (2, 4, 8):
         raise ValueError(f"quantize_bit must be 2, 4 or 8, got {quantize_bit}")
@@ -193,6 +209,10 @@ def _quantize(x, s, z, channel, quantize_bit, dtype, zero_input=False):
     if x.dtype != BF16:
         x = x.to(BF16)
     a = _Addr(x)
+    if zero_input and a.t is not x:
+        # the kernel would zero a private bf16 / contiguous copy and leave the caller's tensor as it was
+        raise ValueError("zero_input=True needs a bfloat16 activation whose channel dimension is contiguous "
+                         "and 16-byte aligned: it is zeroed in place")
     if a.N % 32:
         raise ValueError(f"channel count must be a multiple of 32, got {a.N}")
     s = _vec(s, a.N, "scale")
@@ -203,7 +223,10 @@ def _quantize(x, s, z, channel, quantize_bit, dtype, zero_input=False):
     if channel is not None:
         channel = channel.to(torch.int64).contiguous()
         k = channel.numel()
-        x_outlier = torch.empty((a.B, a.M, k), device=x.device, dtype=BF16)
+        # zero-filled (a few hundred KB): a list position the kernel finds no column for - an index
+        # outside the tensor, the earlier copies of a repeated one - then reads as zeros, not as
+        # whatever the allocator handed out
+        x_outlier = torch.zeros((a.B, a.M, k), device=x.device, dtype=BF16)
     _lib.call("hyc_quant_pack", a.t.data_ptr(), s.data_ptr(), _lib.ptr(z), q.data_ptr(),
               _lib.ptr(channel) if k else None, k, _lib.ptr(x_outlier) if k else None, int(bool(zero_input)),
               a.B, a.M, a.N, a.sb, a.sm, a.hd, a.sh, quantize_bit, _lib.stream_of(x))

@@ -16,10 +16,17 @@ from ._fuse import _prep
 BF16 = torch.bfloat16
 
 
-def _check(xa, b, n):
+def _check(xa, b, n, rows):
+    """Shapes the kernels rely on: they read xa[row, 0..R) for every row of the activation and
+    B[0..R, 0..N), so a short operand would be read out of bounds on the device."""
+    if b.dim() != 2:
+        raise ValueError(f"LoRA-B must be a matrix [R, N], got shape {tuple(b.shape)}")
     r = b.shape[0]
-    if xa.shape[-1] != r:
-        raise ValueError(f"LoRA rank mismatch: x@A has {xa.shape[-1]} columns, B has {r} rows")
+    if xa.dim() < 1 or xa.shape[-1] != r:
+        raise ValueError(f"LoRA rank mismatch: x@A has shape {tuple(xa.shape)}, B has {r} rows")
+    if xa.numel() != rows * r:
+        raise ValueError(f"x@A must hold one row of {r} values per activation row ({rows} rows), "
+                         f"got shape {tuple(xa.shape)}")
     if b.shape[1] != n:
         raise ValueError(f"LoRA-B width {b.shape[1]} does not match the activation width {n}")
     if n % 32:
@@ -57,16 +64,16 @@ def _lora_b(b):
 def lora_add(x_main, xa, b, inplace=False, residual=None):
     """bf16(x_main + bf16(xa @ b)), then - with a residual of x_main's shape - bf16(residual + that);
     `inplace` overwrites x_main (contiguous bf16) and returns it."""
-    _lib.require_gpu(x_main, xa, b, residual)
     n = x_main.shape[-1]
-    r = _check(xa, b, n)
+    r = _check(xa, b, n, x_main.numel() // max(n, 1))
+    if residual is not None and residual.shape != x_main.shape:
+        raise ValueError(f"residual must have the shape of x_main {tuple(x_main.shape)}, got {tuple(residual.shape)}")
+    _lib.require_gpu(x_main, xa, b, residual)
     x = x_main if (inplace and x_main.dtype == BF16 and x_main.is_contiguous() and x_main.data_ptr() % 16 == 0) \
         else _prep(x_main, "x_main")
     y = x if inplace else torch.empty_like(x)
     xa, (b, bt) = _prep(xa, "xa"), _lora_b(b)
     if residual is not None:
-        if residual.shape != x_main.shape:
-            raise ValueError(f"residual must have the shape of x_main {tuple(x_main.shape)}, got {tuple(residual.shape)}")
         residual = _prep(residual, "residual")
     _lib.call("hyc_lora_add", xa.data_ptr(), b.data_ptr(), bt, x.data_ptr(), _lib.ptr(residual), y.data_ptr(),
               x.numel() // n, n, r, _lib.stream_of(x))
@@ -76,11 +83,14 @@ def lora_add(x_main, xa, b, inplace=False, residual=None):
     return y
 
 
-def _vec(t, n, name):
-    t = t.to(BF16).reshape(-1)
-    if t.numel() != n:
+def _vec_ok(t, n, name):
+    if t is not None and t.numel() != n:
         raise ValueError(f"{name} must have {n} elements (one per channel), got {t.numel()}")
-    return _prep(t, name)
+
+
+def _vec(t, n, name):
+    _vec_ok(t, n, name)
+    return _prep(t.to(BF16).reshape(-1), name)
 
 
 ROPE_HEAD_DIM = 128          # the fused rotation needs heads as wide as a column tile
@@ -101,9 +111,13 @@ def lora_add_quant(x_main, xa, b, scale, zero_point=None, quantize_bit=8, inplac
     rotates y as rope_forward would on its [B, M, N / 128, 128] view (heads of 128 dims only)."""
     if quantize_bit not in (2, 4, 8):
         raise ValueError(f"quantize_bit must be 2, 4 or 8, got {quantize_bit}")
-    _lib.require_gpu(x_main, xa, b, scale, zero_point)
+    if x_main.dim() != 3:
+        raise ValueError(f"x_main must be [B, M, N], got shape {tuple(x_main.shape)}")
     B, M, n = x_main.shape
-    r = _check(xa, b, n)
+    r = _check(xa, b, n, B * M)
+    _vec_ok(scale, n, "scale")
+    _vec_ok(zero_point, n, "zero point")
+    _lib.require_gpu(x_main, xa, b, scale, zero_point)
     x = _prep(x_main, "x_main")
     y = x if (inplace and x is x_main) else torch.empty_like(x)
     xa, (b, bt) = _prep(xa, "xa"), _lora_b(b)
@@ -128,12 +142,15 @@ def lora_add_restore(q, scale, xa, b, zero_point=None, quantize_bit=8, rope=None
     writing the dequantised tensor; rope=(cos, sin) rotates the result like lora_add_quant's."""
     if quantize_bit not in (2, 4, 8):
         raise ValueError(f"quantize_bit must be 2, 4 or 8, got {quantize_bit}")
-    _lib.require_gpu(q, scale, xa, b, zero_point)
+    if q.dim() != 3:
+        raise ValueError(f"packed codes must be [B, M, N*bits/8], got shape {tuple(q.shape)}")
     B, M, nbytes = q.shape
-    n = scale.shape[-1]
+    n = scale.numel()
     if nbytes * 8 != n * quantize_bit or q.dtype != torch.uint8:
         raise ValueError(f"packed codes must be uint8 of width {n * quantize_bit // 8}, got {q.dtype} {nbytes}")
-    r = _check(xa, b, n)
+    r = _check(xa, b, n, B * M)
+    _vec_ok(zero_point, n, "zero point")
+    _lib.require_gpu(q, scale, xa, b, zero_point)
     q = q.contiguous()
     xa, (b, bt) = _prep(xa, "xa"), _lora_b(b)
     s = _vec(scale, n, "scale")
@@ -182,13 +199,17 @@ def lora_products(x, u=None, v=None):
     """x [..., N] bf16 read once -> (u^T x as [R, N] or None, x v^T as [..., R] or None), u [..., R], v [R, N]
     (a `weight.T` view of an [N, R] weight is read in place).  fp32 accumulation over the whole
     contraction, one bf16 rounding."""
-    _lib.require_gpu(x, u, v)
     if u is None and v is None:
         raise ValueError("nothing to compute: pass u, v or both")
     n = x.shape[-1]
     r = u.shape[-1] if u is not None else v.shape[0]
     if n % 32 or r % 2 or not 2 <= r <= 64:
         raise ValueError(f"width must be a multiple of 32 and the rank even within 2..64, got {n}, {r}")
+    if u is not None and u.numel() != x.numel() // n * r:
+        raise ValueError(f"u must be [T, {r}] with T = {x.numel() // n}, got {tuple(u.shape)}")
+    if v is not None and tuple(v.shape) != (r, n):
+        raise ValueError(f"v must be [{r}, {n}], got {tuple(v.shape)}")
+    _lib.require_gpu(x, u, v)
     lead = tuple(x.shape[:-1])
     x = _prep(x, "x")
     T = x.numel() // n
@@ -201,14 +222,19 @@ def lora_product_from_codes(q, scale, u, zero_point=None, quantize_bit=8):
     decompression_dequantization[_with_zero_point](q, scale[, zero_point]) would expand first)."""
     if quantize_bit not in (2, 4, 8):
         raise ValueError(f"quantize_bit must be 2, 4 or 8, got {quantize_bit}")
-    _lib.require_gpu(q, scale, u, zero_point)
+    if q.dim() != 3:
+        raise ValueError(f"packed codes must be [B, M, N*bits/8], got shape {tuple(q.shape)}")
     B, M, nbytes = q.shape
-    n = scale.shape[-1]
+    n = scale.numel()
     if nbytes * 8 != n * quantize_bit or q.dtype != torch.uint8:
         raise ValueError(f"packed codes must be uint8 of width {n * quantize_bit // 8}, got {q.dtype} {nbytes}")
     r = u.shape[-1]
     if n % 32 or r % 2 or not 2 <= r <= 64:
         raise ValueError(f"width must be a multiple of 32 and the rank even within 2..64, got {n}, {r}")
+    if u.numel() != B * M * r:
+        raise ValueError(f"u must be [T, {r}] with T = {B * M}, got {tuple(u.shape)}")
+    _vec_ok(zero_point, n, "zero point")
+    _lib.require_gpu(q, scale, u, zero_point)
     s = _vec(scale, n, "scale")
     z = None if zero_point is None else _vec(zero_point, n, "zero point")
     p1, _ = _contract(None, (q.contiguous(), s, z, quantize_bit), u, None, B * M, n, r, q.device)

@@ -9,7 +9,9 @@
  *     allocated, freed or kept between calls, nothing synchronises with the host.
  *     Work is enqueued on `stream` (a hipStream_t passed as void*; NULL = default stream).
  *   - Return value: HYC_OK (0) or a negative HYC_ERR_* code.  On error nothing was
- *     launched.  Entry points are reentrant; any thread may call with its own stream.
+ *     launched.  Entry points are reentrant; any thread may call with its own stream
+ *     (hyc_set_tuning, a benchmarking aid that writes process-wide launch-shape
+ *     settings, is the one exception: call it while no other thread is launching).
  *   - Each declaration cites the function of the reference (thu-ee-acts-lab/HyC-LoRA,
  *     path:line inside its checkout) whose GPU work it replaces.
  */

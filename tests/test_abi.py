@@ -59,7 +59,11 @@ def test_argument_validation_without_launch(L):
     assert h.hyc_quant_pack(None, None, None, None, None, 0, None, 0, 0, 4, 64, 256, 64, 64, 0, 4, None) == 0
     assert h.hyc_set_tuning(b"no_such_key", 1) == -8
     assert h.hyc_set_tuning(b"quant_rows_per_wave", 0) == -8
-    assert h.hyc_set_tuning(b"quant_rows_per_wave", 16) == 0
+    # the knobs are process-wide: put the default back so later tests run with it
+    try:
+        assert h.hyc_set_tuning(b"quant_rows_per_wave", 16) == 0
+    finally:
+        assert h.hyc_set_tuning(b"quant_rows_per_wave", 8) == 0
 
 
 def test_missing_library_is_an_error(L, monkeypatch, tmp_path):

@@ -145,6 +145,58 @@ def test_rmsnorm_backward(ops, dev, n, rows):
     assert_close_bf16(dx, xf.grad - c2, what="dx vs autograd minus the LayerNorm mean term")
 
 
+@pytest.mark.parametrize("n,rows", [(512, 7), (4096, 64), (96, 33), (8192, 4)])
+def test_rmsnorm_backward_mean_term_is_layernorms(ops, dev, n, rows):
+    """The c2 = mean(w*dy) term of the reference's formula (rmsnorm_kernels.py:96-98) is not part of a
+    true RMSNorm's derivative.  On rows whose mean is exactly zero the formula IS LayerNorm's backward
+    (layernorm_kernels.py:92-104), so there the kernel must agree with autograd of F.layer_norm - an
+    independent library routine - and must differ from autograd of RMSNorm by c2 * rstd."""
+    from test_oracle_norm import layernorm_autograd_dx, rmsnorm_autograd_dx, zero_mean_case
+    x, dy, w = zero_mean_case(n, rows, seed=n + rows)
+    xg, dyg, wg = x.to(dev), dy.to(dev), w.to(dev)
+    y, mean, rstd, block, warps = ops.norm.rmsnorm_forward(xg, wg, 1e-5)
+    assert_close_bf16(y, F.layer_norm(x.double(), (n,), w.double(), None, 1e-5), what="rmsnorm_forward vs layer_norm")
+    ln_dx = layernorm_autograd_dx(x, dy, w)
+    rms_dx = rmsnorm_autograd_dx(x, dy, w)
+    c2 = (w.double() * dy.double()).mean(-1, keepdim=True) * rstd.cpu().double().reshape(-1, 1)
+    dx, _ = ops.norm.rmsnorm_backward(dyg, xg, wg, mean, rstd, True, 1e-5, warps, block)
+    dxu, dw = ops.normu.rmsnorm_backward(dyg, xg, wg, mean, rstd, 1e-5, warps, block)
+    res = torch.zeros_like(dyg)
+    dxr, _ = ops.norm.rmsnorm_backward(dyg, xg, wg, mean, rstd, True, 1e-5, warps, block, residual=res)
+    for got, what in ((dx, "rmsnorm_backward"), (dxu, "updatable rmsnorm_backward"), (dxr, "rmsnorm_backward + residual")):
+        assert_close_bf16(got, ln_dx, what=what + " vs autograd of layer_norm")
+        assert_close_bf16(got, rms_dx - c2, what=what + ": difference to true RMSNorm is c2 * rstd")
+        assert (got.cpu().double() - rms_dx).abs().max() / rms_dx.abs().max() > 5e-2, "case does not exercise the mean term"
+    assert_close_bf16(dx, O.rmsnorm_bwd(dy, x, w, rstd.cpu())[0], what="rmsnorm_backward vs oracle")
+    wd = w.double().requires_grad_()
+    F.layer_norm(x.double(), (n,), wd, None, 1e-5).backward(dy.double())
+    assert_close_bf16(dw, wd.grad, what="dw vs autograd of layer_norm")
+
+
+def test_rmsnorm_backward_from_codes_mean_term(ops, dev):
+    """The same pin for the backward that reads the norm's input from its compressed copy.  The rows
+    (v | -v) lie on the grid k/16, |k| <= 127, and every channel has the step 1/16, so the 8-bit
+    codes decode to the rows themselves and these still sum to exactly zero."""
+    from hyclora_amd.operators import compress_function as cf
+    from test_oracle_norm import layernorm_autograd_dx
+    n, rows = 1024, 16
+    g = torch.Generator().manual_seed(11)
+    v = (torch.randn(rows, n // 2, generator=g) * 32).round().clamp(-127, 127) / 16
+    x = torch.cat([v, -v], dim=-1)[:, torch.randperm(n, generator=g)].to(BF16).contiguous()
+    dy = (torch.randn(rows, n, generator=g) + 0.5).to(BF16)
+    w = (1 + 0.1 * torch.randn(n, generator=g)).to(BF16)
+    x3, dy3, wg = x.reshape(1, rows, n).to(dev), dy.reshape(1, rows, n).to(dev), w.to(dev)
+    scale = torch.full((1, n), 1 / 16, dtype=BF16, device=dev)
+    q = cf.compression_quantization(x3, scale, 8)
+    assert torch.equal(cf.decompression_dequantization(q, scale, 8), x3), "the codes do not decode to the rows"
+    _, _, rstd, _, _ = ops.norm.rmsnorm_forward(x3, wg, 1e-5)
+    dx = ops.norm.rmsnorm_backward_from_codes(dy3, q, scale, None, None, 8, wg, rstd)
+    assert_close_bf16(dx.reshape(rows, n), layernorm_autograd_dx(x, dy, w),
+                      what="rmsnorm_backward_from_codes vs autograd of layer_norm")
+    dense, _ = ops.norm.rmsnorm_backward(dy3, x3, wg, None, rstd, True, 1e-5, 0, 0)
+    assert torch.equal(dx, dense), "from-codes backward and dense backward differ"
+
+
 def test_rmsnorm_errors(ops, dev):
     with pytest.raises(RuntimeError):
         ops.norm.rmsnorm_forward(torch.zeros(1, 1, 32776, dtype=BF16, device=dev), torch.ones(32776, dtype=BF16, device=dev), 1e-5)

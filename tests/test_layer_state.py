@@ -14,7 +14,7 @@ def test_extra_state_round_trip(tmp_path):
     assert sd[key]["iteration"] == 0 and sd[key]["static_value"]["x"]["scale"] is None
     layer.iteration = 7
     layer.static_value["x"] = {"outlier_channel_index": torch.tensor([3, 9]),
-                               "scale": torch.tensor([0.5, 0.25]).to(torch.bfloat16)}
+                               "scale": torch.tensor([0.5, 0.25] * 8).to(torch.bfloat16)}
     layer.static_value["a"]["outlier"] = torch.tensor(0.125)
     torch.save(layer.state_dict(), tmp_path / "s.pt")
     other = FusedLlamaLayerIntraInterFullFuse()
@@ -41,3 +41,15 @@ def test_extra_state_of_another_layer_type_is_rejected():
         pytest.skip("same statistics layout")
     with pytest.raises((ValueError, RuntimeError)):
         dst.load_state_dict(src.state_dict())
+
+
+@pytest.mark.parametrize("channels", [[3, 16], [-1, 2], [5, 5]])
+def test_extra_state_with_a_bad_channel_list_is_rejected(channels):
+    """The kernels skip an out-of-range outlier channel and keep one copy of a repeated one, so a
+    list that enters from a checkpoint is checked where it enters."""
+    layer = FusedLlamaLayerIntraInterFullFuse()
+    layer.static_value["x_medium"] = {"outlier_channel_index": torch.tensor(channels),
+                                      "scale": torch.ones(16).to(torch.bfloat16)}
+    state = layer.get_extra_state()
+    with pytest.raises(ValueError, match="outlier channel"):
+        FusedLlamaLayerIntraInterFullFuse().set_extra_state(state)
