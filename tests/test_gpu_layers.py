@@ -20,7 +20,7 @@ class Lin:
         self.weight, self.bias = weight, bias
 
 
-def make_layer_inputs(dev, seed, B=2, S=64, hidden=256, heads=4, kv_heads=4, inter=512, rank=16):
+def make_layer_inputs(dev, seed, B=2, S=64, hidden=256, heads=4, kv_heads=4, inter=512, rank=16, theta=10000.0):
     g = torch.Generator(device=dev).manual_seed(seed)
     rn = lambda *s, sc=1.0: (torch.randn(*s, generator=g, device=dev) * sc).to(BF16)
     hd = hidden // heads
@@ -38,7 +38,7 @@ def make_layer_inputs(dev, seed, B=2, S=64, hidden=256, heads=4, kv_heads=4, int
     nw1 = (1 + 0.1 * torch.randn(hidden, generator=g, device=dev)).to(BF16).requires_grad_()
     nw2 = (1 + 0.1 * torch.randn(hidden, generator=g, device=dev)).to(BF16).requires_grad_()
     pos = torch.arange(S, device=dev, dtype=torch.float32)
-    inv = 1.0 / (10000 ** (torch.arange(0, hd, 2, device=dev, dtype=torch.float32) / hd))
+    inv = 1.0 / (theta ** (torch.arange(0, hd, 2, device=dev, dtype=torch.float32) / hd))
     ang = torch.cat([pos[:, None] * inv[None, :]] * 2, dim=-1)
     cos, sin = ang.cos().to(BF16)[None], ang.sin().to(BF16)[None]
     mask = torch.full((S, S), float("-inf"), device=dev).triu(1).to(BF16)[None, None]
@@ -61,7 +61,7 @@ class RefRMSNorm(torch.autograd.Function):
         return O.rmsnorm_bwd(dy, x, w, rstd)
 
 
-def reference_layer(t):
+def reference_layer(t, sdpa=False):
     from hyclora_amd.models.compute_utils import hidden_to_head_shape, head_to_hidden_shape, repeat_kv
     rope_forward = O.rope                      # differentiable torch ops; the HIP operator works in place
     P = t.P
@@ -77,9 +77,12 @@ def reference_layer(t):
     q = rope_forward(q.transpose(1, 2), t.cos, t.sin).transpose(1, 2)
     k = rope_forward(k.transpose(1, 2), t.cos, t.sin).transpose(1, 2)
     k, v = repeat_kv(k, t.heads // t.kv_heads), repeat_kv(v, t.heads // t.kv_heads)
-    s = q @ k.transpose(-2, -1) / math.sqrt(t.hd) + t.mask
-    a = torch.softmax(s, dim=-1, dtype=BF16)
-    o = head_to_hidden_shape(a @ v)
+    if sdpa:                    # causal attention without a materialised map (long sequences)
+        o = head_to_hidden_shape(F.scaled_dot_product_attention(q, k, v, is_causal=True))
+    else:
+        s = q @ k.transpose(-2, -1) / math.sqrt(t.hd) + t.mask
+        a = torch.softmax(s, dim=-1, dtype=BF16)
+        o = head_to_hidden_shape(a @ v)
     xm = t.x + proj("o", o)
     xn2 = RefRMSNorm.apply(xm, t.nw2)
     had = F.silu(proj("gate", xn2)) * proj("up", xn2)
