@@ -26,7 +26,7 @@ class HycError(RuntimeError):
 
 
 # name -> (restype, argtypes)
-ABI_VERSION = 3          # hyc_abi_version() of the library these signatures describe
+ABI_VERSION = 4          # hyc_abi_version() of the library these signatures describe
 _P, _I, _L = c_void_p, c_int, c_int64
 _SIGNATURES = {
     "hyc_error_string": (c_char_p, [_I]),
@@ -55,6 +55,8 @@ _SIGNATURES = {
     "hyc_rmsnorm_fwd": (_I, [_P, _P, _I, _P, _P, _L, _L, ctypes.c_float, _P]),
     "hyc_rmsnorm_bwd_workspace": (_L, [_L, _L]),
     "hyc_rmsnorm_bwd": (_I, [_P, _P, _P, _I, _P, _P, _P, _P, _L, _L, _L, _P]),
+    "hyc_rmsnorm_bwd_static_max_bytes": (_L, []),
+    "hyc_rmsnorm_bwd_static": (_I, [_P, _P, _P, _I, _P, _P, _P, _L, _L, _P]),
     "hyc_rmsnorm_bwd_add": (_I, [_P, _P, _P, _I, _P, _P, _P, _P, _P, _L, _L, _L, _P]),
     "hyc_rmsnorm_bwd_codes": (_I, [_P, _P, _P, _P, _L, _P, _I, _P, _I, _P, _P, _P, _L, _L, _P]),
     "hyc_silu_bwd": (_I, [_P, _P, _P, _L, _P]),

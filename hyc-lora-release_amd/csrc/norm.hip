@@ -8,6 +8,8 @@
 // spin-lock accumulation (operators/rmsnorm_kernels.py:103-113): each wave accumulates its
 // rows in fp32 registers, the workgroup combines its waves in LDS and writes one partial
 // row; a second kernel adds the partial rows in a fixed order.  Deterministic, no atomics.
+#include <mutex>
+
 #include "hyc_common.hpp"
 
 namespace hyc {
@@ -15,6 +17,16 @@ namespace hyc {
 constexpr int kNormThreads = 256;
 constexpr int kNormWaves = kNormThreads / kWave;
 constexpr int kNormMaxBlocks = 512;
+constexpr int kNormMaxRegisterRow = 8192;      // longest row the backward kernel holds in registers
+
+// Scratch of hyc_rmsnorm_bwd_static: the fp32 partial rows of the weight gradient, for the largest
+// launch the backward kernel makes (kNormMaxBlocks workgroups x rows of kNormMaxRegisterRow
+// channels = 16 MiB).  Lives in every GPU's memory from the moment the library's code object is
+// loaded there until the process ends.  In host code the array's NAME is only a handle: the
+// device address is obtained once per device with hipGetSymbolAddress (static_scratch() below)
+// and only that pointer is ever handed to a kernel.
+constexpr int64_t kStaticScratchBytes = (int64_t)kNormMaxBlocks * kNormMaxRegisterRow * (int64_t)sizeof(float);
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 template <bool W32>
 __device__ __forceinline__ void load_w8(const void* w, int col, float (&wf)[8]) {
@@ -315,6 +327,41 @@ extern "C" int hyc_rmsnorm_bwd(const void* dy, const void* x, const void* weight
                                const float* rstd, void* dx, void* dw, void* workspace, int64_t workspace_bytes,
                                int64_t rows, int64_t N, void* stream) {
     return rmsnorm_bwd_any(dy, x, weight, weight_is_fp32, rstd, nullptr, dx, dw, workspace, workspace_bytes, rows, N, stream);
+}
+
+// Device address of `scratch` on the current device; looked up once per device.
+static int static_scratch(void** out) {
+    constexpr int kMaxDevices = 64;
+    static void* ptrs[kMaxDevices] = {};
+    static std::mutex lock;
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return HYC_ERR_LAUNCH;
+    std::lock_guard<std::mutex> hold(lock);
+    if (!ptrs[dev]) {
+        void* p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) {
+            (void)hipGetLastError();
+            return HYC_ERR_LAUNCH;
+        }
+        ptrs[dev] = p;
+    }
+    *out = ptrs[dev];
+    return HYC_OK;
+}
+
+extern "C" int64_t hyc_rmsnorm_bwd_static_max_bytes(void) { return kStaticScratchBytes; }
+
+extern "C" int hyc_rmsnorm_bwd_static(const void* dy, const void* x, const void* weight, int weight_is_fp32,
+                                      const float* rstd, void* dx, void* dw, int64_t rows, int64_t N, void* stream) {
+    // sizes first, so that a caller learns about an oversized request without any device work
+    if (rows < 0 || N < 0 || N % 8 != 0) return HYC_ERR_SHAPE;
+    if (N > kNormMaxRegisterRow || hyc_rmsnorm_bwd_workspace(rows, N) > kStaticScratchBytes) return HYC_ERR_WORKSPACE;
+    if (rows == 0 || N == 0) return HYC_OK;
+    if (!dw) return HYC_ERR_NULL;
+    void* ws = nullptr;
+    const int rc = static_scratch(&ws);
+    if (rc != HYC_OK) return rc;
+    return rmsnorm_bwd_any(dy, x, weight, weight_is_fp32, rstd, nullptr, dx, dw, ws, kStaticScratchBytes, rows, N, stream);
 }
 
 extern "C" int hyc_rmsnorm_bwd_add(const void* dy, const void* x, const void* weight, int weight_is_fp32,

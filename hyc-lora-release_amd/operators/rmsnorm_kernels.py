@@ -78,6 +78,28 @@ def _backward(dy, x, w, rstd, want_dw, residual=None):
     return dx, dw
 
 
+def rmsnorm_backward_into(dy, x, w, rstd, dx, dw):
+    """rmsnorm_backward with the weight gradient, written into the caller's `dx` (bf16, dy's shape) and
+    `dw` ([N], w's dtype), through the entry point that allocates nothing: its fp32 partial rows live
+    in a fixed device array of the library (16 MiB per GPU), not in a workspace.  For callers that
+    must not allocate device memory (graph capture, serving loops).  All tensors must already be
+    contiguous, bf16 activations, fp32 rstd; calls that overlap in time on one GPU race on that array.
+    Same bits as rmsnorm_updatable_kernels.rmsnorm_backward."""
+    _lib.require_gpu(dy, x, w, rstd, dx, dw)
+    n = x.shape[-1]
+    rows = x.numel() // n if n else 0
+    ok = (dy.dtype == x.dtype == dx.dtype == torch.bfloat16 and dy.shape == x.shape == dx.shape
+          and rstd.dtype == torch.float32 and rstd.numel() == rows and w.numel() == n and dw.shape == w.shape
+          and dw.dtype == w.dtype and w.dtype in (torch.bfloat16, torch.float32)
+          and all(t.is_contiguous() for t in (dy, x, w, rstd, dx, dw)))
+    if not ok:
+        raise ValueError("rmsnorm_backward_into takes contiguous bf16 dy / x / dx of one shape, fp32 rstd [rows], "
+                         "and w / dw [N] of one dtype (bf16 or fp32); nothing is converted or copied")
+    _lib.call("hyc_rmsnorm_bwd_static", dy.data_ptr(), x.data_ptr(), w.data_ptr(), int(w.dtype == torch.float32),
+              rstd.data_ptr(), dx.data_ptr(), dw.data_ptr(), rows, n, _lib.stream_of(x))
+    return dx, dw
+
+
 def backward_from_codes_supported(dy, n, want_dw):
     """Whether rmsnorm_backward_from_codes takes this case (whole 512-column slabs, an even number of
     rows, bf16 gradient, no weight gradient)."""

@@ -270,6 +270,22 @@ int hyc_rmsnorm_bwd(const void *dy, const void *x, const void *weight, int weigh
                     const float *rstd, void *dx, void *dw, void *workspace, int64_t workspace_bytes,
                     int64_t rows, int64_t N, void *stream);
 
+/* hyc_rmsnorm_bwd with the weight gradient for callers that cannot allocate device memory or
+ * carry a workspace: code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  No counterpart in the reference.  Same kernels, same results bit for bit; the fp32
+ * partial rows live in a file-scope device array of the library instead of a caller workspace
+ * (hyc_rmsnorm_bwd_static_max_bytes() = 16 MiB per GPU, resident from the time the library is
+ * loaded on a device until the process ends).  Allocates nothing and frees nothing.
+ *   dw must be given (without it hyc_rmsnorm_bwd needs no workspace either).
+ *   N > 8192, or a shape whose partial rows would exceed the array: HYC_ERR_WORKSPACE, nothing launched.
+ *   Every call on one GPU uses that GPU's one array: calls that overlap in time on the same GPU
+ *   (different streams or threads) race on it; calls on one stream are ordered and safe.  Nothing
+ *   in the array needs clearing between calls: each launch overwrites all it later reads.
+ */
+int64_t hyc_rmsnorm_bwd_static_max_bytes(void);
+int hyc_rmsnorm_bwd_static(const void *dy, const void *x, const void *weight, int weight_is_fp32,
+                           const float *rstd, void *dx, void *dw, int64_t rows, int64_t N, void *stream);
+
 /* The same with the gradient that arrives over the residual connection added in the same pass:
  * dx = bf16(bf16(dx of hyc_rmsnorm_bwd) + residual), i.e. the bits of that call followed by a bf16
  * add.  Replaces `grad_norm_2 + grad_output` / `grad_norm_1 + grad_medium` after the norm backward
