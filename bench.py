@@ -30,10 +30,69 @@ ROOT = Path(__file__).resolve().parent
 sys.path.insert(0, str(ROOT))
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of quant_pack_kernel<4,false,false> on the benchmark tensor, measured with
-# rocprofv3 --pmc FETCH_SIZE (44 162.3 KiB raw, x1.99948 from the copy-kernel calibration) and
-# WRITE_SIZE (22 016 KiB, x1.0): 88 301.6 KiB read + 22 016 KiB written.
-MEASURED_TRAFFIC_BYTES = int((44162.3 * 1.99948 + 22016.0) * 1024)
+SETTLE_MS = 60.0          # every timed arm first runs its own kernels this long: the GPU reaches its
+                          # steady clocks only after tens of milliseconds of work, whatever --warmup says
+# HBM bytes per launch of the dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# `bench.py --only quant` and `--only copy`; `bench.py --pmc-summary DIR` writes this file from their
+# CSVs together with a hash of the kernel sources it was measured on.
+TRAFFIC_JSON = ROOT / "profiles" / "quant_pack_q4_config2_hbm_traffic.json"
+TRAFFIC_SOURCES = ["quant_pack.hip", "hyc_pack.hpp", "hyc_quant_math.h", "hyc_common.hpp"]
+
+
+def kernel_source_hash():
+    import hashlib
+    h = hashlib.sha256()
+    for name in TRAFFIC_SOURCES:
+        h.update((ROOT / "hyc-lora-release_amd" / "csrc" / name).read_bytes())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic():
+    """(bytes per launch or None, note): the counter measurement is only quoted while the kernel
+    sources are the ones it was taken on."""
+    if not TRAFFIC_JSON.exists():
+        return None, "no counter measurement committed"
+    rec = json.loads(TRAFFIC_JSON.read_text())
+    if rec.get("source_sha256_16") != kernel_source_hash():
+        return None, f"counter measurement is of other kernel sources ({rec.get('source_sha256_16')}); re-run the pmc passes"
+    return int(rec["traffic_bytes"]), f"rocprofv3 FETCH_SIZE/WRITE_SIZE at commit {rec.get('commit', '?')}, scale factors {rec['fetch_scale']:.5f}/{rec['write_scale']:.5f}"
+
+
+def pmc_summary(directory):
+    """Reads DIR/pmc_{quant,copy}_{FETCH_SIZE,WRITE_SIZE}/**/*counter_collection.csv (one rocprofv3
+    --pmc run each of `bench.py --only quant` / `--only copy`) and writes TRAFFIC_JSON: KiB per
+    dispatch of the quantiser, each counter scaled by what it reads for a plain copy of known size."""
+    import csv
+    import glob
+    import statistics
+    import subprocess
+
+    def median(mode, counter, match):
+        files = glob.glob(f"{directory}/pmc_{mode}_{counter}/**/*counter_collection.csv", recursive=True)
+        if not files:
+            raise SystemExit(f"no counter CSV under {directory}/pmc_{mode}_{counter}")
+        vals = [float(r["Counter_Value"]) for r in csv.DictReader(open(files[0])) if match in r["Kernel_Name"]]
+        if not vals:
+            raise SystemExit(f"no dispatch of {match} in {files[0]}")
+        return statistics.median(vals), len(vals)
+    B, M, N = 4, 1024, 11008
+    copy_kib = B * M * N * 2 / 1024                       # the copy arm reads and writes one activation
+    cf, ncf = median("copy", "FETCH_SIZE", "copyBuffer")
+    cw, _ = median("copy", "WRITE_SIZE", "copyBuffer")
+    qf, nq = median("quant", "FETCH_SIZE", "quant_pack_kernel<4")
+    qw, _ = median("quant", "WRITE_SIZE", "quant_pack_kernel<4")
+    fs, ws = copy_kib / cf, copy_kib / cw
+    commit = subprocess.run(["git", "-C", str(ROOT), "rev-parse", "--short", "HEAD"], capture_output=True, text=True).stdout.strip()
+    rec = {"kernel": "hyc::quant_pack_kernel<4,false,false>", "workload": "bf16 [4,1024,11008], q_bit 4",
+           "fetch_kib_raw": qf, "write_kib_raw": qw, "copy_fetch_kib_raw": cf, "copy_write_kib_raw": cw,
+           "copy_kib_per_direction": copy_kib, "fetch_scale": fs, "write_scale": ws, "dispatches": nq,
+           "read_bytes": qf * fs * 1024, "written_bytes": qw * ws * 1024,
+           "traffic_bytes": int((qf * fs + qw * ws) * 1024),
+           "algorithmic_bytes": int(B * M * N * 2.5 + 2 * N),
+           "source_sha256_16": kernel_source_hash(), "commit": commit or "unknown"}
+    rec["ratio_to_algorithmic"] = rec["traffic_bytes"] / rec["algorithmic_bytes"]
+    TRAFFIC_JSON.write_text(json.dumps(rec, indent=1) + "\n")
+    print(json.dumps(rec))
 
 
 def parse():
@@ -43,8 +102,10 @@ def parse():
     ap.add_argument("--warmup", type=int, default=1000,
                     help="untimed steps; ~50 ms of work lets the GPU reach its steady clocks (20 steps do not)")
     ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU-oracle timing (for profiler runs)")
-    ap.add_argument("--only", choices=["all", "roundtrip", "quant", "fused", "lora", "copy", "layers", "stack"], default="all",
+    ap.add_argument("--only", choices=["all", "roundtrip", "quant", "fused", "mlp", "lora", "copy", "layers", "stack"], default="all",
                     help="restrict the run to one part (for profiler runs)")
+    ap.add_argument("--pmc-summary", default="", metavar="DIR",
+                    help="no GPU work: turn the rocprofv3 counter CSVs under DIR into profiles/quant_pack_q4_config2_hbm_traffic.json")
     ap.add_argument("--layer-case", default="", help="with --only layers: run only the cases whose name contains this")
     ap.add_argument("--layer-arm", choices=["both", "plain", "compressed"], default="both",
                     help="with --only layers: run only one arm (for profiler runs)")
@@ -133,7 +194,9 @@ def bench_layers(torch, dev, only_case="", arm="both"):
         with torch.autograd.graph.saved_tensors_hooks(pack, lambda v: v):
             y = fn()                                  # what the forward keeps alive for backward
         saved = sum(seen.values())
+        t.x.grad = None
         y.backward(t.grad)
+        result = (y.detach(), t.x.grad.clone())
         for _ in range(warmup):
             fn().backward(t.grad)
         torch.cuda.synchronize()
@@ -143,7 +206,18 @@ def bench_layers(torch, dev, only_case="", arm="both"):
             fn().backward(t.grad)
         e1.record()
         torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / steps, saved
+        return e0.elapsed_time(e1) / steps, saved, result
+
+    def agreement(got, want, q=8):
+        """A wrong but fast layer must not post a number: forward output (never compressed) and the
+        input gradient (carries the codes' quantisation error) against the uncompressed autograd arm."""
+        (y, gx), (y0, gx0) = got, want
+        rel = ((y.float() - y0.float()).abs().max() / y0.float().abs().max()).item()
+        cos = F.cosine_similarity(gx.float().flatten(), gx0.float().flatten(), dim=0).item()
+        assert rel <= 2e-2, f"layer output differs from the uncompressed layer: max rel err {rel:.2e}"
+        floor = 0.4 if q == 2 else 0.8           # 2-bit codes: a quarter of a channel's range per step
+        assert cos >= floor, f"input gradient differs from the uncompressed layer: cosine {cos:.4f} (q_bit {q})"
+        return {"out_max_rel_err": rel, "grad_x_cos": cos}
 
     cfg = lambda lt, q: SimpleNamespace(use_hyclora=True, layer_type=lt, iteration_threshold=2,
                                         softmax_outlier_ratio=0.05, layernorm_outlier_ratio=0.005, q_bit=q)
@@ -159,15 +233,17 @@ def bench_layers(torch, dev, only_case="", arm="both"):
             continue
         t = make(**dims)
         mask = None if sdpa else torch.full((t.S, t.S), float("-inf"), device=dev).triu(1).to(BF16)[None, None]
-        entry, saved_p = {}, 0
+        entry, saved_p, plain = {}, 0, None
         if arm != "compressed":
-            ms_p, saved_p = measure(lambda: run_plain(t, mask, sdpa), t)
+            ms_p, saved_p, plain = measure(lambda: run_plain(t, mask, sdpa), t)
             entry["bf16_uncompressed"] = {"fwd_bwd_ms": ms_p, "saved_activation_MB": saved_p / 1e6}
             # the reference's own comparison arm: its default layer type, hand-written backward, nothing compressed
             base = llama_flash_attn.FusedLlamaLayerBaseline() if maker is None else maker(cfg("baseline", 0))
             base.set_hyclora_config(cfg("baseline", 0))
-            ms_b, saved_b = measure(lambda: run_fused(base, t, mask), t)
-            entry["baseline_layer"] = {"fwd_bwd_ms": ms_b, "saved_activation_MB": saved_b / 1e6}
+            ms_b, saved_b, res_b = measure(lambda: run_fused(base, t, mask), t)
+            entry["baseline_layer"] = {"fwd_bwd_ms": ms_b, "saved_activation_MB": saved_b / 1e6,
+                                       "check_against_uncompressed": agreement(res_b, plain)}
+            del res_b
             del base
         for q in (qbits if arm != "plain" else []):
             if maker is None:
@@ -177,12 +253,13 @@ def bench_layers(torch, dev, only_case="", arm="both"):
                 layer = maker(cfg(lt, q))
             for _ in range(3):                       # run past calibration so the steady state is timed
                 run_fused(layer, t, mask).backward(t.grad)
-            ms_f, saved_f = measure(lambda: run_fused(layer, t, mask), t)
+            ms_f, saved_f, res_f = measure(lambda: run_fused(layer, t, mask), t)
             entry[f"compressed_q{q}"] = {"fwd_bwd_ms": ms_f, "saved_activation_MB": saved_f / 1e6,
-                                         "saved_vs_bf16": saved_p / max(saved_f, 1) if saved_p else None}
-            del layer
+                                         "saved_vs_bf16": saved_p / max(saved_f, 1) if saved_p else None,
+                                         "check_against_uncompressed": agreement(res_f, plain, q) if plain else None}
+            del layer, res_f
         out[name] = entry
-        del t, mask
+        del t, mask, plain
         torch.cuda.empty_cache()
     return out
 
@@ -327,6 +404,9 @@ def bench_stack(torch, dev, n_layers=4, steps=5):
 
 def main():
     args = parse()
+    if args.pmc_summary:
+        pmc_summary(args.pmc_summary)
+        return
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this path has no cross-GPU work (got --gpus {args.gpus}); "
               "run with --gpus 1.", file=sys.stderr)
@@ -356,12 +436,23 @@ def main():
     def randn(*shape, scale=1.0):
         return (torch.randn(*shape, generator=gen, device=dev, dtype=torch.float32) * scale).to(BF16)
 
-    def timed(fn, steps, warmup):
+    def settle(run, min_ms=SETTLE_MS):
+        """Runs `run()` (a batch of the arm's own launches) until min_ms of wall time have passed."""
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        while min_ms > 0:
+            run()
+            torch.cuda.synchronize()
+            if (time.perf_counter() - t0) * 1e3 >= min_ms:
+                break
+
+    def timed(fn, steps, warmup, settle_ms=SETTLE_MS):
         """ms per call: `steps` calls between two events on the launching stream, bracketed
-        by synchronisation; the host clock around the same region is returned as well."""
+        by synchronisation; the host clock around the same region is returned as well.  Before the
+        timed region: `warmup` calls, then the arm's own calls for settle_ms more."""
         for i in range(warmup):
             fn(i)
-        torch.cuda.synchronize()
+        settle(lambda: [fn(i) for i in range(max(steps, 1))], settle_ms)
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         t0 = time.perf_counter()
         e0.record()
@@ -417,7 +508,7 @@ def main():
                 side.wait_stream(st)
         for _ in range(max(1, -(-warmup // steps))):
             graph.replay()
-        torch.cuda.synchronize()
+        settle(graph.replay)
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         t0 = time.perf_counter()
         e0.record()
@@ -457,13 +548,14 @@ def main():
     if args.only in ("all", "quant", "roundtrip"):
         ms_q, _ = timed(quant, K, W)
         ms_d, _ = timed(dequant, K, W)
+        traffic, traffic_note = measured_traffic()
         kernels["quant_pack_q4"] = {"ms": ms_q, "GBps": bytes_quant / ms_q / 1e6}
         kernels["unpack_dequant_q4"] = {"ms": ms_d, "GBps": bytes_quant / ms_d / 1e6}
         roofline = {"bound": "hbm", "kernel": "hyc::quant_pack_kernel<4,false,false>",
                     "achieved": bytes_quant / ms_q / 1e6, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                     "frac": bytes_quant / ms_q / 1e6 / HBM_PEAK_GBS,
                     "algorithmic_bytes_per_launch": bytes_quant, "launch_ms": ms_q,
-                    "traffic": MEASURED_TRAFFIC_BYTES}
+                    "traffic": traffic, "traffic_source": traffic_note}
     else:
         roofline = None
 
@@ -478,20 +570,47 @@ def main():
             sets.append(d)
         s1 = cf.get_statistics_only_quant(sets[0]["x1"], QB, 'per-channel')
         s2 = cf.get_statistics_only_quant(sets[0]["x2"], QB, 'per-channel')
-        saved = {}
+        # outputs are allocated once and the C ABI is called directly, so that both kernels can be
+        # timed as HIP-graph replays like every other kernel that runs shorter than an eager launch costs
+        bt = 0
+        for d in sets:
+            d["q1"] = torch.empty(B, M, N * QB // 8, device=dev, dtype=torch.uint8)
+            d["q2"] = torch.empty_like(d["q1"])
+            d["o"] = torch.empty(B, M, N, device=dev, dtype=BF16)
+            d["ob"], d["gg"], d["gu"] = torch.empty_like(d["o"]), torch.empty_like(d["o"]), torch.empty_like(d["o"])
+        s1v, s2v = s1.reshape(-1).contiguous(), s2.reshape(-1).contiguous()
 
-        def f_fwd(i):
+        def f_fwd(i, st=None):
             d = sets[i % NF]
-            saved[i % NF] = fuse_forward(d["xa1"], d["b1"], d["x1"], s1, d["xa2"], d["b2"], d["x2"], s2, QB)
+            rc = L.hyc_lora_silu_mul_fwd(d["xa1"].data_ptr(), d["b1"].data_ptr(), d["x1"].data_ptr(), s1v.data_ptr(),
+                                         d["xa2"].data_ptr(), d["b2"].data_ptr(), d["x2"].data_ptr(), s2v.data_ptr(),
+                                         d["q1"].data_ptr(), d["q2"].data_ptr(), d["o"].data_ptr(), T, N, R, QB, bt, st or stream)
+            assert rc == 0, _lib.error_string(rc)
 
-        def f_bwd(i):
+        def f_bwd(i, st=None):
             d = sets[i % NF]
-            q1, q2, _ = saved[i % NF]
-            fuse_backward(d["xa1"], d["b1"], q1, s1, d["xa2"], d["b2"], q2, s2, d["g"], QB)
+            rc = L.hyc_lora_silu_mul_bwd(d["xa1"].data_ptr(), d["b1"].data_ptr(), d["q1"].data_ptr(), s1v.data_ptr(),
+                                         d["xa2"].data_ptr(), d["b2"].data_ptr(), d["q2"].data_ptr(), s2v.data_ptr(),
+                                         d["g"].data_ptr(), d["ob"].data_ptr(), d["gg"].data_ptr(), d["gu"].data_ptr(),
+                                         T, N, R, QB, bt, st or stream)
+            assert rc == 0, _lib.error_string(rc)
 
-        Kf, Wf = max(K // 4, 10), max(W // 4, 3)
-        ms_ff, _ = timed(f_fwd, Kf, Wf)
-        ms_fb, _ = timed(f_bwd, Kf, Wf)
+        Kf, Wf = 30, 3
+        f_fwd(0)
+        f_bwd(0)
+        # a wrong but fast kernel must not post a number: the timed entry points against the wrappers'
+        # results and against the unfused fp32 composite
+        d0 = sets[0]
+        q1w, q2w, ow = fuse_forward(d0["xa1"], d0["b1"], d0["x1"], s1, d0["xa2"], d0["b2"], d0["x2"], s2, QB)
+        assert torch.equal(q1w, d0["q1"]) and torch.equal(q2w, d0["q2"]) and torch.equal(ow, d0["o"])
+        ref = F.silu(d0["x1"].float() + d0["xa1"].float() @ d0["b1"].float()) * (d0["x2"].float() + d0["xa2"].float() @ d0["b2"].float())
+        err = ((ow.float() - ref).abs().max() / ref.abs().max()).item()
+        assert err <= 1e-2, f"fused forward differs from the unfused composite: {err:.2e}"
+        del ref, q1w, q2w, ow
+        ms_ff, _ = timed_graph(f_fwd, Kf, Wf)
+        ms_fb, _ = timed_graph(f_bwd, Kf, Wf)
+        ms_ff_eager, _ = timed(f_fwd, Kf, Wf)
+        ms_fb_eager, _ = timed(f_bwd, Kf, Wf)
         bytes_ff = E * (6 + QB / 4) + 2 * T * R * 2 + 2 * R * N * 2 + 4 * N
         bytes_fb = E * (8 + QB / 4) + 2 * T * R * 2 + 2 * R * N * 2 + 4 * N
 
@@ -515,13 +634,109 @@ def main():
         ms_tf, _ = timed(t_fwd, Kf, Wf)
         ms_tfb, _ = timed(t_fwdbwd, Kf, Wf)
         fused = {"fwd_ms": ms_ff, "bwd_ms": ms_fb, "fwd_bwd_ms": ms_ff + ms_fb,
+                 "timing": f"{Kf} launches over {NF} rotating operand sets recorded in one HIP graph, replayed once, "
+                           f"after {SETTLE_MS:.0f} ms of the same replays",
+                 "eager_fwd_ms": ms_ff_eager, "eager_bwd_ms": ms_fb_eager,
                  "fwd_GBps": bytes_ff / ms_ff / 1e6, "bwd_GBps": bytes_fb / ms_fb / 1e6,
                  "fwd_frac_of_hbm_peak": bytes_ff / ms_ff / 1e6 / HBM_PEAK_GBS,
                  "bwd_frac_of_hbm_peak": bytes_fb / ms_fb / 1e6 / HBM_PEAK_GBS,
                  "torch_unfused_fwd_ms": ms_tf, "torch_unfused_fwd_bwd_ms": ms_tfb,
                  "speedup_vs_torch_unfused": ms_tfb / (ms_ff + ms_fb),
                  "note": "the fused kernels also produce/consume the 4-bit saved activations; the torch arm keeps bf16"}
-        del sets, saved
+        del sets
+
+    # ---- the whole MLP block of the layer: x_norm_2 -> gate/up -> LoRA-SiLU-product -> down, forward
+    # and backward with the frozen GEMMs, new kernels against unfused bf16 torch autograd --------------
+    mlp = None
+    if args.only in ("all", "mlp"):
+        import math
+
+        from hyclora_amd.models.compute_utils import lora_backward, lora_forward
+        from hyclora_amd.operators import lora_kernels
+        from hyclora_amd.operators.triton_fuse_lora_silu_hadamard_backward_kernels import triton_fuse_silu_backward
+        from hyclora_amd.operators.triton_fuse_lora_silu_hadamard_forward_kernels import triton_fuse_silu_forward
+
+        def adapter(out_f, in_f):
+            a = torch.empty(R, in_f, device=dev)
+            torch.nn.init.kaiming_uniform_(a, a=math.sqrt(5), generator=gen)      # as PEFT initialises lora_A
+            return a.to(BF16).requires_grad_(), randn(out_f, R, scale=1e-3).requires_grad_()
+        Wm = {"gate": randn(N, H, scale=0.02), "up": randn(N, H, scale=0.02), "down": randn(H, N, scale=0.02)}
+        Ad = {"gate": adapter(N, H), "up": adapter(N, H), "down": adapter(H, N)}
+        NX = 4
+        x_in = [rmsnorm_kernels.rmsnorm_forward(randn(B, M, H), torch.ones(H, device=dev, dtype=BF16), 1e-5)[0] for _ in range(NX)]
+        g_out = [randn(B, M, H) for _ in range(NX)]
+        with torch.no_grad():
+            s_x = cf.get_statistics_only_quant(x_in[0], QB, 'per-channel')
+            s_gate = cf.get_statistics_only_quant(x_in[0] @ Wm["gate"].t(), QB, 'per-channel')
+            s_up = cf.get_statistics_only_quant(x_in[0] @ Wm["up"].t(), QB, 'per-channel')
+        lora_t = {n: (Ad[n][0].detach().t(), Ad[n][1].detach().t()) for n in Ad}       # [in, R], [R, out] views
+
+        def new_fwd(x):
+            """What the full_fuse layer does between its second norm and its output
+            (models/llama/fused_llama_layer_intra_inter_full_fuse.py:218-251), statistics frozen."""
+            gate_main, up_main = x @ Wm["gate"].t(), x @ Wm["up"].t()
+            gate_xa, up_xa = x @ lora_t["gate"][0], x @ lora_t["up"][0]
+            q1, q2, had = triton_fuse_silu_forward(gate_xa, lora_t["gate"][1], gate_main, s_gate,
+                                                   up_xa, lora_t["up"][1], up_main, s_up, QB)
+            xq = cf.compression_quantization(x, s_x, QB)                  # the block's input is kept as codes
+            out, _, down_xa = lora_forward(Wm["down"], None, *lora_t["down"], None, had)
+            return out, (q1, q2, gate_xa, up_xa, xq, down_xa)
+
+        def new_bwd(saved, g):
+            """(…full_fuse.py:359-383): gradients of the block's input and of the six adapter matrices."""
+            q1, q2, gate_xa, up_xa, xq, down_xa = saved
+            a_d, b_d = lora_t["down"]
+            gb_down, g_mid = lora_kernels.lora_products(g, u=down_xa, v=b_d)
+            g_down = lora_kernels.lora_add(g @ Wm["down"], g_mid, a_d.mT, inplace=True)
+            had, g_gate, g_up = triton_fuse_silu_backward(gate_xa, lora_t["gate"][1], q1, s_gate,
+                                                          up_xa, lora_t["up"][1], q2, s_up, g_down, QB)
+            ga_down = lora_kernels.lora_products(had, u=g_mid)[0].t()
+            codes = (xq, s_x, None, QB)
+            ga_g, gb_g, gx = lora_backward(Wm["gate"], None, *lora_t["gate"], None, gate_xa, g_gate, x_codes=codes)
+            ga_u, gb_u, gx = lora_backward(Wm["up"], None, *lora_t["up"], None, up_xa, g_up, x_codes=codes, accumulate=gx)
+            return gx, (ga_g, gb_g, ga_u, gb_u, ga_down, gb_down)
+
+        def new_step(i):
+            with torch.no_grad():
+                out, saved = new_fwd(x_in[i % NX])
+                return out, new_bwd(saved, g_out[i % NX])
+
+        def torch_step(i, want=False):
+            x = x_in[i % NX].detach().requires_grad_()
+
+            def proj(n, inp):
+                return inp @ Wm[n].t() + (inp @ Ad[n][0].t()) @ Ad[n][1].t()
+            out = proj("down", F.silu(proj("gate", x)) * proj("up", x))
+            out.backward(g_out[i % NX])
+            res = (out.detach(), x.grad, [Ad[n][j].grad.clone() for n in ("gate", "up", "down") for j in (0, 1)]) if want else None
+            for n in Ad:
+                Ad[n][0].grad = Ad[n][1].grad = None
+            return res
+
+        # the two arms must agree before either is timed (the new arm keeps 4-bit activations: its
+        # gradients carry their quantisation error, its forward output does not)
+        out_n, (gx_n, gl_n) = new_step(0)
+        out_t, gx_t, gl_t = torch_step(0, want=True)
+        cosine = lambda a, b: F.cosine_similarity(a.float().flatten(), b.float().flatten(), dim=0).item()
+        chk = {"out_max_rel_err": ((out_n.float() - out_t.float()).abs().max() / out_t.float().abs().max()).item(),
+               "out_cos": cosine(out_n, out_t), "grad_x_cos": cosine(gx_n, gx_t),
+               "adapter_grad_cos_min": min(cosine(a, b)
+                                           for a, b in zip((g.t() for g in gl_n), gl_t))}
+        assert chk["out_max_rel_err"] <= 2e-2 and chk["out_cos"] >= 0.9999, f"MLP forward differs from torch: {chk}"
+        assert chk["grad_x_cos"] >= 0.95 and chk["adapter_grad_cos_min"] >= 0.9, f"MLP gradients differ from torch: {chk}"
+        del out_n, gx_n, gl_n, out_t, gx_t, gl_t
+        Km = 10
+        ms_new, _ = timed(new_step, Km, 2)
+        ms_new_f, _ = timed(lambda i: new_fwd(x_in[i % NX]), Km, 2)
+        ms_t, _ = timed(torch_step, Km, 2)
+        gemm_flop = 2 * T * H * N * 3 * 2                       # three frozen GEMMs forward, three for grad_x
+        mlp = {"mlp_fwd_bwd_ms": ms_new, "mlp_fwd_ms": ms_new_f, "torch_mlp_fwd_bwd_ms": ms_t,
+               "speedup_vs_torch_unfused": ms_t / ms_new,
+               "frozen_gemm_TFLOP": gemm_flop / 1e12, "frozen_gemm_floor_ms_at_2.5_PFLOPs": gemm_flop / 2.5e15 * 1e3,
+               "check_against_torch": chk,
+               "note": "both arms run the same six hipBLASLt GEMMs on the frozen weights; the new arm keeps gate/up/x as "
+                       "4-bit codes (saved activations 4x smaller), the torch arm keeps bf16 tensors for autograd"}
+        del Wm, Ad, x_in, g_out
 
     lora = None
     if args.only in ("all", "lora"):
@@ -727,6 +942,7 @@ def main():
         "roofline": roofline,
         "cpu_baseline": cpu,
         "fused": fused,
+        "mlp": mlp,
         "lora": lora,
         "kernels": kernels,
         "layers": layers,
