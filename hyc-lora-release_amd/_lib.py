@@ -41,6 +41,7 @@ _SIGNATURES = {
     "hyc_sparse_num_segments": (_L, [_L]),
     "hyc_sparse_count": (_I, [_P, _L, _P, _I, _P, _P, _P]),
     "hyc_sparse_write": (_I, [_P, _L, _P, _I, _P, _P, _P, _P]),
+    "hyc_sparse_write_bounded": (_I, [_P, _L, _P, _I, _P, _L, _P, _P, _P]),
     "hyc_sparse_segment_offsets": (_I, [_P, _L, _L, _P, _P]),
     "hyc_sparse_restore": (_I, [_P, _P, _P, _L, _P, _P]),
     "hyc_softmax_bwd": (_I, [_P, _P, _P, _L, _L, _P]),

@@ -231,14 +231,18 @@ void sparse_write_kernel(const uint16_t* __restrict__ a, int64_t n,
                                                                    const float* __restrict__ thr_p, int64_t nseg,
                                                                    const int64_t* __restrict__ offsets,
                                                                    int64_t* __restrict__ idx_out,
-                                                                   uint16_t* __restrict__ val_out, uint32_t cmp_mask) {
+                                                                   uint16_t* __restrict__ val_out, uint32_t cmp_mask,
+                                                                   int64_t capacity) {
+    // capacity: entries idx_out / val_out have room for.  Entries whose output position lies at or
+    // past it are not written (the caller sees from seg_offsets' last element that the list did not
+    // fit and writes it again into buffers of the right size).
     __shared__ uint32_t stage[kSegThreads / kWave][kStageEntries];
     const int lane = threadIdx.x & (kWave - 1);
     const int64_t seg = blockIdx.x * (int64_t)(kSegThreads / kWave) + (threadIdx.x >> 6);
     if (seg >= nseg) return;
     const float thr = rbf(*thr_p);
     const int64_t base = offsets[seg];
-    if (offsets[seg + 1] == base) return;          // nothing kept in this segment
+    if (offsets[seg + 1] == base || base >= capacity) return;     // nothing kept in this segment, or no room left
     // all of the segment's loads are issued before anything depends on them; the chunks stay packed
     // (4 registers each) so that enough waves fit on a SIMD
     u32x4 e[kSegSteps];
@@ -281,7 +285,8 @@ void sparse_write_kernel(const uint16_t* __restrict__ a, int64_t n,
         }
         __builtin_amdgcn_wave_barrier();               // LDS writes of this wave are visible to its lanes
         const int64_t first = seg * (int64_t)kSeg;
-        for (uint32_t k = lane; k < total; k += kWave) {
+        const uint32_t room = capacity - base < (int64_t)total ? (uint32_t)(capacity - base) : total;
+        for (uint32_t k = lane; k < room; k += kWave) {
             const uint32_t v = st[k];
             idx_out[base + k] = first + (v >> 16);
             val_out[base + k] = (uint16_t)v;
@@ -295,8 +300,10 @@ void sparse_write_kernel(const uint16_t* __restrict__ a, int64_t n,
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             if (mask[s] & (1u << j)) {
-                idx_out[w] = c * 8 + j;
-                val_out[w] = (uint16_t)chunk_elem(e[s], j);
+                if (w < capacity) {
+                    idx_out[w] = c * 8 + j;
+                    val_out[w] = (uint16_t)chunk_elem(e[s], j);
+                }
                 ++w;
             }
         }
@@ -613,17 +620,29 @@ extern "C" int hyc_sparse_count(const void* a, int64_t n, const float* threshold
     return check_launch();
 }
 
-extern "C" int hyc_sparse_write(const void* a, int64_t n, const float* threshold, int compare_abs,
-                                const int64_t* seg_offsets, int64_t* indices, void* values, void* stream) {
-    if (n < 0) return HYC_ERR_SHAPE;
+static int sparse_write_any(const void* a, int64_t n, const float* threshold, int compare_abs,
+                            const int64_t* seg_offsets, int64_t capacity, int64_t* indices, void* values, void* stream) {
+    if (n < 0 || capacity < 0) return HYC_ERR_SHAPE;
     const int64_t nseg = hyc_sparse_num_segments(n);
     if (nseg == 0) return HYC_OK;
     if (!a || !threshold || !seg_offsets || !indices || !values) return HYC_ERR_NULL;
     if (!aligned16(a)) return HYC_ERR_ALIGN;
     hipLaunchKernelGGL(sparse_write_kernel, dim3((unsigned)cdiv(nseg, 4)), dim3(kSegThreads), 0, (hipStream_t)stream,
                        (const uint16_t*)a, n, threshold, nseg, seg_offsets, indices, (uint16_t*)values,
-                       compare_abs ? 0x7fffu : 0xffffu);
+                       compare_abs ? 0x7fffu : 0xffffu, capacity);
     return check_launch();
+}
+
+extern "C" int hyc_sparse_write(const void* a, int64_t n, const float* threshold, int compare_abs,
+                                const int64_t* seg_offsets, int64_t* indices, void* values, void* stream) {
+    return sparse_write_any(a, n, threshold, compare_abs, seg_offsets, INT64_MAX, indices, values, stream);
+}
+
+extern "C" int hyc_sparse_write_bounded(const void* a, int64_t n, const float* threshold, int compare_abs,
+                                        const int64_t* seg_offsets, int64_t capacity, int64_t* indices, void* values,
+                                        void* stream) {
+    if (capacity == 0) return n < 0 ? HYC_ERR_SHAPE : HYC_OK;      // no room: nothing to write
+    return sparse_write_any(a, n, threshold, compare_abs, seg_offsets, capacity, indices, values, stream);
 }
 
 extern "C" int hyc_sparse_segment_offsets(const int64_t* indices, int64_t nnz, int64_t n, int64_t* seg_offsets,

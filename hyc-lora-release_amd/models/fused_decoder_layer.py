@@ -122,7 +122,7 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
                 w_down, b_down, qs_down, a_down, bb_down,
                 attention_mask, num_heads, head_dim, num_key_value_heads,
                 iteration, iteration_threshold, static_value, softmax_outlier_ratio,
-                layernorm_outlier_ratio, q_bit, spec):
+                layernorm_outlier_ratio, q_bit, spec, host_state=None):
         W = dict(q=(w_q, b_q, qs_q, a_q, bb_q), k=(w_k, b_k, qs_k, a_k, bb_k), v=(w_v, b_v, qs_v, a_v, bb_v),
                  o=(w_o, b_o, qs_o, a_o, bb_o), gate=(w_gate, b_gate, qs_gate, a_gate, bb_gate),
                  up=(w_up, b_up, qs_up, a_up, bb_up), down=(w_down, b_down, qs_down, a_down, bb_down))
@@ -232,6 +232,7 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             (quant_zp if spec.attention == "sdpa" else quant)("k_rope", k, "k")
             quant("v_rep", v, "v")
 
+        map_pending = None
         if spec.attention == "map":
             s = heads_matmul(q, k.transpose(-2, -1))
             del q, k
@@ -259,7 +260,18 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             else:
                 thr = get_statistics_softmax(a, softmax_outlier_ratio) if calib else sv['a']['outlier']
                 stats[("a", "outlier")] = thr
-                saved["a_idx"], saved["a_val"], saved["a_seg"] = compress_attention_map(a, thr, seg)
+                capacity = None if (calib or host_state is None) else host_state.get("map_capacity")
+                if capacity is None:
+                    # sizes the lists from nnz read back from the device, as to_sparse() does
+                    saved["a_idx"], saved["a_val"], saved["a_seg"] = compress_attention_map(a, thr, seg)
+                    if host_state is not None:
+                        _note_map_entries(host_state, saved["a_idx"].numel())
+                else:
+                    # frozen threshold: the lists get room for a little more than the recent steps
+                    # needed and nothing is read back here; whether they fitted is looked at when the
+                    # rest of the forward pass has been enqueued (the map is kept until then)
+                    saved["a_idx"], saved["a_val"], saved["a_seg"], count = compress_attention_map(a, thr, seg, capacity=capacity)
+                    map_pending = (a, thr, count, capacity)
             o = heads_matmul(a, v, out_hidden=True)
             del a, v
         else:
@@ -327,6 +339,13 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
         if whole:
             quant("hadamard", hadamard)
         del hadamard
+        if map_pending is not None:
+            a, thr, count, capacity = map_pending
+            nnz = count.value()                   # waits for the compaction only; the device still has the MLP block to run
+            if nnz > capacity:                    # did not fit: write the lists again at their exact size
+                saved["a_idx"], saved["a_val"], saved["a_seg"] = compress_attention_map(a, thr, saved["a_seg"])
+            _note_map_entries(host_state, nnz)
+            del a, map_pending
 
         ctx.names = list(saved.keys())
         ctx.save_for_backward(*saved.values(), cos, sin, norm_weight_1, norm_weight_2,
@@ -346,7 +365,7 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
     def backward(ctx, grad_output, *_unused):
         spec, q_bit = ctx.spec, ctx.q_bit
         if grad_output is None:
-            return (None,) * 53
+            return (None,) * 54
         tensors = list(ctx.saved_tensors)
         ns = len(ctx.names)
         S = dict(zip(ctx.names, tensors[:ns]))
@@ -537,7 +556,20 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
                 + lora_grads("q") + lora_grads("k") + lora_grads("v") + lora_grads("o")
                 + (grad_nw2, None)
                 + lora_grads("gate") + lora_grads("up") + lora_grads("down")
-                + (None,) * 11)
+                + (None,) * 12)
+
+
+MAP_HISTORY = 8            # steps whose kept-entry counts size the next step's attention-map lists
+MAP_HEADROOM = 1.0 / 16    # room beyond the largest of them
+
+
+def _note_map_entries(host_state, nnz):
+    """Records the kept-entry count of a step and sets the capacity of the next step's lists."""
+    history = host_state.setdefault("map_history", [])
+    history.append(int(nnz))
+    del history[:-MAP_HISTORY]
+    top = max(history)
+    host_state["map_capacity"] = top + int(top * MAP_HEADROOM) + 64
 
 
 def _weight_of(module):
@@ -558,6 +590,10 @@ class FusedDecoderLayer(torch.nn.Module):
         self.spec = LayerSpec(self.layer_type, self.attention, eps)
         self.iteration = 0
         self.static_value = self.spec.empty_static_value()
+        # host-side bookkeeping that is not part of the calibration state (not checkpointed): the
+        # recent kept-entry counts of the attention map, from which the next step's lists are sized
+        # without reading the count back first
+        self.host_state = {}
         self.use_hyclora = False
 
     def set_hyclora_config(self, hyclora_config):
@@ -626,7 +662,7 @@ class FusedDecoderLayer(torch.nn.Module):
             *five(down_proj_base, down_proj_lora_a, down_proj_lora_b),
             attention_mask, num_heads, head_dim, num_key_value_heads,
             self.iteration, self.iteration_threshold, self.static_value,
-            self.softmax_outlier_ratio, self.layernorm_outlier_ratio, self.q_bit, self.spec)
+            self.softmax_outlier_ratio, self.layernorm_outlier_ratio, self.q_bit, self.spec, self.host_state)
         y, stat_values = outs[0], outs[1:]
         if self.iteration < self.iteration_threshold:
             fresh = {}

@@ -308,12 +308,43 @@ def _threshold_tensor(outlier, device) -> torch.Tensor:
     return torch.tensor(float(outlier), device=device, dtype=torch.float32)
 
 
-def compress_attention_map(x: torch.Tensor, outlier, seg_offsets=None, compare_abs=False):
+_PINNED = {}          # device index -> [pinned int64 ring, next slot]
+_PINNED_SLOTS = 256
+
+
+class PendingCount:
+    """A device-side element count on its way to the host without a stream synchronisation: an
+    asynchronous copy into pinned memory followed by an event.  `value()` waits for that event only
+    (the device keeps executing whatever has been enqueued since)."""
+
+    def __init__(self, count: torch.Tensor):
+        ring = _PINNED.get(count.device.index)
+        if ring is None:
+            ring = _PINNED[count.device.index] = [torch.empty(_PINNED_SLOTS, dtype=torch.int64, pin_memory=True), 0]
+        slot = ring[1]
+        ring[1] = (slot + 1) % _PINNED_SLOTS          # a slot is read long before the ring comes round again
+        self._host = ring[0][slot:slot + 1]
+        self._host.copy_(count.reshape(1), non_blocking=True)
+        self._event = torch.cuda.Event()
+        self._event.record(torch.cuda.current_stream(count.device))
+
+    def value(self) -> int:
+        self._event.synchronize()
+        return int(self._host[0])
+
+
+def compress_attention_map(x: torch.Tensor, outlier, seg_offsets=None, compare_abs=False, capacity=None):
     """Kept entries of the flattened map: (indices int64 [nnz] ascending, values bf16 [nnz],
     seg_offsets int64 [nseg + 1]).  An entry is kept when x > outlier (compared in bf16, as
     torch does) and x != 0.  seg_offsets lets restore_attention_map skip the index search.
     `seg_offsets` may be passed in when the producer of x already counted (softmax_forward with a
-    threshold): the counting pass is skipped.  compare_abs: keep by magnitude, |x| > outlier."""
+    threshold): the counting pass is skipped.  compare_abs: keep by magnitude, |x| > outlier.
+
+    `capacity` (an int): no read-back of nnz.  The outputs are sized `capacity`, entries that do not
+    fit are not written, and a fourth result - a PendingCount - tells later how many entries there
+    were; the caller must check `pending.value() <= capacity` before the lists are consumed and call
+    again without `capacity` (passing the same seg_offsets) when they did not fit.  Entries past nnz
+    in the outputs are uninitialised; seg_offsets bounds what the restore kernels read."""
     _lib.require_gpu(x)
     if x.dtype != BF16:
         x = x.to(BF16)
@@ -333,6 +364,13 @@ def compress_attention_map(x: torch.Tensor, outlier, seg_offsets=None, compare_a
         offsets = torch.empty(nseg + 1, device=x.device, dtype=torch.int64)
         _lib.call("hyc_sparse_count", flat.data_ptr(), n, thr.data_ptr(), int(compare_abs), counts.data_ptr(),
                   offsets.data_ptr(), st)
+    if capacity is not None:
+        capacity = int(capacity)
+        idx = torch.empty(capacity, device=x.device, dtype=torch.int64)
+        val = torch.empty(capacity, device=x.device, dtype=BF16)
+        _lib.call("hyc_sparse_write_bounded", flat.data_ptr(), n, thr.data_ptr(), int(compare_abs), offsets.data_ptr(),
+                  capacity, idx.data_ptr(), val.data_ptr(), st)
+        return idx, val, offsets, PendingCount(offsets[-1:])
     nnz = int(offsets[-1].item())      # the one host sync; to_sparse() has the same one
     idx = torch.empty(nnz, device=x.device, dtype=torch.int64)
     val = torch.empty(nnz, device=x.device, dtype=BF16)

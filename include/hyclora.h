@@ -179,6 +179,11 @@ int hyc_hist_select(const uint32_t *hist, int64_t kth, float *threshold, void *s
  *                      entries kept before each segment, last element = total kept (nnz).
  *                      The caller reads nnz back to size the outputs, as to_sparse itself does.
  *   hyc_sparse_write   same a / threshold / seg_offsets; indices int64 [nnz], values bf16 [nnz].
+ *   hyc_sparse_write_bounded    the same into buffers with room for `capacity` entries, sized by
+ *                      the caller without knowing nnz (no read-back before the launch): entries at
+ *                      output positions >= capacity are not written.  The list is complete exactly
+ *                      when seg_offsets[nseg] <= capacity, which the caller checks when it suits it;
+ *                      a truncated list must not be handed to hyc_sparse_restore / hyc_softmax_bwd_restore.
  *   hyc_sparse_segment_offsets  rebuilds seg_offsets from an ascending index list (for sparse
  *                      tensors that did not come from hyc_sparse_count).
  *   hyc_sparse_restore out bf16 [n] (16-byte aligned): zeros, with values[i] at indices[i].
@@ -188,6 +193,9 @@ int hyc_sparse_count(const void *a, int64_t n, const float *threshold, int compa
                      int64_t *seg_offsets, void *stream);
 int hyc_sparse_write(const void *a, int64_t n, const float *threshold, int compare_abs,
                      const int64_t *seg_offsets, int64_t *indices, void *values, void *stream);
+int hyc_sparse_write_bounded(const void *a, int64_t n, const float *threshold, int compare_abs,
+                             const int64_t *seg_offsets, int64_t capacity, int64_t *indices, void *values,
+                             void *stream);
 int hyc_sparse_segment_offsets(const int64_t *indices, int64_t nnz, int64_t n, int64_t *seg_offsets,
                                void *stream);
 int hyc_sparse_restore(const int64_t *indices, const void *values, const int64_t *seg_offsets,

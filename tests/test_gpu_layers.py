@@ -355,6 +355,45 @@ def test_frozen_statistics_path_equals_calibrating_path(dev, layer_type, q_bit):
             assert torch.equal(a, b)
 
 
+def test_attention_map_lists_sized_without_a_read_back(dev):
+    """Once the threshold is frozen the layer sizes the attention map's index / value lists from the
+    kept-entry counts of its recent steps and checks the count of the current step only after the whole
+    forward pass has been enqueued.  The result must be what the exact-size path gives, bit for bit:
+    when the lists fit, and when they do not (capacity forced far too small: the layer writes them
+    again at the exact size)."""
+    import hyclora_amd  # noqa: F401
+    from hyclora_amd.models.llama import make_fused_llama_layer
+
+    def steps(tamper):
+        t = make_layer_inputs(dev, seed=41, S=512, hidden=256, heads=2, kv_heads=2, inter=512)
+        layer = make_fused_llama_layer(config("intra_inter_full_fuse", 4, sm_ratio=0.05, thr=1))
+        outs = []
+        for it in range(3):
+            if it >= 1:
+                tamper(layer)
+            y = run_fused(layer, t)
+            y.backward(t.grad)
+            outs.append((y.detach().clone(), t.x.grad.clone()))
+            t.x.grad = None
+        return layer, outs
+
+    def exact(layer):
+        layer.host_state.pop("map_capacity", None)          # no capacity: nnz is read back, lists sized exactly
+
+    def too_small(layer):
+        layer.host_state["map_capacity"] = 7
+
+    ref_layer, ref = steps(exact)
+    layer, got = steps(lambda layer: None)
+    nnz = ref_layer.host_state["map_history"][-1]
+    assert layer.host_state["map_history"] == [nnz] * 3 and nnz < layer.host_state["map_capacity"] <= nnz * 1.07 + 64
+    small_layer, small = steps(too_small)
+    assert small_layer.host_state["map_history"] == [nnz] * 3
+    for a, b, c in zip(ref, got, small):
+        assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+        assert torch.equal(a[0], c[0]) and torch.equal(a[1], c[1])
+
+
 def test_calibration_state_survives_a_checkpoint(dev, tmp_path):
     """Calibrate, save state_dict, load it into a fresh module (weights_only loader): the resumed
     layer is past calibration and reproduces the original's next step bit for bit."""

@@ -82,6 +82,39 @@ def test_compaction_and_restore(cf, dev, shape):
     assert same_bits(cf.decompression_softmax(ref_sp.to(dev)).cpu(), ref_sp.to_dense())
 
 
+@pytest.mark.parametrize("shape,ratio", [((2, 4, 128, 128), 0.05), ((1, 2, 100, 100), 0.5), ((1, 1, 8, 8), 0.5),
+                                         ((1, 2, 256, 256), 0.9)])         # the last: dense segments (direct stores)
+def test_compaction_into_preallocated_lists(cf, dev, shape, ratio):
+    """The compaction that sizes its outputs before the count is known: with room for everything the
+    lists' first nnz entries are the exact lists and the deferred count is nnz; with too little room
+    the first `capacity` entries are still right, nothing is written past them, and the count tells."""
+    import hyclora_amd  # noqa: F401
+    from hyclora_amd import _lib as L
+    a = attention_map(seed=3, shape=shape).to(dev)
+    thr = cf.get_statistics_softmax(a, ratio)
+    idx, val, seg = cf.compress_attention_map(a, thr)
+    nnz = idx.numel()
+    assert nnz > 8
+    for capacity in (nnz + 100, nnz, nnz - 1, nnz // 2, 1):
+        i2, v2, s2, count = cf.compress_attention_map(a, thr, capacity=capacity)
+        assert count.value() == nnz and torch.equal(s2, seg)
+        keep = min(capacity, nnz)
+        assert i2.numel() == capacity and torch.equal(i2[:keep], idx[:keep]) and torch.equal(v2[:keep], val[:keep])
+        # nothing past the capacity is touched: the C entry point on buffers with a guard zone
+        gi = torch.full((capacity + 64,), -7, device=dev, dtype=torch.int64)
+        gv = torch.full((capacity + 64,), 3.0, device=dev, dtype=BF16)
+        flat = a.reshape(-1)
+        L.call("hyc_sparse_write_bounded", flat.data_ptr(), flat.numel(), thr.data_ptr(), 0, seg.data_ptr(), capacity,
+               gi.data_ptr(), gv.data_ptr(), L.stream_of(a))
+        assert torch.equal(gi[:keep], idx[:keep]) and bool((gi[capacity:] == -7).all()) and bool((gv[capacity:] == 3.0).all())
+    # the counting pass of the producer is reused in the same way
+    i3, v3, s3, count = cf.compress_attention_map(a, thr, seg_offsets=seg, capacity=nnz + 5)
+    assert count.value() == nnz and torch.equal(i3[:nnz], idx) and torch.equal(v3[:nnz], val) and s3 is seg
+    # and the consumers read only what the segment offsets bound
+    back = cf.restore_attention_map(i3, v3, s3, a.shape)
+    assert torch.equal(back, cf.restore_attention_map(idx, val, seg, a.shape))
+
+
 def test_threshold_is_compared_in_bf16_and_zeros_are_dropped(cf, dev):
     a = torch.tensor([1.0078125, 1.0, 0.0, -0.0, 0.5, float("nan"), 1.015625, 2.0] * 8, dtype=BF16)
     thr = torch.tensor(1.0058, dtype=torch.float32)        # rounds to bf16 1.0078125
