@@ -26,7 +26,7 @@ class HycError(RuntimeError):
 
 
 # name -> (restype, argtypes)
-ABI_VERSION = 4          # hyc_abi_version() of the library these signatures describe
+ABI_VERSION = 5          # hyc_abi_version() of the library these signatures describe
 _P, _I, _L = c_void_p, c_int, c_int64
 _SIGNATURES = {
     "hyc_error_string": (c_char_p, [_I]),
@@ -50,6 +50,8 @@ _SIGNATURES = {
     "hyc_layernorm_bwd": (_I, [_P, _P, _P, _I, _P, _P, _P, _L, _L, _P]),
     "hyc_outlier_table": (_I, [_P, _L, _L, _P, _P]),
     "hyc_rmsnorm_fwd_compress": (_I, [_P, _P, _I, _P, _P, _L, _L, ctypes.c_float, _I, _P, _P, _P, _P, _P, _L, _P, _P]),
+    "hyc_rmsnorm_fwd_compress_lora": (_I, [_P, _P, _P, _P, _L, _L, ctypes.c_float, _I, _P, _P, _P, _P, _P, _L, _P,
+                                           _I, _P, _P, _P, _P]),
     "hyc_rope": (_I, [_P, _P, _P, _I, _L, _L, _L, _L, _L, _L, _L, _L, _L, _I, _P]),
     "hyc_softmax_fwd": (_I, [_P, _P, _P, _L, _L, ctypes.c_float, _L, _L, _L, _L, _P, _P, _P, _P]),
     "hyc_softmax_bwd_restore": (_I, [_P, _P, _P, _P, _P, _P, _L, _L, ctypes.c_float, _P]),

@@ -37,6 +37,26 @@ struct NormCompressArgs {
     float eps;
 };
 
+// LoRA-A down contraction out of the same pass (column-slab kernel only): xa = y @ A for up to four
+// blocks of 16 adapter rows, y being the bf16 output the kernel has just formed.  The layers compute
+// `x_norm @ lora_A^T` for q, k and v (gate and up) right after the norm
+// (models/utils/compute_utils.py:22 via fused_llama_layer_intra_inter_full_fuse.py:111-117, :218-226),
+// each a library GEMM that reads the [T, N] output again.
+constexpr int kXaBlocks = 4;
+// Rows per matrix-core tile: 16 (every row of the 16x16x16 form used) where the tiles of all waves fit
+// in LDS, i.e. up to 8 waves = 4096 columns - one workgroup per compute unit then - and 8 (rows 8..15 of
+// the form stay empty) for wider rows.  Halving the tile doubles the adapter bytes pulled from L2 per
+// row, which is what this phase is bound by (measured: ~10 TB/s of L2 hits).
+template <int MAXW> constexpr int kXaRowsFor = MAXW <= 8 ? 16 : 8;
+constexpr int kXaPitch = kWave * 8 + 8;      // bf16 elements per row of a wave's y tile in LDS (16 bytes of padding)
+struct XaArgs {
+    const uint16_t* w[kXaBlocks];    // block b: 16 consecutive rows of an adapter weight [R, N] (lora_A.weight), row-major
+    uint16_t* out[kXaBlocks];        // its 16 result columns: out[b][row * stride[b] + j]
+    int64_t stride[kXaBlocks];
+    int valid[kXaBlocks];            // how many of the 16 rows exist (a rank that is not a multiple of 16)
+    int nb;                          // blocks in use, 0 = no contraction
+};
+
 template <int QBIT>
 __device__ __forceinline__ void quantise_chunk(const float (&f)[8], const uint16_t* scale, int col, int chunk, bool active,
                                                uint8_t* qrow) {
@@ -167,14 +187,22 @@ static int compute_units() {
 
 // MAXW: the most waves a workgroup may have (8: rows up to 4096 columns, 16: up to 8192).  Four
 // waves per SIMD either way: two workgroups of 8 waves or one of 16 on a compute unit.
-template <int QBIT, bool W32, int MAXW>
-__global__ __launch_bounds__(MAXW * kWave) __attribute__((amdgpu_waves_per_eu(4)))
-void rmsnorm_fwd_compress_slab_kernel(const NormCompressArgs a, int rows_per_group) {
+// XA: also the LoRA-A contraction described at XaArgs.  A wave keeps the bf16 output of its slab for
+// a tile of kXaRows rows in LDS, turns it into the A operand of v_mfma_f32_16x16x16_bf16 (K runs over
+// the slab's 512 columns, 32 per step: lane (i, g) supplies columns 32m + 8g .. +7 of row i as two
+// operands, and the adapter rows are loaded in the same column order, 16 bytes a lane, so that two
+// consecutive steps consume whole 128-byte lines), and leaves a [rows x 16] fp32 partial per block;
+// the slabs' partials are added in column order through LDS and rounded once.
+template <int QBIT, bool W32, int MAXW, bool XA>
+__global__ __launch_bounds__(MAXW * kWave) __attribute__((amdgpu_waves_per_eu(XA && MAXW <= 8 ? 2 : 4)))
+void rmsnorm_fwd_compress_slab_kernel(const NormCompressArgs a, const XaArgs xa, int rows_per_group) {
     constexpr int G = kSlabRows;
-    extern __shared__ float slab_part[];                // [2][G][waves][64]
+    constexpr int kXaRows = kXaRowsFor<MAXW>;
+    extern __shared__ float slab_part[];                // [2][G][waves][64], then (XA) [waves][kXaRows][kXaPitch] bf16
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int nw = blockDim.x >> 6;
+    uint16_t* const ytile = reinterpret_cast<uint16_t*>(slab_part + 2 * G * nw * kWave) + wave * (kXaRows * kXaPitch);
     const int chunk = wave * kWave + lane;
     const int col = chunk * 8;
     const int N = a.N;
@@ -209,7 +237,7 @@ void rmsnorm_fwd_compress_slab_kernel(const NormCompressArgs a, int rows_per_gro
 #pragma unroll
         for (int g = 0; g < G; ++g) xv[g] = ld16_nt(a.x + (r + g) * N + col);
     };
-    auto step = [&](int64_t r, int buf, auto ahead_tag, auto fast_tag) __attribute__((always_inline)) {
+    auto step = [&](int64_t r, int buf, int tile_row, auto ahead_tag, auto fast_tag) __attribute__((always_inline)) {
         constexpr bool AHEAD = decltype(ahead_tag)::value;
         constexpr bool FAST = decltype(fast_tag)::value;
         float f[G][8];
@@ -247,6 +275,7 @@ void rmsnorm_fwd_compress_slab_kernel(const NormCompressArgs a, int rows_per_gro
             for (int j = 0; j < 8; ++j) o[j] = (f[g][j] * rstd[g]) * wf[j];
             const u32x4 yv = pack8(o);
             st16_nt(a.y + row * N + col, yv);
+            if constexpr (XA) *reinterpret_cast<u32x4*>(ytile + (tile_row + g) * kXaPitch + 8 * lane) = yv;
             uint32_t lo, hi;
             if (a.q_y) {
                 float fy[8];
@@ -271,19 +300,93 @@ void rmsnorm_fwd_compress_slab_kernel(const NormCompressArgs a, int rows_per_gro
             __builtin_amdgcn_sched_barrier(0);
         }
     };
+    // The LoRA-A contraction of the tile rows [t0, t0 + nrows) that the steps above left in LDS.
+    auto contract = [&](int64_t t0, int nrows) __attribute__((always_inline)) {
+        const int i = lane & 15, g = lane >> 4;
+        f32x4 acc[kXaBlocks];
+        const uint16_t* wp[kXaBlocks];
+#pragma unroll
+        for (int b = 0; b < kXaBlocks; ++b) {
+            acc[b] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            const bool have = b < xa.nb && i < xa.valid[b];
+            wp[b] = have ? xa.w[b] + (int64_t)i * N + wave * (kWave * 8) + 8 * g : nullptr;
+        }
+        const uint16_t* yrow = ytile + i * kXaPitch + 8 * g;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");          // the tile rows written by this wave's other lanes
+        __builtin_amdgcn_wave_barrier();
+        u32x4 bw[2][kXaBlocks];
+        auto fetch = [&](int m, u32x4 (&dst)[kXaBlocks]) __attribute__((always_inline)) {
+#pragma unroll
+            for (int b = 0; b < kXaBlocks; ++b) {
+                dst[b] = u32x4{0, 0, 0, 0};
+                if (b < xa.nb && wp[b]) dst[b] = ld16(wp[b] + 32 * m);
+            }
+        };
+        fetch(0, bw[0]);
+#pragma unroll 2
+        for (int m = 0; m < kWave * 8 / 32; m += 2) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                if (m + h + 1 < kWave * 8 / 32) fetch(m + h + 1, bw[(h + 1) & 1]);
+                u32x4 av = {0, 0, 0, 0};
+                if (i < kXaRows) av = *reinterpret_cast<const u32x4*>(yrow + 32 * (m + h));
+                const s16x4 a0 = __builtin_bit_cast(s16x4, u32x2{av.x, av.y});
+                const s16x4 a1 = __builtin_bit_cast(s16x4, u32x2{av.z, av.w});
+#pragma unroll
+                for (int b = 0; b < kXaBlocks; ++b) {
+                    if (b < xa.nb) {
+                        const u32x4 w4 = bw[h & 1][b];
+                        acc[b] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a0, __builtin_bit_cast(s16x4, u32x2{w4.x, w4.y}), acc[b], 0, 0, 0);
+                        acc[b] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a1, __builtin_bit_cast(s16x4, u32x2{w4.z, w4.w}), acc[b], 0, 0, 0);
+                    }
+                }
+            }
+        }
+        // the slab's partial, rows x (16 per block), into this wave's own tile region (its reads of it
+        // are done: a wave's LDS operations complete in order)
+        float* part = reinterpret_cast<float*>(ytile);
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        if (g < kXaRows / 4) {
+#pragma unroll
+            for (int b = 0; b < kXaBlocks; ++b) {
+                if (b < xa.nb) {
+                    const float e[4] = {acc[b].x, acc[b].y, acc[b].z, acc[b].w};
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) part[(4 * g + v) * (16 * kXaBlocks) + 16 * b + i] = e[v];
+                }
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+        const float* all = reinterpret_cast<const float*>(reinterpret_cast<const uint16_t*>(slab_part + 2 * G * nw * kWave));
+        constexpr int kWaveFloats = kXaRows * kXaPitch / 2;             // a wave's tile region in floats
+        for (int o = threadIdx.x; o < kXaRows * 16 * kXaBlocks; o += blockDim.x) {
+            const int row = o / (16 * kXaBlocks), c = o % (16 * kXaBlocks), b = c >> 4, j = c & 15;
+            if (row < nrows && b < xa.nb && j < xa.valid[b]) {
+                float sum = 0.0f;
+                for (int w = 0; w < nw; ++w) sum += all[w * kWaveFloats + o];          // slabs in column order
+                xa.out[b][(t0 + row) * xa.stride[b] + j] = f_to_bf(sum);
+            }
+        }
+    };
     auto run = [&](auto fast_tag) __attribute__((always_inline)) {
         request(r0);
         int64_t r = r0;
         int buf = 0;
         if (r + G < r1) {
-            step(r, buf, std::true_type{}, fast_tag);
-            for (r += G, buf ^= 1; r + G < r1; r += G, buf ^= 1) step(r, buf, std::true_type{}, fast_tag);
+            step(r, buf, (int)(r - r0), std::true_type{}, fast_tag);
+            for (r += G, buf ^= 1; r + G < r1; r += G, buf ^= 1) step(r, buf, (int)(r - r0), std::true_type{}, fast_tag);
         }
-        step(r, buf, std::false_type{}, fast_tag);
+        step(r, buf, (int)(r - r0), std::false_type{}, fast_tag);
     };
     // every wave of the workgroup makes the same number of steps whichever branch it takes
     if (fast) run(std::true_type{});
     else run(std::false_type{});
+    // With the contraction a workgroup's strip is one tile (the launch sees to that), so this comes
+    // when nothing of the row loop is live any more: its registers are the contraction's.
+    if constexpr (XA) contract(r0, (int)(r1 - r0));
 }
 
 // ------------------------------------------------------------------------------------
@@ -485,9 +588,22 @@ __global__ void otable_mark_kernel(const int64_t* __restrict__ oidx, int k, int 
     }
 }
 
+static bool slab_shape(int64_t rows, int64_t N) {
+    return N % (kWave * 8) == 0 && N / (kWave * 8) <= 16 && rows % kSlabRows == 0;
+}
+
+// Launch with more dynamic LDS than the 64 KiB a kernel may use without asking.
+template <typename K>
+static void launch_slab(K kernel, dim3 grid, dim3 block, size_t lds, hipStream_t st, const NormCompressArgs& a,
+                        const XaArgs& xa, int rows_per_group) {
+    if (lds > 64 * 1024)
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    hipLaunchKernelGGL(kernel, grid, block, lds, st, a, xa, rows_per_group);
+}
+
 template <int QBIT, bool W32>
-static int launch_nc(const NormCompressArgs& a, hipStream_t st) {
-    if (g_slab_enabled && a.N % (kWave * 8) == 0 && a.N / (kWave * 8) <= 16 && a.rows % kSlabRows == 0) {
+static int launch_nc(const NormCompressArgs& a, const XaArgs& xa, hipStream_t st) {
+    if ((g_slab_enabled || xa.nb > 0) && slab_shape(a.rows, a.N)) {
         const int waves = a.N / (kWave * 8);
         // Strip height: all workgroups resident at once (16 waves per compute unit), each walking as
         // long a strip as that allows - the per-column constants are set up once per strip.
@@ -496,17 +612,27 @@ static int launch_nc(const NormCompressArgs& a, hipStream_t st) {
             const int64_t resident = (int64_t)compute_units() * (16 / (waves <= 8 ? waves : 16));
             rows_per_group = (int)(cdiv(cdiv(a.rows, resident), (int64_t)kSlabRows) * kSlabRows);
         }
+        if (xa.nb > 0) rows_per_group = waves <= 8 ? kXaRowsFor<8> : kXaRowsFor<16>;      // one matrix-core tile per workgroup
         const int64_t groups = cdiv(a.rows, (int64_t)rows_per_group);
         if (groups > INT32_MAX) return HYC_ERR_SHAPE;
-        const size_t lds = 2 * kSlabRows * waves * kWave * sizeof(float);
-        if (waves <= 8)
-            hipLaunchKernelGGL((rmsnorm_fwd_compress_slab_kernel<QBIT, W32, 8>), dim3((unsigned)groups), dim3(waves * kWave), lds,
-                               st, a, rows_per_group);
-        else
-            hipLaunchKernelGGL((rmsnorm_fwd_compress_slab_kernel<QBIT, W32, 16>), dim3((unsigned)groups), dim3(waves * kWave), lds,
-                               st, a, rows_per_group);
+        size_t lds = 2 * kSlabRows * waves * kWave * sizeof(float);
+        const dim3 grid((unsigned)groups), block(waves * kWave);
+        if (xa.nb > 0) {
+            if constexpr (W32) {
+                return HYC_ERR_ARG;                             // the contraction is built for bf16 norm weights only
+            } else {
+                lds += (size_t)waves * rows_per_group * kXaPitch * sizeof(uint16_t);
+                if (waves <= 8) launch_slab(rmsnorm_fwd_compress_slab_kernel<QBIT, false, 8, true>, grid, block, lds, st, a, xa, rows_per_group);
+                else launch_slab(rmsnorm_fwd_compress_slab_kernel<QBIT, false, 16, true>, grid, block, lds, st, a, xa, rows_per_group);
+            }
+        } else if (waves <= 8) {
+            launch_slab(rmsnorm_fwd_compress_slab_kernel<QBIT, W32, 8, false>, grid, block, lds, st, a, xa, rows_per_group);
+        } else {
+            launch_slab(rmsnorm_fwd_compress_slab_kernel<QBIT, W32, 16, false>, grid, block, lds, st, a, xa, rows_per_group);
+        }
         return check_launch();
     }
+    if (xa.nb > 0) return HYC_ERR_SHAPE;                        // only the column-slab kernel contracts
     const dim3 grid((unsigned)cdiv(a.rows, (int64_t)kNcWaves)), block(kNcThreads);
 #define HYC_NC(CH) \
     hipLaunchKernelGGL((rmsnorm_fwd_compress_kernel<CH, QBIT, W32>), grid, block, kNcWaves * CH * kWave * 16, st, a)
@@ -549,10 +675,10 @@ extern "C" int hyc_outlier_table(const int64_t* outlier_idx, int64_t k, int64_t 
     return check_launch();
 }
 
-extern "C" int hyc_rmsnorm_fwd_compress(const void* x, const void* weight, int weight_is_fp32, void* y, float* rstd,
-                                        int64_t rows, int64_t N, float eps, int q_bit, const void* scale_y, void* q_y,
-                                        const void* scale_x, void* q_x, const uint16_t* outlier_table, int64_t k,
-                                        void* x_outlier, void* stream) {
+static int norm_compress_any(const void* x, const void* weight, int weight_is_fp32, void* y, float* rstd,
+                             int64_t rows, int64_t N, float eps, int q_bit, const void* scale_y, void* q_y,
+                             const void* scale_x, void* q_x, const uint16_t* outlier_table, int64_t k,
+                             void* x_outlier, const XaArgs& xa, void* stream) {
     if (q_bit != 2 && q_bit != 4 && q_bit != 8) return HYC_ERR_QBIT;
     if (rows < 0 || N < 0 || N % 32 != 0 || N > 8192 || k < 0 || k > 65535) return HYC_ERR_SHAPE;
     if (rows == 0 || N == 0) return HYC_OK;
@@ -571,11 +697,48 @@ extern "C" int hyc_rmsnorm_fwd_compress(const void* x, const void* weight, int w
     a.otable = outlier_table; a.xo = (uint16_t*)x_outlier;
     a.rows = rows; a.N = (int)N; a.k = q_x ? (int)k : 0; a.eps = eps;
     hipStream_t st = (hipStream_t)stream;
-#define HYC_NC_Q(QB) (weight_is_fp32 ? launch_nc<QB, true>(a, st) : launch_nc<QB, false>(a, st))
+#define HYC_NC_Q(QB) (weight_is_fp32 ? launch_nc<QB, true>(a, xa, st) : launch_nc<QB, false>(a, xa, st))
     if (q_bit == 8) return HYC_NC_Q(8);
     if (q_bit == 4) return HYC_NC_Q(4);
     return HYC_NC_Q(2);
 #undef HYC_NC_Q
+}
+
+extern "C" int hyc_rmsnorm_fwd_compress(const void* x, const void* weight, int weight_is_fp32, void* y, float* rstd,
+                                        int64_t rows, int64_t N, float eps, int q_bit, const void* scale_y, void* q_y,
+                                        const void* scale_x, void* q_x, const uint16_t* outlier_table, int64_t k,
+                                        void* x_outlier, void* stream) {
+    XaArgs none{};
+    return norm_compress_any(x, weight, weight_is_fp32, y, rstd, rows, N, eps, q_bit, scale_y, q_y, scale_x, q_x,
+                             outlier_table, k, x_outlier, none, stream);
+}
+
+extern "C" int hyc_rmsnorm_fwd_compress_lora(const void* x, const void* weight, void* y, float* rstd, int64_t rows, int64_t N,
+                                             float eps, int q_bit, const void* scale_y, void* q_y, const void* scale_x,
+                                             void* q_x, const uint16_t* outlier_table, int64_t k, void* x_outlier,
+                                             int n_adapters, const void* const* adapter_weight, const int64_t* adapter_rank,
+                                             void* const* adapter_out, void* stream) {
+    if (n_adapters < 1 || n_adapters > kXaBlocks) return HYC_ERR_ARG;
+    if (!adapter_weight || !adapter_rank || !adapter_out) return HYC_ERR_NULL;
+    if (rows < 0 || N < 0) return HYC_ERR_SHAPE;
+    if (rows > 0 && N > 0 && !slab_shape(rows, N)) return HYC_ERR_SHAPE;
+    XaArgs xa{};
+    for (int g = 0; g < n_adapters; ++g) {
+        const int64_t R = adapter_rank[g];
+        if (R < 1 || R > 16 * kXaBlocks) return HYC_ERR_RANK;
+        if (!adapter_weight[g] || !adapter_out[g]) return HYC_ERR_NULL;
+        if (!aligned16(adapter_weight[g])) return HYC_ERR_ALIGN;
+        for (int64_t r0 = 0; r0 < R; r0 += 16) {               // an adapter of rank R occupies ceil(R / 16) blocks
+            if (xa.nb == kXaBlocks) return HYC_ERR_RANK;
+            xa.w[xa.nb] = (const uint16_t*)adapter_weight[g] + r0 * N;
+            xa.out[xa.nb] = (uint16_t*)adapter_out[g] + r0;
+            xa.stride[xa.nb] = R;
+            xa.valid[xa.nb] = (int)(R - r0 < 16 ? R - r0 : 16);
+            ++xa.nb;
+        }
+    }
+    return norm_compress_any(x, weight, 0, y, rstd, rows, N, eps, q_bit, scale_y, q_y, scale_x, q_x, outlier_table, k,
+                             x_outlier, xa, stream);
 }
 
 extern "C" int hyc_rmsnorm_bwd_codes(const void* dy, const void* q_x, const void* scale_x, const uint16_t* outlier_table,

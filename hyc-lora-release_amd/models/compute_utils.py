@@ -51,12 +51,13 @@ def dense_weight(w: torch.Tensor, quant_state):
     return dequantize_nf4(w, quant_state)
 
 
-def lora_forward(w, w_quant_state, w_lora_a, w_lora_b, b, x, residual=None):
+def lora_forward(w, w_quant_state, w_lora_a, w_lora_b, b, x, residual=None, x_lora_a=None):
     """-> (x @ W^T [+ b] + (x @ A) @ B, the frozen part alone, x @ A).  Reference :18-25.  The LoRA
     product and the add are one MFMA kernel over the frozen part (bf16 operands); other dtypes
     take the torch expression.  `residual` (not in the reference's signature) is added to the first
-    result in the same pass - the `x + o_final` that follows the projection in the layers."""
-    x_main, x_lora_a = lora_parts(w, w_quant_state, w_lora_a, b, x)
+    result in the same pass - the `x + o_final` that follows the projection in the layers.
+    `x_lora_a`: x @ A where the producer of x has already formed it."""
+    x_main, x_lora_a = lora_parts(w, w_quant_state, w_lora_a, b, x, x_lora_a)
     w_lora_b = w_lora_b.to(x_main.dtype)
     if lora_kernels.supported(x_main, x_lora_a, w_lora_b) and (residual is None or residual.dtype == x_main.dtype):
         return lora_kernels.lora_add(x_main, x_lora_a, w_lora_b, residual=residual), x_main, x_lora_a
@@ -64,14 +65,17 @@ def lora_forward(w, w_quant_state, w_lora_a, w_lora_b, b, x, residual=None):
     return (y if residual is None else residual + y), x_main, x_lora_a
 
 
-def lora_parts(w, w_quant_state, w_lora_a, b, x):
-    """-> (x @ W^T [+ b], x @ A): what lora_forward computes before the LoRA add."""
+def lora_parts(w, w_quant_state, w_lora_a, b, x, x_lora_a=None):
+    """-> (x @ W^T [+ b], x @ A): what lora_forward computes before the LoRA add.  x @ A is taken
+    from `x_lora_a` when the caller has it already (the fused norm kernel forms it)."""
     wt = dense_weight(w, w_quant_state).t()
     x = x.to(wt.dtype)
     x_main = x @ wt
     if b is not None:
         x_main = x_main + b.to(wt.dtype)
-    return x_main, x @ w_lora_a.to(wt.dtype)
+    if x_lora_a is None:
+        x_lora_a = x @ w_lora_a.to(wt.dtype)
+    return x_main, x_lora_a.to(wt.dtype)
 
 
 def lora_backward(w, w_quant_state, w_lora_a, w_lora_b, x, x_lora_a, grad_y, x_codes=None, accumulate=None):

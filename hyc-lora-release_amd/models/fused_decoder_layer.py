@@ -51,7 +51,7 @@ from ..operators.compress_function import (compress_attention_map, compression_p
                                            outlier_addition_fuse_decompression_dequantization,
                                            update_dict, validate_channel_list)
 from ..operators.rmsnorm_kernels import _backward as _rmsnorm_backward
-from ..operators.rmsnorm_kernels import (backward_from_codes_supported, rmsnorm_backward_from_codes, rmsnorm_forward,
+from ..operators.rmsnorm_kernels import (backward_from_codes_supported, lora_a_supported, rmsnorm_backward_from_codes, rmsnorm_forward,
                                          rmsnorm_forward_compress)
 from ..operators.silu_kernels import silu_backward, silu_hadamard, silu_hadamard_backward
 from ..operators.softmax_kernels import softmax_backward, softmax_backward_from_compressed, softmax_forward
@@ -133,9 +133,11 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
         raw = spec.mode == "baseline"                   # keep activations as they are
         whole = spec.mode in ("baseline", "intra")      # save whole activations, not the frozen-weight parts
 
+        xa_ready = {}           # projection name -> x @ A formed by the norm kernel that produced x
+
         def proj(name, inp, residual=None):
             w, b, qs, la, lb = W[name]
-            return lora_forward(w, qs, la, lb, b, inp, residual=residual)
+            return lora_forward(w, qs, la, lb, b, inp, residual=residual, x_lora_a=xa_ready.pop(name, None))
 
         def proj_quant(name, inp, zp=False, rotate=False):
             """Projection `name` of inp with the frozen part quantised on the way: -> (output, x @ A,
@@ -144,7 +146,7 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             embedding; the reference quantises `*_main`, adds and rotates in separate passes
             (…full_fuse.py:105-152)."""
             w, b, qs, la, lb = W[name]
-            main, xa = lora_parts(w, qs, la, b, inp)
+            main, xa = lora_parts(w, qs, la, b, inp, xa_ready.pop(name, None))
             lb = lb.to(main.dtype)
             if not (lora_kernels.supported(main, xa, lb) and main.dim() == 3):
                 (quant_zp if zp else quant)(name + "_main", main, name)
@@ -185,26 +187,38 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             stats[(name, "outlier_channel_index")], stats[(name, "scale")] = idx, s
             saved[name + "_o"], saved[name + "_q"], saved[name + "_s"], saved[name + "_idx"] = o, q, s, idx
 
-        def norm_block(xname, nname, t, w):
+        def norm_block(xname, nname, t, w, consumers):
             """RMSNorm of t plus the compressed copies of t (channel base) and of the output.  With
             frozen statistics all three come out of one pass over t; while calibrating the steps of
             the output depend on the output, so the separate operators run (returns done=False and
-            the caller quantises the output itself)."""
+            the caller quantises the output itself).  Where the kernel takes the shape, the same pass
+            also forms `output @ lora_A` for the projections `consumers` that read the output
+            (…full_fuse.py:111-117, :218-226 do one GEMM each): calibrating or not, so that both give
+            the same bits."""
             n = t.shape[-1]
+            adapters = [W[c][3] for c in consumers]
+            with_xa = lora_a_supported(t, w, adapters) and all(W[c][0].dtype == torch.bfloat16 or W[c][2] is not None
+                                                               for c in consumers)
             if raw or calib or t.dtype != torch.bfloat16 or t.dim() != 3 or n % 32 or n > 8192:
-                y, _, rstd, _, _ = rmsnorm_forward(t, w, spec.eps)
+                if with_xa:
+                    y, rstd, _, _, _, xas = rmsnorm_forward_compress(t, w, spec.eps, q_bit or 8, lora_a=adapters)
+                    xa_ready.update(zip(consumers, xas))
+                else:
+                    y, _, rstd, _, _ = rmsnorm_forward(t, w, spec.eps)
                 channel_base(xname, t)
                 return y, rstd, False
             idx, sx, sn = sv[xname]['outlier_channel_index'], sv[xname]['scale'], sv[nname]['scale']
-            y, rstd, q_y, q_x, x_out = rmsnorm_forward_compress(t, w, spec.eps, q_bit, scale_y=sn, scale_x=sx,
-                                                                outlier_idx=idx)
+            y, rstd, q_y, q_x, x_out, *xas = rmsnorm_forward_compress(t, w, spec.eps, q_bit, scale_y=sn, scale_x=sx,
+                                                                      outlier_idx=idx, lora_a=adapters if with_xa else None)
+            if with_xa:
+                xa_ready.update(zip(consumers, xas[0]))
             stats[(xname, "outlier_channel_index")], stats[(xname, "scale")], stats[(nname, "scale")] = idx, sx, sn
             saved[xname + "_o"], saved[xname + "_q"], saved[xname + "_s"], saved[xname + "_idx"] = x_out, q_x, sx, idx
             saved[nname + "_q"], saved[nname + "_s"] = q_y, sn
             return y, rstd, True
 
         # ---- attention block -------------------------------------------------------------------
-        x_norm_1, saved["rstd_1"], norm_1_done = norm_block("x", "x_norm_1", x, norm_weight_1)
+        x_norm_1, saved["rstd_1"], norm_1_done = norm_block("x", "x_norm_1", x, norm_weight_1, ("q", "k", "v"))
         q_rotated = k_rotated = False
         if whole:
             q, _, saved["q_lora_a"] = proj("q", x_norm_1)
@@ -297,15 +311,19 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
         del o
 
         # ---- MLP block ---------------------------------------------------------------------------
-        x_norm_2, saved["rstd_2"], norm_2_done = norm_block("x_medium", "x_norm_2", x_medium, norm_weight_2)
+        x_norm_2, saved["rstd_2"], norm_2_done = norm_block("x_medium", "x_norm_2", x_medium, norm_weight_2, ("gate", "up"))
         if spec.mode == "intra_inter_full_fuse":
             from .compute_utils import dense_weight
             wg, wu = dense_weight(w_gate, qs_gate).t(), dense_weight(w_up, qs_up).t()
             x_norm_2 = x_norm_2.to(wg.dtype)
             gate_main = x_norm_2 @ wg if b_gate is None else x_norm_2 @ wg + b_gate.to(wg.dtype)
             up_main = x_norm_2 @ wu if b_up is None else x_norm_2 @ wu + b_up.to(wu.dtype)
-            gate_lora_a = x_norm_2 @ a_gate.to(wg.dtype)
-            up_lora_a = x_norm_2 @ a_up.to(wu.dtype)
+            gate_lora_a = xa_ready.pop("gate", None)
+            up_lora_a = xa_ready.pop("up", None)
+            if gate_lora_a is None:
+                gate_lora_a = x_norm_2 @ a_gate.to(wg.dtype)
+            if up_lora_a is None:
+                up_lora_a = x_norm_2 @ a_up.to(wu.dtype)
             if calib:
                 gate_s = get_statistics_only_quant(gate_main, q_bit, 'per-channel')
                 up_s = get_statistics_only_quant(up_main, q_bit, 'per-channel')

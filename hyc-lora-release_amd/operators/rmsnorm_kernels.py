@@ -177,14 +177,51 @@ def outlier_table(outlier_idx, n, cached=False):
     return table
 
 
-def rmsnorm_forward_compress(x, weight, eps, q_bit, scale_y=None, scale_x=None, outlier_idx=None, table=None):
+MAX_LORA_BLOCKS = 4          # 16-row blocks of adapter weights the fused norm kernel contracts with
+
+
+def _adapter_weight(a):
+    """lora_A as the kernel reads it: bf16 [R, N] row-major.  The layers pass the `[N, R]` view
+    `lora_A.weight.T`, whose transpose is that weight as it lies in memory."""
+    if a.dim() != 2:
+        raise ValueError(f"a LoRA-A operand must be a matrix, got shape {tuple(a.shape)}")
+    w = a.t()
+    if w.dtype != torch.bfloat16:
+        w = w.to(torch.bfloat16)
+    if not w.is_contiguous() or w.data_ptr() % 16:
+        w = w.contiguous().clone() if w.is_contiguous() else w.contiguous()
+    return w
+
+
+def lora_a_supported(x, weight, lora_a):
+    """Whether rmsnorm_forward_compress(..., lora_a=lora_a) takes this case: bf16 [B, M, N] activations
+    whose rows are whole 512-column slabs (N <= 8192), an even row count, a bf16 norm weight and
+    adapters `[N, R]` whose ranks, rounded up to multiples of 16, add up to at most 64."""
+    if not (x.is_cuda and x.dtype == torch.bfloat16 and x.dim() == 3 and weight.dtype == torch.bfloat16):
+        return False
+    n = x.shape[-1]
+    if n % 512 or n > 8192 or x.numel() == 0 or (x.numel() // n) % 2:
+        return False
+    if not lora_a or any(a.dim() != 2 or a.shape[0] != n or not 1 <= a.shape[1] <= 64 or a.dtype != torch.bfloat16
+                         for a in lora_a):
+        return False
+    return sum(-(-a.shape[1] // 16) for a in lora_a) <= MAX_LORA_BLOCKS
+
+
+def rmsnorm_forward_compress(x, weight, eps, q_bit, scale_y=None, scale_x=None, outlier_idx=None, table=None, lora_a=None):
     """RMSNorm forward that also produces, from the same read of x, the packed codes of the
     normalised output (steps `scale_y`) and the channel-base compressed input (steps `scale_x`,
     outlier channels `outlier_idx`): what rmsnorm_forward + compression_pack_quant_base(y) +
     compression_pack_channel_base(x) produce with frozen statistics, bit for bit
     (fused_llama_layer_intra_inter_full_fuse.py:97-126).
 
-    -> (y, rstd, q_y or None, q_x or None, x_outlier or None)."""
+    -> (y, rstd, q_y or None, q_x or None, x_outlier or None).
+
+    lora_a: a list of LoRA-A operands `[N, R]` (the `lora_A.weight.T` views the layers pass around) of
+    the projections that consume y.  Then a sixth result is returned, the list of `y @ a` as
+    [B, M, R] bf16 - lora_forward's `x @ w_lora_a` (models/utils/compute_utils.py:22) for each of them,
+    formed while y is still on the chip instead of by one library GEMM each over y in memory
+    (see lora_a_supported for the shapes this takes)."""
     _lib.require_gpu(x, weight)
     if x.dtype != torch.bfloat16 or x.dim() != 3:
         raise NotImplementedError("rmsnorm_forward_compress takes bfloat16 [batch, seq, hidden] activations")
@@ -217,6 +254,19 @@ def rmsnorm_forward_compress(x, weight, eps, q_bit, scale_y=None, scale_x=None, 
         x_out = torch.empty((b, m, k), dtype=torch.bfloat16, device=dev)
         if k and table is None:
             table = outlier_table(outlier_idx, n, cached=True)
+    if lora_a is not None:
+        import ctypes
+        if not lora_a_supported(x, weight, lora_a):
+            raise NotImplementedError("rmsnorm_forward_compress(lora_a=...): see lora_a_supported for the shapes it takes")
+        ws = [_adapter_weight(a) for a in lora_a]
+        outs = [torch.empty((b, m, a.shape[1]), dtype=torch.bfloat16, device=dev) for a in lora_a]
+        g = len(ws)
+        _lib.call("hyc_rmsnorm_fwd_compress_lora", x.data_ptr(), w.data_ptr(), y.data_ptr(), rstd.data_ptr(), rows, n,
+                  float(eps), q_bit, _lib.ptr(scale_y), _lib.ptr(q_y), _lib.ptr(scale_x), _lib.ptr(q_x),
+                  _lib.ptr(table) if k else None, k, _lib.ptr(x_out) if k else None, g,
+                  (ctypes.c_void_p * g)(*[t.data_ptr() for t in ws]), (ctypes.c_int64 * g)(*[t.shape[0] for t in ws]),
+                  (ctypes.c_void_p * g)(*[t.data_ptr() for t in outs]), _lib.stream_of(x))
+        return y, rstd, q_y, q_x, x_out, outs
     _lib.call("hyc_rmsnorm_fwd_compress", x.data_ptr(), w.data_ptr(), w32, y.data_ptr(), rstd.data_ptr(), rows, n,
               float(eps), q_bit, _lib.ptr(scale_y), _lib.ptr(q_y), _lib.ptr(scale_x), _lib.ptr(q_x),
               _lib.ptr(table) if k else None, k, _lib.ptr(x_out) if k else None, _lib.stream_of(x))

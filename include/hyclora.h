@@ -377,6 +377,28 @@ int hyc_rmsnorm_fwd_compress(const void *x, const void *weight, int weight_is_fp
                              const void *scale_x, void *q_x, const uint16_t *outlier_table, int64_t k,
                              void *x_outlier, void *stream);
 
+/* hyc_rmsnorm_fwd_compress that also forms, from the normalised output while it is still on the chip,
+ * the LoRA-A down projections of up to four adapters that take this output as their input:
+ * adapter_out[g] = bf16( y @ adapter_weight[g]^T ), fp32 accumulation over the whole row, one rounding.
+ * Replaces `x_norm @ lora_A^T` of lora_forward for q, k and v (gate and up), each of which reads the
+ * [rows, N] output again (models/utils/compute_utils.py:22 as called from
+ * models/llama/fused_llama_layer_intra_inter_full_fuse.py:111-117, :218-226).
+ *   n_adapters 1..4; adapter_weight / adapter_rank / adapter_out are HOST arrays of that length:
+ *   adapter_weight[g]  bf16 [rank, N] row-major on the device (lora_A.weight as nn.Linear keeps it), 16-byte aligned;
+ *   adapter_rank[g]    1..64; the ranks, each rounded up to a multiple of 16, may add up to 64 at most
+ *                      (HYC_ERR_RANK otherwise);
+ *   adapter_out[g]     bf16 [rows, rank] contiguous on the device.
+ *   The norm weight is bf16.  q_y, q_x may be NULL (no compressed copy), as in hyc_rmsnorm_fwd_compress;
+ *   y, rstd and the codes are the same bits as from that call.
+ * Only for rows that are a whole number of 512-column slabs (N % 512 == 0, N <= 8192) and an even
+ * number of rows: HYC_ERR_SHAPE otherwise (callers then use a library GEMM on y).
+ */
+int hyc_rmsnorm_fwd_compress_lora(const void *x, const void *weight, void *y, float *rstd, int64_t rows, int64_t N,
+                                  float eps, int q_bit, const void *scale_y, void *q_y, const void *scale_x,
+                                  void *q_x, const uint16_t *outlier_table, int64_t k, void *x_outlier,
+                                  int n_adapters, const void *const *adapter_weight, const int64_t *adapter_rank,
+                                  void *const *adapter_out, void *stream);
+
 /* ---------------------------------------------------------------------------------------
  * Rotary position embedding, in place: for every (b, s, h) the head x[b,s,h,:] = (x1 | x2) becomes
  * (x1*cos[s] - x2*sin[s] | x2*cos[s] + x1*sin[s]); backward != 0 uses -sin.

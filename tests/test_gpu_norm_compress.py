@@ -158,3 +158,59 @@ def test_outlier_table_and_errors(ops, dev):
         ops.norm.rmsnorm_forward_compress(x, w, 1e-5, 3, scale_y=torch.ones(64, device=dev, dtype=BF16))
     with pytest.raises(ValueError):
         ops.norm.rmsnorm_forward_compress(x, w, 1e-5, 4, scale_y=torch.ones(32, device=dev, dtype=BF16))
+
+
+@pytest.mark.parametrize("shape", [(2, 34, 4096), (1, 8, 512), (4, 1, 1024), (1, 20, 5120), (1, 12, 8192), (2, 513, 2048)])
+@pytest.mark.parametrize("ranks", [(16, 16, 16), (16, 16), (8,), (64,), (32, 4), (12, 16, 16, 16)])
+def test_lora_a_contraction_in_the_norm_pass(ops, dev, shape, ranks):
+    """y @ lora_A^T for every adapter fed by the norm's output, formed inside the norm kernel
+    (compute_utils.py:22 via ...full_fuse.py:111-117, :218-226): against the float64 product of the
+    kernel's own y rounded once (the oracle's lora_products: >= 99 % of the values the same bits, all
+    within tolerance), with every other output of the call unchanged bit for bit; row counts that do
+    not fill the last 8-row tile, ranks that do not fill a 16-row block, 1 to 16 waves per workgroup."""
+    q_bit = 4
+    x, _ = activation_with_outlier_channels(seed=shape[1] + len(ranks), shape=shape, frac=0.01)
+    g = torch.Generator().manual_seed(7)
+    n = shape[-1]
+    w = (1 + 0.1 * torch.randn(n, generator=g)).to(BF16)
+    weights = [(torch.randn(r, n, generator=g) / n ** 0.5).to(BF16).to(dev) for r in ranks]     # lora_A.weight: [R, N]
+    views = [a.t() for a in weights]                                                             # what the layers pass: [N, R]
+    xd, wd = x.to(dev), w.to(dev)
+    idx, s_x = ops.cf.get_statistics_channel_base(xd, 0.01, q_bit, 'per-channel')
+    y_ref, _, _, _, _ = ops.norm.rmsnorm_forward(xd, wd, 1e-5)
+    s_y = ops.cf.get_statistics_only_quant(y_ref, q_bit, 'per-channel')
+    assert ops.norm.lora_a_supported(xd, wd, views)
+    base = ops.norm.rmsnorm_forward_compress(xd, wd, 1e-5, q_bit, scale_y=s_y, scale_x=s_x, outlier_idx=idx)
+    got = ops.norm.rmsnorm_forward_compress(xd, wd, 1e-5, q_bit, scale_y=s_y, scale_x=s_x, outlier_idx=idx, lora_a=views)
+    for a, b in zip(base, got[:5]):
+        assert torch.equal(a, b), "an output of the norm changes when the contraction is switched on"
+    plain = ops.norm.rmsnorm_forward_compress(xd, wd, 1e-5, q_bit, lora_a=views)                 # no compressed copies
+    assert torch.equal(plain[0], base[0]) and torch.equal(plain[1], base[1]) and plain[2] is None and plain[3] is None
+    y = got[0].cpu()
+    for r, a, xa, xa2 in zip(ranks, weights, got[5], plain[5]):
+        assert xa.shape == (*shape[:2], r) and xa.dtype == BF16 and xa.is_contiguous()
+        assert torch.equal(xa, xa2)
+        _, want = O.lora_products(y, v=a.cpu())
+        assert_close_bf16(xa, want, what=f"rank {r} x@A vs float64 product")
+        same = (xa.cpu().view(torch.int16) == want.view(torch.int16)).float().mean().item()
+        assert same >= 0.99, f"rank {r}: only {same:.4f} of the values are the same bits as the float64 product"
+        assert_close_bf16(xa, got[0] @ a.t(), what=f"rank {r} x@A vs the library GEMM")
+    # repeated calls give the same bits (fixed summation order, no atomics)
+    again = ops.norm.rmsnorm_forward_compress(xd, wd, 1e-5, q_bit, scale_y=s_y, scale_x=s_x, outlier_idx=idx, lora_a=views)
+    for xa, xb in zip(got[5], again[5]):
+        assert torch.equal(xa, xb)
+
+
+def test_lora_a_contraction_limits(ops, dev):
+    z = lambda *sh: torch.zeros(*sh, dtype=BF16, device=dev)
+    w = torch.ones(1024, dtype=BF16, device=dev)
+    ok = [z(1024, 16)]
+    assert ops.norm.lora_a_supported(z(2, 4, 1024), w, ok)
+    assert not ops.norm.lora_a_supported(z(2, 4, 1024), w.float(), ok)            # fp32 norm weight
+    assert not ops.norm.lora_a_supported(z(1, 3, 1024), w, ok)                     # odd row count
+    assert not ops.norm.lora_a_supported(z(2, 4, 1024 + 32), torch.ones(1056, dtype=BF16, device=dev), [z(1056, 16)])
+    assert not ops.norm.lora_a_supported(z(2, 4, 1024), w, [z(1024, 16)] * 5)      # five blocks
+    assert not ops.norm.lora_a_supported(z(2, 4, 1024), w, [z(1024, 48), z(1024, 32)])
+    assert not ops.norm.lora_a_supported(z(2, 4, 1024), w, [z(512, 16)])           # adapter of another width
+    with pytest.raises(NotImplementedError):
+        ops.norm.rmsnorm_forward_compress(z(1, 3, 1024), w, 1e-5, 4, lora_a=ok)
