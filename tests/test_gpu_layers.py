@@ -119,6 +119,8 @@ def config(layer_type, q_bit, sm_ratio=0.999, ln_ratio=0.005, thr=5):
 # batch element 0, no zero point) clips one-sided activations such as silu(gate) even at 8 bits.
 # Parity of the layer logic is checked tightly against the oracle layer below.
 COS_FLOOR = {8: 0.95, 4: 0.93, 2: 0.4}
+# (max |a-b| / max |b|, cosine) of a gradient of the fused layer against the oracle layer, per code width
+ORACLE_LAYER_BOUND = {8: (1.5e-2, 0.9999), 4: (2e-2, 0.9999), 2: (0.2, 0.999)}
 
 
 @pytest.mark.parametrize("layer_type", ["intra", "intra_inter", "intra_inter_full_fuse"])
@@ -204,14 +206,20 @@ def test_layer_matches_oracle_layer(dev, layer_type, q_bit, kv_heads):
     for n in ("q", "k", "v", "o", "gate", "up", "down"):
         expect += [G[(n, "A")].sum(0).t(), G[(n, "B")].sum(0).t()]
     names = ["x", "norm_w1", "norm_w2"] + [f"{n}.lora_{ab}" for n in ("q", "k", "v", "o", "gate", "up", "down") for ab in "AB"]
+    worst = (0.0, 1.0)
     for name, got, want in zip(names, grads, expect):
         if want is None:
             continue
         rel, cos = rel_err_and_cos(got, want)
-        # the two sides run the same GEMMs, but a recomputed bf16 value that differs in its last bit
-        # can flip a code, and one flipped 2-bit code is a quarter of the range
-        rel_tol = 0.2 if q_bit == 2 else 2e-2
-        assert rel <= rel_tol and cos >= 0.999, f"{layer_type} q{q_bit} kv{kv_heads} grad {name}: rel {rel:.2e} cos {cos:.5f}"
+        worst = (max(worst[0], rel), min(worst[1], cos))
+        # Both sides compress the same way, so nothing of this difference is quantisation error as such:
+        # it is kernel error (the operator tolerance, 1e-2 / 0.9999) amplified by the codes - the two
+        # sides accumulate their products in different orders, a recomputed bf16 value that differs in
+        # its last bit can flip a code, and a flipped code is 1/255, 1/15 or 1/3 of a channel's range.
+        # The quantisation error itself is what test_layer_matches_uncompressed_autograd bounds loosely.
+        rel_tol, cos_tol = ORACLE_LAYER_BOUND[q_bit]
+        assert rel <= rel_tol and cos >= cos_tol, f"{layer_type} q{q_bit} kv{kv_heads} grad {name}: rel {rel:.2e} cos {cos:.5f}"
+    print(f"{layer_type} q{q_bit} kv{kv_heads}: worst rel {worst[0]:.2e}, worst cos {worst[1]:.6f}")
 
 
 @pytest.mark.parametrize("layer_type", ["baseline", "intra", "intra_inter", "intra_inter_full_fuse"])
