@@ -546,15 +546,18 @@ def main():
                               "eager_ms_per_step": ms_eager, "eager_wall_ms_per_step": wall_eager,
                               "eager_GBps": bytes_round / (ms_eager * 1e-3) / 1e9}
     if args.only in ("all", "quant", "roundtrip"):
-        ms_q, _ = timed(quant, K, W)
-        ms_d, _ = timed(dequant, K, W)
+        # the single-kernel loops time at least 400 launches: with fewer, the start-up of the first launch
+        # into an empty queue (~10 us) is a visible share of the average
+        Kq = max(K, 400)
+        ms_q, _ = timed(quant, Kq, W)
+        ms_d, _ = timed(dequant, Kq, W)
         traffic, traffic_note = measured_traffic()
         kernels["quant_pack_q4"] = {"ms": ms_q, "GBps": bytes_quant / ms_q / 1e6}
         kernels["unpack_dequant_q4"] = {"ms": ms_d, "GBps": bytes_quant / ms_d / 1e6}
         roofline = {"bound": "hbm", "kernel": "hyc::quant_pack_kernel<4,false,false>",
                     "achieved": bytes_quant / ms_q / 1e6, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                     "frac": bytes_quant / ms_q / 1e6 / HBM_PEAK_GBS,
-                    "algorithmic_bytes_per_launch": bytes_quant, "launch_ms": ms_q,
+                    "algorithmic_bytes_per_launch": bytes_quant, "launch_ms": ms_q, "launches_timed": Kq,
                     "traffic": traffic, "traffic_source": traffic_note}
     else:
         roofline = None
@@ -821,42 +824,61 @@ def main():
 
     if args.only == "all":
         Kx, Wx = max(K // 4, 10), max(W // 4, 3)
+        Kg = 40
+
+        def tg(fn):
+            """ms per call of a wrapper that allocates and launches but never synchronises: Kg calls recorded
+            into one HIP graph (outputs come from the graph's private pool), replayed once.  These kernels
+            run 5-25 us, less than an eager call through the Python wrapper costs on the host."""
+            fn(0)
+            torch.cuda.synchronize()
+            return timed_graph(lambda i, st: fn(i), Kg, 3)[0]
         NH = 16                                   # 16 x 33.5 MB: past the 256 MiB last-level cache
         x_h = [randn(B, M, H) for _ in range(NH)]
         w_h = torch.ones(H, device=dev, dtype=BF16)
-        ms, _ = timed(lambda i: rmsnorm_kernels.rmsnorm_forward(x_h[i % NH], w_h, 1e-5), Kx, Wx)
+        ms = tg(lambda i: rmsnorm_kernels.rmsnorm_forward(x_h[i % NH], w_h, 1e-5))
         kernels["rmsnorm_fwd_4096"] = {"ms": ms, "GBps": T * H * 4 / ms / 1e6}
         y, mean, rstd, bs, nw = rmsnorm_kernels.rmsnorm_forward(x_h[0], w_h, 1e-5)
-        ms, _ = timed(lambda i: rmsnorm_kernels.rmsnorm_backward(x_h[(i + 1) % NH], x_h[i % NH], w_h, mean, rstd, True, 1e-5, nw, bs), Kx, Wx)
+        ms = tg(lambda i: rmsnorm_kernels.rmsnorm_backward(x_h[(i + 1) % NH], x_h[i % NH], w_h, mean, rstd, True, 1e-5, nw, bs))
         kernels["rmsnorm_bwd_4096"] = {"ms": ms, "GBps": T * H * 6 / ms / 1e6}
-        ms, _ = timed(lambda i: silu_kernels.silu_backward(xs[i % NB], xs[(i + 1) % NB]), Kx, Wx)
+        ms = tg(lambda i: silu_kernels.silu_backward(xs[i % NB], xs[(i + 1) % NB]))
         kernels["silu_bwd"] = {"ms": ms, "GBps": E * 6 / ms / 1e6}
         idx = torch.randperm(H, device=dev)[:20].contiguous()
         _, sc = cf.get_statistics_channel_base(x_h[0], 0.005, QB, 'per-channel')
-        ms, _ = timed(lambda i: cf.outlier_subtraction_fuse_compression_quantization(x_h[i % NH], sc, idx, QB), Kx, Wx)
+        ms = tg(lambda i: cf.outlier_subtraction_fuse_compression_quantization(x_h[i % NH], sc, idx, QB))
         kernels["quant_pack_q4_outlier_4096"] = {"ms": ms, "GBps": T * H * 2.5 / ms / 1e6}
         sy = cf.get_statistics_only_quant(y, QB, 'per-channel')
         tbl = rmsnorm_kernels.outlier_table(idx, H)
-        ms, _ = timed(lambda i: rmsnorm_kernels.rmsnorm_forward_compress(x_h[i % NH], w_h, 1e-5, QB, scale_y=sy, scale_x=sc,
-                                                                         outlier_idx=idx, table=tbl), Kx, Wx)
-        ms3, _ = timed(lambda i: (rmsnorm_kernels.rmsnorm_forward(x_h[i % NH], w_h, 1e-5),
-                                  cf.outlier_subtraction_fuse_compression_quantization(x_h[i % NH], sc, idx, QB),
-                                  cf.compression_quantization(x_h[(i + 1) % NH], sy, QB)), Kx, Wx)
+        ms = tg(lambda i: rmsnorm_kernels.rmsnorm_forward_compress(x_h[i % NH], w_h, 1e-5, QB, scale_y=sy, scale_x=sc,
+                                                                   outlier_idx=idx, table=tbl))
+        ms3 = tg(lambda i: (rmsnorm_kernels.rmsnorm_forward(x_h[i % NH], w_h, 1e-5),
+                            cf.outlier_subtraction_fuse_compression_quantization(x_h[i % NH], sc, idx, QB),
+                            cf.compression_quantization(x_h[(i + 1) % NH], sy, QB)))
         kernels["rmsnorm_fwd_compress_4096"] = {"ms": ms, "GBps": T * H * (4 + 2 * QB / 8) / ms / 1e6,
                                                 "three_separate_kernels_ms": ms3}
-        ms, _ = timed(lambda i: cf.get_statistics_channel_base(x_h[i % NH], 0.005, QB, 'per-channel'), Kx, Wx)
+        # the same pass that also forms x_norm @ lora_A^T for the three adapters fed by the norm (q, k, v),
+        # against the fused norm followed by one library GEMM per adapter
+        a_w = [randn(R, H, scale=H ** -0.5) for _ in range(3)]
+        a_v = [a.t() for a in a_w]
+        ms = tg(lambda i: rmsnorm_kernels.rmsnorm_forward_compress(x_h[i % NH], w_h, 1e-5, QB, scale_y=sy, scale_x=sc,
+                                                                   outlier_idx=idx, table=tbl, lora_a=a_v))
+        ms_lib = tg(lambda i: [x_h[i % NH] @ v for v in a_v])
+        kernels["rmsnorm_fwd_compress_lora3_4096"] = {"ms": ms, "GBps": T * H * (4 + 2 * QB / 8) / ms / 1e6,
+                                                      "three_library_gemms_ms": ms_lib,
+                                                      "norm_then_three_library_gemms_ms": kernels["rmsnorm_fwd_compress_4096"]["ms"] + ms_lib}
+        ms = tg(lambda i: cf.get_statistics_channel_base(x_h[i % NH], 0.005, QB, 'per-channel'))
         kernels["calibration_stats_4096"] = {"ms": ms}
         # norm backward straight from the channel-base compressed input, residual gradient added, against
         # restore + backward with the same add
         xo_h, qx_h = cf.outlier_subtraction_fuse_compression_quantization(x_h[0].clone(), sc, idx, QB)
-        ms, _ = timed(lambda i: rmsnorm_kernels.rmsnorm_backward_from_codes(x_h[i % NH], qx_h, sc, xo_h, idx, QB, w_h, rstd,
-                                                                            residual=x_h[(i + 1) % NH], table=tbl), Kx, Wx)
-        ms2, _ = timed(lambda i: rmsnorm_kernels._backward(
+        ms = tg(lambda i: rmsnorm_kernels.rmsnorm_backward_from_codes(x_h[i % NH], qx_h, sc, xo_h, idx, QB, w_h, rstd,
+                                                                      residual=x_h[(i + 1) % NH], table=tbl))
+        ms2 = tg(lambda i: rmsnorm_kernels._backward(
             x_h[i % NH], cf.outlier_addition_fuse_decompression_dequantization(qx_h, sc, xo_h, idx, QB), w_h, rstd,
-            want_dw=False, residual=x_h[(i + 1) % NH]), Kx, Wx)
+            want_dw=False, residual=x_h[(i + 1) % NH]))
         kernels["rmsnorm_bwd_from_codes_4096"] = {"ms": ms, "GBps": T * H * (6 + QB / 8) / ms / 1e6,
                                                   "restore_then_backward_ms": ms2}
-        ms, _ = timed(lambda i: silu_kernels.silu_hadamard_backward(xs[i % NB], xs[(i + 1) % NB], xs[(i + 2) % NB]), Kx, Wx)
+        ms = tg(lambda i: silu_kernels.silu_hadamard_backward(xs[i % NB], xs[(i + 1) % NB], xs[(i + 2) % NB]))
         kernels["silu_mul_bwd"] = {"ms": ms, "GBps": E * 10 / ms / 1e6}
         # attention map (configuration 3 shape): compaction, restore, softmax backward
         a = torch.softmax(torch.randn(4, 32, 1024, 1024, generator=gen, device=dev) * 0.707
