@@ -8,6 +8,11 @@ hyc_oracle.py (device-agnostic: runs wherever the input tensors live).  One devi
 the implementation under test: the input-norm outliers are restored with the input-norm channel list
 (the reference's intra_inter/full_fuse files pass the post-attention list, :484).
 
+The map-free variant (attention="flash") follows models/llama_flash_attn/fused_llama_layer_intra_inter.py:
+zero-point codes for q and k (:128-139), causal attention through the flash kernel with its row log-sum-exps
+kept (:156-180), and the kernel's backward formula applied to the rebuilt q, k, v and the dequantised output
+(:450-468) - restated here with dense fp32 matrices.
+
 Calibration is always "fresh" (iteration < threshold): statistics are computed from the tensors at hand.
 """
 import math
@@ -52,10 +57,44 @@ def _rope(x, cos, sin, sign=1.0):
     return torch.cat([x1 * c - x2 * s, x2 * c + x1 * s], dim=-1).to(x.dtype)
 
 
+def _flash_forward(q, k, v, scale):
+    """Causal attention as the flash kernels define it (llama_flash_attn/fused_llama_layer_intra_inter.py:156-180,
+    flash_attn 2.5.8 `_flash_attn_varlen_forward`, causal=True, no dropout): fp32 scores, row log-sum-exps kept,
+    output rounded once.  -> (o [B,H,S,D] in q's dtype, lse fp32 [B,H,S])."""
+    s = (q.float() @ k.float().transpose(-2, -1)) * scale
+    n = s.shape[-1]
+    s = s + torch.full((n, n), float("-inf"), device=s.device).triu(1)
+    lse = torch.logsumexp(s, dim=-1)
+    p = torch.exp(s - lse.unsqueeze(-1))
+    return (p @ v.float()).to(q.dtype), lse
+
+
+def _flash_backward(g_o, q, k, v, out, lse, scale):
+    """What `_flash_attn_varlen_backward` computes from the tensors it is GIVEN (…intra_inter.py:450-468: q, k, v
+    rebuilt from their codes and `out` dequantised, `softmax_lse` the one saved in forward): the probabilities are
+    recomputed from q, k and the saved log-sum-exps, the row term is sum(dO * out) of the given output.
+    -> (grad_q, grad_k, grad_v)."""
+    s = (q.float() @ k.float().transpose(-2, -1)) * scale
+    n = s.shape[-1]
+    s = s + torch.full((n, n), float("-inf"), device=s.device).triu(1)
+    p = torch.exp(s - lse.unsqueeze(-1))
+    gof = g_o.float()
+    d_p = gof @ v.float().transpose(-2, -1)
+    delta = (gof * out.float()).sum(dim=-1, keepdim=True)
+    d_s = p * (d_p - delta)
+    g_q = (d_s @ k.float()) * scale
+    g_k = (d_s.transpose(-2, -1) @ q.float()) * scale
+    g_v = p.transpose(-2, -1) @ gof
+    return g_q.to(q.dtype), g_k.to(q.dtype), g_v.to(q.dtype)
+
+
 def layer_forward_backward(x, nw1, nw2, cos, sin, weights, mask, heads, kv_heads, grad_out, *, mode, q_bit,
-                           softmax_ratio, layernorm_ratio, eps=1e-5):
+                           softmax_ratio, layernorm_ratio, eps=1e-5, attention="map"):
     """weights: name -> (W [out,in], A [r,in], B [out,r]) for q,k,v,o,gate,up,down (plain tensors).
-    Returns (x_out, grads) with grads = {'x': .., (name,'A'): .., (name,'B'): ..}."""
+    Returns (x_out, grads) with grads = {'x': .., (name,'A'): .., (name,'B'): ..}.
+    attention="flash": the map-free variant (models/llama_flash_attn/fused_llama_layer_intra_inter.py): causal
+    attention without a saved map, q and k compressed with a zero point (:128-139), backward through the flash
+    kernel's formula on the rebuilt q, k, v and the dequantised output (:450-468); `mask` is not used."""
     hd = x.shape[-1] // heads
     n_rep = heads // kv_heads
     At = {n: w[1].t() for n, w in weights.items()}      # [in, r]
@@ -79,6 +118,13 @@ def layer_forward_backward(x, nw1, nw2, cos, sin, weights, mask, heads, kv_heads
         s = O.scale_only_quant(t, q_bit)
         return O.compress(t, s, q_bit), s
 
+    def cqz(t):                                          # compression_pack_quant_zp_base, calibrating
+        s, z = O.scale_zero_point(t, q_bit)
+        return O.compress(t, s, q_bit, z), s, z
+
+    flash = attention == "flash"
+    cqk = cqz if flash else cq                           # q and k: with a zero point in the map-free variant
+
     def ccb(t):                                          # compression_pack_channel_base, calibrating
         idx, s = O.channel_stats(t, layernorm_ratio, q_bit)
         xo, q = O.compress_channel_base(t, s, idx, q_bit)
@@ -92,21 +138,25 @@ def layer_forward_backward(x, nw1, nw2, cos, sin, weights, mask, heads, kv_heads
     v, v_main, v_xa = lora_fwd("v", xn1)
     xn1_sv = cq(xn1)
     if mode != "intra":
-        q_sv, k_sv, v_sv = cq(q_main), cq(k_main), cq(v_main)
+        q_sv, k_sv, v_sv = cqk(q_main), cqk(k_main), cq(v_main)
     q, k, v = _heads(q, heads), _heads(k, kv_heads), _heads(v, kv_heads)
     q = _rope(q.transpose(1, 2), cos, sin).transpose(1, 2)
     k = _rope(k.transpose(1, 2), cos, sin).transpose(1, 2)
     k, v = _repeat(k, n_rep), _repeat(v, n_rep)
     if mode == "intra":
-        q_sv, k_sv, v_sv = cq(q), cq(k), cq(v)           # 4-D inputs are read as [B, S, H*D]
-    s = q @ k.transpose(-2, -1) / math.sqrt(hd)
-    if mask is not None:
-        s = s + mask
-    a = torch.softmax(s, dim=-1, dtype=v.dtype)
-    thr = O.softmax_threshold(a, softmax_ratio)
-    a_idx, a_val = O.softmax_compress(a, thr)
-    a_shape = a.shape
-    o = _hidden(a @ v)
+        q_sv, k_sv, v_sv = cqk(q), cqk(k), cq(v)         # 4-D inputs are read as [B, S, H*D]
+    if flash:
+        o, lse = _flash_forward(q, k, v, 1.0 / math.sqrt(hd))
+        o = _hidden(o)
+    else:
+        s = q @ k.transpose(-2, -1) / math.sqrt(hd)
+        if mask is not None:
+            s = s + mask
+        a = torch.softmax(s, dim=-1, dtype=v.dtype)
+        thr = O.softmax_threshold(a, softmax_ratio)
+        a_idx, a_val = O.softmax_compress(a, thr)
+        a_shape = a.shape
+        o = _hidden(a @ v)
     o_final, _, o_xa = lora_fwd("o", o)
     o_sv = cq(o)
     xm = x + o_final
@@ -164,23 +214,30 @@ def layer_forward_backward(x, nw1, nw2, cos, sin, weights, mask, heads, kv_heads
     xm_r = O.decompress_channel_base(xm_sv[1], xm_sv[3], xm_sv[0], xm_sv[2], q_bit)
     g_norm2, G["nw2"] = O.rmsnorm_bwd(g_gate_up, xm_r, nw2, rstd2)
     g_medium = g_norm2 + go
-    G[("o", "A")], G[("o", "B")], g_o = lora_bwd("o", dq(o_sv), o_xa, g_medium)
+    o_r = dq(o_sv)
+    G[("o", "A")], G[("o", "B")], g_o = lora_bwd("o", o_r, o_xa, g_medium)
     g_o = _heads(g_o, heads)
-    a_r = O.softmax_restore(a_idx, a_val, a_shape)
+    dqk = (lambda sv, **kw: O.decompress(sv[0], sv[1], q_bit, sv[2], **kw).to(x.device)) if flash else dq
     if mode == "intra":
-        q_r, k_r, v_r = (dq(sv, is_head=True, num_heads=heads) for sv in (q_sv, k_sv, v_sv))
+        q_r, k_r = (dqk(sv, is_head=True, num_heads=heads) for sv in (q_sv, k_sv))
+        v_r = dq(v_sv, is_head=True, num_heads=heads)
     else:
         v_r = _repeat(_heads(dq(v_sv) + v_xa @ Bt["v"], kv_heads), n_rep)
-        q_r = _heads(dq(q_sv) + q_xa @ Bt["q"], heads)
+        q_r = _heads(dqk(q_sv) + q_xa @ Bt["q"], heads)
         q_r = _rope(q_r.transpose(1, 2), cos, sin).transpose(1, 2)
-        k_r = _heads(dq(k_sv) + k_xa @ Bt["k"], kv_heads)
+        k_r = _heads(dqk(k_sv) + k_xa @ Bt["k"], kv_heads)
         k_r = _repeat(_rope(k_r.transpose(1, 2), cos, sin).transpose(1, 2), n_rep)
-    g_v = a_r.transpose(-2, -1) @ g_o
-    g_a = g_o @ v_r.transpose(-2, -1)
-    g_v = _repeat_bwd(g_v, n_rep)
-    g_s = O.softmax_bwd(a_r, g_a) / math.sqrt(hd)
-    g_k = _repeat_bwd(g_s.transpose(-2, -1) @ q_r, n_rep)
-    g_q = g_s @ k_r
+    if flash:
+        g_q, g_k, g_v = _flash_backward(g_o, q_r, k_r, v_r, _heads(o_r, heads), lse, 1.0 / math.sqrt(hd))
+        g_k, g_v = _repeat_bwd(g_k, n_rep), _repeat_bwd(g_v, n_rep)
+    else:
+        a_r = O.softmax_restore(a_idx, a_val, a_shape)
+        g_v = a_r.transpose(-2, -1) @ g_o
+        g_a = g_o @ v_r.transpose(-2, -1)
+        g_v = _repeat_bwd(g_v, n_rep)
+        g_s = O.softmax_bwd(a_r, g_a) / math.sqrt(hd)
+        g_k = _repeat_bwd(g_s.transpose(-2, -1) @ q_r, n_rep)
+        g_q = g_s @ k_r
     g_q = _rope(g_q.transpose(1, 2), cos, sin, -1.0).transpose(1, 2)
     g_k = _rope(g_k.transpose(1, 2), cos, sin, -1.0).transpose(1, 2)
     g_q, g_k, g_v = _hidden(g_q), _hidden(g_k), _hidden(g_v)

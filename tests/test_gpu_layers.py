@@ -282,6 +282,50 @@ def test_sdpa_variant_and_norm_weight_grads(dev):
         assert layer.static_value['q']['zero_point'] is not None and 'a' not in layer.static_value
 
 
+@pytest.mark.parametrize("layer_type", ["intra", "intra_inter", "intra_inter_full_fuse"])
+@pytest.mark.parametrize("q_bit", [8, 4])
+@pytest.mark.parametrize("kv_heads", [4, 2])
+def test_map_free_layer_matches_oracle_layer(dev, layer_type, q_bit, kv_heads):
+    """The map-free variant (no saved attention map; q and k kept as zero-point codes; backward through the
+    flash kernel with the dequantised output, models/llama_flash_attn/fused_llama_layer_intra_inter.py:128-180,
+    :450-468) against the oracle's restatement of it with dense fp32 attention matrices: same compression on
+    both sides, so the bounds are those of test_layer_matches_oracle_layer."""
+    import hyclora_amd  # noqa: F401
+    from hyclora_amd.models import llama_flash_attn as lf
+    from oracle import layer_oracle
+    cls = {"intra": lf.FusedLlamaLayerIntra, "intra_inter": lf.FusedLlamaLayerIntraInter,
+           "intra_inter_full_fuse": lf.FusedLlamaLayerIntraInterFullFuse}[layer_type]
+    t = make_layer_inputs(dev, seed=61 + q_bit, S=128, kv_heads=kv_heads)
+    layer = cls()
+    layer.set_hyclora_config(config(layer_type, q_bit))
+    out = run_fused(layer, t, use_mask=False)
+    grads = grads_of(t, out)
+    weights = {n: tuple(m.weight.detach() for m in t.P[n]) for n in t.P}
+    with torch.no_grad():
+        ref_out, G = layer_oracle.layer_forward_backward(
+            t.x.detach(), t.nw1.detach(), t.nw2.detach(), t.cos, t.sin, weights, None, t.heads, t.kv_heads,
+            t.grad, mode=layer_type, q_bit=q_bit, softmax_ratio=0.0, layernorm_ratio=0.005, attention="flash")
+    rel, cos = rel_err_and_cos(out, ref_out)
+    assert rel <= 1e-2 and cos >= 0.9999, f"forward: rel {rel:.2e} cos {cos:.6f}"
+    expect = [G["x"], G["nw1"], G["nw2"]]
+    for n in ("q", "k", "v", "o", "gate", "up", "down"):
+        expect += [G[(n, "A")].sum(0).t(), G[(n, "B")].sum(0).t()]
+    names = ["x", "norm_w1", "norm_w2"] + [f"{n}.lora_{ab}" for n in ("q", "k", "v", "o", "gate", "up", "down") for ab in "AB"]
+    worst = (0.0, 1.0)
+    for name, got, want in zip(names, grads, expect):
+        assert got is not None and got.shape == want.shape, name        # this variant also trains the norm weights
+        rel, cos = rel_err_and_cos(got, want)
+        worst = (max(worst[0], rel), min(worst[1], cos))
+        # the flash kernel rounds its probabilities to bf16 before the products of its backward and sums
+        # the norm-weight gradient over all rows in another order; the restatement keeps fp32 matrices:
+        # the element-wise bound is wider than in the map variant, the direction as tight
+        # (and at 4 bits its output differs from the dense one in enough last bits to flip codes of the saved
+        # attention output, which the 256 rows of this case do not average out in the norm-weight gradients)
+        rel_tol, cos_tol = (5e-2, 0.9999) if q_bit == 8 else (0.15, 0.999)
+        assert rel <= rel_tol and cos >= cos_tol, f"{layer_type} q{q_bit} kv{kv_heads} grad {name}: rel {rel:.2e} cos {cos:.5f}"
+    print(f"map-free {layer_type} q{q_bit} kv{kv_heads}: worst rel {worst[0]:.2e}, worst cos {worst[1]:.6f}")
+
+
 def test_map_free_backward_from_saved_lse_equals_recomputation(dev, monkeypatch):
     """The map-free layers keep the flash kernel's log-sum-exps and call its backward directly; with
     uncompressed activations (layer type 'baseline') that must give the gradients of recomputing the
