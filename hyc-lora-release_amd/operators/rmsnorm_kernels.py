@@ -188,8 +188,10 @@ def _adapter_weight(a):
     w = a.t()
     if w.dtype != torch.bfloat16:
         w = w.to(torch.bfloat16)
-    if not w.is_contiguous() or w.data_ptr() % 16:
-        w = w.contiguous().clone() if w.is_contiguous() else w.contiguous()
+    if not w.is_contiguous():
+        w = w.contiguous()
+    if w.data_ptr() % 16:
+        w = w.clone()
     return w
 
 
