@@ -66,6 +66,37 @@ def test_argument_validation_without_launch(L):
         assert h.hyc_set_tuning(b"quant_rows_per_wave", 8) == 0
 
 
+def test_argument_validation_of_the_newer_entry_points(L):
+    """Error codes that come back before any launch (fake pointers are never dereferenced)."""
+    h = L.lib()
+    fake = ctypes.c_void_p(0x1000)
+    one_ptr = (ctypes.c_void_p * 1)(0x1000)
+    five_ptr = (ctypes.c_void_p * 5)(*[0x1000] * 5)
+    rank = lambda *r: (ctypes.c_int64 * len(r))(*r)
+
+    def norm_lora(rows, n, n_adapters, weights, ranks, outs):
+        return h.hyc_rmsnorm_fwd_compress_lora(fake, fake, fake, fake, rows, n, 1e-5, 4, None, None, None, None, None, 0,
+                                               None, n_adapters, weights, ranks, outs, None)
+    assert norm_lora(8, 1024, 0, one_ptr, rank(16), one_ptr) == -8               # no adapter
+    assert norm_lora(8, 1024, 5, five_ptr, rank(16, 16, 16, 16, 16), five_ptr) == -8
+    assert norm_lora(8, 1024, 1, one_ptr, rank(0), one_ptr) == -5                # rank out of range
+    assert norm_lora(8, 1024, 1, one_ptr, rank(65), one_ptr) == -5
+    two_ptr = (ctypes.c_void_p * 2)(0x1000, 0x1000)
+    assert norm_lora(8, 1024, 2, two_ptr, rank(48, 32), two_ptr) == -5           # five 16-row blocks
+    assert norm_lora(8, 1056, 1, one_ptr, rank(16), one_ptr) == -3               # not whole 512-column slabs
+    assert norm_lora(7, 1024, 1, one_ptr, rank(16), one_ptr) == -3               # odd row count
+    assert norm_lora(8, 1024, 1, None, rank(16), one_ptr) == -1
+    assert norm_lora(8, 1024, 1, (ctypes.c_void_p * 1)(0x1008), rank(16), one_ptr) == -4   # adapter rows not 16-byte aligned
+    # bounded compaction: a negative capacity is a shape error, no room at all is a no-op
+    assert h.hyc_sparse_write_bounded(fake, 4096, fake, 0, fake, -1, fake, fake, None) == -3
+    assert h.hyc_sparse_write_bounded(fake, 4096, fake, 0, fake, 0, fake, fake, None) == 0
+    assert h.hyc_sparse_write_bounded(None, 4096, fake, 0, fake, 10, fake, fake, None) == -1
+    # the entry point with its own scratch memory: sizes first
+    assert h.hyc_rmsnorm_bwd_static(fake, fake, fake, 0, fake, fake, fake, 16, 8200, None) == -7
+    assert h.hyc_rmsnorm_bwd_static(fake, fake, fake, 0, fake, fake, None, 16, 64, None) == -1
+    assert h.hyc_rmsnorm_bwd_static_max_bytes() == 512 * 8192 * 4
+
+
 def test_missing_library_is_an_error(L, monkeypatch, tmp_path):
     monkeypatch.setattr(L, "_lib", None)
     monkeypatch.setattr(L, "LIB_PATH", tmp_path / "libhyclora.so")
