@@ -469,6 +469,19 @@ __global__ __launch_bounds__(kSegThreads) void softmax_bwd_restore_kernel(const 
     const int64_t seg = blockIdx.x * (int64_t)(kSegThreads / kWave) + wave;
     const bool live = seg < nseg;
     u32x4* st = reinterpret_cast<u32x4*>(stage[wave]);
+    // The segment's share of the gradient is requested before anything else: its latency then covers
+    // the two dependent round trips of the rebuild (offsets, then indices and values) instead of
+    // following them.  Not for rows of 2048: the 32 registers that hold it there cost a wave per SIMD
+    // and more than the overlap gains (measured 290 against 275 us on [2, 32, 2048, 2048]).
+    constexpr bool kAhead = SPR != 4;
+    u32x4 gall[kAhead ? kSegSteps : 1];
+    if constexpr (kAhead) {
+#pragma unroll
+        for (int c = 0; c < kSegSteps; ++c) {
+            gall[c] = u32x4{0, 0, 0, 0};
+            if (live) gall[c] = ld16_nt(g + seg * kSeg + (int64_t)(c * kWave + lane) * 8);
+        }
+    }
 #pragma unroll
     for (int s = 0; s < kSegSteps; ++s) st[s * kWave + lane] = u32x4{0, 0, 0, 0};
     __syncthreads();
@@ -490,7 +503,8 @@ __global__ __launch_bounds__(kSegThreads) void softmax_bwd_restore_kernel(const 
         for (int s = 0; s < SPR; ++s) {
             const int c = (r * SPR + s) * kWave + lane;      // chunk inside the segment
             yv[s] = st[c];
-            gv[s] = ld16_nt(g + seg * kSeg + (int64_t)c * 8);
+            if constexpr (kAhead) gv[s] = gall[r * SPR + s];
+            else gv[s] = ld16_nt(g + seg * kSeg + (int64_t)c * 8);
         }
 #pragma unroll
         for (int s = 0; s < SPR; ++s) {
@@ -509,7 +523,7 @@ __global__ __launch_bounds__(kSegThreads) void softmax_bwd_restore_kernel(const 
             unpack8(gv[s], gf);
 #pragma unroll
             for (int j = 0; j < 8; ++j) of[j] = rbf((gf[j] - acc) * yf[j]) * out_scale;   // bf16 result, then the bf16 scaling
-            st16_nt(o_out + seg * kSeg + (int64_t)c * 8, pack8(of));
+            st16_nt(o_out + seg * kSeg + (int64_t)c * 8, pack8(of));       // ordinary stores: 166 against 149 us
             if (a_out) st16_nt(a_out + seg * kSeg + (int64_t)c * 8, yv[s]);
         }
     }
