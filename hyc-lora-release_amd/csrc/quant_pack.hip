@@ -75,6 +75,11 @@ struct QuantArgs {
 struct OutlierLane {
     uint32_t mask = 0;        // bit j: column col0 + j is an outlier
     uint32_t pos[4] = {0, 0, 0, 0};  // 16-bit list positions, two per dword
+    // dword p of the lane's chunk with its outlier columns cleared: d & keep(p)
+    __device__ __forceinline__ uint32_t keep(int p) const {
+        const uint32_t two = mask >> (2 * p);
+        return ~(((two & 1u) ? 0x0000ffffu : 0u) | ((two & 2u) ? 0xffff0000u : 0u));
+    }
 };
 
 __device__ __forceinline__ OutlierLane find_outliers(const int64_t* oidx, int k, int wave_col0, int col0, int lane) {
@@ -104,6 +109,51 @@ __device__ __forceinline__ OutlierLane find_outliers(const int64_t* oidx, int k,
 
 __device__ __forceinline__ uint32_t outlier_pos(const OutlierLane& o, int j) {
     return (o.pos[j >> 1] >> (16 * (j & 1))) & 0xffffu;
+}
+
+// One of four dwords by a run-time index (three selects; the operands stay in registers).
+__device__ __forceinline__ uint32_t pick4(uint32_t d0, uint32_t d1, uint32_t d2, uint32_t d3, int p) {
+    const uint32_t lo = (p & 1) ? d1 : d0, hi = (p & 1) ? d3 : d2;
+    return (p & 2) ? hi : lo;
+}
+__device__ __forceinline__ uint32_t outlier_pos_dyn(const OutlierLane& o, int j) {
+    return (pick4(o.pos[0], o.pos[1], o.pos[2], o.pos[3], j >> 1) >> (16 * (j & 1))) & 0xffffu;
+}
+
+// The quantiser's outlier step.  A lane owns at most one outlier column as a rule, so the first one
+// is handled without a branch: its value is picked out of the row's chunk in compute (first_value)
+// and stored next to the row's codes, as one more predicated store whose place in the order of
+// memory operations is fixed.  Whatever a lane holds beyond that - and all of them when the input
+// is to be zeroed in place - goes through extract_rest: a loop over the set bits with stores
+// inside, which makes the compiler wait for every outstanding load and store before it, and which
+// is deliberately not unrolled (eight predicated copies of the body per row once made this kernel
+// sixty thousand instructions long).
+struct OutlierFirst {
+    int j = 0;            // the lane's lowest outlier column (0 if it has none)
+    uint32_t pos = 0;     // its position in the list
+    uint32_t rest = 0;    // mask bits beyond it
+    OutlierFirst() = default;
+    __device__ __forceinline__ explicit OutlierFirst(const OutlierLane& o) {
+        if (o.mask) {
+            j = __ffs((int)o.mask) - 1;
+            pos = outlier_pos_dyn(o, j);
+            rest = o.mask & (o.mask - 1);
+        }
+    }
+    __device__ __forceinline__ uint32_t first_value(const u32x4& v) const {
+        return (pick4(v.x, v.y, v.z, v.w, j >> 1) >> (16 * (j & 1))) & 0xffffu;
+    }
+};
+
+__device__ __forceinline__ void extract_rest(const OutlierLane& o, uint32_t bits, const u32x4& v, uint16_t* xo_row,
+                                             uint16_t* x_chunk, bool zero_input) {
+#pragma clang loop unroll(disable)
+    while (bits) {
+        const int j = __ffs((int)bits) - 1;
+        bits &= bits - 1;
+        xo_row[outlier_pos_dyn(o, j)] = (uint16_t)(pick4(v.x, v.y, v.z, v.w, j >> 1) >> (16 * (j & 1)));
+        if (zero_input) x_chunk[j] = 0;
+    }
 }
 
 // Walks the rows t = b*M + m of a [B, M, .] tensor with independent batch and row strides
@@ -139,9 +189,10 @@ __device__ __forceinline__ int64_t chunk_offset(int col0, int head_dim, int64_t 
 // row1 are skipped) and advances the cursor.
 template <bool FULL>
 __device__ __forceinline__ void load_rows(const QuantArgs& a, RowCursor& cur, int64_t t0, int64_t row1, bool active,
-                                          int64_t coff, u32x4 (&v)[kRowUnroll]) {
+                                          int64_t coff, u32x4 (&v)[kRowUnroll], int64_t (&roff)[kRowUnroll]) {
 #pragma unroll
     for (int u = 0; u < kRowUnroll; ++u) {
+        roff[u] = cur.off;                 // element offset of the row (only the outlier step reads it)
         if constexpr (FULL) {
             v[u] = ld16_nt(a.x + cur.off + coff);
         } else {
@@ -170,31 +221,26 @@ __device__ __forceinline__ void quant_rows(const QuantArgs& a, int64_t row0, int
     if (row0 >= row1) return;
     RowCursor cur(row0, a.M, a.stride_b, a.stride_m);
     u32x4 v[kRowUnroll];
-    load_rows<FULL>(a, cur, row0, row1, active, coff, v);
+    int64_t roff[kRowUnroll];
+    load_rows<FULL>(a, cur, row0, row1, active, coff, v, roff);
     // the first rows are already on their way while the wave looks up its outlier columns
     OutlierLane ol;
     if constexpr (OUTL) ol = find_outliers(a.oidx, a.k, (chunk & ~(kWave - 1)) * 8, chunk * 8, chunk & (kWave - 1));
+    const OutlierFirst of(ol);
+    const bool in_place = OUTL && a.zero_input != 0;
+    const uint32_t loop_bits = in_place ? ol.mask : of.rest;     // what extract_rest handles, per lane
+    const bool store_first = OUTL && ol.mask != 0 && !in_place;
+    uint32_t first[OUTL ? kRowUnroll : 1];
     auto compute = [&](u32x4 (&v)[kRowUnroll], int64_t t0, uint32_t (&lo)[kRowUnroll], uint32_t (&hi)[kRowUnroll]) {
 #pragma unroll
         for (int u = 0; u < kRowUnroll; ++u) {
             const int64_t t = t0 + u;
             if constexpr (OUTL) {
-                if (ol.mask && (FULL || (active && t < row1))) {
-                    uint32_t d[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
-#pragma unroll
-                    for (int j = 0; j < 8; ++j) {
-                        if (ol.mask & (1u << j)) {
-                            const uint32_t sh = 16 * (j & 1);
-                            a.xo[t * a.k + outlier_pos(ol, j)] = (uint16_t)(d[j >> 1] >> sh);
-                            d[j >> 1] &= ~(0xffffu << sh);
-                            if (a.zero_input) {
-                                const RowCursor here(t, a.M, a.stride_b, a.stride_m);
-                                a.x[here.off + coff + j] = 0;
-                            }
-                        }
-                    }
-                    v[u] = u32x4{d[0], d[1], d[2], d[3]};
-                }
+                first[u] = of.first_value(v[u]);
+                asm volatile("" : "+v"(first[u]));     // picked here, not at the store: the row's registers take the next loads
+                if (loop_bits && (FULL || (active && t < row1)))
+                    extract_rest(ol, loop_bits, v[u], a.xo + t * a.k, a.x + roff[u] + coff, in_place);
+                v[u] = u32x4{v[u].x & ol.keep(0), v[u].y & ol.keep(1), v[u].z & ol.keep(2), v[u].w & ol.keep(3)};
             }
             float f[8];
             unpack8(v[u], f);
@@ -207,6 +253,9 @@ __device__ __forceinline__ void quant_rows(const QuantArgs& a, int64_t row0, int
         for (int u = 0; u < kRowUnroll; ++u) {
             const int64_t t = t0 + u;
             store_merged<QBIT, false>(a.q + t * row_bytes, chunk, FULL || (active && t < row1), lo[u], hi[u]);
+            if constexpr (OUTL) {
+                if (store_first && (FULL || (active && t < row1))) a.xo[t * a.k + of.pos] = (uint16_t)first[u];
+            }
         }
     };
     // The first group is peeled so that the loop is always entered with "4 loads, then 4 stores"
@@ -216,11 +265,11 @@ __device__ __forceinline__ void quant_rows(const QuantArgs& a, int64_t row0, int
     int64_t t0 = row0;
     compute(v, t0, lo, hi);
     if (t0 + kRowUnroll < row1) {
-        load_rows<FULL>(a, cur, t0 + kRowUnroll, row1, active, coff, v);
+        load_rows<FULL>(a, cur, t0 + kRowUnroll, row1, active, coff, v, roff);
         store(t0, lo, hi);
         for (t0 += kRowUnroll; t0 + kRowUnroll < row1; t0 += kRowUnroll) {
             compute(v, t0, lo, hi);
-            load_rows<FULL>(a, cur, t0 + kRowUnroll, row1, active, coff, v);
+            load_rows<FULL>(a, cur, t0 + kRowUnroll, row1, active, coff, v, roff);
             store(t0, lo, hi);
         }
         compute(v, t0, lo, hi);                                // last group: nothing left to load
@@ -289,6 +338,7 @@ __global__ __launch_bounds__(kQuantThreads) void unpack_dequant_kernel(const Qua
         }
     }
     OutlierLane ol;
+    OutlierFirst of;
 
     const int64_t coff = active ? chunk_offset(col0, a.head_dim, a.stride_h) : 0;
     const int64_t row0 = (row_tile * kQuantWaves + wave) * (int64_t)a.rows_per_wave;
@@ -316,20 +366,17 @@ __global__ __launch_bounds__(kQuantThreads) void unpack_dequant_kernel(const Qua
                 }
             }
         };
-        // Outlier values travel with the codes of their row, one load per flagged column, so
-        // that the row's store waits for one round of memory latency and not for two.
-        uint32_t ov[OUTL ? kDeqUnroll : 1][8];
+        // The value of a lane's first outlier column travels with the codes of its row, so that the
+        // row's store waits for one round of memory latency and not for two.  Further outlier columns
+        // of the same lane (rare) are fetched where they are inserted.
+        uint32_t ovf[OUTL ? kDeqUnroll : 1];
         auto load_outliers = [&](int64_t t0) {
             if constexpr (OUTL) {
                 if (ol.mask) {
 #pragma unroll
                     for (int u = 0; u < kDeqUnroll; ++u) {
                         const int64_t t = t0 + u;
-                        if (FULL || (active && t < row1)) {
-#pragma unroll
-                            for (int j = 0; j < 8; ++j)
-                                if (ol.mask & (1u << j)) ov[u][j] = a.xo[t * a.k + outlier_pos(ol, j)];
-                        }
+                        if (FULL || (active && t < row1)) ovf[u] = a.xo[t * a.k + of.pos];
                     }
                 }
             }
@@ -358,13 +405,18 @@ __global__ __launch_bounds__(kQuantThreads) void unpack_dequant_kernel(const Qua
                 cur.next(a.M, a.stride_b, a.stride_m);
                 if constexpr (OUTL) {
                     if (ol.mask && (FULL || (active && t < row1))) {
-                        uint32_t d[4] = {o[u].x, o[u].y, o[u].z, o[u].w};
+                        uint32_t d[4] = {o[u].x & ol.keep(0), o[u].y & ol.keep(1), o[u].z & ol.keep(2), o[u].w & ol.keep(3)};
+                        auto insert = [&](int j, uint32_t value) {
 #pragma unroll
-                        for (int j = 0; j < 8; ++j) {
-                            if (ol.mask & (1u << j)) {
-                                const uint32_t sh = 16 * (j & 1);
-                                d[j >> 1] = (d[j >> 1] & ~(0xffffu << sh)) | (ov[u][j] << sh);
-                            }
+                            for (int p = 0; p < 4; ++p) d[p] |= (j >> 1) == p ? value << (16 * (j & 1)) : 0u;
+                        };
+                        insert(of.j, ovf[u]);
+                        uint32_t bits = of.rest;
+#pragma clang loop unroll(disable)
+                        while (bits) {
+                            const int j = __ffs((int)bits) - 1;
+                            bits &= bits - 1;
+                            insert(j, a.xo[t * a.k + outlier_pos_dyn(ol, j)]);
                         }
                         o[u] = u32x4{d[0], d[1], d[2], d[3]};
                     }
@@ -379,7 +431,10 @@ __global__ __launch_bounds__(kQuantThreads) void unpack_dequant_kernel(const Qua
         // next group's loads go out before this group's stores (see quant_rows)
         load_codes(row0);
         // the first codes are already on their way while the wave looks up its outlier columns
-        if constexpr (OUTL) ol = find_outliers(a.oidx, a.k, col_tile * kWave * 8, col0, lane);
+        if constexpr (OUTL) {
+            ol = find_outliers(a.oidx, a.k, col_tile * kWave * 8, col0, lane);
+            of = OutlierFirst(ol);
+        }
         load_outliers(row0);
         int64_t t0 = row0;
         compute(t0);                              // first group peeled, as in quant_rows

@@ -124,6 +124,12 @@ def test_outliers_many_unsorted_adjacent(cf, dev):
     assert same_bits(xo.cpu(), xo_ref) and torch.equal(p.cpu(), p_ref)
     back = cf.outlier_addition_fuse_decompression_dequantization(p, s.to(dev), xo, idx.to(dev), 4)
     assert same_bits(back.cpu(), O.decompress_channel_base(p_ref, s, xo_ref, idx, 4))
+    # the in-place zeroing with several outlier columns inside one lane's chunk
+    xg = x.to(dev)
+    xo2, p2 = cf.outlier_subtraction_fuse_compression_quantization(xg, s.to(dev), idx.to(dev), 4, zero_input=True)
+    assert torch.equal(p2, p) and torch.equal(xo2, xo)
+    xz = x.clone(); xz[:, :, idx] = 0
+    assert same_bits(xg.cpu(), xz)
 
 
 @pytest.mark.parametrize("q_bit", QBITS)
