@@ -52,6 +52,7 @@ struct ContractArgs {
     int64_t T;
     int N, C, R;
     int tiles_per_group, groups, v_transposed;
+    int passes;                          // the rank is covered 16*NB at a time; see the kernel
     int64_t n_blocks;                    // strips * groups
 };
 
@@ -64,7 +65,7 @@ __device__ __forceinline__ s16x4 pick_column(const u32x4 (&xv)[4], int u8) {
     return __builtin_bit_cast(s16x4, pk);
 }
 
-template <int QBIT, bool ZP, bool P1, bool P2, int NB>
+template <int QBIT, bool ZP, bool P1, bool P2, int NB, bool MULTI = false>
 __global__ __launch_bounds__(kCtThreads) void lora_contract_kernel(const ContractArgs a) {
     static_assert(QBIT == 0 || !P2, "the column contraction reads dense X only");
     __shared__ float red[P1 ? kCtWaves * 16 * kCtTile : 1];
@@ -91,6 +92,17 @@ __global__ __launch_bounds__(kCtThreads) void lora_contract_kernel(const Contrac
     constexpr float kHalf = (float)(1 << (QB - 1));
     const int row_bytes = a.N * QB / 8;
 
+    // Ranks beyond 16*NB are covered in passes over the workgroup's tiles, 16*NB LoRA rows at a time:
+    // every accumulator and operand of the contraction scales with the number of rank blocks held at
+    // once (about 100 registers per block), and with more than one block the kernel is down to one wave
+    // per SIMD with nothing to hide its loads behind.  A later pass finds the tiles in the cache the
+    // first one pulled them through.
+    // (MULTI is a template parameter: with the loop bound read from the arguments the one-pass kernel
+    // of the usual ranks ran 42 instead of 31 us.)
+    const int passes = MULTI ? a.passes : 1;
+    const int rows_all = 16 * NB * passes;                    // LoRA rows of a partial plane
+    for (int pass = 0; pass < passes; ++pass) {
+    const int rb = pass * 16 * NB;
     f32x4 acc2[P2 ? kCtSteps : 1][NB];
     if constexpr (P2) {
 #pragma unroll
@@ -117,7 +129,7 @@ __global__ __launch_bounds__(kCtThreads) void lora_contract_kernel(const Contrac
                 uint32_t e[NB][8][4];
 #pragma unroll
                 for (int nb = 0; nb < NB; ++nb) {
-                    const int r = 16 * nb + j;
+                    const int r = rb + 16 * nb + j;
 #pragma unroll
                     for (int s8 = 0; s8 < 8; ++s8) {
                         const int col = c0 + 16 * s8 + 4 * g;
@@ -140,7 +152,7 @@ __global__ __launch_bounds__(kCtThreads) void lora_contract_kernel(const Contrac
             } else {
 #pragma unroll
                 for (int nb = 0; nb < NB; ++nb) {
-                    const int r = 16 * nb + j;
+                    const int r = rb + 16 * nb + j;
 #pragma unroll
                     for (int s8 = 0; s8 < 8; ++s8) {
                         const int col = c0 + 16 * s8 + 4 * g;
@@ -197,7 +209,7 @@ __global__ __launch_bounds__(kCtThreads) void lora_contract_kernel(const Contrac
                 // U operand: lane (r = 16nb + j, g), rows t0 + 4g .. +3 (whole dwords, see above)
 #pragma unroll
                 for (int nb = 0; nb < (P1 ? NB : 0); ++nb) {
-                    const int r = 16 * nb + j;
+                    const int r = rb + 16 * nb + j;
 #pragma unroll
                     for (int kk = 0; kk < 4; ++kk) {
                         const int64_t t = t0 + 4 * g + kk;
@@ -286,7 +298,7 @@ __global__ __launch_bounds__(kCtThreads) void lora_contract_kernel(const Contrac
                     for (int w = 1; w < kCtWaves; ++w)
 #pragma unroll
                         for (int e = 0; e < 8; ++e) sum[e] += red[(w * 16 + r) * kCtTile + cc + e];
-                    float* dst = a.part1 + ((strip * (16 * NB) + 16 * nb + r) * (int64_t)a.N + c0 + cc);
+                    float* dst = a.part1 + ((strip * rows_all + rb + 16 * nb + r) * (int64_t)a.N + c0 + cc);
                     *reinterpret_cast<f32x4*>(dst) = f32x4{sum[0], sum[1], sum[2], sum[3]};
                     *reinterpret_cast<f32x4*>(dst + 4) = f32x4{sum[4], sum[5], sum[6], sum[7]};
                 }
@@ -304,10 +316,11 @@ __global__ __launch_bounds__(kCtThreads) void lora_contract_kernel(const Contrac
 #pragma unroll
                 for (int vv = 0; vv < 4; ++vv) {
                     const int64_t t = row_base + 16 * st + 4 * g + vv;
-                    if (t < a.T) a.part2[((int64_t)group * a.T + t) * (16 * NB) + 16 * nb + j] = e[vv];
+                    if (t < a.T) a.part2[((int64_t)group * a.T + t) * rows_all + rb + 16 * nb + j] = e[vv];
                 }
             }
     }
+    }   // pass
 }
 
 // out[i][c] = bf16( sum_k part[k][i][c] ), i < rows_out, c < cols_out, partial planes of
@@ -357,12 +370,16 @@ __global__ __launch_bounds__(256) void contract_reduce_kernel(const ReduceJob j0
 
 // ------------------------------------------------------------------------------------
 template <int QBIT, bool ZP, bool P1, bool P2>
-static void contract_launch_nb(const ContractArgs& a, dim3 grid, int nb, hipStream_t st) {
+static void contract_launch_nb(ContractArgs a, dim3 grid, int nb, hipStream_t st) {
+    // nb = rank blocks of 16.  One or two are held at once; three run as three passes of one, four as
+    // two passes of two (measured on [4096, 11008], both products: 101 and 109 us against 120 and 279 us
+    // for kernels that held three or four blocks at once and spilled).
     const dim3 block(kCtThreads);
+    a.passes = nb <= 2 ? 1 : (nb == 3 ? 3 : 2);
     if (nb == 1) hipLaunchKernelGGL((lora_contract_kernel<QBIT, ZP, P1, P2, 1>), grid, block, 0, st, a);
     else if (nb == 2) hipLaunchKernelGGL((lora_contract_kernel<QBIT, ZP, P1, P2, 2>), grid, block, 0, st, a);
-    else if (nb == 3) hipLaunchKernelGGL((lora_contract_kernel<QBIT, ZP, P1, P2, 3>), grid, block, 0, st, a);
-    else hipLaunchKernelGGL((lora_contract_kernel<QBIT, ZP, P1, P2, 4>), grid, block, 0, st, a);
+    else if (nb == 3) hipLaunchKernelGGL((lora_contract_kernel<QBIT, ZP, P1, P2, 1, true>), grid, block, 0, st, a);
+    else hipLaunchKernelGGL((lora_contract_kernel<QBIT, ZP, P1, P2, 2, true>), grid, block, 0, st, a);
 }
 
 static int64_t contract_geometry(int64_t T, int64_t N, int64_t R, int* tiles_per_group, int* groups, int64_t* strips,

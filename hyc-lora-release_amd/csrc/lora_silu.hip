@@ -25,8 +25,17 @@ constexpr int kFuseThreads = 256;                  // 4 waves
 // tensors), i.e. two waves per SIMD.  Telling the compiler so makes it schedule for latency hiding
 // inside the wave instead of chasing a third wave it cannot get without spilling
 // (measured on [4096 x 11008], q=4: 126 -> 93 us forward, 122 -> 99 us backward).
-#define HYC_FUSE_KERNEL __global__ __launch_bounds__(kFuseThreads) __attribute__((amdgpu_waves_per_eu(2, 2)))
+#define HYC_FUSE_KERNEL(DEEP) __global__ __launch_bounds__(kFuseThreads) __attribute__((amdgpu_waves_per_eu(KSTEPS >= DEEP ? 1 : 2, KSTEPS >= DEEP ? 1 : 2)))
 constexpr int kFuseWaves = kFuseThreads / kWave;
+#ifndef HYC_FWD_DEEP
+#define HYC_FWD_DEEP 2
+#endif
+#ifndef HYC_BWD_DEEP
+#define HYC_BWD_DEEP 3
+#endif
+#ifndef HYC_ROLL_DEEP
+#define HYC_ROLL_DEEP 1
+#endif
 
 // Strip heights (backward, forward; see hyc_set_tuning).  0 = by size: a wave sets up its LoRA-B
 // operands and per-column constants once per strip, which in the [N, R] layout of LoRA-B is 16
@@ -173,7 +182,7 @@ __device__ __forceinline__ void fuse_fwd_rows_full(const FuseArgs& a, int64_t ro
 }
 
 template <int QBIT, int KSTEPS>
-HYC_FUSE_KERNEL void lora_silu_fwd_kernel(const FuseArgs a) {
+HYC_FUSE_KERNEL(HYC_FWD_DEEP) void lora_silu_fwd_kernel(const FuseArgs a) {
     constexpr int CT = kColTilesPerGroup<QBIT>, RS = kFuseWaves / CT;
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -202,7 +211,7 @@ HYC_FUSE_KERNEL void lora_silu_fwd_kernel(const FuseArgs a) {
     const bool full = (col_tile + 1) * (kTileCols / 8) <= a.C && (row_end - row_begin) % kTileRows == 0;   // uniform
     if (__ballot(!(c1.fast && c2.fast)) != 0ull)
         fuse_fwd_rows<QBIT, KSTEPS, false>(a, row_begin, row_end, lane, chunk, active, c1, c2, B1, B2);
-    else if (KSTEPS == 1 && full)                  // deeper ranks have no registers to spare for it
+    else if ((KSTEPS == 1 || (HYC_ROLL_DEEP && KSTEPS >= HYC_FWD_DEEP)) && full)                  // deeper ranks have no registers to spare for it
         fuse_fwd_rows_full<QBIT, KSTEPS>(a, row_begin, row_end, lane, chunk, c1, c2, B1, B2);
     else
         fuse_fwd_rows<QBIT, KSTEPS, true>(a, row_begin, row_end, lane, chunk, active, c1, c2, B1, B2);
@@ -210,7 +219,7 @@ HYC_FUSE_KERNEL void lora_silu_fwd_kernel(const FuseArgs a) {
 
 // ------------------------------------------------------------------------------------
 template <int QBIT, int KSTEPS>
-HYC_FUSE_KERNEL void lora_silu_bwd_kernel(const FuseArgs a) {
+HYC_FUSE_KERNEL(HYC_BWD_DEEP) void lora_silu_bwd_kernel(const FuseArgs a) {
     constexpr int CT = kColTilesPerGroup<QBIT>, RS = kFuseWaves / CT;
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -264,7 +273,7 @@ HYC_FUSE_KERNEL void lora_silu_bwd_kernel(const FuseArgs a) {
 
     // Interior strips at rank 16: the rolling prefetch of fuse_fwd_rows_full - a row's registers
     // are requested again for the next tile as soon as the row has been taken out of them.
-    const bool full = KSTEPS == 1 && (col_tile + 1) * (kTileCols / 8) <= a.C && row_begin < row_end &&
+    const bool full = (KSTEPS == 1 || (HYC_ROLL_DEEP && KSTEPS >= HYC_BWD_DEEP)) && (col_tile + 1) * (kTileCols / 8) <= a.C && row_begin < row_end &&
                       (row_end - row_begin) % kTileRows == 0;      // uniform across the wave
     if (full) {
         const int i = lane & 15;

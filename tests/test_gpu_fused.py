@@ -46,7 +46,8 @@ def mlp_inputs(seed, B, M, H, I, R):
 
 @pytest.mark.parametrize("q_bit", QBITS)
 @pytest.mark.parametrize("dims", [(2, 64, 256, 1024, 16), (1, 37, 128, 160, 16), (1, 16, 64, 11008, 16),
-                                  (2, 20, 64, 256, 8), (1, 33, 64, 384, 32), (1, 16, 64, 128, 64), (1, 5, 64, 96, 4)])
+                                  (2, 20, 64, 256, 8), (1, 33, 64, 384, 32), (1, 16, 64, 128, 64), (1, 5, 64, 96, 4),
+                                  (2, 100, 64, 384, 48), (1, 130, 64, 256, 64)])
 def test_fused_forward_and_backward(fz, dev, q_bit, dims):
     B, M, H, I, R = dims
     t = mlp_inputs(q_bit + I, B, M, H, I, R)
@@ -62,7 +63,9 @@ def test_fused_forward_and_backward(fz, dev, q_bit, dims):
     # unfused composition in fp32
     gate = x1.float() + xa1.float() @ b1.float()
     up = x2.float() + xa2.float() @ b2.float()
-    assert_close_bf16(o, F.silu(gate) * up, what="fused forward o vs unfused fp32")
+    # (the bar is the oracle comparison above; this one measures the reference's own bf16-per-operation
+    # arithmetic against fp32, and the rounded LoRA term of a rank-64 adapter is a larger share of it)
+    assert_close_bf16(o, F.silu(gate) * up, rel_tol=1e-2 if R <= 32 else 1.5e-2, what="fused forward o vs unfused fp32")
 
     g = torch.randn(B, M, I, generator=torch.Generator().manual_seed(1)).to(BF16)
     ob, gg, gu = fz.bwd(*d(xa1, b1), q1, s1.to(dev), *d(xa2, b2), q2, s2.to(dev), g.to(dev), q_bit)
@@ -80,7 +83,7 @@ def test_fused_forward_and_backward(fz, dev, q_bit, dims):
 
 
 @pytest.mark.parametrize("q_bit", QBITS)
-@pytest.mark.parametrize("R", [16, 8])
+@pytest.mark.parametrize("R", [16, 8, 48, 64])      # 48 and 64: the deep-rank instantiations walk the same way
 def test_fused_results_do_not_depend_on_the_strip_height(fz, dev, q_bit, R):
     # Interior strips are walked with the next tile requested ahead: one tile per strip takes only
     # the closing step of that walk, two tiles the opening and the closing one, more the loop in

@@ -40,7 +40,8 @@ def nearly_same_bits(a, b, what):
 
 
 SHAPES = [((2, 64), 256, 16), ((1, 37), 160, 16), ((300,), 11008, 16), ((2, 20), 256, 8), ((1, 33), 384, 32),
-          ((1, 16), 128, 64), ((5,), 96, 4), ((3, 50), 4096, 16), ((2, 513), 512, 48), ((1, 1), 32, 2), ((700,), 1024, 12)]
+          ((1, 16), 128, 64), ((5,), 96, 4), ((3, 50), 4096, 16), ((2, 513), 512, 48), ((1, 1), 32, 2), ((700,), 1024, 12),
+          ((520,), 8192, 64), ((300,), 4224, 40)]      # ranks past 32: several passes over several tiles per workgroup
 
 
 @pytest.mark.parametrize("lead,N,R", SHAPES)
@@ -64,7 +65,8 @@ def test_both_products_from_one_pass(K, dev, lead, N, R):
 
 @pytest.mark.parametrize("q_bit", [2, 4, 8])
 @pytest.mark.parametrize("zp", [False, True])
-@pytest.mark.parametrize("B,M,N,R", [(2, 64, 256, 16), (1, 37, 160, 16), (1, 300, 11008, 16), (2, 50, 4096, 32), (3, 7, 96, 8)])
+@pytest.mark.parametrize("B,M,N,R", [(2, 64, 256, 16), (1, 37, 160, 16), (1, 300, 11008, 16), (2, 50, 4096, 32), (3, 7, 96, 8),
+                                     (1, 300, 1024, 64), (2, 40, 8192, 48)])
 def test_row_product_straight_from_codes(K, dev, q_bit, zp, B, M, N, R):
     x, u, _ = inputs(q_bit + N, (B, M), N, R)
     if zp:
