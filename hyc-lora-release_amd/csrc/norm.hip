@@ -220,19 +220,48 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_bwd_kernel(const uint16_
     }
 }
 
-// dw[c] = sum over partial rows, fixed order; output in the weight's dtype.
+// dw[c] = sum over partial rows, fixed order; output in the weight's dtype.  A workgroup owns 64
+// columns; thread (g = tid / 16, c4 = tid % 16) adds rows g, g + 16, g + 32, ... of four columns, four
+// loads in flight, and the 16 row groups are then added in order through LDS.  (One thread per column
+// walking all partial rows by itself was a chain of several hundred dependent loads on 16 workgroups:
+// 70 us for 4 MB.)
 template <bool W32>
-__global__ void rmsnorm_dw_reduce_kernel(const float* __restrict__ partial, int nparts, int N, void* __restrict__ dw) {
-    const int c = blockIdx.x * blockDim.x + threadIdx.x;
-    if (c >= N) return;
-    float s = 0.0f;
-    for (int p = 0; p < nparts; ++p) s += partial[(int64_t)p * N + c];
-    if constexpr (W32) ((float*)dw)[c] = s;
-    else ((uint16_t*)dw)[c] = f_to_bf(s);
+__global__ __launch_bounds__(256) void rmsnorm_dw_reduce_kernel(const float* __restrict__ partial, int nparts, int N,
+                                                                void* __restrict__ dw) {
+    __shared__ f32x4 red[16][16];
+    const int c4 = threadIdx.x & 15, g = threadIdx.x >> 4;
+    const int col = (blockIdx.x * 16 + c4) * 4;
+    f32x4 s = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (col < N) {
+        const float* p0 = partial + col;
+        int p = g;
+        for (; p + 48 < nparts; p += 64) {
+            f32x4 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) v[u] = *reinterpret_cast<const f32x4*>(p0 + (int64_t)(p + 16 * u) * N);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) s += v[u];
+        }
+        for (; p < nparts; p += 16) s += *reinterpret_cast<const f32x4*>(p0 + (int64_t)p * N);
+    }
+    red[g][c4] = s;
+    __syncthreads();
+    if (g != 0 || col >= N) return;
+    f32x4 t = red[0][c4];
+#pragma unroll
+    for (int k = 1; k < 16; ++k) t += red[k][c4];
+    if constexpr (W32) {
+        *reinterpret_cast<f32x4*>((float*)dw + col) = t;
+    } else {
+        *reinterpret_cast<u32x2*>((uint16_t*)dw + col) = u32x2{pk_bf16(t.x, t.y), pk_bf16(t.z, t.w)};
+    }
 }
 
-static int bwd_blocks(int64_t rows) {
-    int64_t b = cdiv(rows, kNormWaves * 4);
+// Workgroups of the backward launch that also leaves dw partials (one partial row each).  Rows of up to
+// 4096 channels leave room for two such waves per SIMD, longer ones for one: [4096 x 4096] takes 32 us
+// with two rows per wave against 37 with four, [4096 x 8192] 73 us with four against 84 with two.
+static int bwd_blocks(int64_t rows, int64_t N) {
+    int64_t b = cdiv(rows, kNormWaves * (N <= 4096 ? 2 : 4));
     if (b > kNormMaxBlocks) b = kNormMaxBlocks;
     if (b < 1) b = 1;
     return (int)b;
@@ -243,10 +272,16 @@ static int launch_fwd(const uint16_t* x, const void* w, uint16_t* y, float* rstd
                       hipStream_t st) {
     const dim3 grid((unsigned)cdiv(rows, kNormWaves)), block(kNormThreads);
 #define HYC_FWD(CH) hipLaunchKernelGGL((rmsnorm_fwd_kernel<CH, W32>), grid, block, 0, st, x, w, y, rstd, rows, N, eps)
+    // a row is held in registers, CH chunks of 8 per lane; the steps between the powers of two keep
+    // rows of 3072, 5120, 6144 and 7168 from paying for registers they do not fill
     if (N <= 512) HYC_FWD(1);
     else if (N <= 1024) HYC_FWD(2);
     else if (N <= 2048) HYC_FWD(4);
+    else if (N <= 3072) HYC_FWD(6);
     else if (N <= 4096) HYC_FWD(8);
+    else if (N <= 5120) HYC_FWD(10);
+    else if (N <= 6144) HYC_FWD(12);
+    else if (N <= 7168) HYC_FWD(14);
     else if (N <= 8192) HYC_FWD(16);
     else hipLaunchKernelGGL((rmsnorm_fwd_long_kernel<W32>), grid, block, 0, st, x, w, y, rstd, rows, N, eps);
 #undef HYC_FWD
@@ -261,7 +296,11 @@ static int launch_bwd_r(const uint16_t* dy, const uint16_t* x, const void* w, co
     if (N <= 512) HYC_BWD(1);
     else if (N <= 1024) HYC_BWD(2);
     else if (N <= 2048) HYC_BWD(4);
+    else if (N <= 3072) HYC_BWD(6);
     else if (N <= 4096) HYC_BWD(8);
+    else if (N <= 5120) HYC_BWD(10);
+    else if (N <= 6144) HYC_BWD(12);
+    else if (N <= 7168) HYC_BWD(14);
     else HYC_BWD(16);
 #undef HYC_BWD
     return check_launch();
@@ -291,7 +330,7 @@ extern "C" int hyc_rmsnorm_fwd(const void* x, const void* weight, int weight_is_
 
 extern "C" int64_t hyc_rmsnorm_bwd_workspace(int64_t rows, int64_t N) {
     if (rows <= 0 || N <= 0) return 0;
-    return (int64_t)bwd_blocks(rows) * N * (int64_t)sizeof(float);
+    return (int64_t)bwd_blocks(rows, N) * N * (int64_t)sizeof(float);
 }
 
 static int rmsnorm_bwd_any(const void* dy, const void* x, const void* weight, int weight_is_fp32, const float* rstd,
@@ -303,16 +342,17 @@ static int rmsnorm_bwd_any(const void* dy, const void* x, const void* weight, in
     if (!aligned16(dy) || !aligned16(x) || !aligned16(weight) || !aligned16(dx) || !aligned16(residual)) return HYC_ERR_ALIGN;
     const uint16_t* res = (const uint16_t*)residual;
     hipStream_t st = (hipStream_t)stream;
-    const int blocks = bwd_blocks(rows);
+    const int blocks = bwd_blocks(rows, N);
     int rc;
     if (dw) {
         if (!workspace) return HYC_ERR_NULL;
+        if (!aligned16(workspace) || !aligned16(dw)) return HYC_ERR_ALIGN;
         if (workspace_bytes < hyc_rmsnorm_bwd_workspace(rows, N)) return HYC_ERR_WORKSPACE;
         rc = weight_is_fp32
                  ? launch_bwd<true, true>((const uint16_t*)dy, (const uint16_t*)x, weight, rstd, res, (uint16_t*)dx, (float*)workspace, rows, (int)N, blocks, st)
                  : launch_bwd<false, true>((const uint16_t*)dy, (const uint16_t*)x, weight, rstd, res, (uint16_t*)dx, (float*)workspace, rows, (int)N, blocks, st);
         if (rc != HYC_OK) return rc;
-        const dim3 grid((unsigned)cdiv(N, 256)), block(256);
+        const dim3 grid((unsigned)cdiv(N, 64)), block(256);
         if (weight_is_fp32) hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel<true>, grid, block, 0, st, (const float*)workspace, blocks, (int)N, dw);
         else hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel<false>, grid, block, 0, st, (const float*)workspace, blocks, (int)N, dw);
         return check_launch();

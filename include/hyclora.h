@@ -270,8 +270,9 @@ int hyc_rmsnorm_fwd(const void *x, const void *weight, int weight_is_fp32, void 
  * requested, _rms_norm_bwd_dwdb (operators/rmsnorm_updatable_kernels.py:117-137) — with a
  * deterministic two-stage fp32 reduction instead of the spin-lock accumulation.
  *   dy, x, dx  bf16 [rows, N] contiguous; N % 8 == 0, N <= 8192.
- *   dw         [N] in the weight's dtype, or NULL.  When given, workspace must hold
- *              hyc_rmsnorm_bwd_workspace(rows, N) bytes (fp32 partial rows).
+ *   dw         [N] in the weight's dtype, 16-byte aligned, or NULL.  When given, workspace
+ *              (16-byte aligned) must hold hyc_rmsnorm_bwd_workspace(rows, N) bytes (fp32
+ *              partial rows).
  */
 int64_t hyc_rmsnorm_bwd_workspace(int64_t rows, int64_t N);
 int hyc_rmsnorm_bwd(const void *dy, const void *x, const void *weight, int weight_is_fp32,
