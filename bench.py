@@ -107,12 +107,13 @@ def parse():
     ap.add_argument("--pmc-summary", default="", metavar="DIR",
                     help="no GPU work: turn the rocprofv3 counter CSVs under DIR into profiles/quant_pack_q4_config2_hbm_traffic.json")
     ap.add_argument("--layer-case", default="", help="with --only layers: run only the cases whose name contains this")
+    ap.add_argument("--layer-seq", type=int, default=0, help="with --only layers: sequence length instead of the configuration's")
     ap.add_argument("--layer-arm", choices=["both", "plain", "compressed"], default="both",
                     help="with --only layers: run only one arm (for profiler runs)")
     return ap.parse_args()
 
 
-def bench_layers(torch, dev, only_case="", arm="both"):
+def bench_layers(torch, dev, only_case="", arm="both", seq=0):
     """Forward+backward of one decoder layer with random-init bf16 weights N(0, 0.02) and LoRA r=16 on
     all seven linears: the compressed layer of this package against an uncompressed bf16
     torch-autograd layer of the same architecture, with the activation bytes each keeps for backward."""
@@ -231,6 +232,9 @@ def bench_layers(torch, dev, only_case="", arm="both"):
     for name, dims, maker, lt, qbits, sdpa in cases:
         if only_case not in name:
             continue
+        if seq:                                       # another sequence length than the configuration's
+            dims = dict(dims, S=seq)
+            name = f"{name}_at_s{seq}"
         t = make(**dims)
         mask = None if sdpa else torch.full((t.S, t.S), float("-inf"), device=dev).triu(1).to(BF16)[None, None]
         entry, saved_p, plain = {}, 0, None
@@ -935,7 +939,7 @@ def main():
         for buffers in (xs, qs, xh):
             buffers.clear()
         torch.cuda.empty_cache()
-        layers = bench_layers(torch, dev, args.layer_case, args.layer_arm)
+        layers = bench_layers(torch, dev, args.layer_case, args.layer_arm, args.layer_seq)
     stack = None
     if args.only in ("all", "stack"):
         for buffers in (xs, qs, xh):

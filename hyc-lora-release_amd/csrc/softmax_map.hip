@@ -366,10 +366,14 @@ __global__ __launch_bounds__(kSegThreads) void sparse_restore_kernel(const int64
 // (models/llama/fused_llama_layer_intra_inter_full_fuse.py:159-167) in one read and one write.
 // One wave per row, the row held in registers (CH chunks of 8 per lane).  Row r uses mask row
 // (r / rows_per_batch) * mask_stride_b + (r % mask_rows) * mask_stride_row.
-// COUNT: a wave walks the 4096/n rows of one compaction segment and also leaves the number of
+// COUNT = 1: a wave walks the 4096/n rows of one compaction segment and also leaves the number of
 // entries the compaction will keep (a > threshold, a != 0) in counts[segment], which saves
 // hyc_sparse_count's pass over the map.
-template <int CH, bool COUNT>
+// COUNT = 2: the same for row lengths that do not divide a segment (n <= 4096, a multiple of 8): a
+// wave's rows (at most 4096 elements) lie in at most two segments, a chunk of 8 never straddles
+// one, and the wave adds its two counts to counts[] with integer atomics (zeroed by the caller;
+// the sums do not depend on the order of the additions).
+template <int CH, int COUNT>
 __global__ __launch_bounds__(256) void softmax_fwd_kernel(const uint16_t* __restrict__ s, const uint16_t* __restrict__ mask,
                                                           uint16_t* __restrict__ out, int64_t rows, int n, float scale,
                                                           int mask_rows, int64_t rows_per_batch, int64_t mask_stride_b,
@@ -378,10 +382,16 @@ __global__ __launch_bounds__(256) void softmax_fwd_kernel(const uint16_t* __rest
     const int lane = threadIdx.x & (kWave - 1);
     const int64_t w = blockIdx.x * 4ll + (threadIdx.x >> 6);
     const int64_t row_begin = w * rows_per_wave;
-    if (row_begin >= rows) return;
+    __shared__ uint32_t wg_counts[COUNT == 2 ? 6 : 1];
+    if constexpr (COUNT == 2) {                     // every wave of the workgroup reaches both barriers
+        if (threadIdx.x < 6) wg_counts[threadIdx.x] = 0;
+        __syncthreads();
+    }
+    if (COUNT != 2 && row_begin >= rows) return;
     float thr = 0.0f;
-    if constexpr (COUNT) thr = rbf(*thr_p);
-    uint32_t cnt = 0;
+    if constexpr (COUNT != 0) thr = rbf(*thr_p);
+    uint32_t cnt = 0, cnt_next = 0;
+    const int64_t seg_first = (row_begin * n) / kSeg;
     for (int r = 0; r < rows_per_wave; ++r) {
         const int64_t row = row_begin + r;
         if (row >= rows) break;
@@ -434,18 +444,39 @@ __global__ __launch_bounds__(256) void softmax_fwd_kernel(const uint16_t* __rest
                 for (int j = 0; j < 8; ++j) t[c][j] *= inv;
                 const u32x4 ov = pack8(t[c]);
                 st16_nt(out + base + col, ov);
-                if constexpr (COUNT) {
+                if constexpr (COUNT != 0) {
                     const uint32_t d[4] = {ov.x, ov.y, ov.z, ov.w};
+                    uint32_t c8 = 0;
 #pragma unroll
-                    for (int j = 0; j < 8; ++j) cnt += keep((d[j >> 1] >> (16 * (j & 1))) & 0xffffu, thr) ? 1u : 0u;
+                    for (int j = 0; j < 8; ++j) c8 += keep((d[j >> 1] >> (16 * (j & 1))) & 0xffffu, thr) ? 1u : 0u;
+                    if (COUNT == 1 || (base + col) / kSeg == seg_first) cnt += c8;
+                    else cnt_next += c8;
                 }
             }
         }
     }
-    if constexpr (COUNT) {
+    if constexpr (COUNT != 0) {
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) cnt += (uint32_t)__shfl_xor((int)cnt, o, kWave);
-        if (lane == 0) counts[w] = cnt;
+        if constexpr (COUNT == 1) {
+            if (lane == 0) counts[w] = cnt;
+        } else {
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) cnt_next += (uint32_t)__shfl_xor((int)cnt_next, o, kWave);
+            // the workgroup's waves hold neighbouring rows, mostly of the same segments: their counts
+            // meet in LDS first (the workgroup's rows span at most 4 * 4096 elements, 5 segments) and
+            // one thread per segment adds to memory
+            const int64_t seg_wg = (blockIdx.x * 4ll * rows_per_wave * n) / kSeg;
+            if (lane == 0) {
+                if (cnt) atomicAdd(&wg_counts[seg_first - seg_wg], cnt);
+                if (cnt_next) atomicAdd(&wg_counts[seg_first + 1 - seg_wg], cnt_next);
+            }
+        }
+    }
+    if constexpr (COUNT == 2) {
+        __syncthreads();
+        if (threadIdx.x < 6 && wg_counts[threadIdx.x])
+            atomicAdd(&counts[(blockIdx.x * 4ll * rows_per_wave * n) / kSeg + threadIdx.x], wg_counts[threadIdx.x]);
     }
 }
 
@@ -525,6 +556,88 @@ __global__ __launch_bounds__(kSegThreads) void softmax_bwd_restore_kernel(const 
             for (int j = 0; j < 8; ++j) of[j] = rbf((gf[j] - acc) * yf[j]) * out_scale;   // bf16 result, then the bf16 scaling
             st16_nt(o_out + seg * kSeg + (int64_t)c * 8, pack8(of));       // ordinary stores: 166 against 149 us
             if (a_out) st16_nt(a_out + seg * kSeg + (int64_t)c * 8, yv[s]);
+        }
+    }
+}
+
+// The same for any row length n <= 4096 that is a multiple of 8 (sequence lengths that are not a
+// power of two): a wave takes the whole rows that fit into one stage of 4096 elements, which lie in
+// at most two segments of the compressed map; it walks the entries of those segments and keeps the
+// ones that fall into its rows.  A row is STEPS = ceil(n / 512) wave-wide steps, lanes past the end
+// of the row idle; chunk c of a row belongs to lane c % 64 as in softmax_bwd_kernel, so the row sums
+// are added in the same order and the results are the same bits as restore followed by that kernel.
+template <int STEPS, int NRMAX>
+__global__ __launch_bounds__(kSegThreads) void softmax_bwd_restore_rows_kernel(const int64_t* __restrict__ idx,
+                                                                               const uint16_t* __restrict__ val,
+                                                                               const int64_t* __restrict__ offsets,
+                                                                               const uint16_t* __restrict__ g, int64_t rows,
+                                                                               int n, int rows_per_wave,
+                                                                               uint16_t* __restrict__ a_out,
+                                                                               uint16_t* __restrict__ o_out, float out_scale) {
+    // NRMAX bounds rows_per_wave (the host chooses both from n), so that the gradient of all the wave's
+    // rows can be requested before the rebuild, as in the kernel above.
+    __shared__ __attribute__((aligned(16))) uint16_t stage[kSegThreads / kWave][kSeg];
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x >> 6;
+    const int64_t r0 = (blockIdx.x * (int64_t)(kSegThreads / kWave) + wave) * rows_per_wave;
+    if (r0 >= rows) return;                                  // waves share nothing: no workgroup barrier below
+    const int nr = rows - r0 < rows_per_wave ? (int)(rows - r0) : rows_per_wave;
+    const int cpr = n / 8;                                   // chunks per row
+    const int64_t flat0 = r0 * n;
+    const int span = nr * n;
+    u32x4 gall[NRMAX][STEPS];
+#pragma unroll
+    for (int r = 0; r < NRMAX; ++r)
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) {
+            const int c = s * kWave + lane;
+            gall[r][s] = u32x4{0, 0, 0, 0};
+            if (r < nr && c < cpr) gall[r][s] = ld16_nt(g + flat0 + (int64_t)r * n + c * 8);
+        }
+    u32x4* st = reinterpret_cast<u32x4*>(stage[wave]);
+    for (int c = lane; c < nr * cpr; c += kWave) st[c] = u32x4{0, 0, 0, 0};
+    const int64_t seg_a = flat0 / kSeg, seg_b = (flat0 + span - 1) / kSeg;
+    const int64_t e0 = offsets[seg_a], e1 = offsets[seg_b + 1];
+    // a wave's LDS operations are carried out in the order it issues them: the zeros above land first
+    for (int64_t e = e0 + lane; e < e1; e += kWave) {
+        const int64_t rel = idx[e] - flat0;
+        if (rel >= 0 && rel < span) stage[wave][rel] = val[e];
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int r = 0; r < NRMAX; ++r) {
+        if (r >= nr) break;                                  // uniform over the wave
+        const int64_t row_at = flat0 + (int64_t)r * n;
+        u32x4 yv[STEPS];
+        float acc = 0.0f;
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) {
+            const int c = s * kWave + lane;
+            yv[s] = u32x4{0, 0, 0, 0};
+            if (c < cpr) yv[s] = st[r * cpr + c];
+        }
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) {
+            float yf[8], gf[8];
+            unpack8(yv[s], yf);
+            unpack8(gall[r][s], gf);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc += rbf(yf[j] * gf[j]);
+        }
+        acc = wave_sum(acc);
+#pragma unroll
+        for (int s = 0; s < STEPS; ++s) {
+            const int c = s * kWave + lane;
+            if (c >= cpr) continue;
+            float yf[8], gf[8], of[8];
+            unpack8(yv[s], yf);
+            unpack8(gall[r][s], gf);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) of[j] = rbf((gf[j] - acc) * yf[j]) * out_scale;
+            st16_nt(o_out + row_at + c * 8, pack8(of));
+            if (a_out) st16_nt(a_out + row_at + c * 8, yv[s]);
         }
     }
 }
@@ -703,12 +816,36 @@ extern "C" int hyc_softmax_bwd(const void* y, const void* grad_y, void* out, int
 extern "C" int hyc_softmax_bwd_restore(const int64_t* indices, const void* values, const int64_t* seg_offsets,
                                        const void* grad_y, void* a_out, void* out, int64_t rows, int64_t n,
                                        float out_scale, void* stream) {
-    if (rows < 0 || n < 0) return HYC_ERR_SHAPE;
-    if (n != 512 && n != 1024 && n != 2048 && n != 4096) return HYC_ERR_SHAPE;
+    if (rows < 0 || n < 8 || n > 4096 || n % 8 != 0) return HYC_ERR_SHAPE;
     if (rows == 0) return HYC_OK;
-    if ((rows * n) % kSeg != 0) return HYC_ERR_SHAPE;
     if (!seg_offsets || !grad_y || !out) return HYC_ERR_NULL;
     if (!aligned16(grad_y) || !aligned16(out) || (a_out && !aligned16(a_out))) return HYC_ERR_ALIGN;
+    if ((n != 512 && n != 1024 && n != 2048 && n != 4096) || (rows * n) % kSeg != 0) {
+        // rows that do not tile the segments of the map
+        // rows per wave: what fits one 4096-element stage, at most 8 (short rows leave lanes idle instead)
+        const int steps = (int)cdiv(n, (int64_t)kWave * 8);
+        const int rpw = kSeg / n > 8 ? 8 : (int)(kSeg / n);
+        const int64_t waves = cdiv(rows, (int64_t)rpw);
+        if (cdiv(waves, 4) > INT32_MAX) return HYC_ERR_SHAPE;
+        const dim3 grid((unsigned)cdiv(waves, 4)), block(kSegThreads);
+        hipStream_t st = (hipStream_t)stream;
+#define HYC_SBR(STEPS, NRMAX)                                                                                   \
+        hipLaunchKernelGGL((softmax_bwd_restore_rows_kernel<STEPS, NRMAX>), grid, block, 0, st, indices,        \
+                           (const uint16_t*)values, seg_offsets, (const uint16_t*)grad_y, rows, (int)n, rpw,    \
+                           (uint16_t*)a_out, (uint16_t*)out, out_scale)
+        switch (steps) {                                    // NRMAX = the largest rpw of that range of n
+            case 1: HYC_SBR(1, 8); break;                   // n <= 512
+            case 2: HYC_SBR(2, 7); break;                   // 520 .. 1024: 7 .. 4 rows
+            case 3: HYC_SBR(3, 3); break;                   // 1032 .. 1536: 3 or 2
+            case 4: HYC_SBR(4, 2); break;                   // 1544 .. 2048
+            case 5: HYC_SBR(5, 1); break;
+            case 6: HYC_SBR(6, 1); break;
+            case 7: HYC_SBR(7, 1); break;
+            default: HYC_SBR(8, 1); break;
+        }
+#undef HYC_SBR
+        return check_launch();
+    }
     const int64_t nseg = rows * n / kSeg;
     if (cdiv(nseg, 4) > INT32_MAX) return HYC_ERR_SHAPE;
     const dim3 grid((unsigned)cdiv(nseg, 4)), block(kSegThreads);
@@ -731,7 +868,13 @@ extern "C" int hyc_softmax_fwd(const void* s, const void* mask, void* out, int64
     if (n % 8 != 0 || n > 8192) return HYC_ERR_SHAPE;
     const bool count = threshold || seg_counts || seg_offsets;
     if (count && !(threshold && seg_counts && seg_offsets)) return HYC_ERR_NULL;
-    if (count && (n < 512 || kSeg % n != 0 || (rows * n) % kSeg != 0)) return HYC_ERR_SHAPE;
+    if (count && n > kSeg) return HYC_ERR_SHAPE;
+    // rows that tile the segments: one count per wave; otherwise atomic sums into zeroed counts
+#ifdef HYC_FORCE_GENERAL
+    const bool tiled = false;
+#else
+    const bool tiled = count && n >= 512 && kSeg % n == 0 && (rows * n) % kSeg == 0;
+#endif
     if (rows == 0 || n == 0) {
         if (count) hipLaunchKernelGGL(seg_scan_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, seg_counts, (int64_t)0, seg_offsets);
         return count ? check_launch() : HYC_OK;
@@ -744,7 +887,13 @@ extern "C" int hyc_softmax_fwd(const void* s, const void* mask, void* out, int64
     } else {
         mask_rows = rows_per_batch = 1;
     }
-    const int rpw = count ? (int)(kSeg / n) : 1;
+    const int rpw = tiled ? (int)(kSeg / n) : 1;
+    const int64_t nseg = count ? cdiv(rows * n, (int64_t)kSeg) : 0;
+    if (count && !tiled) {
+        const int64_t fb = cdiv(nseg, 256);
+        hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)(fb > 1024 ? 1024 : fb)), dim3(256), 0, (hipStream_t)stream,
+                           seg_counts, nseg, 0u);
+    }
     const int64_t waves = cdiv(rows, (int64_t)rpw);
     if (cdiv(waves, 4) > INT32_MAX) return HYC_ERR_SHAPE;
     const dim3 grid((unsigned)cdiv(waves, 4)), block(256);
@@ -754,11 +903,14 @@ extern "C" int hyc_softmax_fwd(const void* s, const void* mask, void* out, int64
     uint16_t* op = (uint16_t*)out;
 #define HYC_SMF(CH)                                                                                                     \
     do {                                                                                                                \
-        if (count)                                                                                                      \
-            hipLaunchKernelGGL((softmax_fwd_kernel<CH, true>), grid, block, 0, st, sp, mp, op, rows, (int)n, scale,      \
+        if (tiled)                                                                                                      \
+            hipLaunchKernelGGL((softmax_fwd_kernel<CH, 1>), grid, block, 0, st, sp, mp, op, rows, (int)n, scale,         \
+                               (int)mask_rows, rows_per_batch, mask_stride_b, mask_stride_row, threshold, seg_counts, rpw); \
+        else if (count)                                                                                                 \
+            hipLaunchKernelGGL((softmax_fwd_kernel<CH, 2>), grid, block, 0, st, sp, mp, op, rows, (int)n, scale,         \
                                (int)mask_rows, rows_per_batch, mask_stride_b, mask_stride_row, threshold, seg_counts, rpw); \
         else                                                                                                            \
-            hipLaunchKernelGGL((softmax_fwd_kernel<CH, false>), grid, block, 0, st, sp, mp, op, rows, (int)n, scale,     \
+            hipLaunchKernelGGL((softmax_fwd_kernel<CH, 0>), grid, block, 0, st, sp, mp, op, rows, (int)n, scale,         \
                                (int)mask_rows, rows_per_batch, mask_stride_b, mask_stride_row, threshold, seg_counts, rpw); \
     } while (0)
     if (n <= 512) HYC_SMF(1);
@@ -768,7 +920,6 @@ extern "C" int hyc_softmax_fwd(const void* s, const void* mask, void* out, int64
     else HYC_SMF(16);
 #undef HYC_SMF
     if (count) {
-        const int64_t nseg = rows * n / kSeg;
         hipLaunchKernelGGL(seg_scan_kernel, dim3((unsigned)(nseg > 1024 ? cdiv(nseg, 1024) : 1)), dim3(1024), 0, st, seg_counts, nseg, seg_offsets);
     }
     return check_launch();

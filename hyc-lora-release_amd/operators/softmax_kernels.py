@@ -20,13 +20,17 @@ def softmax_backward(y: torch.Tensor, grad_y: torch.Tensor) -> torch.Tensor:
     return o
 
 
-FUSED_ROW_LENGTHS = (512, 1024, 2048, 4096)
+def fused_row_length(n: int) -> bool:
+    """Row lengths the one-pass kernels take (the kept-entry count inside softmax_forward, restore +
+    backward in softmax_backward_from_compressed): multiples of 8 up to 4096.  512, 1024, 2048 and
+    4096 tile the 4096-element segments of the compressed map and run the tuned forms."""
+    return 8 <= n <= 4096 and n % 8 == 0
 
 
 def softmax_backward_from_compressed(idx, val, seg_offsets, grad_y, want_map=True, out_scale=1.0):
     """(restored map or None, softmax backward) straight from a compressed attention map
     (`compress_attention_map`) and the upstream gradient `grad_y` of the map's shape [..., n].
-    One pass instead of restore + backward when n is 512, 1024, 2048 or 4096; other row lengths
+    One pass instead of restore + backward when n is a multiple of 8 up to 4096; other row lengths
     take the two-kernel route.  `out_scale` multiplies the bf16 gradient (and rounds again), which
     is what the layers' `grad_s = grad_s / math.sqrt(head_dim)` does on the device."""
     from .compress_function import restore_attention_map
@@ -36,7 +40,7 @@ def softmax_backward_from_compressed(idx, val, seg_offsets, grad_y, want_map=Tru
     shape = tuple(grad_y.shape)
     n = shape[-1]
     numel = grad_y.numel()
-    if n not in FUSED_ROW_LENGTHS or numel % 4096 or numel == 0:
+    if not fused_row_length(n) or numel == 0:
         a = restore_attention_map(idx, val, seg_offsets, shape)
         o = softmax_backward(a, grad_y)
         return (a if want_map else None), (o if out_scale == 1.0 else o * out_scale)
@@ -49,9 +53,6 @@ def softmax_backward_from_compressed(idx, val, seg_offsets, grad_y, want_map=Tru
               seg_offsets.data_ptr(), grad_y.data_ptr(), _lib.ptr(a), o.data_ptr(), numel // n, n,
               float(out_scale), _lib.stream_of(grad_y))
     return a, o
-
-
-COUNTED_ROW_LENGTHS = FUSED_ROW_LENGTHS
 
 
 def softmax_forward(s, scale, mask=None, threshold=None, inplace=False):
@@ -87,10 +88,10 @@ def softmax_forward(s, scale, mask=None, threshold=None, inplace=False):
         mptr, mask_rows, rows_per_batch = mask.data_ptr(), s.shape[2], s.shape[1] * s.shape[2]
         msb, msr = (mask.stride(0) if mask.shape[0] > 1 else 0), mask.stride(2)
     counts = offsets = thr = None
-    if threshold is not None and n in COUNTED_ROW_LENGTHS and s.numel() % 4096 == 0 and s.numel():
+    if threshold is not None and fused_row_length(n) and s.numel():
         from .compress_function import _threshold_tensor
         thr = _threshold_tensor(threshold, s.device)
-        nseg = s.numel() // 4096
+        nseg = -(-s.numel() // 4096)
         counts = torch.empty(nseg, device=s.device, dtype=torch.int32)
         offsets = torch.empty(nseg + 1, device=s.device, dtype=torch.int64)
     _lib.call("hyc_softmax_fwd", s.data_ptr(), mptr, out.data_ptr(), rows, n, float(scale), mask_rows, rows_per_batch,

@@ -225,8 +225,11 @@ int hyc_softmax_bwd(const void *y, const void *grad_y, void *out, int64_t rows, 
  *             mask for all batches, stride_row = 0 one mask row for all queries, as a padding mask).
  *   threshold, seg_counts, seg_offsets   all NULL, or all given: then seg_counts / seg_offsets are
  *             filled exactly as hyc_sparse_count(out, rows*n, threshold, ...) would fill them, without
- *             another pass over the map.  Needs n in {512,1024,2048,4096} and rows*n % 4096 == 0
- *             (otherwise HYC_ERR_SHAPE: call hyc_sparse_count afterwards instead).
+ *             another pass over the map (seg_counts holds ceil(rows*n / 4096) counters).  Needs
+ *             n <= 4096 (otherwise HYC_ERR_SHAPE: call hyc_sparse_count afterwards instead).  Rows of
+ *             512, 1024, 2048 or 4096 elements with rows*n % 4096 == 0 tile the segments and give one
+ *             count per wave; other row lengths add their counts with integer atomics into counters
+ *             the call zeroes first (one more small launch; the result is the same).
  */
 int hyc_softmax_fwd(const void *s, const void *mask, void *out, int64_t rows, int64_t n, float scale,
                     int64_t mask_rows, int64_t rows_per_batch, int64_t mask_stride_b, int64_t mask_stride_row,
@@ -244,8 +247,11 @@ int hyc_softmax_fwd(const void *s, const void *mask, void *out, int64_t rows, in
  *   out_scale     the bf16 gradient is multiplied by this and rounded again: 1.0f, or 1/sqrt(head_dim) to fold
  *                 in the layer's grad_s = grad_s / math.sqrt(head_dim) (…full_fuse.py:436; a multiplication by
  *                 the fp32 reciprocal in torch's device kernel);
- *   n in {512, 1024, 2048, 4096} and rows*n a multiple of 4096; other shapes: HYC_ERR_SHAPE (use
- *   hyc_sparse_restore + hyc_softmax_bwd).
+ *   n a multiple of 8, 8 <= n <= 4096; other row lengths: HYC_ERR_SHAPE (use hyc_sparse_restore +
+ *   hyc_softmax_bwd).  Rows of 512, 1024, 2048 or 4096 elements with rows*n % 4096 == 0 tile the
+ *   map's segments (one segment per wave); for other shapes a wave takes the whole rows that fit
+ *   into 4096 elements and filters the entries of the one or two segments they lie in.  Either way
+ *   the results are the bits of hyc_sparse_restore followed by hyc_softmax_bwd.
  */
 int hyc_softmax_bwd_restore(const int64_t *indices, const void *values, const int64_t *seg_offsets,
                             const void *grad_y, void *a_out, void *out, int64_t rows, int64_t n,

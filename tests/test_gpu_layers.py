@@ -229,7 +229,8 @@ def test_layer_matches_oracle_layer(dev, layer_type, q_bit, kv_heads):
                                   dict(B=2, S=48, hidden=256, heads=2, kv_heads=1, inter=256, rank=16)])   # heads of 128 dims: rotation fused into the LoRA add
 def test_layer_on_ragged_shapes(dev, layer_type, dims):
     """Shapes that fill none of the kernels' tiles evenly (rows not a multiple of 16 or 256, widths
-    not a multiple of 128, a sequence length the fused softmax does not take, ranks 4 / 8 / 32):
+    not a multiple of 128, sequence lengths the one-pass softmax kernels take in their row-group form
+    (40, 48, 264) or not at all (17), ranks 4 / 8 / 32):
     every layer type against the oracle layer (baseline: against autograd of the same graph)."""
     import hyclora_amd  # noqa: F401
     from hyclora_amd.models import llama
@@ -388,9 +389,10 @@ def test_frozen_statistics_path_equals_calibrating_path(dev, layer_type, q_bit):
     frozen statistics equal the fresh ones, so the two code paths must agree bit for bit."""
     import hyclora_amd  # noqa: F401
     from hyclora_amd.models.llama import make_fused_llama_layer
-    t = make_layer_inputs(dev, seed=31, S=128, hidden=512, heads=4, kv_heads=4, inter=1024)   # rows of 128: not counted in the softmax pass
-    t2 = make_layer_inputs(dev, seed=32, S=512, hidden=256, heads=2, kv_heads=2, inter=512)   # rows of 512: counted
-    for tt in (t, t2):
+    t = make_layer_inputs(dev, seed=31, S=128, hidden=512, heads=4, kv_heads=4, inter=1024)   # rows of 128: counted with atomic sums
+    t2 = make_layer_inputs(dev, seed=32, S=512, hidden=256, heads=2, kv_heads=2, inter=512)   # rows of 512: one count per wave
+    t3 = make_layer_inputs(dev, seed=33, S=200, hidden=256, heads=2, kv_heads=2, inter=512)   # rows that straddle the map's segments
+    for tt in (t, t2, t3):
         layer = make_fused_llama_layer(config(layer_type, q_bit, sm_ratio=0.05, thr=1))
         outs = []
         for it in range(2):
