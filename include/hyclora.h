@@ -51,7 +51,9 @@ int hyc_abi_version(void);
  * row count, the default),
  * "fuse_rows_per_wave" (same for both fused LoRA-SiLU kernels, multiple of 16; defaults: backward 32,
  * forward 0 = 96 for tensors of 2^24 elements and more, else 32;
- * "fuse_fwd_rows_per_wave" / "fuse_bwd_rows_per_wave" set one of them).  Unknown key or bad value: HYC_ERR_ARG.  No
+ * "fuse_fwd_rows_per_wave" / "fuse_bwd_rows_per_wave" set one of them),
+ * "contract_max_groups" (column groups hyc_lora_contract cuts a row strip into, default 32; changes the
+ * workspace hyc_lora_contract_workspace asks for).  Unknown key or bad value: HYC_ERR_ARG.  No
  * counterpart in the reference (its launch shapes come from triton.autotune). */
 int hyc_set_tuning(const char *key, int value);
 
