@@ -380,12 +380,26 @@ def compress_attention_map(x: torch.Tensor, outlier, seg_offsets=None, compare_a
     return idx, val, offsets
 
 
+def check_map_lists(idx, val, seg_offsets, numel: int) -> None:
+    """The kernels that rebuild a map read idx / val up to seg_offsets' last entry and seg_offsets up to
+    the map's last 4096-element segment: lists of another map would be read out of bounds on the device."""
+    if idx.dtype != torch.int64 or idx.numel() != val.numel():
+        raise ValueError(f"compressed map: int64 indices and as many values expected, got {idx.dtype} "
+                         f"x {idx.numel()} and {val.numel()} values")
+    if seg_offsets is not None:
+        nseg = -(-numel // 4096)
+        if seg_offsets.dtype != torch.int64 or seg_offsets.numel() != nseg + 1:
+            raise ValueError(f"seg_offsets must be int64 [{nseg + 1}] for a map of {numel} elements, got "
+                             f"{seg_offsets.dtype} [{seg_offsets.numel()}]")
+
+
 def restore_attention_map(idx, val, seg_offsets, shape):
     """Dense bf16 tensor of `shape`: zeros with val[i] at flat position idx[i]."""
-    _lib.require_gpu(idx, val)
     n = 1
     for d in shape:
         n *= int(d)
+    check_map_lists(idx, val, seg_offsets, n)
+    _lib.require_gpu(idx, val)
     idx = idx.reshape(-1).contiguous()
     val = val.to(BF16).reshape(-1).contiguous()
     st = _lib.stream_of(val)

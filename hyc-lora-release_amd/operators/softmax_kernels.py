@@ -33,13 +33,14 @@ def softmax_backward_from_compressed(idx, val, seg_offsets, grad_y, want_map=Tru
     One pass instead of restore + backward when n is a multiple of 8 up to 4096; other row lengths
     take the two-kernel route.  `out_scale` multiplies the bf16 gradient (and rounds again), which
     is what the layers' `grad_s = grad_s / math.sqrt(head_dim)` does on the device."""
-    from .compress_function import restore_attention_map
-    _lib.require_gpu(idx, val, seg_offsets, grad_y)
-    if grad_y.dtype != torch.bfloat16:
-        raise NotImplementedError("softmax backward computes in bfloat16")
+    from .compress_function import check_map_lists, restore_attention_map
     shape = tuple(grad_y.shape)
     n = shape[-1]
     numel = grad_y.numel()
+    check_map_lists(idx, val, seg_offsets, numel)
+    _lib.require_gpu(idx, val, seg_offsets, grad_y)
+    if grad_y.dtype != torch.bfloat16:
+        raise NotImplementedError("softmax backward computes in bfloat16")
     if not fused_row_length(n) or numel == 0:
         a = restore_attention_map(idx, val, seg_offsets, shape)
         o = softmax_backward(a, grad_y)

@@ -103,3 +103,16 @@ def test_channel_list_validation():
     for bad in ([64], [-1], [3, 3]):
         with pytest.raises(ValueError, match="outlier channel"):
             cf.validate_channel_list(torch.tensor(bad), 64)
+
+
+def test_compressed_map_lists_must_belong_to_the_map():
+    from hyclora_amd.operators import softmax_kernels as sk
+    g = t(1, 2, 40, 104)                                   # 8320 elements: 3 segments, 4 offsets
+    idx, val, seg = torch.zeros(5, dtype=torch.int64), t(5), torch.zeros(4, dtype=torch.int64)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        sk.softmax_backward_from_compressed(idx, val, seg, g)
+    for bad in ((idx[:4], val, seg), (idx.int(), val, seg), (idx, val, seg[:3]), (idx, val, seg.int())):
+        with pytest.raises(ValueError, match="compressed map|seg_offsets"):
+            sk.softmax_backward_from_compressed(*bad, g)
+        with pytest.raises(ValueError, match="compressed map|seg_offsets"):
+            cf.restore_attention_map(*bad, g.shape)
