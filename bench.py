@@ -108,12 +108,14 @@ def parse():
                     help="no GPU work: turn the rocprofv3 counter CSVs under DIR into profiles/quant_pack_q4_config2_hbm_traffic.json")
     ap.add_argument("--layer-case", default="", help="with --only layers: run only the cases whose name contains this")
     ap.add_argument("--layer-seq", type=int, default=0, help="with --only layers: sequence length instead of the configuration's")
+    ap.add_argument("--layer-dims", default="", help="with --only layers: override dimensions of the configuration, "
+                    "e.g. hidden=5120,heads=40,kv=40,inter=13824")
     ap.add_argument("--layer-arm", choices=["both", "plain", "compressed"], default="both",
                     help="with --only layers: run only one arm (for profiler runs)")
     return ap.parse_args()
 
 
-def bench_layers(torch, dev, only_case="", arm="both", seq=0):
+def bench_layers(torch, dev, only_case="", arm="both", seq=0, dims_override=None):
     """Forward+backward of one decoder layer with random-init bf16 weights N(0, 0.02) and LoRA r=16 on
     all seven linears: the compressed layer of this package against an uncompressed bf16
     torch-autograd layer of the same architecture, with the activation bytes each keeps for backward."""
@@ -235,6 +237,9 @@ def bench_layers(torch, dev, only_case="", arm="both", seq=0):
         if seq:                                       # another sequence length than the configuration's
             dims = dict(dims, S=seq)
             name = f"{name}_at_s{seq}"
+        if dims_override:                             # other widths (e.g. hidden=5120,heads=40,kv=40,inter=13824)
+            dims = dict(dims, **dims_override)
+            name = name + "_with_" + "_".join(f"{k}{v}" for k, v in sorted(dims_override.items()))
         t = make(**dims)
         mask = None if sdpa else torch.full((t.S, t.S), float("-inf"), device=dev).triu(1).to(BF16)[None, None]
         entry, saved_p, plain = {}, 0, None
@@ -939,7 +944,8 @@ def main():
         for buffers in (xs, qs, xh):
             buffers.clear()
         torch.cuda.empty_cache()
-        layers = bench_layers(torch, dev, args.layer_case, args.layer_arm, args.layer_seq)
+        layer_dims = {k: int(v) for k, v in (kv.split("=") for kv in args.layer_dims.split(",") if kv)}
+        layers = bench_layers(torch, dev, args.layer_case, args.layer_arm, args.layer_seq, layer_dims)
     stack = None
     if args.only in ("all", "stack"):
         for buffers in (xs, qs, xh):
