@@ -333,6 +333,11 @@ extern "C" int64_t hyc_rmsnorm_bwd_workspace(int64_t rows, int64_t N) {
     return (int64_t)bwd_blocks(rows, N) * N * (int64_t)sizeof(float);
 }
 
+namespace hyc {
+int rmsnorm_bwd_dense_slab(const void* dy, const void* x, const void* weight, int weight_is_fp32, const float* rstd,
+                           const void* residual, void* dx, int64_t rows, int64_t N, void* stream);   // norm_compress.hip
+}
+
 static int rmsnorm_bwd_any(const void* dy, const void* x, const void* weight, int weight_is_fp32, const float* rstd,
                            const void* residual, void* dx, void* dw, void* workspace, int64_t workspace_bytes,
                            int64_t rows, int64_t N, void* stream) {
@@ -356,6 +361,12 @@ static int rmsnorm_bwd_any(const void* dy, const void* x, const void* weight, in
         if (weight_is_fp32) hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel<true>, grid, block, 0, st, (const float*)workspace, blocks, (int)N, dw);
         else hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel<false>, grid, block, 0, st, (const float*)workspace, blocks, (int)N, dw);
         return check_launch();
+    }
+    // Rows longer than 4096 channels leave a row-per-wave kernel one or two waves per SIMD (3.4 - 3.9 TB/s);
+    // the column-slab kernel of the fused norm files takes them where the shape fits (same bits).
+    if (N > 4096) {
+        rc = hyc::rmsnorm_bwd_dense_slab(dy, x, weight, weight_is_fp32, rstd, residual, dx, rows, N, stream);
+        if (rc <= 0) return rc;
     }
     // without dw the grid need not be capped, but the same persistent loop is used
     return weight_is_fp32

@@ -400,6 +400,7 @@ void rmsnorm_fwd_compress_slab_kernel(const NormCompressArgs a, const XaArgs xa,
 // dense backward kernel's summation order, so dx is the same bits as from dequantise + backward.
 // Optionally adds the residual connection's gradient, like hyc_rmsnorm_bwd_add.
 struct NormBwdCodesArgs {
+    const uint16_t* x;                                  // the norm's input itself (QBIT = 0) instead of its compressed copy
     const uint16_t* dy; const uint8_t* q_x; const uint16_t* scale_x;
     const uint16_t* otable; const uint16_t* xo;
     const void* w; const float* rstd; const uint16_t* res; uint16_t* dx;
@@ -418,8 +419,12 @@ void rmsnorm_bwd_codes_slab_kernel(const NormBwdCodesArgs a, int rows_per_group)
     const int chunk = wave * kWave + lane;
     const int col = chunk * 8;
     const int N = a.N;
-    const int row_bytes = N * QBIT / 8;
-    constexpr float kHalf = (float)(1 << (QBIT - 1));
+    // QBIT = 0: x is read as it is (the stand-alone backward for rows longer than a wave holds well);
+    // everything after the load is the same code, so the results are the same bits
+    constexpr bool DENSE = QBIT == 0;
+    constexpr int QB = DENSE ? 8 : QBIT;
+    const int row_bytes = N * QB / 8;
+    constexpr float kHalf = (float)(1 << (QB - 1));
     const int64_t r0 = (int64_t)blockIdx.x * rows_per_group;
     int64_t r1 = r0 + rows_per_group;
     if (r1 > a.rows) r1 = a.rows;
@@ -445,11 +450,12 @@ void rmsnorm_bwd_codes_slab_kernel(const NormBwdCodesArgs a, int rows_per_group)
             unpack8(wp, out);
         }
     };
-    const u32x4 sp = ld16(a.scale_x + col);
+    u32x4 sp = {0, 0, 0, 0};
+    if constexpr (!DENSE) sp = ld16(a.scale_x + col);
     // Outlier columns of this lane: the first two are fetched ahead with the row (slots 1 and 2 of
     // `oslot`, two bits a column), any further one when it is used (slot 3).  Few lanes have any.
     u32x4 tv = {0, 0, 0, 0};
-    if (a.k > 0) tv = ld16(a.otable + col);
+    if (!DENSE && a.k > 0) tv = ld16(a.otable + col);
     const uint32_t td[4] = {tv.x, tv.y, tv.z, tv.w};
     uint32_t oslot = 0, opos0 = 0, opos1 = 0;
     {
@@ -465,10 +471,11 @@ void rmsnorm_bwd_codes_slab_kernel(const NormBwdCodesArgs a, int rows_per_group)
             }
         }
     }
-    const PackedSlot<QBIT> slot(chunk);
+    const PackedSlot<QB> slot(chunk);
     const float inv_n = 1.0f / (float)N;
 
     u32x2 cw[G];
+    u32x4 xd[DENSE ? G : 1];
     u32x4 gv[G];
     float rs[G];
     uint32_t ov[G][2];
@@ -476,10 +483,11 @@ void rmsnorm_bwd_codes_slab_kernel(const NormBwdCodesArgs a, int rows_per_group)
 #pragma unroll
         for (int g = 0; g < G; ++g) {
             const int64_t row = r + g;
-            cw[g] = ld8(a.q_x + row * row_bytes + slot.offset);
+            if constexpr (DENSE) xd[g] = ld16_nt(a.x + row * N + col);
+            else cw[g] = ld8(a.q_x + row * row_bytes + slot.offset);
             gv[g] = ld16_nt(a.dy + row * N + col);
             rs[g] = a.rstd[row];
-            if (oslot) {
+            if (!DENSE && oslot) {
                 ov[g][0] = a.xo[row * a.k + opos0];
                 if (oslot & 0xaaaau) ov[g][1] = a.xo[row * a.k + opos1];        // a second outlier column
             }
@@ -495,12 +503,15 @@ void rmsnorm_bwd_codes_slab_kernel(const NormBwdCodesArgs a, int rows_per_group)
 #pragma unroll
         for (int g = 0; g < G; ++g) {
             float c[8], gf[8], x[8], sf[8], w8[8];
-            slot.decode(cw[g], c);
             unpack8(gv[g], gf);
-            unpack8(sp, sf);
             weight8(w8);
             gp[g] = gv[g];
             rstd[g] = rs[g];
+            if constexpr (DENSE) {
+                xp[g] = xd[g];
+            } else {
+            slot.decode(cw[g], c);
+            unpack8(sp, sf);
 #pragma unroll
             for (int j = 0; j < 8; ++j) x[j] = (c[j] - kHalf) * sf[j];  // the dequantiser's arithmetic ...
             if (oslot) {
@@ -516,6 +527,7 @@ void rmsnorm_bwd_codes_slab_kernel(const NormBwdCodesArgs a, int rows_per_group)
                 }
             }
             xp[g] = pack8(x);                                           // ... and its rounding to bf16
+            }
             unpack8(xp[g], x);
             float p1 = 0.0f, p2 = 0.0f;
 #pragma unroll
@@ -741,22 +753,9 @@ extern "C" int hyc_rmsnorm_fwd_compress_lora(const void* x, const void* weight, 
                              x_outlier, xa, stream);
 }
 
-extern "C" int hyc_rmsnorm_bwd_codes(const void* dy, const void* q_x, const void* scale_x, const uint16_t* outlier_table,
-                                     int64_t k, const void* x_outlier, int q_bit, const void* weight, int weight_is_fp32,
-                                     const float* rstd, const void* residual, void* dx, int64_t rows, int64_t N,
-                                     void* stream) {
-    if (q_bit != 2 && q_bit != 4 && q_bit != 8) return HYC_ERR_QBIT;
-    if (rows < 0 || N < 0 || k < 0 || k > 65535) return HYC_ERR_SHAPE;
-    if (N % (kWave * 8) != 0 || N / (kWave * 8) > 16 || rows % kSlabRows != 0) return HYC_ERR_SHAPE;
-    if (rows == 0 || N == 0) return HYC_OK;
-    if (!dy || !q_x || !scale_x || !weight || !rstd || !dx || (k > 0 && (!outlier_table || !x_outlier))) return HYC_ERR_NULL;
-    if (!aligned16(dy) || !aligned16(scale_x) || !aligned16(weight) || !aligned16(dx) || !aligned16(residual) ||
-        (outlier_table && !aligned16(outlier_table)) || (reinterpret_cast<uintptr_t>(q_x) & 7u))
-        return HYC_ERR_ALIGN;
-    NormBwdCodesArgs a;
-    a.dy = (const uint16_t*)dy; a.q_x = (const uint8_t*)q_x; a.scale_x = (const uint16_t*)scale_x;
-    a.otable = outlier_table; a.xo = (const uint16_t*)x_outlier; a.w = weight; a.rstd = rstd;
-    a.res = (const uint16_t*)residual; a.dx = (uint16_t*)dx; a.rows = rows; a.N = (int)N; a.k = (int)k;
+// Shared launch of the slab backward: q_bit 2 / 4 / 8 = x from its codes, 0 = x itself.
+static int launch_bwd_slab(const NormBwdCodesArgs& a, int q_bit, int weight_is_fp32, hipStream_t st) {
+    const int64_t rows = a.rows;
     const int waves = a.N / (kWave * 8);
     int rows_per_group = g_slab_rows_per_group;
     if (rows_per_group == 0) {
@@ -767,7 +766,6 @@ extern "C" int hyc_rmsnorm_bwd_codes(const void* dy, const void* q_x, const void
     if (groups > INT32_MAX) return HYC_ERR_SHAPE;
     const size_t lds = 2 * kSlabRows * 2 * waves * kWave * sizeof(float);
     const dim3 grid((unsigned)groups), block(waves * kWave);
-    hipStream_t st = (hipStream_t)stream;
 #define HYC_NBC(QB, W32, MAXW)                                                                                          \
     do {                                                                                                                \
         if (a.res) hipLaunchKernelGGL((rmsnorm_bwd_codes_slab_kernel<QB, W32, MAXW, true>), grid, block, lds, st, a, rows_per_group); \
@@ -780,8 +778,41 @@ extern "C" int hyc_rmsnorm_bwd_codes(const void* dy, const void* q_x, const void
     } while (0)
     if (q_bit == 8) HYC_NBC_W(8);
     else if (q_bit == 4) HYC_NBC_W(4);
-    else HYC_NBC_W(2);
+    else if (q_bit == 2) HYC_NBC_W(2);
+    else HYC_NBC_W(0);
 #undef HYC_NBC_W
 #undef HYC_NBC
     return check_launch();
+}
+
+namespace hyc {
+// RMSNorm backward (dx only) of a dense input in the column-slab form; norm.hip sends rows longer than
+// 4096 channels here.  Returns 1 when the shape does not fit the slabs (the caller keeps its own kernel).
+int rmsnorm_bwd_dense_slab(const void* dy, const void* x, const void* weight, int weight_is_fp32, const float* rstd,
+                           const void* residual, void* dx, int64_t rows, int64_t N, void* stream) {
+    if (!slab_shape(rows, N)) return 1;
+    NormBwdCodesArgs a{};
+    a.x = (const uint16_t*)x; a.dy = (const uint16_t*)dy; a.w = weight; a.rstd = rstd;
+    a.res = (const uint16_t*)residual; a.dx = (uint16_t*)dx; a.rows = rows; a.N = (int)N; a.k = 0;
+    return launch_bwd_slab(a, 0, weight_is_fp32, (hipStream_t)stream);
+}
+}  // namespace hyc
+
+extern "C" int hyc_rmsnorm_bwd_codes(const void* dy, const void* q_x, const void* scale_x, const uint16_t* outlier_table,
+                                     int64_t k, const void* x_outlier, int q_bit, const void* weight, int weight_is_fp32,
+                                     const float* rstd, const void* residual, void* dx, int64_t rows, int64_t N,
+                                     void* stream) {
+    if (q_bit != 2 && q_bit != 4 && q_bit != 8) return HYC_ERR_QBIT;
+    if (rows < 0 || N < 0 || k < 0 || k > 65535) return HYC_ERR_SHAPE;
+    if (N % (kWave * 8) != 0 || N / (kWave * 8) > 16 || rows % kSlabRows != 0) return HYC_ERR_SHAPE;
+    if (rows == 0 || N == 0) return HYC_OK;
+    if (!dy || !q_x || !scale_x || !weight || !rstd || !dx || (k > 0 && (!outlier_table || !x_outlier))) return HYC_ERR_NULL;
+    if (!aligned16(dy) || !aligned16(scale_x) || !aligned16(weight) || !aligned16(dx) || !aligned16(residual) ||
+        (outlier_table && !aligned16(outlier_table)) || (reinterpret_cast<uintptr_t>(q_x) & 7u))
+        return HYC_ERR_ALIGN;
+    NormBwdCodesArgs a{};
+    a.dy = (const uint16_t*)dy; a.q_x = (const uint8_t*)q_x; a.scale_x = (const uint16_t*)scale_x;
+    a.otable = outlier_table; a.xo = (const uint16_t*)x_outlier; a.w = weight; a.rstd = rstd;
+    a.res = (const uint16_t*)residual; a.dx = (uint16_t*)dx; a.rows = rows; a.N = (int)N; a.k = (int)k;
+    return launch_bwd_slab(a, q_bit, weight_is_fp32, (hipStream_t)stream);
 }

@@ -90,7 +90,7 @@ def test_elementwise_extremes(ops, dev):
         assert torch.isfinite(o).all() and torch.allclose(o, r, atol=1e-2, rtol=1e-2)
 
 
-@pytest.mark.parametrize("n", [4096, 512, 96, 1024, 8192, 16384, 2048 + 64])
+@pytest.mark.parametrize("n", [4096, 512, 96, 1024, 8192, 16384, 2048 + 64, 3072, 5120, 6144, 7168])
 @pytest.mark.parametrize("wdtype", [BF16, torch.float32])
 def test_rmsnorm_forward(ops, dev, n, wdtype):
     g = torch.Generator().manual_seed(n)
@@ -108,7 +108,7 @@ def test_rmsnorm_forward(ops, dev, n, wdtype):
     assert_close_bf16(y, ref, what="rmsnorm_forward vs fp64 formula")
 
 
-@pytest.mark.parametrize("n", [4096, 512, 96, 1024, 8192])
+@pytest.mark.parametrize("n", [4096, 512, 96, 1024, 8192, 3072, 5120, 7168, 6144 + 8])   # beyond 4096: even row counts take the column-slab kernel
 @pytest.mark.parametrize("rows", [(2, 33), (1, 1), (4, 300)])
 def test_rmsnorm_backward(ops, dev, n, rows):
     g = torch.Generator().manual_seed(n + rows[1])
