@@ -22,9 +22,12 @@ Pinning status (what independent evidence holds each function in place):
     by unit row sums, exact zeros under a -inf mask and shift invariance.
   * softmax_bwd, rmsnorm_fwd, silu_*, gelu_bwd, fused_*: pinned to tolerance against
     torch.autograd of the fp32 composite.  rmsnorm_bwd follows the reference's
-    formula (which keeps LayerNorm's mean term) and is pinned only against a
-    float64 evaluation of that same formula and against autograd for inputs where the
-    extra term vanishes: "parity unpinned" for the c2 term beyond reading the source.
+    formula, which keeps LayerNorm's mean term c2 = mean(w * dy).  That term is pinned on rows
+    whose mean is exactly zero (built as v | -v): there the formula IS the backward of
+    F.layer_norm, so the oracle must equal float64 autograd of layer_norm and must differ
+    from autograd of a true RMSNorm by exactly c2 * rstd - a dropped or sign-flipped term
+    fails both (tests/test_oracle_norm.py; the same check on the GPU kernel in
+    tests/test_gpu_elementwise_norm.py).
   * layernorm_fwd / layernorm_bwd: pinned against torch.nn.functional.layer_norm and its
     autograd in float64 (an independent library routine), tests/test_oracle_layernorm.py.
   * nf4_dequant: bitsandbytes (0.43.2, pinned in the reference's requirements.txt) is not installed,
