@@ -121,6 +121,7 @@ def rmsnorm_backward_from_codes(dy, q_x, scale_x, x_outlier, outlier_idx, q_bit,
     k = 0 if outlier_idx is None else int(outlier_idx.numel())
     if k and table is None:
         table = outlier_table(outlier_idx, n, cached=True)
+    _check_table(table, n, k)
     if q_x.dtype != torch.uint8 or q_x.numel() != rows * n * q_bit // 8:
         raise ValueError("q_x does not hold the packed codes of a tensor of dy's shape")
     q_x = q_x.contiguous()
@@ -152,6 +153,13 @@ def rmsnorm_backward(dy, x, w, m, v, needs_inputs_grad, eps, num_warps, BLOCK_SI
         return None, None
     dx, _ = _backward(dy, x, w, v, want_dw=False, residual=residual)
     return dx, None
+
+
+def _check_table(table, n, k):
+    """A table handed in by the caller is read with one entry per channel."""
+    if k and (table.dtype != torch.int16 or table.numel() != n or not table.is_contiguous()):
+        raise ValueError(f"outlier table must be a contiguous int16 [{n}] (outlier_table(idx, {n})), got "
+                         f"{table.dtype} {tuple(table.shape)}")
 
 
 _TABLES = {}          # id(channel-list tensor) -> (weak reference to it, its version, n, table)
@@ -256,6 +264,7 @@ def rmsnorm_forward_compress(x, weight, eps, q_bit, scale_y=None, scale_x=None, 
         x_out = torch.empty((b, m, k), dtype=torch.bfloat16, device=dev)
         if k and table is None:
             table = outlier_table(outlier_idx, n, cached=True)
+        _check_table(table, n, k)
     if lora_a is not None:
         import ctypes
         if not lora_a_supported(x, weight, lora_a):
