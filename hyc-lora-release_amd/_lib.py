@@ -26,7 +26,7 @@ class HycError(RuntimeError):
 
 
 # name -> (restype, argtypes)
-ABI_VERSION = 5          # hyc_abi_version() of the library these signatures describe
+ABI_VERSION = 6          # hyc_abi_version() of the library these signatures describe
 _P, _I, _L = c_void_p, c_int, c_int64
 _SIGNATURES = {
     "hyc_error_string": (c_char_p, [_I]),
@@ -64,6 +64,7 @@ _SIGNATURES = {
     "hyc_rmsnorm_bwd_codes": (_I, [_P, _P, _P, _P, _L, _P, _I, _P, _I, _P, _P, _P, _L, _L, _P]),
     "hyc_silu_bwd": (_I, [_P, _P, _P, _L, _P]),
     "hyc_silu_mul": (_I, [_P, _P, _P, _L, _P]),
+    "hyc_silu_once_mul": (_I, [_P, _P, _P, _L, _P]),
     "hyc_silu_mul_bwd": (_I, [_P, _P, _P, _P, _P, _L, _P]),
     "hyc_gelu_bwd": (_I, [_P, _P, _P, _L, _P]),
     "hyc_lora_silu_mul_fwd": (_I, [_P] * 11 + [_L, _L, _L, _I, _I, _P]),

@@ -27,6 +27,11 @@ struct SiluMul {   // o = (sig(x1) * x1) * x2
         return rbf(rbf(sigmoidf_(x1)) * x1) * x2;
     }
 };
+struct SiluOnceMul {   // o = bf16(silu(x1)) * x2 with silu evaluated in fp32 and rounded once, as torch's F.silu
+    __device__ __forceinline__ float operator()(float x1, float x2) const {
+        return rbf(x1 * sigmoidf_(x1)) * x2;
+    }
+};
 struct GeluBwd {   // d/dx of 0.5 x (1 + tanh(gamma (x + kappa x^3))), times g; fp32 throughout
     __device__ __forceinline__ float operator()(float x, float g) const {
         constexpr float gamma = 0.7978845608028654f, kappa = 0.044715f;
@@ -71,16 +76,17 @@ __global__ __launch_bounds__(kEwThreads) void binary_kernel(const uint16_t* __re
 }
 
 // Backward of o = silu(x) * u in one pass: grad_x = silu_backward(x, bf16(g * u)) and
-// grad_u = g * silu(x), with silu(x) = bf16(bf16(sig(x)) * x) as SiluMul forms it.  The layers that do
-// not use the fused LoRA kernels compute this with F.silu, two products and silu_backward
-// (models/llama/fused_llama_layer_intra_inter.py:361-381, whose comment asks for this kernel).
+// grad_u = g * silu(x), with silu(x) = bf16(x * sig(x)) evaluated in fp32 and rounded once - what
+// torch.nn.functional.silu gives.  The layers that do not use the fused LoRA kernels compute exactly
+// this with F.silu, two products and silu_backward
+// (models/llama/fused_llama_layer_intra_inter.py:362-381, whose comment asks for this kernel).
 __global__ __launch_bounds__(kEwThreads) void silu_mul_bwd_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ u,
                                                                   const uint16_t* __restrict__ g, uint16_t* __restrict__ gx,
                                                                   uint16_t* __restrict__ gu, int64_t n) {
     const SiluBwd dsilu;
     auto one = [&](float xf, float uf, float gf, float& ox, float& ou) {
         ox = dsilu(xf, rbf(gf * uf));
-        ou = gf * rbf(rbf(sigmoidf_(xf)) * xf);
+        ou = gf * rbf(xf * sigmoidf_(xf));
     };
     const int64_t chunks = n / 8;
     constexpr int kUnroll = 2;
@@ -140,6 +146,9 @@ extern "C" int hyc_silu_bwd(const void* x, const void* g, void* out, int64_t n, 
 }
 extern "C" int hyc_silu_mul(const void* x1, const void* x2, void* out, int64_t n, void* stream) {
     return launch_binary<SiluMul>(x1, x2, out, n, stream);
+}
+extern "C" int hyc_silu_once_mul(const void* x1, const void* x2, void* out, int64_t n, void* stream) {
+    return launch_binary<SiluOnceMul>(x1, x2, out, n, stream);
 }
 extern "C" int hyc_gelu_bwd(const void* x, const void* g, void* out, int64_t n, void* stream) {
     return launch_binary<GeluBwd>(x, g, out, n, stream);

@@ -31,7 +31,8 @@ Deliberate differences from the reference:
     modify their input);
   * backward restores the input-norm outliers with the *input-norm* channel list; the reference's
     intra_inter / full_fuse files pass the post-attention list there
-    (fused_llama_layer_intra_inter_full_fuse.py:484), which its own 'intra' file does not (:492);
+    (fused_llama_layer_intra_inter_full_fuse.py:484), which its own 'intra' file does not (:492) and
+    which is not the gradient of the layer; `reference_outlier_list=True` reproduces that statement;
   * RMSNorm eps is a parameter (default 1e-5, the value the reference hard-codes, :99,203).
 """
 from __future__ import annotations
@@ -53,7 +54,7 @@ from ..operators.compress_function import (compress_attention_map, compression_p
 from ..operators.rmsnorm_kernels import _backward as _rmsnorm_backward
 from ..operators.rmsnorm_kernels import (backward_from_codes_supported, lora_a_supported, rmsnorm_backward_from_codes, rmsnorm_forward,
                                          rmsnorm_forward_compress)
-from ..operators.silu_kernels import silu_backward, silu_hadamard, silu_hadamard_backward
+from ..operators.silu_kernels import silu_backward, silu_hadamard, silu_hadamard_backward, silu_once_hadamard
 from ..operators.softmax_kernels import softmax_backward, softmax_backward_from_compressed, softmax_forward
 from ..operators.triton_fuse_lora_silu_hadamard_backward_kernels import triton_fuse_silu_backward
 from ..operators.triton_fuse_lora_silu_hadamard_forward_kernels import triton_fuse_silu_forward
@@ -77,6 +78,10 @@ class LayerSpec:
     mode: str = "intra_inter_full_fuse"
     attention: str = "map"          # 'map' | 'sdpa'
     eps: float = 1e-5
+    # True: backward puts the input-norm outliers back at the post-attention norm's channels, as the
+    # reference's intra_inter / full_fuse files are written (…full_fuse.py:484 passes
+    # ctx.post_layernorm_channel); False: at their own channels, as its 'intra' file does (:492)
+    reference_outlier_list: bool = False
 
     def __post_init__(self):
         if self.mode not in MODES:
@@ -430,23 +435,24 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             main = deq(name + "_main")
             return main + (xa @ lb).to(main.dtype), False
 
-        def channel_base_restored(name):
+        def channel_base_restored(name, channels):
             if name + "_raw" in S:
                 return S[name + "_raw"]
             return outlier_addition_fuse_decompression_dequantization(
-                S[name + "_q"], S[name + "_s"], S[name + "_o"], S[name + "_idx"], q_bit)
+                S[name + "_q"], S[name + "_s"], S[name + "_o"], S[channels + "_idx"], q_bit)
 
-        def norm_backward(dy, name, weight, rstd, want_dw, residual):
+        def norm_backward(dy, name, weight, rstd, want_dw, residual, channels=None):
             """Backward of the norm whose input the layer saved under `name`, plus the gradient of the
             residual connection (`grad_norm + residual` in the reference, …full_fuse.py:386-393,486-493).
             A compressed input is read from its codes where the kernel takes the shape; otherwise it
             is restored first.  The residual is added inside the kernel where it can be."""
+            channels = channels or name
             fused_add = residual.dtype == dy.dtype == torch.bfloat16 and residual.shape == dy.shape
             if name + "_raw" not in S and fused_add and backward_from_codes_supported(dy, dy.shape[-1], want_dw):
-                dx = rmsnorm_backward_from_codes(dy, S[name + "_q"], S[name + "_s"], S[name + "_o"], S[name + "_idx"],
+                dx = rmsnorm_backward_from_codes(dy, S[name + "_q"], S[name + "_s"], S[name + "_o"], S[channels + "_idx"],
                                                  q_bit, weight, rstd, residual=residual)
                 return dx, None
-            xin = channel_base_restored(name)
+            xin = channel_base_restored(name, channels)
             if fused_add:
                 return _rmsnorm_backward(dy, xin, weight, rstd, want_dw=want_dw, residual=residual)
             dx, dw = _rmsnorm_backward(dy, xin, weight, rstd, want_dw=want_dw)
@@ -483,7 +489,10 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             fn = None
             if spec.mode == "intra_inter":
                 gate, up = rebuilt_hidden("gate")[0], rebuilt_hidden("up")[0]
-                hadamard = silu_hadamard(gate, up)            # as forward formed it
+                if gate.dtype == up.dtype == torch.bfloat16:
+                    hadamard = silu_once_hadamard(gate, up)   # up * F.silu(gate), as the reference recomputes it
+                else:
+                    hadamard = up * F.silu(gate)
             else:
                 hadamard, up, fn, gate = deq("hadamard"), deq("up"), deq("fn"), deq("gate")
             grad_down = back("down", hadamard, S["down_lora_a"], grad_output)
@@ -565,7 +574,9 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
         grad_x = back("k", "x_norm_1", S["k_lora_a"], grad_k, accumulate=grad_x)
         grad_x = back("v", "x_norm_1", S["v_lora_a"], grad_v, accumulate=grad_x)
         del grad_q, grad_k, grad_v
-        grad_input, grad_nw1 = norm_backward(grad_x, "x", norm_weight_1, S["rstd_1"], ctx.norm_grads[0], grad_medium)
+        as_reference = spec.reference_outlier_list and spec.mode in ("intra_inter", "intra_inter_full_fuse")
+        grad_input, grad_nw1 = norm_backward(grad_x, "x", norm_weight_1, S["rstd_1"], ctx.norm_grads[0], grad_medium,
+                                             channels="x_medium" if as_reference else "x")
 
         def lora_grads(name):
             return (None, None, None) + G[name]
@@ -603,9 +614,9 @@ class FusedDecoderLayer(torch.nn.Module):
     layer_type = "intra_inter_full_fuse"
     attention = "map"
 
-    def __init__(self, eps: float = 1e-5):
+    def __init__(self, eps: float = 1e-5, reference_outlier_list: bool = False):
         super().__init__()
-        self.spec = LayerSpec(self.layer_type, self.attention, eps)
+        self.spec = LayerSpec(self.layer_type, self.attention, eps, reference_outlier_list)
         self.iteration = 0
         self.static_value = self.spec.empty_static_value()
         # host-side bookkeeping that is not part of the calibration state (not checkpointed): the

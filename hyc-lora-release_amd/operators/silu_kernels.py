@@ -15,11 +15,18 @@ def silu_hadamard(x, g):
     return binary("hyc_silu_mul", x, g)
 
 
+def silu_once_hadamard(x, u):
+    """u * F.silu(x): SiLU evaluated in fp32 and rounded to bf16 once, then the product - the form in which
+    the reference's backward recomputes the gated product
+    (models/llama/fused_llama_layer_intra_inter.py:362,370), one pass instead of two."""
+    return binary("hyc_silu_once_mul", x, u)
+
+
 def silu_hadamard_backward(x, u, g):
-    """Backward of silu_hadamard(x, u) for an upstream gradient g, in one pass over the three tensors:
-    -> (grad_x, grad_u) = (silu_backward(x, g * u), g * silu(x)).  No counterpart in the reference, whose
-    layers compose it from F.silu, two products and silu_backward
-    (models/llama/fused_llama_layer_intra_inter.py:361-381)."""
+    """Backward of the gated product silu(x) * u for an upstream gradient g, in one pass over the three
+    tensors: -> (grad_x, grad_u) = (silu_backward(x, g * u), g * F.silu(x)).  No counterpart in the
+    reference, whose layers compose exactly this from F.silu, two products and silu_backward
+    (models/llama/fused_llama_layer_intra_inter.py:362-381)."""
     assert x.shape == u.shape == g.shape
     _lib.require_gpu(x, u, g)
     if not (x.dtype == u.dtype == g.dtype == torch.bfloat16):

@@ -430,14 +430,19 @@ int hyc_rope(void *x, const void *cos, const void *sin, int table_is_fp32, int64
  *   hyc_silu_bwd  out = g * (sig * (1 + x*(1 - sig))), sig = bf16(sigmoid(x)), bf16 after
  *                 every operation.  Replaces silu_backward_kernel (operators/silu_kernels.py:12-45).
  *   hyc_silu_mul  out = (sig(x1) * x1) * x2.  Replaces triton_silu_hadamard_kernel (:73-106).
+ *   hyc_silu_once_mul  out = bf16(silu(x1)) * x2, silu evaluated in fp32 and rounded once.  Replaces
+ *                 `fn = torch.nn.functional.silu(gate); hadamard = up * fn`, the form in which the backward
+ *                 of the layers without the fused LoRA kernels recomputes the gated product
+ *                 (models/llama/fused_llama_layer_intra_inter.py:362,370).
  *   hyc_gelu_bwd  out = d/dx[tanh-GELU](x) * g, evaluated in fp32.  Replaces
  *                 gelu_backward_kernel (operators/gelu_kernels.py:19-58).
  */
 int hyc_silu_bwd(const void *x, const void *g, void *out, int64_t n, void *stream);
 int hyc_silu_mul(const void *x1, const void *x2, void *out, int64_t n, void *stream);
+int hyc_silu_once_mul(const void *x1, const void *x2, void *out, int64_t n, void *stream);
 /* Backward of o = silu(x) * u in one pass: grad_x = hyc_silu_bwd(x, bf16(g * u)), grad_u = g * silu(x) with
- * silu(x) as hyc_silu_mul forms it.  Replaces F.silu + two products + silu_backward in the layers that
- * do not use the fused LoRA kernels (models/llama/fused_llama_layer_intra_inter.py:361-381). */
+ * silu(x) as hyc_silu_once_mul forms it (F.silu).  Replaces F.silu + two products + silu_backward in the layers
+ * that do not use the fused LoRA kernels (models/llama/fused_llama_layer_intra_inter.py:362-381). */
 int hyc_silu_mul_bwd(const void *x, const void *u, const void *g, void *grad_x, void *grad_u, int64_t n,
                      void *stream);
 int hyc_gelu_bwd(const void *x, const void *g, void *out, int64_t n, void *stream);

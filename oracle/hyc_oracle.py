@@ -50,7 +50,10 @@ from typing import Optional, Tuple
 
 import torch
 
-BF16 = torch.bfloat16
+BF16 = torch.bfloat16       # what the arithmetic rounds to after each operation.  Tests may bind this name to
+                            # float64 to run the same code without intermediate rounding.
+WIRE = torch.bfloat16       # dtype of a dequantised activation: part of the format (the product code * step is
+                            # rounded to bf16 once, compress_function_kernel.py:200-204), not of the arithmetic
 F32 = torch.float32
 
 
@@ -226,7 +229,7 @@ def dequant(c: torch.Tensor, s: torch.Tensor, q_bit: int,
     v = c.to(BF16) - (2 ** (q_bit - 1))
     if z is not None:
         v = v - z.to(BF16).reshape(1, 1, -1)
-    return (v * s).to(BF16)
+    return (v * s).to(WIRE)
 
 
 def decompress(p, s, q_bit, z=None, is_head=False, num_heads=1):
@@ -249,7 +252,7 @@ def compress_channel_base(x, s, idx, q_bit):
 def decompress_channel_base(p, s, x_outlier, idx, q_bit, is_head=False, num_heads=1):
     """outlier_addition_fuse_decompression_dequantization (compress_function.py:147-174)."""
     x = decompress(p, s, q_bit)
-    x[:, :, idx] = x_outlier
+    x[:, :, idx] = x_outlier.to(x.dtype)
     if is_head:
         x = hidden_to_head_shape(x, num_heads)
     return x
@@ -378,11 +381,11 @@ def silu_mul(x1, x2):
 
 
 def silu_mul_bwd(x, u, g):
-    """Backward of silu_mul(x, u): (silu_bwd(x, g*u), g * (sig(x)*x)), every product rounded to bf16 -
-    the composition the layers write out (fused_llama_layer_intra_inter.py:361-381) with silu(x) as
-    silu_mul forms it."""
+    """Backward of the gated product silu(x) * u: (silu_bwd(x, g*u), g * F.silu(x)), every product rounded to
+    bf16 and silu itself evaluated in fp32 and rounded once - the composition the layers write out
+    (fused_llama_layer_intra_inter.py:362-381)."""
     x = x.to(BF16); u = u.to(BF16); g = g.to(BF16)
-    return silu_bwd(x, g * u), g * (_sig_bf16(x) * x)
+    return silu_bwd(x, g * u), g * torch.nn.functional.silu(x)
 
 
 GELU_GAMMA = 0.7978845608028654
@@ -441,9 +444,14 @@ def fused_fwd(xa1, b1, x1, s1, xa2, b2, x2, s2, q_bit):
 def fused_bwd(xa1, b1, q1, s1, xa2, b2, q2, s2, grad_o, q_bit):
     """triton_fuse_silu_backward (…backward_kernels.py:106-149,152-178)
     -> (o, grad_gate, grad_up)."""
+    return fused_bwd_dense(xa1, b1, decompress(q1, s1, q_bit), xa2, b2, decompress(q2, s2, q_bit), grad_o)
+
+
+def fused_bwd_dense(xa1, b1, x1, xa2, b2, x2, grad_o):
+    """The arithmetic of fused_bwd after its two dequantisations (…backward_kernels.py:124-149): x1, x2 are the
+    frozen-weight parts of gate and up as the kernel holds them at that point."""
     g = grad_o.to(BF16)
-    x1 = decompress(q1, s1, q_bit)
-    x2 = decompress(q2, s2, q_bit)
+    x1 = x1.to(BF16); x2 = x2.to(BF16)
     y1 = x1 + _lora_term(xa1, b1)
     y2 = x2 + _lora_term(xa2, b2)
     sig = _sig_bf16(y1)

@@ -93,3 +93,35 @@ def scalar_unpack_dequant(q, s, z, q_bit):
         None if zb is None else zb.ctypes.data_as(ctypes.c_void_p), out.ctypes.data_as(ctypes.c_void_p),
         ctypes.c_long(B), ctypes.c_long(M), ctypes.c_long(N), ctypes.c_int(q_bit))
     return from_bits(out)
+
+
+def layer_saved_state(out: torch.Tensor, heads: int) -> dict:
+    """What a fused decoder layer kept for backward, read off the autograd node of its output and renamed to
+    the reference's save-list names (the keys oracle/layer_oracle.py's backward reads).  Call it before
+    backward runs: the node drops its tensors afterwards.  The attention map's lists are cut to the entries
+    that were written (the layer may have sized them with headroom)."""
+    node = out.grad_fn
+    raw = dict(zip(node.names, node.saved_tensors))
+    prefix = {"q_rope": "q", "k_rope": "k", "v_rep": "v", "o_lora_a": "o_final_lora_a"}
+    suffix = {"_s": "_scale", "_z": "_zero_point", "_idx": "_channel_idx"}
+    S = {}
+    for name, t in raw.items():
+        if name in ("a_idx", "a_val", "a_seg", "sdpa_rng", "sdpa_unused") or name.endswith("_raw"):
+            continue
+        for old, new in prefix.items():
+            if name == old or name.startswith(old + "_"):
+                name = new + name[len(old):]
+                break
+        for old, new in suffix.items():
+            if name.endswith(old):
+                name = name[:-len(old)] + new
+                break
+        S[name] = t
+    if "sdpa_lse" in S:
+        S["softmax_lse"] = S.pop("sdpa_lse")
+    if "a_idx" in raw:
+        nnz = int(raw["a_seg"][-1].item())
+        S["a_o_indices"], S["a_o_values"] = raw["a_idx"][:nnz], raw["a_val"][:nnz]
+        b, s = out.shape[0], out.shape[1]
+        S["a_shape"] = (b, heads, s, s)
+    return S
