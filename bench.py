@@ -102,10 +102,11 @@ def parse():
     ap.add_argument("--warmup", type=int, default=1000,
                     help="untimed steps; ~50 ms of work lets the GPU reach its steady clocks (20 steps do not)")
     ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU-oracle timing (for profiler runs)")
-    ap.add_argument("--only", choices=["all", "roundtrip", "quant", "fused", "mlp", "lora", "copy", "layers", "stack"], default="all",
+    ap.add_argument("--only", choices=["all", "roundtrip", "quant", "fused", "fused4", "mlp", "lora", "copy", "layers", "stack"], default="all",
                     help="restrict the run to one part (for profiler runs)")
     ap.add_argument("--pmc-summary", default="", metavar="DIR",
                     help="no GPU work: turn the rocprofv3 counter CSVs under DIR into profiles/quant_pack_q4_config2_hbm_traffic.json")
+    ap.add_argument("--fused4-bits", default="2,4,8", help="with --only fused4: the code widths to run")
     ap.add_argument("--layer-case", default="", help="with --only layers: run only the cases whose name contains this")
     ap.add_argument("--layer-seq", type=int, default=0, help="with --only layers: sequence length instead of the configuration's")
     ap.add_argument("--layer-dims", default="", help="with --only layers: override dimensions of the configuration, "
@@ -572,23 +573,25 @@ def main():
         roofline = None
 
     # ---- the other kernels of the path, same shape ---------------------------------------------
-    fused = None
-    if args.only in ("all", "fused"):
+    def fused_at(Bf, Mf, Nf, qb, with_torch):
+        """Fused LoRA-SiLU-Hadamard forward and backward on [Bf, Mf, Nf] at qb bits through the C ABI, checked
+        against the wrappers and the unfused composite before timing; HIP-graph replays."""
         NF = 3
+        Tf, Ef = Bf * Mf, Bf * Mf * Nf
         sets = []
         for _ in range(NF):
-            d = dict(x1=randn(B, M, N), x2=randn(B, M, N), xa1=randn(B, M, R), xa2=randn(B, M, R),
-                     b1=randn(R, N, scale=0.05), b2=randn(R, N, scale=0.05), g=randn(B, M, N))
+            d = dict(x1=randn(Bf, Mf, Nf), x2=randn(Bf, Mf, Nf), xa1=randn(Bf, Mf, R), xa2=randn(Bf, Mf, R),
+                     b1=randn(R, Nf, scale=0.05), b2=randn(R, Nf, scale=0.05), g=randn(Bf, Mf, Nf))
             sets.append(d)
-        s1 = cf.get_statistics_only_quant(sets[0]["x1"], QB, 'per-channel')
-        s2 = cf.get_statistics_only_quant(sets[0]["x2"], QB, 'per-channel')
+        s1 = cf.get_statistics_only_quant(sets[0]["x1"], qb, 'per-channel')
+        s2 = cf.get_statistics_only_quant(sets[0]["x2"], qb, 'per-channel')
         # outputs are allocated once and the C ABI is called directly, so that both kernels can be
         # timed as HIP-graph replays like every other kernel that runs shorter than an eager launch costs
         bt = 0
         for d in sets:
-            d["q1"] = torch.empty(B, M, N * QB // 8, device=dev, dtype=torch.uint8)
+            d["q1"] = torch.empty(Bf, Mf, Nf * qb // 8, device=dev, dtype=torch.uint8)
             d["q2"] = torch.empty_like(d["q1"])
-            d["o"] = torch.empty(B, M, N, device=dev, dtype=BF16)
+            d["o"] = torch.empty(Bf, Mf, Nf, device=dev, dtype=BF16)
             d["ob"], d["gg"], d["gu"] = torch.empty_like(d["o"]), torch.empty_like(d["o"]), torch.empty_like(d["o"])
         s1v, s2v = s1.reshape(-1).contiguous(), s2.reshape(-1).contiguous()
 
@@ -596,7 +599,7 @@ def main():
             d = sets[i % NF]
             rc = L.hyc_lora_silu_mul_fwd(d["xa1"].data_ptr(), d["b1"].data_ptr(), d["x1"].data_ptr(), s1v.data_ptr(),
                                          d["xa2"].data_ptr(), d["b2"].data_ptr(), d["x2"].data_ptr(), s2v.data_ptr(),
-                                         d["q1"].data_ptr(), d["q2"].data_ptr(), d["o"].data_ptr(), T, N, R, QB, bt, st or stream)
+                                         d["q1"].data_ptr(), d["q2"].data_ptr(), d["o"].data_ptr(), Tf, Nf, R, qb, bt, st or stream)
             assert rc == 0, _lib.error_string(rc)
 
         def f_bwd(i, st=None):
@@ -604,7 +607,7 @@ def main():
             rc = L.hyc_lora_silu_mul_bwd(d["xa1"].data_ptr(), d["b1"].data_ptr(), d["q1"].data_ptr(), s1v.data_ptr(),
                                          d["xa2"].data_ptr(), d["b2"].data_ptr(), d["q2"].data_ptr(), s2v.data_ptr(),
                                          d["g"].data_ptr(), d["ob"].data_ptr(), d["gg"].data_ptr(), d["gu"].data_ptr(),
-                                         T, N, R, QB, bt, st or stream)
+                                         Tf, Nf, R, qb, bt, st or stream)
             assert rc == 0, _lib.error_string(rc)
 
         Kf, Wf = 30, 3
@@ -613,18 +616,29 @@ def main():
         # a wrong but fast kernel must not post a number: the timed entry points against the wrappers'
         # results and against the unfused fp32 composite
         d0 = sets[0]
-        q1w, q2w, ow = fuse_forward(d0["xa1"], d0["b1"], d0["x1"], s1, d0["xa2"], d0["b2"], d0["x2"], s2, QB)
+        q1w, q2w, ow = fuse_forward(d0["xa1"], d0["b1"], d0["x1"], s1, d0["xa2"], d0["b2"], d0["x2"], s2, qb)
         assert torch.equal(q1w, d0["q1"]) and torch.equal(q2w, d0["q2"]) and torch.equal(ow, d0["o"])
+        assert torch.equal(q1w, cf.compression_quantization(d0["x1"], s1, qb)), "fused codes differ from the quantiser's"
+        obw, ggw, guw = fuse_backward(d0["xa1"], d0["b1"], q1w, s1, d0["xa2"], d0["b2"], q2w, s2, d0["g"], qb)
+        assert torch.equal(obw, d0["ob"]) and torch.equal(ggw, d0["gg"]) and torch.equal(guw, d0["gu"])
         ref = F.silu(d0["x1"].float() + d0["xa1"].float() @ d0["b1"].float()) * (d0["x2"].float() + d0["xa2"].float() @ d0["b2"].float())
         err = ((ow.float() - ref).abs().max() / ref.abs().max()).item()
         assert err <= 1e-2, f"fused forward differs from the unfused composite: {err:.2e}"
-        del ref, q1w, q2w, ow
+        del ref, q1w, q2w, ow, obw, ggw, guw
         ms_ff, _ = timed_graph(f_fwd, Kf, Wf)
         ms_fb, _ = timed_graph(f_bwd, Kf, Wf)
-        ms_ff_eager, _ = timed(f_fwd, Kf, Wf)
-        ms_fb_eager, _ = timed(f_bwd, Kf, Wf)
-        bytes_ff = E * (6 + QB / 4) + 2 * T * R * 2 + 2 * R * N * 2 + 4 * N
-        bytes_fb = E * (8 + QB / 4) + 2 * T * R * 2 + 2 * R * N * 2 + 4 * N
+        bytes_ff = Ef * (6 + qb / 4) + 2 * Tf * R * 2 + 2 * R * Nf * 2 + 4 * Nf
+        bytes_fb = Ef * (8 + qb / 4) + 2 * Tf * R * 2 + 2 * R * Nf * 2 + 4 * Nf
+        res = {"fwd_ms": ms_ff, "bwd_ms": ms_fb, "fwd_bwd_ms": ms_ff + ms_fb,
+               "timing": f"{Kf} launches over {NF} rotating operand sets recorded in one HIP graph, replayed once, "
+                         f"after {SETTLE_MS:.0f} ms of the same replays",
+               "fwd_GBps": bytes_ff / ms_ff / 1e6, "bwd_GBps": bytes_fb / ms_fb / 1e6,
+               "fwd_frac_of_hbm_peak": bytes_ff / ms_ff / 1e6 / HBM_PEAK_GBS,
+               "bwd_frac_of_hbm_peak": bytes_fb / ms_fb / 1e6 / HBM_PEAK_GBS}
+        if not with_torch:
+            return res
+        res["eager_fwd_ms"], _ = timed(f_fwd, Kf, Wf)
+        res["eager_bwd_ms"], _ = timed(f_bwd, Kf, Wf)
 
         # unfused bf16 torch on the same GPU: LoRA add, SiLU, product and their autograd backward
         def t_fwdbwd(i):
@@ -645,17 +659,19 @@ def main():
 
         ms_tf, _ = timed(t_fwd, Kf, Wf)
         ms_tfb, _ = timed(t_fwdbwd, Kf, Wf)
-        fused = {"fwd_ms": ms_ff, "bwd_ms": ms_fb, "fwd_bwd_ms": ms_ff + ms_fb,
-                 "timing": f"{Kf} launches over {NF} rotating operand sets recorded in one HIP graph, replayed once, "
-                           f"after {SETTLE_MS:.0f} ms of the same replays",
-                 "eager_fwd_ms": ms_ff_eager, "eager_bwd_ms": ms_fb_eager,
-                 "fwd_GBps": bytes_ff / ms_ff / 1e6, "bwd_GBps": bytes_fb / ms_fb / 1e6,
-                 "fwd_frac_of_hbm_peak": bytes_ff / ms_ff / 1e6 / HBM_PEAK_GBS,
-                 "bwd_frac_of_hbm_peak": bytes_fb / ms_fb / 1e6 / HBM_PEAK_GBS,
-                 "torch_unfused_fwd_ms": ms_tf, "torch_unfused_fwd_bwd_ms": ms_tfb,
-                 "speedup_vs_torch_unfused": ms_tfb / (ms_ff + ms_fb),
-                 "note": "the fused kernels also produce/consume the 4-bit saved activations; the torch arm keeps bf16"}
-        del sets
+        res.update({"torch_unfused_fwd_ms": ms_tf, "torch_unfused_fwd_bwd_ms": ms_tfb,
+                    "speedup_vs_torch_unfused": ms_tfb / (ms_ff + ms_fb),
+                    "note": "the fused kernels also produce/consume the 4-bit saved activations; the torch arm keeps bf16"})
+        return res
+
+    fused = fused_at(B, M, N, QB, True) if args.only in ("all", "fused") else None
+    # configuration 4's MLP width and its sweep of code widths: [2, 2048, 14336] at 2, 4 and 8 bits
+    fused_config4 = None
+    if args.only in ("all", "fused4"):
+        widths = [int(w) for w in args.fused4_bits.split(",")]
+        fused_config4 = {"shape": [2, 2048, 14336], "rank": R}
+        for qb in widths:
+            fused_config4[f"q{qb}"] = fused_at(2, 2048, 14336, qb, False)
 
     # ---- the whole MLP block of the layer: x_norm_2 -> gate/up -> LoRA-SiLU-product -> down, forward
     # and backward with the frozen GEMMs, new kernels against unfused bf16 torch autograd --------------
@@ -992,6 +1008,7 @@ def main():
         "roofline": roofline,
         "cpu_baseline": cpu,
         "fused": fused,
+        "fused_config4": fused_config4,
         "mlp": mlp,
         "lora": lora,
         "kernels": kernels,

@@ -149,7 +149,13 @@ struct PackedSlot {
     }
     // the 8 codes of the chunk as floats
     __device__ __forceinline__ void decode(u32x2 w, float (&c)[8]) const {
-        const uint32_t lo = (w.x >> shift) & mask, hi = (w.y >> shift) & mask;
+        uint32_t lo = (w.x >> shift) & mask, hi = (w.y >> shift) & mask;
+        if constexpr (QBIT != 8) {
+            // the masked words are made opaque: a code is then one byte-to-float conversion of them; left to
+            // itself the compiler extracts every code from the packed word with a bit-field instruction first
+            asm("" : "+v"(lo));
+            asm("" : "+v"(hi));
+        }
 #pragma unroll
         for (int j = 0; j < 8; ++j) c[j] = (float)(((j < 4 ? lo : hi) >> (8 * (j & 3))) & 0xffu);
     }

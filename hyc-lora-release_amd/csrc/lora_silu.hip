@@ -36,12 +36,28 @@ constexpr int kFuseWaves = kFuseThreads / kWave;
 #ifndef HYC_ROLL_DEEP
 #define HYC_ROLL_DEEP 1
 #endif
+// Cache policy of the packed codes.  At 2 and 4 bits a tile's codes are a quarter / half of a 128-byte line
+// and the rest of the line belongs to a neighbouring wave: ordinary stores and loads, so that the pieces
+// meet in L2.  At 8 bits a wave writes and reads whole lines that nobody else touches: streaming accesses
+// (forward 95.0 -> 91.2 us, backward 117.7 -> 116.4 us on [4096, 14336]).
+template <int QBIT> constexpr bool kStreamCodes = QBIT == 8;
 
-// Strip heights (backward, forward; see hyc_set_tuning).  0 = by size: a wave sets up its LoRA-B
-// operands and per-column constants once per strip, which in the [N, R] layout of LoRA-B is 16
+// Strip heights (backward, forward; see hyc_set_tuning).  0 = by code width and size: a wave sets up its
+// LoRA-B operands and per-column constants once per strip, which in the [N, R] layout of LoRA-B is 16
 // scattered 8-byte loads per lane; 96-row strips spread that over six tiles once the tensor is
-// large enough to fill the machine with such strips (forward 70 -> 66 us on [4096, 11008]).
-static int g_fuse_rows_per_wave[2] = {32, 0};
+// large enough to fill the machine with such strips (forward 70 -> 66 us on [4096, 11008]).  At 8 bits a
+// workgroup is four strips of ONE column tile, and short strips do better: measured on [4096, 11008] and
+// [4096, 14336], forward 32 rows (69.9 / 64.4 % of peak against 70.7 / 60.0 % at 96), backward 16 rows
+// (65.1 / 67.0 % against 66.9 / 63.1 % at 32).
+static int g_fuse_rows_per_wave[2] = {0, 0};
+
+static int fuse_rows_per_wave(bool fwd, int q_bit, int64_t T, int64_t N) {
+    const int set = g_fuse_rows_per_wave[fwd ? 1 : 0];
+    if (set) return set;
+    if (!fwd) return q_bit == 8 ? 16 : 32;
+    if (q_bit == 8) return 32;
+    return T * N >= ((int64_t)1 << 24) ? 96 : 32;
+}
 
 struct FuseArgs {
     const uint16_t* xa1; const uint16_t* b1; const uint16_t* s1;
@@ -156,9 +172,9 @@ __device__ __forceinline__ void fuse_fwd_rows_full(const FuseArgs& a, int64_t ro
             if constexpr (AHEAD) request_row(row0 + kTileRows, v);
             uint32_t lo, hi;
             codes_to_words<QBIT, false, true>(f1, c1, zero8, lo, hi);
-            store_packed<QBIT, false>(a.q1 + r * row_bytes, chunk, true, lo, hi);
+            store_packed<QBIT, kStreamCodes<QBIT>>(a.q1 + r * row_bytes, chunk, true, lo, hi);
             codes_to_words<QBIT, false, true>(f2, c2, zero8, lo, hi);
-            store_packed<QBIT, false>(a.q2 + r * row_bytes, chunk, true, lo, hi);
+            store_packed<QBIT, kStreamCodes<QBIT>>(a.q2 + r * row_bytes, chunk, true, lo, hi);
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 float y1 = rbf(f1[j] + lora_elem(L1[v], j));
@@ -231,12 +247,17 @@ HYC_FUSE_KERNEL(HYC_BWD_DEEP) void lora_silu_bwd_kernel(const FuseArgs a) {
     const int g = lane >> 4;
     constexpr float kHalf = (float)(1 << (QBIT - 1));
 
-    float s1[8], s2[8];
+    // dequantisation is (code - 2^(q-1)) * step rounded to bf16; as code * step + (-2^(q-1) * step) in one
+    // fused multiply-add it is the same number (both products and their sum are exact in fp32: at most 8 x 8
+    // significant bits) and the code's byte converts with a single instruction
+    float s1[8], s2[8], n1[8], n2[8];
     {
         u32x4 v1 = {0, 0, 0, 0}, v2 = {0, 0, 0, 0};
         if (active) { v1 = ld16(a.s1 + col0); v2 = ld16(a.s2 + col0); }
         unpack8(v1, s1);
         unpack8(v2, s2);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) { n1[j] = -kHalf * s1[j]; n2[j] = -kHalf * s2[j]; }
     }
     BOperand<KSTEPS> B1, B2;
     B1.load(a.b1, a.N, a.R, col0, active, g, a.b_transposed != 0);
@@ -250,12 +271,14 @@ HYC_FUSE_KERNEL(HYC_BWD_DEEP) void lora_silu_bwd_kernel(const FuseArgs a) {
 
     // one row of 8 element pairs: codes + upstream gradient -> hadamard, grad_gate, grad_up
     auto row_math = [&](const float (&cd1)[8], const float (&cd2)[8], const float (&gf)[8], const uint32_t (&La)[4],
-                        const uint32_t (&Lb)[4], int64_t t) {
+                        const uint32_t (&Lb)[4], uint16_t* o_at, uint16_t* gg_at, uint16_t* gu_at) {
         float of[8], gg[8], gu[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            const float x1 = rbf((cd1[j] - kHalf) * s1[j]);
-            const float x2 = rbf((cd2[j] - kHalf) * s2[j]);
+            // at 2 bits the four values -2s, -s, 0, s are bf16 numbers already
+            const float d1 = fmaf(cd1[j], s1[j], n1[j]), d2 = fmaf(cd2[j], s2[j], n2[j]);
+            const float x1 = QBIT == 2 ? d1 : rbf(d1);
+            const float x2 = QBIT == 2 ? d2 : rbf(d2);
             const float y1 = rbf(x1 + lora_elem(La, j));
             const float y2 = rbf(x2 + lora_elem(Lb, j));
             const float sig = rbf(sigmoidf_(y1));
@@ -266,28 +289,42 @@ HYC_FUSE_KERNEL(HYC_BWD_DEEP) void lora_silu_bwd_kernel(const FuseArgs a) {
             const float dsilu = rbf(sig * rbf(1.0f + rbf(y1 * rbf(1.0f - sig))));
             gg[j] = gh1 * dsilu;
         }
-        st16_nt(a.o + t * a.N + col0, pack8(of));
-        st16_nt(a.gg + t * a.N + col0, pack8(gg));
-        st16_nt(a.gu + t * a.N + col0, pack8(gu));
+        st16_nt(o_at, pack8(of));
+        st16_nt(gg_at, pack8(gg));
+        st16_nt(gu_at, pack8(gu));
     };
 
     // Interior strips at rank 16: the rolling prefetch of fuse_fwd_rows_full - a row's registers
     // are requested again for the next tile as soon as the row has been taken out of them.
     const bool full = (KSTEPS == 1 || (HYC_ROLL_DEEP && KSTEPS >= HYC_BWD_DEEP)) && (col_tile + 1) * (kTileCols / 8) <= a.C && row_begin < row_end &&
-                      (row_end - row_begin) % kTileRows == 0;      // uniform across the wave
+                      (row_end - row_begin) % kTileRows == 0 && a.N <= (1 << 24);      // uniform across the wave
     if (full) {
         const int i = lane & 15;
         u32x2 w1[4], w2[4], A1[KSTEPS], A2[KSTEPS];
         u32x4 gv[4];
+        // addresses as (wave-uniform row base) + (lane offset that never changes): the row bases are advanced
+        // with scalar instructions, one vector add per access is left
+        const uint32_t lane_q = (uint32_t)(4 * g * row_bytes + slot.offset);
+        const uint32_t lane_x = (uint32_t)(4 * g * a.N + col0) * 2u;
+        auto in_row = [](const void* base, int64_t uniform_bytes, uint32_t lane_bytes) {
+            return reinterpret_cast<const char*>(base) + uniform_bytes + lane_bytes;
+        };
+        auto out_row = [](void* base, int64_t uniform_bytes, uint32_t lane_bytes) {
+            return reinterpret_cast<uint16_t*>(reinterpret_cast<char*>(base) + uniform_bytes + lane_bytes);
+        };
         auto request_a = [&](int64_t row0) {
             request_lora_a<KSTEPS>(a.xa1, a.R, row0 + i, g, A1);
             request_lora_a<KSTEPS>(a.xa2, a.R, row0 + i, g, A2);
         };
         auto request_row = [&](int64_t row0, int v) {
-            const int64_t t = row0 + 4 * g + v;
-            w1[v] = ld8(a.q1 + t * row_bytes + slot.offset);
-            w2[v] = ld8(a.q2 + t * row_bytes + slot.offset);
-            gv[v] = ld16_nt(a.g + t * a.N + col0);
+            if constexpr (kStreamCodes<QBIT>) {
+                w1[v] = ld8_nt(in_row(a.q1, (row0 + v) * row_bytes, lane_q));
+                w2[v] = ld8_nt(in_row(a.q2, (row0 + v) * row_bytes, lane_q));
+            } else {
+                w1[v] = ld8(in_row(a.q1, (row0 + v) * row_bytes, lane_q));
+                w2[v] = ld8(in_row(a.q2, (row0 + v) * row_bytes, lane_q));
+            }
+            gv[v] = ld16_nt(in_row(a.g, (row0 + v) * a.N * 2, lane_x));
         };
         auto work = [&](int64_t row0, auto ahead_tag) {
             constexpr bool AHEAD = decltype(ahead_tag)::value;
@@ -306,7 +343,8 @@ HYC_FUSE_KERNEL(HYC_BWD_DEEP) void lora_silu_bwd_kernel(const FuseArgs a) {
                 slot.decode(w2[v], cd2);
                 unpack8(gv[v], gf);
                 if constexpr (AHEAD) request_row(row0 + kTileRows, v);
-                row_math(cd1, cd2, gf, L1[v], L2[v], row0 + 4 * g + v);
+                const int64_t ub = (row0 + v) * a.N * 2;
+                row_math(cd1, cd2, gf, L1[v], L2[v], out_row(a.o, ub, lane_x), out_row(a.gg, ub, lane_x), out_row(a.gu, ub, lane_x));
                 __builtin_amdgcn_sched_barrier(0);
             }
         };
@@ -348,7 +386,7 @@ HYC_FUSE_KERNEL(HYC_BWD_DEEP) void lora_silu_bwd_kernel(const FuseArgs a) {
             slot.decode(w1[v], cd1);
             slot.decode(w2[v], cd2);
             unpack8(gv[v], gf);
-            row_math(cd1, cd2, gf, L1[v], L2[v], t);
+            row_math(cd1, cd2, gf, L1[v], L2[v], a.o + t * a.N + col0, a.gg + t * a.N + col0, a.gu + t * a.N + col0);
             __builtin_amdgcn_sched_barrier(0);
         }
     }
@@ -396,8 +434,7 @@ static int fuse_launch(FuseArgs& a, int64_t T, int64_t N, int64_t R, int q_bit, 
     a.N = (int)N;
     a.C = (int)(N / 8);
     a.R = (int)R;
-    a.rows_per_wave = g_fuse_rows_per_wave[fwd ? 1 : 0];
-    if (a.rows_per_wave == 0) a.rows_per_wave = T * N >= ((int64_t)1 << 24) ? 96 : 32;
+    a.rows_per_wave = fuse_rows_per_wave(fwd, q_bit, T, N);
     const int ct = 8 / q_bit;                                  // kColTilesPerGroup
     a.col_tiles = (int)cdiv(cdiv(N, kTileCols), ct);           // workgroups along the columns
     const int64_t row_tiles = cdiv(T, (int64_t)(kFuseWaves / ct) * a.rows_per_wave);
@@ -416,7 +453,6 @@ int tune_fuse(const char* key, int value) {
     const bool bwd = both || strcmp(key, "fuse_bwd_rows_per_wave") == 0;
     if (fwd || bwd) {
         if (value < 0 || value > 65536 || value % kTileRows != 0) return HYC_ERR_ARG;     // 0: by size
-        if (value == 0 && bwd) value = 32;
         if (bwd) g_fuse_rows_per_wave[0] = value;
         if (fwd) g_fuse_rows_per_wave[1] = value;
         return HYC_OK;

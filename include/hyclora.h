@@ -49,9 +49,9 @@ int hyc_abi_version(void);
  * "norm_compress_slab" (0 / 1: whether hyc_rmsnorm_fwd_compress may use its column-slab kernel, default 1)
  * and "norm_compress_rows_per_group" (rows a workgroup of that kernel walks, even; 0 = chosen from the
  * row count, the default),
- * "fuse_rows_per_wave" (same for both fused LoRA-SiLU kernels, multiple of 16; defaults: backward 32,
- * forward 0 = 96 for tensors of 2^24 elements and more, else 32;
- * "fuse_fwd_rows_per_wave" / "fuse_bwd_rows_per_wave" set one of them),
+ * "fuse_rows_per_wave" (same for both fused LoRA-SiLU kernels, multiple of 16; default 0 = by code width
+ * and size: backward 32, 16 at 8 bits; forward 96 for tensors of 2^24 elements and more, else 32, and 32
+ * at 8 bits; "fuse_fwd_rows_per_wave" / "fuse_bwd_rows_per_wave" set one of them),
  * "contract_max_groups" (column groups hyc_lora_contract cuts a row strip into, default 32; changes the
  * workspace hyc_lora_contract_workspace asks for).  Unknown key or bad value: HYC_ERR_ARG.  No
  * counterpart in the reference (its launch shapes come from triton.autotune). */

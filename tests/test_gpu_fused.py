@@ -47,7 +47,8 @@ def mlp_inputs(seed, B, M, H, I, R):
 @pytest.mark.parametrize("q_bit", QBITS)
 @pytest.mark.parametrize("dims", [(2, 64, 256, 1024, 16), (1, 37, 128, 160, 16), (1, 16, 64, 11008, 16),
                                   (2, 20, 64, 256, 8), (1, 33, 64, 384, 32), (1, 16, 64, 128, 64), (1, 5, 64, 96, 4),
-                                  (2, 100, 64, 384, 48), (1, 130, 64, 256, 64)])
+                                  (2, 100, 64, 384, 48), (1, 130, 64, 256, 64),
+                                  (2, 112, 64, 384, 32), (1, 200, 64, 256, 24)])      # ranks 17..32 over several strips
 def test_fused_forward_and_backward(fz, dev, q_bit, dims):
     B, M, H, I, R = dims
     t = mlp_inputs(q_bit + I, B, M, H, I, R)
@@ -83,7 +84,8 @@ def test_fused_forward_and_backward(fz, dev, q_bit, dims):
 
 
 @pytest.mark.parametrize("q_bit", QBITS)
-@pytest.mark.parametrize("R", [16, 8, 48, 64])      # 48 and 64: the deep-rank instantiations walk the same way
+@pytest.mark.parametrize("R", [16, 8, 48, 64, 32, 24])      # 48 and 64: the deep-rank instantiations walk the same way;
+                                                             # 32 and 24: forward on the rolling path, backward on the guarded one
 def test_fused_results_do_not_depend_on_the_strip_height(fz, dev, q_bit, R):
     # Interior strips are walked with the next tile requested ahead: one tile per strip takes only
     # the closing step of that walk, two tiles the opening and the closing one, more the loop in
@@ -105,8 +107,7 @@ def test_fused_results_do_not_depend_on_the_strip_height(fz, dev, q_bit, R):
             ob, gg, gu = fz.bwd(*d(xa1, b1), q1, s1.to(dev), *d(xa2, b2), q2, s2.to(dev), g.to(dev), q_bit)
             outs.append((q1, q2, o, ob, gg, gu))
     finally:
-        _lib.set_tuning("fuse_bwd_rows_per_wave", 32)      # the library's defaults
-        _lib.set_tuning("fuse_fwd_rows_per_wave", 0)
+        _lib.set_tuning("fuse_rows_per_wave", 0)           # the library's defaults
     for other in outs[1:]:
         for a, b in zip(outs[0], other):
             assert torch.equal(a, b)
