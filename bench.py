@@ -102,7 +102,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=1000,
                     help="untimed steps; ~50 ms of work lets the GPU reach its steady clocks (20 steps do not)")
     ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU-oracle timing (for profiler runs)")
-    ap.add_argument("--only", choices=["all", "roundtrip", "quant", "fused", "fused4", "mlp", "lora", "copy", "layers", "stack"], default="all",
+    ap.add_argument("--only", choices=["all", "roundtrip", "quant", "fused", "fused4", "mlp", "lora", "kernels", "copy", "layers", "stack"], default="all",
                     help="restrict the run to one part (for profiler runs)")
     ap.add_argument("--pmc-summary", default="", metavar="DIR",
                     help="no GPU work: turn the rocprofv3 counter CSVs under DIR into profiles/quant_pack_q4_config2_hbm_traffic.json")
@@ -853,7 +853,7 @@ def main():
             lora[wname] = e
             del x_l, y_l, q_l, wss
 
-    if args.only == "all":
+    if args.only in ("all", "kernels"):
         Kx, Wx = max(K // 4, 10), max(W // 4, 3)
         Kg = 40
 
@@ -910,7 +910,50 @@ def main():
                                                       "three_library_gemms_ms": ms_lib,
                                                       "norm_then_three_library_gemms_ms": kernels["rmsnorm_fwd_compress_4096"]["ms"] + ms_lib}
         ms = tg(lambda i: cf.get_statistics_channel_base(x_h[i % NH], 0.005, QB, 'per-channel'))
-        kernels["calibration_stats_4096"] = {"ms": ms}
+        kernels["calibration_stats_4096"] = {"ms": ms, "what": "get_statistics_channel_base of [4, 1024, 4096] (batch element 0, "
+                                                                "20 outlier channels): statistics pass, strip fold and channel choice"}
+
+        # the calibration kernels one by one, through the C ABI on preallocated buffers, at the batch-0 slices of
+        # configuration 1 ([512, 4096], 20 outlier channels) and configuration 4 ([2048, 14336], 71)
+        def calibration_kernels(Mc, Nc, kc):
+            nbuf = max(2, min(160, -(-600_000_000 // (Mc * Nc * 2))))         # rotate past the 256 MiB cache
+            xc = [randn(1, Mc, Nc) for _ in range(nbuf)]
+            strips = int(L.hyc_channel_stats_strips(Mc, Nc))
+            stats_c = torch.empty(strips * 3 + 1, Nc, device=dev, dtype=torch.float32)
+            idx_c = torch.empty(kc, device=dev, dtype=torch.int64)
+            sc_c = torch.empty(Nc, device=dev, dtype=BF16)
+
+            def k_stats(i, st):
+                rc = L.hyc_channel_stats(xc[i % nbuf].data_ptr(), Mc, Nc, Nc, Nc, 0, stats_c.data_ptr(), stats_c.numel() * 4, st)
+                assert rc == 0, _lib.error_string(rc)
+
+            def k_select(i, st):
+                rc = L.hyc_channel_select(stats_c.data_ptr(), strips, Nc, kc, QB, 1, idx_c.data_ptr(), sc_c.data_ptr(), None, st)
+                assert rc == 0, _lib.error_string(rc)
+
+            def k_steps_only(i, st):
+                rc = L.hyc_channel_select(stats_c.data_ptr(), strips, Nc, 0, QB, 0, None, sc_c.data_ptr(), None, st)
+                assert rc == 0, _lib.error_string(rc)
+
+            k_stats(0, stream)
+            k_select(0, stream)
+            want_idx, want_s = cf.get_statistics_channel_base(xc[0], kc / Nc + 1e-9, QB, 'per-channel')
+            assert torch.equal(idx_c, want_idx) and torch.equal(sc_c, want_s.reshape(-1)), "timed calibration kernels differ from the wrapper"
+            assert torch.equal(stats_c[1], xc[0][0].max(dim=0).values.float()), "channel maxima differ from torch.max"
+            ms_s = timed_graph(k_stats, Kg, 3)[0]
+            k_stats(0, stream)
+            ms_k = timed_graph(k_select, Kg, 3)[0]
+            k_stats(0, stream)
+            ms_0 = timed_graph(k_steps_only, Kg, 3)[0]
+            nb = Mc * Nc * 2
+            return {"channel_stats": {"ms": ms_s, "bytes": nb, "GBps": nb / ms_s / 1e6, "frac_of_hbm_peak": nb / ms_s / 1e6 / HBM_PEAK_GBS,
+                                      "row_strips": strips},
+                    "channel_select": {"ms": ms_k, "channels": Nc, "chosen": kc,
+                                       "note": "fold of the strips + steps (one thread per channel), then the choice of "
+                                               "the outlier channels by a single workgroup: latency, not bandwidth"},
+                    "channel_select_no_outliers": {"ms": ms_0, "channels": Nc}}
+        kernels["calibration_config1_512x4096"] = calibration_kernels(512, 4096, 20)
+        kernels["calibration_config4_2048x14336"] = calibration_kernels(2048, 14336, 71)
         # norm backward straight from the channel-base compressed input, residual gradient added, against
         # restore + backward with the same add
         xo_h, qx_h = cf.outlier_subtraction_fuse_compression_quantization(x_h[0].clone(), sc, idx, QB)
@@ -931,6 +974,27 @@ def main():
         thr = cf.get_statistics_softmax(a, 0.05)
         ms, _ = timed(lambda i: cf.get_statistics_softmax(a, 0.05), 5, 2)
         kernels["softmax_threshold_kth"] = {"ms": ms, "GBps": Ea * 2 / ms / 1e6}
+        # its two kernels one by one (the histogram is cleared by a fill kernel inside hyc_hist16)
+        hist_c = torch.empty(65536, device=dev, dtype=torch.int32)
+        thr_c = torch.empty((), device=dev, dtype=torch.float32)
+        kth_c = int(Ea * (1 - 0.05))
+
+        def k_hist(i, st):
+            rc = L.hyc_hist16(a.data_ptr(), Ea, hist_c.data_ptr(), st)
+            assert rc == 0, _lib.error_string(rc)
+
+        def k_hsel(i, st):
+            rc = L.hyc_hist_select(hist_c.data_ptr(), kth_c, thr_c.data_ptr(), st)
+            assert rc == 0, _lib.error_string(rc)
+
+        k_hist(0, stream)
+        k_hsel(0, stream)
+        assert thr_c.item() == thr.item() == torch.kthvalue(a.float().flatten(), kth_c).values.item()
+        ms_h = timed_graph(k_hist, 10, 2)[0]
+        ms_hs = timed_graph(k_hsel, Kg, 3)[0]
+        kernels["hist16"] = {"ms": ms_h, "bytes": Ea * 2, "GBps": Ea * 2 / ms_h / 1e6, "frac_of_hbm_peak": Ea * 2 / ms_h / 1e6 / HBM_PEAK_GBS,
+                             "shape": [4, 32, 1024, 1024]}
+        kernels["hist_select"] = {"ms": ms_hs, "bins": 65536, "note": "single workgroup: latency, not bandwidth"}
         idx_a, val_a, seg_a = cf.compress_attention_map(a, thr)
         nnz = idx_a.numel()
         ms, _ = timed(lambda i: cf.compress_attention_map(a, thr), 5, 2)

@@ -26,7 +26,7 @@ class HycError(RuntimeError):
 
 
 # name -> (restype, argtypes)
-ABI_VERSION = 6          # hyc_abi_version() of the library these signatures describe
+ABI_VERSION = 7          # hyc_abi_version() of the library these signatures describe
 _P, _I, _L = c_void_p, c_int, c_int64
 _SIGNATURES = {
     "hyc_error_string": (c_char_p, [_I]),
@@ -34,8 +34,9 @@ _SIGNATURES = {
     "hyc_set_tuning": (_I, [c_char_p, _I]),
     "hyc_quant_pack": (_I, [_P, _P, _P, _P, _P, _L, _P, _I, _L, _L, _L, _L, _L, _L, _L, _I, _P]),
     "hyc_unpack_dequant": (_I, [_P, _P, _P, _P, _P, _L, _P, _L, _L, _L, _L, _L, _L, _L, _I, _P]),
-    "hyc_channel_stats": (_I, [_P, _L, _L, _L, _L, _L, _P, _P]),
-    "hyc_channel_select": (_I, [_P, _L, _L, _I, _I, _P, _P, _P, _P]),
+    "hyc_channel_stats_strips": (_L, [_L, _L]),
+    "hyc_channel_stats": (_I, [_P, _L, _L, _L, _L, _L, _P, _L, _P]),
+    "hyc_channel_select": (_I, [_P, _L, _L, _L, _I, _I, _P, _P, _P, _P]),
     "hyc_hist16": (_I, [_P, _L, _P, _P]),
     "hyc_hist_select": (_I, [_P, _L, _P, _P]),
     "hyc_sparse_num_segments": (_L, [_L]),

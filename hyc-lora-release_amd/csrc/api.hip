@@ -16,7 +16,7 @@ extern "C" const char* hyc_error_string(int code) {
     }
 }
 
-extern "C" int hyc_abi_version(void) { return 6; }
+extern "C" int hyc_abi_version(void) { return 7; }
 
 extern "C" int hyc_set_tuning(const char* key, int value) {
     if (!key) return HYC_ERR_NULL;
@@ -29,6 +29,8 @@ extern "C" int hyc_set_tuning(const char* key, int value) {
     rc = hyc::tune_contract(key, value);
     if (rc != 1) return rc;
     rc = hyc::tune_norm_compress(key, value);
+    if (rc != 1) return rc;
+    rc = hyc::tune_stats(key, value);
     if (rc != 1) return rc;
     return HYC_ERR_ARG;
 }

@@ -106,6 +106,19 @@ __device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
     return v;
 }
 
+// Inclusive prefix sum over the 64 lanes with DPP moves only (no LDS traffic): a shift-and-add scan
+// inside each row of 16 lanes (lanes without a source add 0), then the last lane of row 0 / 2 is
+// added to row 1 / 3, then lane 31 (sum of rows 0-1) to rows 2-3.
+__device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v) {
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x111, 0xf, 0xf, true);    // row_shr:1
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x112, 0xf, 0xf, true);    // row_shr:2
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x114, 0xf, 0xf, true);    // row_shr:4
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x118, 0xf, 0xf, true);    // row_shr:8
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x142, 0xa, 0xf, false);   // row_bcast:15 -> rows 1, 3
+    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x143, 0xc, 0xf, false);   // row_bcast:31 -> rows 2, 3
+    return v;
+}
+
 // logistic function; the callers round the result to bf16, so the 1-ulp hardware
 // reciprocal and exponential are ample
 __device__ __forceinline__ float sigmoidf_(float x) { return __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
@@ -125,5 +138,6 @@ int tune_fuse(const char* key, int value);
 int tune_add(const char* key, int value);
 int tune_contract(const char* key, int value);
 int tune_norm_compress(const char* key, int value);
+int tune_stats(const char* key, int value);
 
 }  // namespace hyc

@@ -77,30 +77,45 @@ __global__ __launch_bounds__(kHistThreads) void hist16_kernel(const uint16_t* __
     }
 }
 
-// Single workgroup: the k-th smallest value (1-based) from the histogram.
+// Single workgroup: the k-th smallest value (1-based) from the histogram.  Wave w takes bins
+// 4096w .. 4096w+4095 in sixteen coalesced 1 KiB loads (load i: lane l holds bins 4096w + 256i + 4l .. +3),
+// so the bins stay in registers in ascending order by (wave, load, lane, component).  Their running count is
+// a lane scan per load, a carry from load to load, and the waves' totals through LDS.
 __global__ __launch_bounds__(1024) void hist_select_kernel(const uint32_t* __restrict__ hist, int64_t kth,
                                                            float* __restrict__ thr) {
-    __shared__ unsigned long long incl[1024];
-    const int t = threadIdx.x;
-    unsigned long long sum = 0;
-    for (int i = 0; i < 64; ++i) sum += hist[t * 64 + i];
-    incl[t] = sum;
-    __syncthreads();
-    for (int o = 1; o < 1024; o <<= 1) {
-        const unsigned long long add = t >= o ? incl[t - o] : 0;
-        __syncthreads();
-        incl[t] += add;
-        __syncthreads();
+    __shared__ unsigned long long wave_total[1024 / kWave];
+    const int t = threadIdx.x, lane = t & (kWave - 1), wave = t >> 6;
+    u32x4 h[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) h[i] = ld16(hist + wave * 4096 + i * 256 + lane * 4);
+    // (the bins hold 32-bit counts of a tensor of fewer than 2^32 elements, so a wave's running count fits 32 bits)
+    uint32_t incl[16];                    // count of the wave's bins up to and including this lane's four of load i
+    uint32_t carry = 0;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const uint32_t v = wave_inclusive_scan(h[i].x + h[i].y + h[i].z + h[i].w);
+        incl[i] = carry + v;
+        carry += (uint32_t)__builtin_amdgcn_readlane((int)v, kWave - 1);
     }
-    const unsigned long long hi = incl[t], lo = hi - sum, k = (unsigned long long)kth;
-    if (lo < k && k <= hi) {
-        unsigned long long cum = lo;
-        for (int i = 0; i < 64; ++i) {
-            cum += hist[t * 64 + i];
-            if (cum >= k) {
-                *thr = __builtin_bit_cast(float, key_to_bf16((uint32_t)(t * 64 + i)) << 16);
-                break;
+    if (lane == 0) wave_total[wave] = carry;
+    __syncthreads();
+    unsigned long long before = 0;
+    for (int w = 0; w < wave; ++w) before += wave_total[w];
+    const unsigned long long k = (unsigned long long)kth;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const uint32_t c[4] = {h[i].x, h[i].y, h[i].z, h[i].w};
+        const unsigned long long hi = before + incl[i];
+        unsigned long long cum = hi - ((unsigned long long)c[0] + c[1] + c[2] + c[3]);
+        if (cum < k && k <= hi) {          // true for exactly one (thread, load)
+            int bin = 3;
+#pragma unroll
+            for (int j = 3; j >= 0; --j) {
+                unsigned long long upto = cum;
+                for (int jj = 0; jj <= j; ++jj) upto += c[jj];
+                if (upto >= k) bin = j;
             }
+            *thr = __builtin_bit_cast(float, key_to_bf16((uint32_t)(wave * 4096 + i * 256 + lane * 4 + bin)) << 16);
         }
     }
 }
@@ -113,19 +128,6 @@ __global__ __launch_bounds__(1024) void hist_select_kernel(const uint32_t* __res
 __device__ __forceinline__ bool keep(uint32_t bits, float thr) {
     const float v = bf_to_f((uint16_t)bits);
     return (v > thr || v != v) && v != 0.0f;
-}
-
-// Inclusive prefix sum over the 64 lanes with DPP moves only (no LDS traffic): a shift-and-add scan
-// inside each row of 16 lanes (lanes without a source add 0), then the last lane of row 0 / 2 is
-// added to row 1 / 3, then lane 31 (sum of rows 0-1) to rows 2-3.
-__device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v) {
-    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x111, 0xf, 0xf, true);    // row_shr:1
-    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x112, 0xf, 0xf, true);    // row_shr:2
-    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x114, 0xf, 0xf, true);    // row_shr:4
-    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x118, 0xf, 0xf, true);    // row_shr:8
-    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x142, 0xa, 0xf, false);   // row_bcast:15 -> rows 1, 3
-    v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x143, 0xc, 0xf, false);   // row_bcast:31 -> rows 2, 3
-    return v;
 }
 
 // Loads the 8 elements of chunk `c` of the flattened tensor, zero-filling past n.

@@ -95,7 +95,8 @@ def _require_per_channel(q_method: str) -> None:
 
 
 def _batch0_stats(x: torch.Tensor):
-    """(stats fp32 [3, N], N): min / max / sum of squares per channel over batch element 0."""
+    """(stats, strips, N): per-strip min / max / sum of squares per channel over batch element 0, fp32
+    [strips*3 + 1, N] as hyc_channel_select takes it."""
     _lib.require_gpu(x)
     if x.dtype != BF16:
         x = x.to(BF16)
@@ -104,9 +105,11 @@ def _batch0_stats(x: torch.Tensor):
         raise ValueError(f"channel count must be a multiple of 32, got {a.N}")
     if a.B == 0:
         raise ValueError("statistics need at least one batch element")
-    stats = torch.empty((3, a.N), device=x.device, dtype=torch.float32)
-    _lib.call("hyc_channel_stats", a.t.data_ptr(), a.M, a.N, a.sm, a.hd, a.sh, stats.data_ptr(), _lib.stream_of(x))
-    return stats, a.N
+    strips = int(_lib.lib().hyc_channel_stats_strips(a.M, a.N))
+    stats = torch.empty((strips * 3 + 1, a.N), device=x.device, dtype=torch.float32)
+    _lib.call("hyc_channel_stats", a.t.data_ptr(), a.M, a.N, a.sm, a.hd, a.sh, stats.data_ptr(),
+              stats.numel() * 4, _lib.stream_of(x))
+    return stats, strips, a.N
 
 
 # ---------------------------------------------------------------------------------------
@@ -146,9 +149,9 @@ def get_statistics_only_quant(x: torch.Tensor, q_bit: int = 8, q_method: str = '
     """Per-channel step bf16 [1, N] from batch element 0.  Reference :45-59."""
     _require_per_channel(q_method)
     _check_bits(q_bit)
-    stats, n = _batch0_stats(x)
+    stats, strips, n = _batch0_stats(x)
     scale = torch.empty((1, n), device=x.device, dtype=BF16)
-    _lib.call("hyc_channel_select", stats.data_ptr(), n, 0, q_bit, 0, None, scale.data_ptr(), None,
+    _lib.call("hyc_channel_select", stats.data_ptr(), strips, n, 0, q_bit, 0, None, scale.data_ptr(), None,
               _lib.stream_of(x))
     return scale
 
@@ -157,10 +160,10 @@ def get_statistics_only_quant_zero_point(x: torch.Tensor, q_bit: int = 8, q_meth
     """(step bf16 [1, N], zero point int8 [1, N]).  Reference :62-77."""
     _require_per_channel(q_method)
     _check_bits(q_bit)
-    stats, n = _batch0_stats(x)
+    stats, strips, n = _batch0_stats(x)
     scale = torch.empty((1, n), device=x.device, dtype=BF16)
     zp = torch.empty((1, n), device=x.device, dtype=torch.int8)
-    _lib.call("hyc_channel_select", stats.data_ptr(), n, 0, q_bit, 0, None, scale.data_ptr(), zp.data_ptr(),
+    _lib.call("hyc_channel_select", stats.data_ptr(), strips, n, 0, q_bit, 0, None, scale.data_ptr(), zp.data_ptr(),
               _lib.stream_of(x))
     return scale, zp
 
@@ -171,11 +174,11 @@ def get_statistics_channel_base(x: torch.Tensor, outlier_ratio: float, q_bit: in
     No clone of x is made: the statistics of the zeroed tensor follow from those of x."""
     _require_per_channel(q_method)
     _check_bits(q_bit)
-    stats, n = _batch0_stats(x)
+    stats, strips, n = _batch0_stats(x)
     k = int(n * outlier_ratio)
     idx = torch.empty((k,), device=x.device, dtype=torch.int64)
     scale = torch.empty((1, n), device=x.device, dtype=BF16)
-    _lib.call("hyc_channel_select", stats.data_ptr(), n, k, q_bit, 1, idx.data_ptr() if k else None,
+    _lib.call("hyc_channel_select", stats.data_ptr(), strips, n, k, q_bit, 1, idx.data_ptr() if k else None,
               scale.data_ptr(), None, _lib.stream_of(x))
     return idx, scale
 
@@ -444,8 +447,8 @@ def get_statistics_structed_pruning(x: torch.Tensor, outlier_ratio: float):
     out = torch.empty((flat.shape[0], k), device=x.device, dtype=torch.int64)
     scale = torch.empty((1, n), device=x.device, dtype=BF16)
     for b in range(flat.shape[0]):
-        stats, _ = _batch0_stats(flat[b:b + 1])
-        _lib.call("hyc_channel_select", stats.data_ptr(), n, k, 8, 0, out[b].data_ptr() if k else None,
+        stats, strips, _ = _batch0_stats(flat[b:b + 1])
+        _lib.call("hyc_channel_select", stats.data_ptr(), strips, n, k, 8, 0, out[b].data_ptr() if k else None,
                   scale.data_ptr(), None, _lib.stream_of(x))
     return out.reshape(*lead, k)
 

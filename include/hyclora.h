@@ -53,7 +53,9 @@ int hyc_abi_version(void);
  * and size: backward 32, 16 at 8 bits; forward 96 for tensors of 2^24 elements and more, else 32, and 32
  * at 8 bits; "fuse_fwd_rows_per_wave" / "fuse_bwd_rows_per_wave" set one of them),
  * "contract_max_groups" (column groups hyc_lora_contract cuts a row strip into, default 32; changes the
- * workspace hyc_lora_contract_workspace asks for).  Unknown key or bad value: HYC_ERR_ARG.  No
+ * workspace hyc_lora_contract_workspace asks for), "stats_waves" (waves hyc_channel_stats aims to launch,
+ * default 4096; sets the number of row strips hyc_channel_stats_strips returns and so the order in which the
+ * sums of squares are added).  Unknown key or bad value: HYC_ERR_ARG.  No
  * counterpart in the reference (its launch shapes come from triton.autotune). */
 int hyc_set_tuning(const char *key, int value);
 
@@ -109,7 +111,8 @@ int hyc_unpack_dequant(const void *q, const void *scale, const void *zero_point,
 
 /* ---------------------------------------------------------------------------------------
  * Calibration statistics, step 1: per-channel minimum, maximum and sum of squares over the
- * M rows of ONE batch element (the reference calibrates on batch element 0 only).
+ * M rows of ONE batch element (the reference calibrates on batch element 0 only), as one partial
+ * result per strip of rows.
  *
  * Replaces the torch reductions in get_statistics_only_quant (operators/compress_function.py:50-54),
  * get_statistics_only_quant_zero_point (:67-72) and get_statistics_channel_base (:86,93-97),
@@ -117,11 +120,18 @@ int hyc_unpack_dequant(const void *q, const void *scale, const void *zero_point,
  *
  *   x      bf16 [M, N] of batch element 0, element (m, c) at
  *          x + m*stride_m + (c / head_dim)*stride_h + (c % head_dim)
- *   stats  fp32 [3, N] output: row 0 = min, row 1 = max (NaN propagates as in torch),
- *          row 2 = sum of squares (fp32 accumulation in a fixed order).
+ *   stats  fp32 [strips*3 + 1, N] device buffer, strips = hyc_channel_stats_strips(M, N) (it follows the
+ *          launch size, hyc_set_tuning "stats_waves").  Output: rows 3s, 3s+1, 3s+2 = min, max (NaN
+ *          propagates as in torch) and sum of squares over the rows of strip s.  The sums are fp32, added
+ *          in a fixed order: a lane of the kernel adds every eighth row of its strip in ascending order,
+ *          the eight waves of a workgroup are added in order (and hyc_channel_select adds the strips in
+ *          order, 32 at a time) - the same bits on every run for given M, N and "stats_waves".  The last row is scratch
+ *          for hyc_channel_select.
+ *   stats_bytes  size of that buffer; HYC_ERR_WORKSPACE when smaller than (strips*3 + 1)*N*4.
  */
+int64_t hyc_channel_stats_strips(int64_t M, int64_t N);
 int hyc_channel_stats(const void *x, int64_t M, int64_t N, int64_t stride_m, int64_t head_dim,
-                      int64_t stride_h, float *stats, void *stream);
+                      int64_t stride_h, float *stats, int64_t stats_bytes, void *stream);
 
 /* ---------------------------------------------------------------------------------------
  * Calibration statistics, step 2: outlier channels and per-channel step / zero point.
@@ -130,7 +140,8 @@ int hyc_channel_stats(const void *x, int64_t M, int64_t N, int64_t stride_m, int
  * (operators/compress_function.py:86-105), get_statistics_only_quant (:50-59) and
  * get_statistics_only_quant_zero_point (:67-77).
  *
- *   stats       fp32 [3, N] from hyc_channel_stats.
+ *   stats       fp32 [strips*3 + 1, N] as hyc_channel_stats left it.  Modified: on return rows 0, 1, 2 hold
+ *               the minimum, maximum and sum of squares over all rows, the last row the channels' sort keys.
  *   k           number of outlier channels (0 = none).  Chosen by bf16 norm
  *               bf16(sqrt(sum of squares)) descending, ties by channel index ascending —
  *               torch.topk leaves tie order unspecified, this rule is fixed.  N <= 32768
@@ -142,7 +153,7 @@ int hyc_channel_stats(const void *x, int64_t M, int64_t N, int64_t stride_m, int
  *   zero_point  int8 [N] output or NULL: -round_half_even(min / step) - 2^(q_bit-1), every
  *               operation rounded to bf16, then converted like a C cast (:72,77).
  */
-int hyc_channel_select(const float *stats, int64_t N, int64_t k, int q_bit, int add_eps,
+int hyc_channel_select(float *stats, int64_t strips, int64_t N, int64_t k, int q_bit, int add_eps,
                        int64_t *outlier_idx, void *scale, int8_t *zero_point, void *stream);
 
 /* ---------------------------------------------------------------------------------------

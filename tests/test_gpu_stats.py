@@ -123,3 +123,54 @@ def test_calibration_dispatch_and_static_values(cf, dev):
         cf.get_statistics_only_quant(xg, 4, 'per-tensor')
     with pytest.raises(ValueError):
         cf.get_statistics_only_quant(xg, 4, 'per-row')
+
+
+@pytest.mark.parametrize("shape", [(1, 2048, 14336), (2, 512, 4096), (1, 37, 96), (1, 7, 32), (1, 1000, 1024)])
+def test_statistics_do_not_depend_on_the_strip_count(cf, dev, shape):
+    """The rows are split into strips whose number follows the launch size aimed for ("stats_waves"); minimum
+    and maximum cannot depend on it, the fp32 sum of squares only in its last bits - so steps and zero points
+    must be the same bits for every setting and equal the oracle's, and a channel list may differ from the
+    oracle's only in channels whose norm is within a bf16 step of the k-th (the order of the additions)."""
+    from hyclora_amd import _lib
+    x = _rand(shape, seed=shape[1], scale=1.5)
+    x[0, :, 5] *= 40
+    k = int(shape[2] * 0.02)
+    got = []
+    try:
+        for waves in (4, 64, 2048, 1 << 16):
+            _lib.set_tuning("stats_waves", waves)
+            s, z = cf.get_statistics_only_quant_zero_point(x.to(dev), 4, 'per-channel')
+            idx, sc = cf.get_statistics_channel_base(x.to(dev), 0.02, 4, 'per-channel')
+            got.append((s.cpu(), z.cpu(), idx.cpu(), sc.cpu()))
+    finally:
+        _lib.set_tuning("stats_waves", 4096)
+    s_ref, z_ref = O.scale_zero_point(x, 4)
+    nrm = O.channel_norms(x).float()
+    ref = set(O.outlier_channels(x, 0.02).tolist())
+    kth = torch.sort(nrm, descending=True).values[k - 1] if k else None
+    for s, z, idx, sc in got:
+        assert same_bits(s, s_ref) and torch.equal(z, z_ref)
+        assert idx.numel() == k and torch.unique(idx).numel() == k
+        for c in set(idx.tolist()) ^ ref:
+            assert abs(nrm[c].item() - kth.item()) <= kth.item() * 2 ** -7, f"channel {c} is not a boundary tie"
+        if k:
+            assert idx[0].item() == 5
+            # descending norms, ties by ascending channel
+            keys = [(-nrm[c].item(), c) for c in idx.tolist()]
+            assert all(a[0] <= b[0] for a, b in zip(keys, keys[1:]))
+        _, sc_ref = O.channel_stats(x, 0.02, 4, idx=idx)
+        assert same_bits(sc, sc_ref)
+
+
+@pytest.mark.parametrize("n,k", [(4096, 1024), (4096, 1025), (2048, 2048), (1024, 1), (32768, 163), (96, 95)])
+def test_channel_lists_of_any_length(cf, dev, n, k):
+    """Lists of up to 1024 channels are found by a radix select and ordered by counting, longer ones by rounds
+    of a block-wide maximum; both must give `norm descending, channel ascending`.  Exactly representable norms
+    (every channel constant, its value a small integer) make the expected list exact, ties included."""
+    g = torch.Generator().manual_seed(n + k)
+    level = torch.randint(0, 200, (n,), generator=g).float()          # many ties
+    x = level.reshape(1, 1, n).expand(1, 4, n).to(BF16).contiguous()
+    idx, _ = cf.get_statistics_channel_base(x.to(dev), k / n + 1e-9, 4, 'per-channel')
+    assert idx.numel() == k
+    order = sorted(range(n), key=lambda c: (-level[c].item(), c))[:k]
+    assert idx.cpu().tolist() == order
