@@ -1013,7 +1013,42 @@ def main():
         kernels["softmax_fwd_scale_mask"]["torch_three_passes_ms"] = ms
         ms, _ = timed(lambda i: softmax_kernels.softmax_backward_from_compressed(idx_a, val_a, seg_a, g_a), 10, 2)
         kernels["softmax_restore_bwd_one_pass"] = {"ms": ms, "GBps": (6 * Ea + 10 * nnz) / ms / 1e6}
-        del a, g_a, idx_a, val_a
+        del a, g_a, idx_a, val_a, seg_a
+
+        # the same kernels on configuration 4's map: [2, 32, 2048, 2048], rows of 2048
+        S4 = 2048
+        g4 = randn(2, 32, S4, S4)
+        E4 = g4.numel()
+        causal4 = torch.full((S4, S4), float("-inf"), device=dev).triu(1).to(BF16)[None, None]
+        a4 = softmax_kernels.softmax_forward(g4, 0.0884, causal4)
+        ref4 = torch.softmax(((g4.float() * torch.tensor(0.0884, device=dev)).to(BF16) + causal4).float(), dim=-1)
+        assert ((a4.float() - ref4).abs().max() / ref4.max()).item() <= 1e-2, "softmax_forward differs from the torch composite at rows of 2048"
+        del ref4
+        thr4 = cf.get_statistics_softmax(a4, 0.05)
+        a4c, seg4 = softmax_kernels.softmax_forward(g4, 0.0884, causal4, threshold=thr4)
+        idx4, val4, seg4b = cf.compress_attention_map(a4, thr4, seg4)
+        nnz4 = idx4.numel()
+        assert torch.equal(a4c, a4) and torch.equal(seg4b, seg4)
+        a_two, o_two = cf.restore_attention_map(idx4, val4, seg4, a4.shape), None
+        o_two = softmax_kernels.softmax_backward(a_two, g4)
+        a_one, o_one = softmax_kernels.softmax_backward_from_compressed(idx4, val4, seg4, g4)
+        assert torch.equal(a_one, a_two) and torch.equal(o_one, o_two), "one-pass restore + backward differs from the two kernels"
+        del a_two, o_two, a_one, o_one, a4c
+        m4 = {}
+        ms, _ = timed(lambda i: softmax_kernels.softmax_forward(g4, 0.0884, causal4), 10, 2)
+        m4["softmax_fwd_scale_mask"] = {"ms": ms, "GBps": 4 * E4 / ms / 1e6, "frac_of_hbm_peak": 4 * E4 / ms / 1e6 / HBM_PEAK_GBS}
+        ms, _ = timed(lambda i: softmax_kernels.softmax_forward(g4, 0.0884, causal4, threshold=thr4), 10, 2)
+        m4["softmax_fwd_scale_mask_count"] = {"ms": ms, "GBps": 4 * E4 / ms / 1e6, "frac_of_hbm_peak": 4 * E4 / ms / 1e6 / HBM_PEAK_GBS}
+        cap4 = nnz4 + nnz4 // 16 + 64
+        ms, _ = timed(lambda i: cf.compress_attention_map(a4, thr4, seg4, capacity=cap4), 10, 2)
+        nb = 2 * E4 + 10 * nnz4
+        m4["sparse_write"] = {"ms": ms, "GBps": nb / ms / 1e6, "frac_of_hbm_peak": nb / ms / 1e6 / HBM_PEAK_GBS, "nnz": nnz4,
+                              "note": "lists sized from a capacity, no read-back; counts come from the forward kernel"}
+        ms, _ = timed(lambda i: softmax_kernels.softmax_backward_from_compressed(idx4, val4, seg4, g4), 10, 2)
+        nb = 6 * E4 + 10 * nnz4
+        m4["softmax_restore_bwd_one_pass"] = {"ms": ms, "GBps": nb / ms / 1e6, "frac_of_hbm_peak": nb / ms / 1e6 / HBM_PEAK_GBS}
+        kernels["attention_map_config4_2x32x2048x2048"] = m4
+        del a4, g4, idx4, val4, seg4
 
     # ---- whole decoder layers (benchmark configurations 2, 4, 5): fwd+bwd ms and saved bytes ----
     layers = None

@@ -504,9 +504,11 @@ __global__ __launch_bounds__(kSegThreads) void softmax_bwd_restore_kernel(const 
     u32x4* st = reinterpret_cast<u32x4*>(stage[wave]);
     // The segment's share of the gradient is requested before anything else: its latency then covers
     // the two dependent round trips of the rebuild (offsets, then indices and values) instead of
-    // following them.  Not for rows of 2048: the 32 registers that hold it there cost a wave per SIMD
-    // and more than the overlap gains (measured 290 against 275 us on [2, 32, 2048, 2048]).
-    constexpr bool kAhead = SPR != 4;
+    // following them.  For rows of 2048 and 4096 the 32 registers that hold it would cost waves per SIMD if the
+    // row's map values were kept in registers between the row sum and the output as well, so there the
+    // values are read from LDS a second time instead (kReread).
+    constexpr bool kAhead = true;
+    constexpr bool kReread = SPR >= 4;
     u32x4 gall[kAhead ? kSegSteps : 1];
     if constexpr (kAhead) {
 #pragma unroll
@@ -552,12 +554,18 @@ __global__ __launch_bounds__(kSegThreads) void softmax_bwd_restore_kernel(const 
         for (int s = 0; s < SPR; ++s) {
             const int c = (r * SPR + s) * kWave + lane;
             float yf[8], gf[8], of[8];
-            unpack8(yv[s], yf);
+            u32x4 y = yv[s];
+            if constexpr (kReread) {
+                // made opaque so that the compiler reads LDS again here instead of keeping the first read alive
+                asm volatile("" ::: "memory");
+                y = st[c];
+            }
+            unpack8(y, yf);
             unpack8(gv[s], gf);
 #pragma unroll
             for (int j = 0; j < 8; ++j) of[j] = rbf((gf[j] - acc) * yf[j]) * out_scale;   // bf16 result, then the bf16 scaling
             st16_nt(o_out + seg * kSeg + (int64_t)c * 8, pack8(of));       // ordinary stores: 166 against 149 us
-            if (a_out) st16_nt(a_out + seg * kSeg + (int64_t)c * 8, yv[s]);
+            if (a_out) st16_nt(a_out + seg * kSeg + (int64_t)c * 8, y);
         }
     }
 }
