@@ -198,15 +198,23 @@ def bench_layers(torch, dev, only_case="", arm="both", seq=0, dims_override=None
         with torch.autograd.graph.saved_tensors_hooks(pack, lambda v: v):
             y = fn()                                  # what the forward keeps alive for backward
         saved = sum(seen.values())
-        t.x.grad = None
+        adapters = [m.weight for n in t.P for m in t.P[n][1:]]
+
+        def clear():          # as optimizer.zero_grad(set_to_none=True): no gradient-accumulation kernels in the timed steps
+            t.x.grad = None
+            for p in adapters:
+                p.grad = None
+        clear()
         y.backward(t.grad)
-        result = (y.detach(), t.x.grad.clone())
+        result = (y.detach(), t.x.grad.clone(), [p.grad.clone() for p in adapters])
         for _ in range(warmup):
+            clear()
             fn().backward(t.grad)
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         for _ in range(steps):
+            clear()
             fn().backward(t.grad)
         e1.record()
         torch.cuda.synchronize()
@@ -215,13 +223,17 @@ def bench_layers(torch, dev, only_case="", arm="both", seq=0, dims_override=None
     def agreement(got, want, q=8):
         """A wrong but fast layer must not post a number: forward output (never compressed) and the
         input gradient (carries the codes' quantisation error) against the uncompressed autograd arm."""
-        (y, gx), (y0, gx0) = got, want
+        (y, gx, ga), (y0, gx0, ga0) = got, want
         rel = ((y.float() - y0.float()).abs().max() / y0.float().abs().max()).item()
         cos = F.cosine_similarity(gx.float().flatten(), gx0.float().flatten(), dim=0).item()
         assert rel <= 2e-2, f"layer output differs from the uncompressed layer: max rel err {rel:.2e}"
         floor = 0.4 if q == 2 else 0.8           # 2-bit codes: a quarter of a channel's range per step
         assert cos >= floor, f"input gradient differs from the uncompressed layer: cosine {cos:.4f} (q_bit {q})"
-        return {"out_max_rel_err": rel, "grad_x_cos": cos}
+        # every one of the fourteen adapter gradients as well: a broken one (zero, wrong sign, another projection's)
+        # would sit far below these floors however coarse the codes are
+        cos_a = [F.cosine_similarity(a.float().flatten(), b.float().flatten(), dim=0).item() for a, b in zip(ga, ga0)]
+        assert min(cos_a) >= floor, f"an adapter gradient differs from the uncompressed layer's: cosines {cos_a} (q_bit {q})"
+        return {"out_max_rel_err": rel, "grad_x_cos": cos, "min_adapter_grad_cos": min(cos_a)}
 
     cfg = lambda lt, q: SimpleNamespace(use_hyclora=True, layer_type=lt, iteration_threshold=2,
                                         softmax_outlier_ratio=0.05, layernorm_outlier_ratio=0.005, q_bit=q)
@@ -243,7 +255,7 @@ def bench_layers(torch, dev, only_case="", arm="both", seq=0, dims_override=None
             name = name + "_with_" + "_".join(f"{k}{v}" for k, v in sorted(dims_override.items()))
         t = make(**dims)
         mask = None if sdpa else torch.full((t.S, t.S), float("-inf"), device=dev).triu(1).to(BF16)[None, None]
-        entry, saved_p, plain = {}, 0, None
+        entry, saved_p, plain, res_b = {}, 0, None, None
         if arm != "compressed":
             ms_p, saved_p, plain = measure(lambda: run_plain(t, mask, sdpa), t)
             entry["bf16_uncompressed"] = {"fwd_bwd_ms": ms_p, "saved_activation_MB": saved_p / 1e6}
@@ -253,7 +265,6 @@ def bench_layers(torch, dev, only_case="", arm="both", seq=0, dims_override=None
             ms_b, saved_b, res_b = measure(lambda: run_fused(base, t, mask), t)
             entry["baseline_layer"] = {"fwd_bwd_ms": ms_b, "saved_activation_MB": saved_b / 1e6,
                                        "check_against_uncompressed": agreement(res_b, plain)}
-            del res_b
             del base
         for q in (qbits if arm != "plain" else []):
             if maker is None:
@@ -266,10 +277,11 @@ def bench_layers(torch, dev, only_case="", arm="both", seq=0, dims_override=None
             ms_f, saved_f, res_f = measure(lambda: run_fused(layer, t, mask), t)
             entry[f"compressed_q{q}"] = {"fwd_bwd_ms": ms_f, "saved_activation_MB": saved_f / 1e6,
                                          "saved_vs_bf16": saved_p / max(saved_f, 1) if saved_p else None,
-                                         "check_against_uncompressed": agreement(res_f, plain, q) if plain else None}
+                                         "check_against_uncompressed": agreement(res_f, plain, q) if plain else None,
+                                         "check_against_baseline_layer": agreement(res_f, res_b, q) if res_b else None}
             del layer, res_f
         out[name] = entry
-        del t, mask, plain
+        del t, mask, plain, res_b
         torch.cuda.empty_cache()
     return out
 

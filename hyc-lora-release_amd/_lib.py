@@ -26,8 +26,17 @@ class HycError(RuntimeError):
 
 
 # name -> (restype, argtypes)
-ABI_VERSION = 7          # hyc_abi_version() of the library these signatures describe
+ABI_VERSION = 8          # hyc_abi_version() of the library these signatures describe
 _P, _I, _L = c_void_p, c_int, c_int64
+
+
+class LoraAddMember(ctypes.Structure):
+    """hyc_lora_add_member of include/hyclora.h: one operand set of a grouped LoRA-add launch."""
+    _fields_ = [("xa", _P), ("b", _P), ("x", _P), ("scale", _P), ("zero_point", _P), ("q", _P), ("y", _P),
+                ("cos_t", _P), ("sin_t", _P), ("seq_len", _L), ("stride_cos", _L), ("stride_sin", _L), ("N", _L),
+                ("b_transposed", _I), ("table_is_fp32", _I)]
+
+
 _SIGNATURES = {
     "hyc_error_string": (c_char_p, [_I]),
     "hyc_abi_version": (_I, []),
@@ -77,6 +86,8 @@ _SIGNATURES = {
     "hyc_lora_add_restore": (_I, [_P, _P, _I] + [_P] * 4 + [_L, _L, _L, _I, _P]),
     "hyc_lora_add_quant_rope": (_I, [_P, _P, _I] + [_P] * 7 + [_I, _L, _L, _L, _L, _L, _L, _I, _P]),
     "hyc_lora_add_restore_rope": (_I, [_P, _P, _I] + [_P] * 6 + [_I, _L, _L, _L, _L, _L, _L, _I, _P]),
+    "hyc_lora_add_quant_group": (_I, [_P, _I, _L, _L, _I, _P]),
+    "hyc_lora_add_restore_group": (_I, [_P, _I, _L, _L, _I, _P]),
 }
 
 

@@ -153,12 +153,12 @@ __device__ __forceinline__ void lora_add_rows(const LoraAddArgs& a, int64_t row_
 }
 
 template <int QBIT, int KSTEPS, int MODE, bool ZP>
-__global__ __launch_bounds__(kAddThreads) void lora_add_kernel(const LoraAddArgs a) {
+__device__ __forceinline__ void lora_add_block(const LoraAddArgs& a, int block) {
     constexpr int CT = MODE == kAddPlain ? 1 : kColTilesPerGroup<QBIT>, RS = kAddWaves / CT;
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int col_tile = (blockIdx.x % a.col_tiles) * CT + wave % CT;     // a.col_tiles counts groups of CT tiles
-    const int64_t row_tile = blockIdx.x / a.col_tiles;
+    const int col_tile = (block % a.col_tiles) * CT + wave % CT;     // a.col_tiles counts groups of CT tiles
+    const int64_t row_tile = block / a.col_tiles;
     const int chunk = col_tile * (kTileCols / 8) + (lane & 15);
     const bool active = chunk < a.C;
     const int col0 = chunk * 8;
@@ -214,7 +214,41 @@ __global__ __launch_bounds__(kAddThreads) void lora_add_kernel(const LoraAddArgs
     lora_add_rows<QBIT, KSTEPS, MODE, ZP, false>(a, row_begin, row_end, lane, chunk, active, qc, z, B);
 }
 
+template <int QBIT, int KSTEPS, int MODE, bool ZP>
+__global__ __launch_bounds__(kAddThreads) void lora_add_kernel(const LoraAddArgs a) {
+    lora_add_block<QBIT, KSTEPS, MODE, ZP>(a, (int)blockIdx.x);
+}
+
+// Several operand sets in one launch (the q, k and v projections of a layer: same rows, rank and code
+// width, each its own width, steps, adapter, rotation tables or none): the grid is the members' grids one
+// after the other.  A [4096, 4096] or [4096, 1024] operand alone is one short generation of waves - its
+// launch is mostly ramp and drain; together the members run like one wide operand.
+constexpr int kAddGroupMax = 4;
+struct LoraAddGroup {
+    LoraAddArgs m[kAddGroupMax];
+    int first_block[kAddGroupMax + 1];
+    int count;
+};
+
+template <int QBIT, int KSTEPS, int MODE, bool ZP>
+__global__ __launch_bounds__(kAddThreads) void lora_add_group_kernel(const LoraAddGroup g) {
+    int mi = 0;
+#pragma unroll
+    for (int i = 1; i < kAddGroupMax; ++i)
+        if (i < g.count && (int)blockIdx.x >= g.first_block[i]) mi = i;
+    lora_add_block<QBIT, KSTEPS, MODE, ZP>(g.m[mi], (int)blockIdx.x - g.first_block[mi]);
+}
+
 // ------------------------------------------------------------------------------------
+template <int QB, int MODE, bool ZP>
+static void add_group_launch_k(const LoraAddGroup& g, dim3 grid, int ksteps, hipStream_t st) {
+    const dim3 block(kAddThreads);
+    if (ksteps == 1) hipLaunchKernelGGL((lora_add_group_kernel<QB, 1, MODE, ZP>), grid, block, 0, st, g);
+    else if (ksteps == 2) hipLaunchKernelGGL((lora_add_group_kernel<QB, 2, MODE, ZP>), grid, block, 0, st, g);
+    else if (ksteps == 3) hipLaunchKernelGGL((lora_add_group_kernel<QB, 3, MODE, ZP>), grid, block, 0, st, g);
+    else hipLaunchKernelGGL((lora_add_group_kernel<QB, 4, MODE, ZP>), grid, block, 0, st, g);
+}
+
 template <int QB, int MODE, bool ZP>
 static void add_launch_k(const LoraAddArgs& a, dim3 grid, int ksteps, hipStream_t st) {
     const dim3 block(kAddThreads);
@@ -224,8 +258,11 @@ static void add_launch_k(const LoraAddArgs& a, dim3 grid, int ksteps, hipStream_
     else hipLaunchKernelGGL((lora_add_kernel<QB, 4, MODE, ZP>), grid, block, 0, st, a);
 }
 
+// Checks one operand set and fills in its launch shape: 1 = launch `blocks` workgroups, HYC_OK = nothing to do,
+// negative = error.
 template <int MODE>
-static int add_launch(LoraAddArgs& a, int64_t T, int64_t N, int64_t R, int q_bit, void* stream) {
+static int add_prepare(LoraAddArgs& a, int64_t T, int64_t N, int64_t R, int q_bit, int64_t& blocks) {
+    blocks = 0;
     if (MODE != kAddPlain && q_bit != 2 && q_bit != 4 && q_bit != 8) return HYC_ERR_QBIT;
     if (T < 0 || N < 0 || N % 32 != 0 || N > (1 << 28) || T > ((int64_t)1 << 40)) return HYC_ERR_SHAPE;
     if (R < 4 || R > 64 || R % 4 != 0) return HYC_ERR_RANK;
@@ -255,7 +292,16 @@ static int add_launch(LoraAddArgs& a, int64_t T, int64_t N, int64_t R, int q_bit
     a.col_tiles = (int)cdiv(cdiv(N, kTileCols), ct);
     const int64_t row_tiles = cdiv(T, (int64_t)(kAddWaves / ct) * a.rows_per_wave);
     if (row_tiles * a.col_tiles > INT32_MAX) return HYC_ERR_SHAPE;
-    const dim3 grid((unsigned)(row_tiles * a.col_tiles));
+    blocks = row_tiles * a.col_tiles;
+    return 1;
+}
+
+template <int MODE>
+static int add_launch(LoraAddArgs& a, int64_t T, int64_t N, int64_t R, int q_bit, void* stream) {
+    int64_t blocks;
+    const int rc = add_prepare<MODE>(a, T, N, R, q_bit, blocks);
+    if (rc <= 0) return rc;
+    const dim3 grid((unsigned)blocks);
     const int ksteps = (int)cdiv(R, 16);
     hipStream_t st = (hipStream_t)stream;
     if constexpr (MODE == kAddPlain) {
@@ -266,6 +312,53 @@ static int add_launch(LoraAddArgs& a, int64_t T, int64_t N, int64_t R, int q_bit
         else if (q_bit == 4) { if (zp) add_launch_k<4, MODE, true>(a, grid, ksteps, st); else add_launch_k<4, MODE, false>(a, grid, ksteps, st); }
         else { if (zp) add_launch_k<2, MODE, true>(a, grid, ksteps, st); else add_launch_k<2, MODE, false>(a, grid, ksteps, st); }
     }
+    return check_launch();
+}
+
+static void member_args(const hyc_lora_add_member& m, LoraAddArgs& a, bool quant) {
+    a = LoraAddArgs{};
+    a.b_transposed = m.b_transposed;
+    a.xa = (const uint16_t*)m.xa; a.b = (const uint16_t*)m.b; a.y = (uint16_t*)m.y;
+    if (quant) a.x = (const uint16_t*)m.x;
+    a.s = (const uint16_t*)m.scale; a.zp = (const uint16_t*)m.zero_point; a.q = (uint8_t*)m.q;
+    a.cos_t = m.cos_t; a.sin_t = m.sin_t; a.rope_f32 = m.table_is_fp32; a.S = (int)m.seq_len;
+    a.stride_cos = m.stride_cos; a.stride_sin = m.stride_sin;
+}
+
+template <int MODE>
+static int add_group_launch(const hyc_lora_add_member* members, int count, int64_t T, int64_t R, int q_bit, void* stream) {
+    if (!members) return HYC_ERR_NULL;
+    if (count < 1 || count > kAddGroupMax) return HYC_ERR_ARG;
+    LoraAddGroup g{};
+    int64_t total = 0;
+    int n = 0;
+    const bool zp = members[0].zero_point != nullptr;
+    for (int i = 0; i < count; ++i) {
+        const hyc_lora_add_member& m = members[i];
+        if ((m.zero_point != nullptr) != zp) return HYC_ERR_ARG;            // one kernel: all with a zero point or none
+        if ((m.cos_t != nullptr) != (m.sin_t != nullptr)) return HYC_ERR_NULL;
+        if (m.cos_t && (m.seq_len <= 0 || m.seq_len > INT32_MAX)) return HYC_ERR_SHAPE;
+        LoraAddArgs a;
+        member_args(m, a, MODE == kAddQuant);
+        int64_t blocks;
+        const int rc = add_prepare<MODE>(a, T, m.N, R, q_bit, blocks);
+        if (rc < 0) return rc;
+        if (rc == 0) continue;                                              // an empty member
+        g.m[n] = a;
+        g.first_block[n] = (int)total;
+        total += blocks;
+        if (total > INT32_MAX) return HYC_ERR_SHAPE;
+        ++n;
+    }
+    if (n == 0) return HYC_OK;
+    g.count = n;
+    g.first_block[n] = (int)total;
+    const dim3 grid((unsigned)total);
+    const int ksteps = (int)cdiv(R, 16);
+    hipStream_t st = (hipStream_t)stream;
+    if (q_bit == 8) { if (zp) add_group_launch_k<8, MODE, true>(g, grid, ksteps, st); else add_group_launch_k<8, MODE, false>(g, grid, ksteps, st); }
+    else if (q_bit == 4) { if (zp) add_group_launch_k<4, MODE, true>(g, grid, ksteps, st); else add_group_launch_k<4, MODE, false>(g, grid, ksteps, st); }
+    else { if (zp) add_group_launch_k<2, MODE, true>(g, grid, ksteps, st); else add_group_launch_k<2, MODE, false>(g, grid, ksteps, st); }
     return check_launch();
 }
 
@@ -343,4 +436,14 @@ extern "C" int hyc_lora_add_restore_rope(const void* xa, const void* b, int b_tr
     a.cos_t = cos_t; a.sin_t = sin_t; a.rope_f32 = table_is_fp32; a.S = (int)seq_len;
     a.stride_cos = stride_cos; a.stride_sin = stride_sin;
     return add_launch<kAddRestore>(a, T, N, R, q_bit, stream);
+}
+
+extern "C" int hyc_lora_add_quant_group(const hyc_lora_add_member* members, int count, int64_t T, int64_t R, int q_bit,
+                                        void* stream) {
+    return add_group_launch<kAddQuant>(members, count, T, R, q_bit, stream);
+}
+
+extern "C" int hyc_lora_add_restore_group(const hyc_lora_add_member* members, int count, int64_t T, int64_t R,
+                                          int q_bit, void* stream) {
+    return add_group_launch<kAddRestore>(members, count, T, R, q_bit, stream);
 }

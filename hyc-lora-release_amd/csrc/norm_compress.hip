@@ -24,6 +24,15 @@
 
 namespace hyc {
 
+// Entry j of a lane's eight outlier-table entries: 1 + position in the channel list, 0 for an ordinary channel.
+// A position past the list (a table built for another, longer list) is read as "ordinary channel": the
+// kernels index x_outlier[row * k + position] with it.
+__device__ __forceinline__ uint32_t table_pos(const uint32_t (&td)[4], int j, int k) {
+    const uint32_t p = (td[j >> 1] >> (16 * (j & 1))) & 0xffffu;
+    return p <= (uint32_t)k ? p : 0u;
+}
+
+
 constexpr int kNcThreads = 256;
 constexpr int kNcWaves = kNcThreads / kWave;
 
@@ -139,7 +148,7 @@ void rmsnorm_fwd_compress_kernel(const NormCompressArgs a) {
                     const uint32_t xd[4] = {xc.x, xc.y, xc.z, xc.w};
 #pragma unroll
                     for (int j = 0; j < 8; ++j) {
-                        const uint32_t p = (td[j >> 1] >> (16 * (j & 1))) & 0xffffu;
+                        const uint32_t p = table_pos(td, j, a.k);
                         if (p) {
                             a.xo[row * a.k + (p - 1)] = (uint16_t)(xd[j >> 1] >> (16 * (j & 1)));
                             f[j] = 0.0f;
@@ -287,7 +296,7 @@ void rmsnorm_fwd_compress_slab_kernel(const NormCompressArgs a, const XaArgs xa,
                 if (has_outlier) {
 #pragma unroll
                     for (int j = 0; j < 8; ++j) {
-                        const uint32_t p = (td[j >> 1] >> (16 * (j & 1))) & 0xffffu;
+                        const uint32_t p = table_pos(td, j, a.k);
                         if (p) {
                             a.xo[row * a.k + (p - 1)] = (uint16_t)(__float_as_uint(f[g][j]) >> 16);
                             f[g][j] = 0.0f;
@@ -462,7 +471,7 @@ void rmsnorm_bwd_codes_slab_kernel(const NormBwdCodesArgs a, int rows_per_group)
         int cnt = 0;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            const uint32_t p = (td[j >> 1] >> (16 * (j & 1))) & 0xffffu;
+            const uint32_t p = table_pos(td, j, a.k);
             if (p) {
                 oslot |= (uint32_t)(cnt < 2 ? cnt + 1 : 3) << (2 * j);
                 if (cnt == 0) opos0 = p - 1;
@@ -521,7 +530,7 @@ void rmsnorm_bwd_codes_slab_kernel(const NormBwdCodesArgs a, int rows_per_group)
                     if (code == 1) x[j] = __uint_as_float(ov[g][0] << 16);
                     else if (code == 2) x[j] = __uint_as_float(ov[g][1] << 16);
                     else if (code == 3) {
-                        const uint32_t p = (td[j >> 1] >> (16 * (j & 1))) & 0xffffu;
+                        const uint32_t p = table_pos(td, j, a.k);
                         x[j] = __uint_as_float((uint32_t)a.xo[(r + g) * a.k + (p - 1)] << 16);
                     }
                 }
@@ -790,7 +799,7 @@ namespace hyc {
 // 4096 channels here.  Returns 1 when the shape does not fit the slabs (the caller keeps its own kernel).
 int rmsnorm_bwd_dense_slab(const void* dy, const void* x, const void* weight, int weight_is_fp32, const float* rstd,
                            const void* residual, void* dx, int64_t rows, int64_t N, void* stream) {
-    if (!slab_shape(rows, N)) return 1;
+    if (!g_slab_enabled || !slab_shape(rows, N)) return 1;       // "norm_compress_slab" 0: the row-per-wave kernel
     NormBwdCodesArgs a{};
     a.x = (const uint16_t*)x; a.dy = (const uint16_t*)dy; a.w = weight; a.rstd = rstd;
     a.res = (const uint16_t*)residual; a.dx = (uint16_t*)dx; a.rows = rows; a.N = (int)N; a.k = 0;

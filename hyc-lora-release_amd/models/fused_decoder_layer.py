@@ -144,28 +144,41 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             w, b, qs, la, lb = W[name]
             return lora_forward(w, qs, la, lb, b, inp, residual=residual, x_lora_a=xa_ready.pop(name, None))
 
-        def proj_quant(name, inp, zp=False, rotate=False):
-            """Projection `name` of inp with the frozen part quantised on the way: -> (output, x @ A,
-            whether the output is already rotated).  One kernel reads the frozen part once, writes its
-            codes, adds the LoRA product and - for q and k with heads of 128 dims - applies the rotary
-            embedding; the reference quantises `*_main`, adds and rotates in separate passes
-            (…full_fuse.py:105-152)."""
-            w, b, qs, la, lb = W[name]
-            main, xa = lora_parts(w, qs, la, b, inp, xa_ready.pop(name, None))
-            lb = lb.to(main.dtype)
-            if not (lora_kernels.supported(main, xa, lb) and main.dim() == 3):
-                (quant_zp if zp else quant)(name + "_main", main, name)
-                return main + xa @ lb, xa, False
-            rope = (cos, sin) if rotate and head_dim == lora_kernels.ROPE_HEAD_DIM else None
-            if zp:
-                s_, z_ = get_statistics_only_quant_zero_point(main, q_bit, 'per-channel') if calib else \
-                    (sv[name]['scale'], sv[name]['zero_point'])
-                stats[(name, "zero_point")] = saved[name + "_main_z"] = z_
-            else:
-                s_, z_ = get_statistics_only_quant(main, q_bit, 'per-channel') if calib else sv[name]['scale'], None
-            stats[(name, "scale")] = saved[name + "_main_s"] = s_
-            saved[name + "_main_q"], y = lora_kernels.lora_add_quant(main, xa, lb, s_, z_, q_bit, inplace=True, rope=rope)
-            return y, xa, rope is not None
+        def proj_quant_group(names, inp, zp=(), rotate=()):
+            """Projections `names` of inp with their frozen parts quantised on the way:
+            -> {name: (output, x @ A, whether the output is already rotated)}.  One kernel reads a frozen
+            part once, writes its codes, adds the LoRA product and - for the names in `rotate`, with heads of
+            128 dims - applies the rotary embedding; the reference quantises `*_main`, adds and rotates in
+            separate passes (…full_fuse.py:105-152).  The members that share a kind of code (with / without a
+            zero point) go into one launch."""
+            out, ready = {}, []
+            for name in names:
+                w, b, qs, la, lb = W[name]
+                main, xa = lora_parts(w, qs, la, b, inp, xa_ready.pop(name, None))
+                lb = lb.to(main.dtype)
+                with_zp = name in zp
+                if not (lora_kernels.supported(main, xa, lb) and main.dim() == 3):
+                    (quant_zp if with_zp else quant)(name + "_main", main, name)
+                    out[name] = (main + xa @ lb, xa, False)
+                    continue
+                rope = (cos, sin) if name in rotate and head_dim == lora_kernels.ROPE_HEAD_DIM else None
+                if with_zp:
+                    s_, z_ = get_statistics_only_quant_zero_point(main, q_bit, 'per-channel') if calib else \
+                        (sv[name]['scale'], sv[name]['zero_point'])
+                    stats[(name, "zero_point")] = saved[name + "_main_z"] = z_
+                else:
+                    s_, z_ = get_statistics_only_quant(main, q_bit, 'per-channel') if calib else sv[name]['scale'], None
+                stats[(name, "scale")] = saved[name + "_main_s"] = s_
+                ready.append((name, dict(x_main=main, xa=xa, b=lb, scale=s_, zero_point=z_, rope=rope)))
+            for with_zp in (True, False):
+                group = [(n, it) for n, it in ready if (it["zero_point"] is not None) == with_zp]
+                for g0 in range(0, len(group), lora_kernels.GROUP_MAX):
+                    part = group[g0:g0 + lora_kernels.GROUP_MAX]
+                    results = lora_kernels.lora_add_quant_group([it for _, it in part], q_bit, inplace=True)
+                    for (n, it), (q_, y_) in zip(part, results):
+                        saved[n + "_main_q"] = q_
+                        out[n] = (y_, it["xa"], it["rope"] is not None)
+            return out
 
         def quant(name, t, key=None):
             if raw:
@@ -230,9 +243,12 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             k, _, saved["k_lora_a"] = proj("k", x_norm_1)
             v, _, saved["v_lora_a"] = proj("v", x_norm_1)
         else:
-            q, saved["q_lora_a"], q_rotated = proj_quant("q", x_norm_1, zp=spec.attention == "sdpa", rotate=True)
-            k, saved["k_lora_a"], k_rotated = proj_quant("k", x_norm_1, zp=spec.attention == "sdpa", rotate=True)
-            v, saved["v_lora_a"], _ = proj_quant("v", x_norm_1)
+            qkv = proj_quant_group(("q", "k", "v"), x_norm_1, zp=("q", "k") if spec.attention == "sdpa" else (),
+                                   rotate=("q", "k"))
+            q, saved["q_lora_a"], q_rotated = qkv["q"]
+            k, saved["k_lora_a"], k_rotated = qkv["k"]
+            v, saved["v_lora_a"], _ = qkv["v"]
+            del qkv
         if not norm_1_done:
             quant("x_norm_1", x_norm_1)
         del x_norm_1
@@ -287,8 +303,8 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
                         _note_map_entries(host_state, saved["a_idx"].numel())
                 else:
                     # frozen threshold: the lists get room for a little more than the recent steps
-                    # needed and nothing is read back here; whether they fitted is looked at when the
-                    # rest of the forward pass has been enqueued (the map is kept until then)
+                    # needed and nothing is read back here; whether they fitted is looked at after the
+                    # o projection has been enqueued (the map is kept until then)
                     saved["a_idx"], saved["a_val"], saved["a_seg"], count = compress_attention_map(a, thr, seg, capacity=capacity)
                     map_pending = (a, thr, count, capacity)
             o = heads_matmul(a, v, out_hidden=True)
@@ -314,6 +330,17 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
         x_medium, _, saved["o_lora_a"] = proj("o", o, residual=x)       # x + o_proj(o) in the projection's add pass
         quant("o", o)
         del o
+        if map_pending is not None:
+            # The dense map (B*H*S*S bf16, 537 MB at 2 x 32 x 2048^2) is let go before the MLP block allocates
+            # its gate / up tensors.  The wait is for the compaction only, which was enqueued before the two
+            # attention products and the o projection the device still has to run.
+            a, thr, count, capacity = map_pending
+            nnz = count.value()
+            if nnz > capacity:                    # did not fit: write the lists again at their exact size
+                saved["a_idx"], saved["a_val"], saved["a_seg"] = compress_attention_map(a, thr, saved["a_seg"])
+            _note_map_entries(host_state, nnz)
+            del a, map_pending
+            map_pending = None
 
         # ---- MLP block ---------------------------------------------------------------------------
         x_norm_2, saved["rstd_2"], norm_2_done = norm_block("x_medium", "x_norm_2", x_medium, norm_weight_2, ("gate", "up"))
@@ -341,8 +368,9 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             del gate_main, up_main
         else:
             if spec.mode == "intra_inter":
-                gate, gate_lora_a, _ = proj_quant("gate", x_norm_2)
-                up, up_lora_a, _ = proj_quant("up", x_norm_2)
+                gu = proj_quant_group(("gate", "up"), x_norm_2)
+                (gate, gate_lora_a, _), (up, up_lora_a, _) = gu["gate"], gu["up"]
+                del gu
                 hadamard = silu_hadamard(gate, up)
             else:                                           # 'intra' and 'baseline'
                 gate, _, gate_lora_a = proj("gate", x_norm_2)
@@ -362,13 +390,6 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
         if whole:
             quant("hadamard", hadamard)
         del hadamard
-        if map_pending is not None:
-            a, thr, count, capacity = map_pending
-            nnz = count.value()                   # waits for the compaction only; the device still has the MLP block to run
-            if nnz > capacity:                    # did not fit: write the lists again at their exact size
-                saved["a_idx"], saved["a_val"], saved["a_seg"] = compress_attention_map(a, thr, saved["a_seg"])
-            _note_map_entries(host_state, nnz)
-            del a, map_pending
 
         ctx.names = list(saved.keys())
         ctx.save_for_backward(*saved.values(), cos, sin, norm_weight_1, norm_weight_2,
@@ -422,18 +443,30 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             G[name] = (ga, gb)
             return gx
 
-        def rebuilt_hidden(name, rotate=False):
-            """Output of projection `name` as forward produced it, from the codes of its frozen part
-            and the saved x @ A: dequantise + LoRA add (+ the rotary embedding for q and k with heads
-            of 128 dims) in one kernel (…full_fuse.py:416-417,439-452).  -> (tensor, rotated or not)."""
-            xa, lb = S[name + "_lora_a"], W[name][4]
-            lb = lb.to(xa.dtype)
-            q_, s_, z_ = S[name + "_main_q"], S[name + "_main_s"], S.get(name + "_main_z")
-            if lora_kernels.supported_restore(q_, xa, lb):
-                rope = (cos, sin) if rotate and D == lora_kernels.ROPE_HEAD_DIM else None
-                return lora_kernels.lora_add_restore(q_, s_, xa, lb, z_, q_bit, rope=rope), rope is not None
-            main = deq(name + "_main")
-            return main + (xa @ lb).to(main.dtype), False
+        def rebuilt_hidden_group(names, rotate=()):
+            """Outputs of projections `names` as forward produced them, from the codes of their frozen parts
+            and the saved x @ A: dequantise + LoRA add (+ the rotary embedding for the names in `rotate`, with
+            heads of 128 dims) in one kernel, the members with the same kind of code in one launch
+            (…full_fuse.py:416-417,439-452).  -> {name: (tensor, rotated or not)}."""
+            out, ready = {}, []
+            for name in names:
+                xa, lb = S[name + "_lora_a"], W[name][4]
+                lb = lb.to(xa.dtype)
+                q_, s_, z_ = S[name + "_main_q"], S[name + "_main_s"], S.get(name + "_main_z")
+                if lora_kernels.supported_restore(q_, xa, lb):
+                    rope = (cos, sin) if name in rotate and D == lora_kernels.ROPE_HEAD_DIM else None
+                    ready.append((name, dict(q=q_, scale=s_, xa=xa, b=lb, zero_point=z_, rope=rope)))
+                else:
+                    main = deq(name + "_main")
+                    out[name] = (main + (xa @ lb).to(main.dtype), False)
+            for with_zp in (True, False):
+                group = [(n, it) for n, it in ready if (it["zero_point"] is not None) == with_zp]
+                for g0 in range(0, len(group), lora_kernels.GROUP_MAX):
+                    part = group[g0:g0 + lora_kernels.GROUP_MAX]
+                    results = lora_kernels.lora_add_restore_group([it for _, it in part], q_bit)
+                    for (n, it), y_ in zip(part, results):
+                        out[n] = (y_, it["rope"] is not None)
+            return out
 
         def channel_base_restored(name, channels):
             if name + "_raw" in S:
@@ -488,7 +521,9 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
         else:
             fn = None
             if spec.mode == "intra_inter":
-                gate, up = rebuilt_hidden("gate")[0], rebuilt_hidden("up")[0]
+                gu = rebuilt_hidden_group(("gate", "up"))
+                gate, up = gu["gate"][0], gu["up"][0]
+                del gu
                 if gate.dtype == up.dtype == torch.bfloat16:
                     hadamard = silu_once_hadamard(gate, up)   # up * F.silu(gate), as the reference recomputes it
                 else:
@@ -518,18 +553,20 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
         grad_o = back("o", "o", S["o_lora_a"], grad_medium)
         grad_o = hidden_to_head_shape(grad_o, H)
 
-        def rebuilt(name, heads):
-            """q/k/v in head shape as the forward attention saw them (before repeat_kv)."""
-            t, rotated = rebuilt_hidden(name, rotate=name != "v")
-            t = hidden_to_head_shape(t, heads)
-            if name != "v" and not rotated:
-                t = rope_forward(t.transpose(1, 2), cos, sin).transpose(1, 2)
-            return t
-
         if spec.mode in ("baseline", "intra"):
             q, k, v = (deq(n, is_head=True, num_heads=H) for n in ("q_rope", "k_rope", "v_rep"))
         else:
+            qkv = rebuilt_hidden_group(("q", "k", "v"), rotate=("q", "k"))
+
+            def rebuilt(name, heads):
+                """q/k/v in head shape as the forward attention saw them (before repeat_kv)."""
+                t, rotated = qkv[name]
+                t = hidden_to_head_shape(t, heads)
+                if name != "v" and not rotated:
+                    t = rope_forward(t.transpose(1, 2), cos, sin).transpose(1, 2)
+                return t
             q, k, v = rebuilt("q", H), repeat_kv(rebuilt("k", KV), n_rep), repeat_kv(rebuilt("v", KV), n_rep)
+            del qkv
 
         if spec.attention == "map":
             # grad_a first, then the restored map and the softmax backward come out of one pass over

@@ -169,6 +169,105 @@ def lora_add_restore(q, scale, xa, b, zero_point=None, quantize_bit=8, rope=None
     return y
 
 
+GROUP_MAX = 4                # operand sets one grouped launch takes
+
+
+def _member(xa, b, bt, x, s, z, q, y, rope_tables, n):
+    m = _lib.LoraAddMember()
+    m.xa, m.b, m.b_transposed, m.x = xa.data_ptr(), b.data_ptr(), bt, _lib.ptr(x)
+    m.scale, m.zero_point, m.q, m.y, m.N = s.data_ptr(), _lib.ptr(z), q.data_ptr(), y.data_ptr(), n
+    if rope_tables is not None:
+        cos, sin, seq = rope_tables
+        m.cos_t, m.sin_t, m.table_is_fp32 = cos.data_ptr(), sin.data_ptr(), int(cos.dtype == torch.float32)
+        m.seq_len, m.stride_cos, m.stride_sin = seq, cos.stride(0), sin.stride(0)
+    return m
+
+
+def lora_add_quant_group(items, quantize_bit=8, inplace=False):
+    """lora_add_quant for up to GROUP_MAX operand sets in one launch -> [(q, y), ...], each pair the same bits
+    as its own call.  items: dicts with x_main [B, M, N_i], xa [B, M, R], b [R, N_i], scale, and optionally
+    zero_point (all items or none) and rope=(cos, sin); B, M and R are shared."""
+    if quantize_bit not in (2, 4, 8):
+        raise ValueError(f"quantize_bit must be 2, 4 or 8, got {quantize_bit}")
+    if not 1 <= len(items) <= GROUP_MAX:
+        raise ValueError(f"a group holds 1 to {GROUP_MAX} operand sets, got {len(items)}")
+    B, M = items[0]["x_main"].shape[:2]
+    members, outs, keep = [], [], []
+    rank = None
+    for it in items:
+        x_main, xa, b, scale, zp, rope = it["x_main"], it["xa"], it["b"], it["scale"], it.get("zero_point"), it.get("rope")
+        if x_main.dim() != 3 or tuple(x_main.shape[:2]) != (B, M):
+            raise ValueError(f"every x_main must be [{B}, {M}, N], got shape {tuple(x_main.shape)}")
+        n = x_main.shape[-1]
+        r = _check(xa, b, n, B * M)
+        if rank not in (None, r):
+            raise ValueError("the members of a group share one LoRA rank")
+        rank = r
+        if (zp is None) != (items[0].get("zero_point") is None):
+            raise ValueError("either every member of a group has a zero point or none has")
+        _vec_ok(scale, n, "scale")
+        _vec_ok(zp, n, "zero point")
+        _lib.require_gpu(x_main, xa, b, scale, zp)
+        x = _prep(x_main, "x_main")
+        y = x if (inplace and x is x_main) else torch.empty_like(x)
+        xa, (b, bt) = _prep(xa, "xa"), _lora_b(b)
+        s = _vec(scale, n, "scale")
+        z = None if zp is None else _vec(zp, n, "zero point")
+        q = torch.empty((B, M, n * quantize_bit // 8), device=x.device, dtype=torch.uint8)
+        tables = None
+        if rope is not None:
+            if n % ROPE_HEAD_DIM:
+                raise ValueError(f"the fused rotation needs a width that is a multiple of {ROPE_HEAD_DIM}, got {n}")
+            tables = _rope_tables(rope, M) + (M,)
+        members.append(_member(xa, b, bt, x, s, z, q, y, tables, n))
+        keep.append((x, xa, b, s, z, tables))
+        outs.append((q, y))
+    arr = (_lib.LoraAddMember * len(members))(*members)
+    _lib.call("hyc_lora_add_quant_group", arr, len(members), B * M, rank, quantize_bit, _lib.stream_of(outs[0][0]))
+    return outs
+
+
+def lora_add_restore_group(items, quantize_bit=8):
+    """lora_add_restore for up to GROUP_MAX operand sets in one launch -> [y, ...].  items: dicts with q
+    [B, M, N_i*bits/8], scale, xa, b and optionally zero_point (all or none) and rope=(cos, sin)."""
+    if quantize_bit not in (2, 4, 8):
+        raise ValueError(f"quantize_bit must be 2, 4 or 8, got {quantize_bit}")
+    if not 1 <= len(items) <= GROUP_MAX:
+        raise ValueError(f"a group holds 1 to {GROUP_MAX} operand sets, got {len(items)}")
+    B, M = items[0]["q"].shape[:2]
+    members, outs, keep = [], [], []
+    rank = None
+    for it in items:
+        q, scale, xa, b, zp, rope = it["q"], it["scale"], it["xa"], it["b"], it.get("zero_point"), it.get("rope")
+        n = scale.numel()
+        if q.dim() != 3 or tuple(q.shape[:2]) != (B, M) or q.shape[2] * 8 != n * quantize_bit or q.dtype != torch.uint8:
+            raise ValueError(f"packed codes must be uint8 [{B}, {M}, {n * quantize_bit // 8}], got {q.dtype} {tuple(q.shape)}")
+        r = _check(xa, b, n, B * M)
+        if rank not in (None, r):
+            raise ValueError("the members of a group share one LoRA rank")
+        rank = r
+        if (zp is None) != (items[0].get("zero_point") is None):
+            raise ValueError("either every member of a group has a zero point or none has")
+        _vec_ok(zp, n, "zero point")
+        _lib.require_gpu(q, scale, xa, b, zp)
+        q = q.contiguous()
+        xa, (b, bt) = _prep(xa, "xa"), _lora_b(b)
+        s = _vec(scale, n, "scale")
+        z = None if zp is None else _vec(zp, n, "zero point")
+        y = torch.empty((B, M, n), device=q.device, dtype=BF16)
+        tables = None
+        if rope is not None:
+            if n % ROPE_HEAD_DIM:
+                raise ValueError(f"the fused rotation needs a width that is a multiple of {ROPE_HEAD_DIM}, got {n}")
+            tables = _rope_tables(rope, M) + (M,)
+        members.append(_member(xa, b, bt, None, s, z, q, y, tables, n))
+        keep.append((q, xa, b, s, z, tables))
+        outs.append(y)
+    arr = (_lib.LoraAddMember * len(members))(*members)
+    _lib.call("hyc_lora_add_restore_group", arr, len(members), B * M, rank, quantize_bit, _lib.stream_of(outs[0]))
+    return outs
+
+
 def contract_supported(x, n, r):
     """Whether lora_products takes a wide operand of this dtype / width and this rank."""
     return x.is_cuda and x.dtype == BF16 and n % 32 == 0 and 2 <= r <= 64 and r % 2 == 0 and x.numel() > 0

@@ -46,7 +46,8 @@ int hyc_abi_version(void);
  * default 8), "dequant_rows_per_wave" (same for hyc_unpack_dequant, default 2),
  * "quant_outlier_rows_per_wave" / "dequant_outlier_rows_per_wave" (the same two when called with
  * an outlier list; default 8 each: a wave first has to find its outlier columns in the list),
- * "norm_compress_slab" (0 / 1: whether hyc_rmsnorm_fwd_compress may use its column-slab kernel, default 1)
+ * "norm_compress_slab" (0 / 1: whether hyc_rmsnorm_fwd_compress and, for rows wider than 4096 channels,
+ * hyc_rmsnorm_bwd without a weight gradient may use the column-slab kernels, default 1)
  * and "norm_compress_rows_per_group" (rows a workgroup of that kernel walks, even; 0 = chosen from the
  * row count, the default),
  * "fuse_rows_per_wave" (same for both fused LoRA-SiLU kernels, multiple of 16; default 0 = by code width
@@ -543,6 +544,34 @@ int hyc_lora_add_restore_rope(const void *xa, const void *b, int b_transposed, c
                               const void *scale, const void *zero_point, void *y, const void *cos,
                               const void *sin, int table_is_fp32, int64_t seq_len, int64_t stride_cos,
                               int64_t stride_sin, int64_t T, int64_t N, int64_t R, int q_bit, void *stream);
+
+/* Up to four operand sets of hyc_lora_add_quant[_rope] / hyc_lora_add_restore[_rope] in ONE launch: the q, k
+ * and v projections of a layer share their rows, rank and code width, and each alone ([4096, 4096] or, with
+ * grouped-query heads, [4096, 1024]) is one short generation of waves whose launch is mostly ramp and drain.
+ * Each member's outputs are the same bits as its own call.  All members with a zero point or all without
+ * (HYC_ERR_ARG otherwise); cos / sin NULL: no rotation for that member.
+ * Replaces the three lora_forward + quantiser sequences of the q, k, v projections and their three
+ * dequantise + add (+ rope) sequences in backward
+ * (models/llama/fused_llama_layer_intra_inter_full_fuse.py:105-152, :416-452). */
+typedef struct hyc_lora_add_member {
+    const void *xa;             /* bf16 [T, R] */
+    const void *b;              /* bf16 [R, N] or, with b_transposed, [N, R] */
+    const void *x;              /* quantise: the frozen part, bf16 [T, N]; restore: unused */
+    const void *scale;          /* bf16 [N] */
+    const void *zero_point;     /* bf16 [N] or NULL */
+    void *q;                    /* uint8 [T, N*q_bit/8]: output of quantise, input of restore */
+    void *y;                    /* bf16 [T, N] */
+    const void *cos_t;          /* rotation tables as in hyc_rope, or NULL */
+    const void *sin_t;
+    int64_t seq_len, stride_cos, stride_sin;
+    int64_t N;
+    int b_transposed;
+    int table_is_fp32;
+} hyc_lora_add_member;
+int hyc_lora_add_quant_group(const hyc_lora_add_member *members, int count, int64_t T, int64_t R, int q_bit,
+                             void *stream);
+int hyc_lora_add_restore_group(const hyc_lora_add_member *members, int count, int64_t T, int64_t R, int q_bit,
+                               void *stream);
 
 /* ---------------------------------------------------------------------------------------
  * The skinny LoRA products that stream a whole [T, N] tensor X for a rank-R result, from one read

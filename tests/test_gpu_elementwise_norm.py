@@ -260,3 +260,33 @@ def test_layernorm_errors(ln, dev):
         ln.layernorm_forward(torch.zeros(2, 24, device=dev), torch.ones(24, device=dev), torch.ones(24, device=dev), 1e-5)
     with pytest.raises(Exception):
         ln.layernorm_forward(torch.zeros(2, 24, dtype=BF16), torch.ones(24, dtype=BF16), torch.ones(24, dtype=BF16), 1e-5)
+
+
+@pytest.mark.parametrize("n", [5120, 6144, 8192])
+@pytest.mark.parametrize("wdtype", [BF16, torch.float32])
+def test_rmsnorm_backward_wide_rows_both_kernels_same_bits(ops, dev, n, wdtype):
+    """Rows wider than 4096 channels: an even row count goes to the column-slab kernel, an odd one (or the
+    "norm_compress_slab" switch off) to the row-per-wave kernel.  The same rows through both must be the same
+    bits, with and without the residual add."""
+    from hyclora_amd import _lib
+    g = torch.Generator().manual_seed(n)
+    rows = 64
+    x = (torch.randn(1, rows, n, generator=g) * 2).to(BF16).to(dev)
+    dy = torch.randn(1, rows, n, generator=g).to(BF16).to(dev)
+    res = torch.randn(1, rows, n, generator=g).to(BF16).to(dev)
+    w = (1 + 0.1 * torch.randn(n, generator=g)).to(wdtype).to(dev)
+    rstd = ops.norm.rmsnorm_forward(x, w, 1e-5)[2]
+    got = {}
+    try:
+        for slab in (1, 0):
+            _lib.set_tuning("norm_compress_slab", slab)
+            got[slab] = (ops.norm._backward(dy, x, w, rstd, want_dw=False)[0],
+                         ops.norm._backward(dy, x, w, rstd, want_dw=False, residual=res)[0])
+    finally:
+        _lib.set_tuning("norm_compress_slab", 1)
+    assert torch.equal(got[1][0], got[0][0]) and torch.equal(got[1][1], got[0][1])
+    # an odd row count takes the row-per-wave kernel whatever the switch says: the first 63 rows must agree too
+    odd = ops.norm._backward(dy[:, :63], x[:, :63], w, rstd[:63], want_dw=False)[0]
+    assert torch.equal(odd, got[1][0][:, :63])
+    dx_ref, _ = O.rmsnorm_bwd(dy.cpu(), x.cpu(), w.cpu(), rstd.cpu())
+    assert_close_bf16(got[1][0], dx_ref, what="wide-row backward vs oracle")

@@ -147,6 +147,29 @@ def _saved_bytes(t, fn):
     return y, sum(seen.values())
 
 
+def map_variant_saved_bytes(out, T, H, KV, I, R, k, q_bit):
+    """Bytes the map variant keeps for backward, from the reference's save list
+    (models/llama/fused_llama_layer_intra_inter_full_fuse.py:254-285) with the shapes its producers give the
+    entries: packed codes of x, x_norm_1, q_main, o, x_medium, x_norm_2 (T*H*q/8 each), k_main, v_main
+    (T*KV*q/8), gate_main, up_main (T*I*q/8); the outlier columns of x and x_medium (T*k bf16); x @ A of the seven
+    projections (T*R bf16); rstd of the two norms (T fp32; the reference also keeps the `mean` buffers its RMSNorm
+    never fills, T fp32 each - not kept here); the steps (bf16 per channel) and the two channel lists (int64); and
+    the sparse map, 10 bytes per kept entry (int64 position + bf16 value).  The layer keeps two things more, both
+    read off its autograd node here: room for up to 1/16 + 64 more entries than the step kept (its lists are
+    sized from earlier steps' counts, without a read-back), and one int64 offset per 4096-element segment of
+    the map.  -> (expected bytes, kept entries, list slots)."""
+    node = out.grad_fn
+    raw = dict(zip(node.names, node.saved_tensors))
+    slots, nnz = raw["a_idx"].numel(), int(raw["a_seg"][-1].item())
+    assert raw["a_val"].numel() == slots and nnz <= slots <= nnz + nnz // 16 + 64, (nnz, slots)
+    code = lambda n: T * n * q_bit // 8
+    expected = 6 * code(H) + 2 * code(KV) + 2 * code(I)
+    expected += 2 * T * k * 2 + 7 * T * R * 2 + 2 * T * 4
+    expected += (6 * H + 2 * KV + 2 * I) * 2 + 2 * k * 8
+    expected += slots * 10 + raw["a_seg"].numel() * 8
+    return expected, nnz, slots
+
+
 # Parity of the layers' backward is held at the operator tolerance (1e-2 / 0.9999, all code widths) by running
 # the oracle's backward from the fused layer's own saved state (tests/test_gpu_layer_saved_state.py and (a0)
 # below).  The end-to-end comparison - forward AND backward redone by the oracle, so that its codes may differ
@@ -179,8 +202,13 @@ def test_mistral_layer_config4(dev, q_bit):
     results = []
     from test_gpu_layer_saved_state import compare, oracle_backward_from_saved_state
     for it in range(2):                       # 0: calibrating kernels, 1: frozen statistics, fused producers
-        out = L.run_fused(layer, t)
+        out, saved_bytes = _saved_bytes(t, lambda: L.run_fused(layer, t))
         if it == 1:
+            # the bytes kept for backward against the reference's save list (4096 tokens, 20 outlier channels)
+            want, nnz, slots = map_variant_saved_bytes(out, 4096, 4096, 1024, 14336, 16, 20, q_bit)
+            print(f"config 4 q{q_bit}: keeps {saved_bytes / 1e6:.1f} MB for backward, save list {want / 1e6:.1f} MB "
+                  f"({nnz} map entries in {slots} slots)")
+            assert abs(saved_bytes - want) <= 1e-3 * want, (saved_bytes, want)
             # (a0) parity proper: the oracle's backward from this very saved state, operator tolerance
             same_state = oracle_backward_from_saved_state(t, out, "intra_inter_full_fuse", q_bit, "map")
         results.append((out.detach().clone(), L.grads_of(t, out)))
@@ -308,3 +336,29 @@ def test_map_free_layer_config5(dev):
             bad.append(report[-1])
     print("config 5 q4 vs uncompressed layer: " + "; ".join(report))
     assert not bad, f"compressed gradients below the cosine floor against the uncompressed layer: {bad}"
+
+
+def test_saved_bytes_of_the_map_variant_config2(dev):
+    """Configuration 2's layer (Llama-2-7B shape, batch 4 x sequence 1024, q_bit 4, 5 % of the map kept): the bytes
+    the full_fuse layer keeps for backward equal the reference's save list, entry by entry in
+    map_variant_saved_bytes - 113.8 MB of codes, outlier columns and x @ A plus 10 bytes per kept map entry,
+    about 180 MB in all."""
+    L = _layer_tools()
+    from hyclora_amd.models import llama
+    dims = dict(B=4, S=1024, hidden=4096, heads=32, kv_heads=32, inter=11008, rank=16)
+    t = L.make_layer_inputs(dev, seed=200, **dims)
+    t.nw1.requires_grad_(False)
+    t.nw2.requires_grad_(False)
+    layer = llama.make_fused_llama_layer(L.config("intra_inter_full_fuse", 4, sm_ratio=0.05, thr=1))
+    for _ in range(2):                                      # past calibration: lists sized from the earlier counts
+        L.run_fused(layer, t).backward(t.grad)
+    out, saved_bytes = _saved_bytes(t, lambda: L.run_fused(layer, t))
+    want, nnz, slots = map_variant_saved_bytes(out, 4096, 4096, 4096, 11008, 16, 20, 4)
+    dense = 4 * 32 * 1024 * 1024
+    assert 0.03 * dense <= nnz <= 0.05 * dense + 1, f"{nnz} of {dense} map entries kept at ratio 0.05"
+    codes_etc = want - slots * 10
+    assert abs(codes_etc - 113.8e6) < 0.2e6, codes_etc      # 8*T*H/2 + 2*T*I/2 + 2*T*k*2 + 7*T*R*2 + small
+    assert 175e6 < want < 190e6, want                       # + 10 bytes for each of the ~6.7 M kept map entries
+    print(f"config 2 q4: keeps {saved_bytes / 1e6:.1f} MB for backward, save list {want / 1e6:.1f} MB ({nnz} map entries)")
+    assert abs(saved_bytes - want) <= 1e-3 * want, (saved_bytes, want)
+    out.backward(t.grad)

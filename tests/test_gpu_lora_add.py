@@ -219,3 +219,52 @@ def test_argument_checks(K, dev):
         K.add_restore(torch.zeros(1, 4, 16, device=dev, dtype=torch.uint8), d(s), d(xa), d(b), None, 4)
     with pytest.raises(RuntimeError):
         K.add(main, xa, b)                                          # CPU tensors: no fallback
+
+
+@pytest.mark.parametrize("q_bit", [2, 4, 8])
+@pytest.mark.parametrize("with_zp", [False, True])
+@pytest.mark.parametrize("dims", [(2, 96, (512, 128, 128), 16), (1, 37, (256, 256, 256, 384), 8), (3, 50, (1024,), 16),
+                                  (1, 200, (4096, 1024, 1024), 16)])
+def test_grouped_launch_equals_the_single_calls(K, dev, q_bit, with_zp, dims):
+    """q, k and v (different widths, rotation on some members only) through ONE launch of the quantise form
+    and ONE of the restore form: every member's codes and sums must be the bits its own call gives."""
+    from hyclora_amd.operators import compress_function as cf
+    from hyclora_amd.operators import lora_kernels
+    B, M, widths, R = dims
+    g = torch.Generator().manual_seed(M + q_bit)
+    pos = torch.arange(M, dtype=torch.float32)
+    inv = 1.0 / (10000.0 ** (torch.arange(0, 128, 2, dtype=torch.float32) / 128))
+    ang = torch.cat([pos[:, None] * inv[None, :]] * 2, dim=-1)
+    cos, sin = ang.cos().to(BF16).to(dev)[None], ang.sin().to(BF16).to(dev)[None]
+    items, singles = [], []
+    for i, n in enumerate(widths):
+        main, xa, b = inputs(1000 * i + n + R, B, M, n, R, shift=0.5 if with_zp else 0.0)
+        main, xa, b = main.to(dev), xa.to(dev), b.to(dev)
+        if with_zp:
+            s, z = cf.get_statistics_only_quant_zero_point(main, q_bit, 'per-channel')
+        else:
+            s, z = cf.get_statistics_only_quant(main, q_bit, 'per-channel'), None
+        rope = (cos, sin) if (n % 128 == 0 and i != len(widths) - 1) else None       # the last member is not rotated
+        items.append(dict(x_main=main, xa=xa, b=b, scale=s, zero_point=z, rope=rope))
+        singles.append(lora_kernels.lora_add_quant(main, xa, b, s, z, q_bit, rope=rope))
+    grouped = lora_kernels.lora_add_quant_group(items, q_bit)
+    for (q1, y1), (q2, y2) in zip(singles, grouped):
+        assert torch.equal(q1, q2) and torch.equal(y1, y2)
+    back_items = [dict(q=q_, scale=it["scale"], xa=it["xa"], b=it["b"], zero_point=it["zero_point"], rope=it["rope"])
+                  for it, (q_, _) in zip(items, grouped)]
+    back = lora_kernels.lora_add_restore_group(back_items, q_bit)
+    for it, y in zip(back_items, back):
+        assert torch.equal(y, lora_kernels.lora_add_restore(it["q"], it["scale"], it["xa"], it["b"], it["zero_point"], q_bit,
+                                                            rope=it["rope"]))
+
+
+def test_grouped_launch_rejects_mixed_zero_points(K, dev):
+    from hyclora_amd.operators import compress_function as cf
+    from hyclora_amd.operators import lora_kernels
+    main, xa, b = (t.to(dev) for t in inputs(5, 1, 32, 128, 16))
+    s, z = cf.get_statistics_only_quant_zero_point(main, 4, 'per-channel')
+    with pytest.raises(ValueError):
+        lora_kernels.lora_add_quant_group([dict(x_main=main, xa=xa, b=b, scale=s, zero_point=z),
+                                           dict(x_main=main, xa=xa, b=b, scale=s)], 4)
+    with pytest.raises(ValueError):
+        lora_kernels.lora_add_quant_group([dict(x_main=main, xa=xa, b=b, scale=s)] * 5, 4)

@@ -214,3 +214,30 @@ def test_lora_a_contraction_limits(ops, dev):
     assert not ops.norm.lora_a_supported(z(2, 4, 1024), w, [z(512, 16)])           # adapter of another width
     with pytest.raises(NotImplementedError):
         ops.norm.rmsnorm_forward_compress(z(1, 3, 1024), w, 1e-5, 4, lora_a=ok)
+
+
+@pytest.mark.parametrize("shape", [(1, 8, 512), (2, 34, 4096)])
+def test_a_table_of_a_longer_list_does_not_reach_past_the_outlier_buffer(ops, dev, shape):
+    """The kernels index x_outlier[row * k + position] with the positions of the caller's table.  A table built
+    for a longer channel list than the one passed (k entries) has positions past k: those channels are treated
+    as ordinary ones - the result is that of the list's first k channels - instead of being written or read
+    past the [rows, k] buffer."""
+    q_bit, n = 4, shape[-1]
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(*shape, generator=g).to(BF16).to(dev)
+    w = (1 + 0.1 * torch.randn(n, generator=g)).to(BF16).to(dev)
+    dy = torch.randn(*shape, generator=g).to(BF16).to(dev)
+    longer = torch.randperm(n, generator=g)[:12].to(dev)
+    short = longer[:5].contiguous()
+    s_x = ops.cf.get_statistics_only_quant(x, q_bit, 'per-channel')
+    s_y = ops.cf.get_statistics_only_quant(ops.norm.rmsnorm_forward(x, w, 1e-5)[0], q_bit, 'per-channel')
+    t_long, t_short = ops.norm.outlier_table(longer, n), ops.norm.outlier_table(short, n)
+    want = ops.norm.rmsnorm_forward_compress(x, w, 1e-5, q_bit, scale_y=s_y, scale_x=s_x, outlier_idx=short, table=t_short)
+    got = ops.norm.rmsnorm_forward_compress(x, w, 1e-5, q_bit, scale_y=s_y, scale_x=s_x, outlier_idx=short, table=t_long)
+    for a, b in zip(want[:5], got[:5]):
+        assert torch.equal(a, b)
+    y, rstd, q_y, q_x, xo = want[:5]
+    assert xo.shape[-1] == 5
+    d_want = ops.norm.rmsnorm_backward_from_codes(dy, q_x, s_x, xo, short, q_bit, w, rstd, table=t_short)
+    d_got = ops.norm.rmsnorm_backward_from_codes(dy, q_x, s_x, xo, short, q_bit, w, rstd, table=t_long)
+    assert torch.equal(d_want, d_got)
