@@ -5,6 +5,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/hyclora.h"
 #include "hyc_quant_math.h"
 
@@ -130,6 +132,16 @@ inline int check_launch() {
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 __host__ __device__ inline int64_t cdiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 
+
+// A launch-shape knob behind hyc_set_tuning (a benchmarking aid): an entry point reads it once per launch,
+// hyc_set_tuning writes it, both relaxed - a caller on another thread gets the old or the new value for its
+// launch, never a torn one.
+struct Knob {
+    std::atomic<int> v;
+    constexpr Knob(int x) : v(x) {}
+    int get() const { return v.load(std::memory_order_relaxed); }
+    void set(int x) { v.store(x, std::memory_order_relaxed); }
+};
 
 // Per-file tuning hooks behind hyc_set_tuning: HYC_OK / HYC_ERR_* if the key belongs to the
 // file, 1 if it does not.

@@ -25,7 +25,7 @@ namespace hyc {
 
 constexpr int kAddThreads = 256;
 constexpr int kAddWaves = kAddThreads / kWave;
-static int g_add_rows_per_wave[3] = {32, 48, 48};   // plain, quantise, restore; see hyc_set_tuning
+static Knob g_add_rows_per_wave[3]{32, 48, 48};   // plain, quantise, restore; see hyc_set_tuning
 
 enum { kAddPlain = 0, kAddQuant = 1, kAddRestore = 2 };
 
@@ -287,7 +287,7 @@ static int add_prepare(LoraAddArgs& a, int64_t T, int64_t N, int64_t R, int q_bi
     a.N = (int)N;
     a.C = (int)(N / 8);
     a.R = (int)R;
-    a.rows_per_wave = g_add_rows_per_wave[MODE];
+    a.rows_per_wave = g_add_rows_per_wave[MODE].get();
     const int ct = MODE == kAddPlain ? 1 : 8 / q_bit;
     a.col_tiles = (int)cdiv(cdiv(N, kTileCols), ct);
     const int64_t row_tiles = cdiv(T, (int64_t)(kAddWaves / ct) * a.rows_per_wave);
@@ -367,7 +367,7 @@ int tune_add(const char* key, int value) {
     for (int m = 0; m < 3; ++m) {
         if (strcmp(key, keys[m]) == 0) {
             if (value < kTileRows || value > 65536 || value % kTileRows != 0) return HYC_ERR_ARG;
-            g_add_rows_per_wave[m] = value;
+            g_add_rows_per_wave[m].set(value);
             return HYC_OK;
         }
     }

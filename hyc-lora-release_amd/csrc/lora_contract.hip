@@ -39,7 +39,7 @@ constexpr int kCtSteps = HYC_CT_STEPS;                    // 16-row steps per wa
 constexpr int kCtStrip = kCtWaves * kCtSteps * 16;        // 256 rows per workgroup
 constexpr int kCtTile = 128;                              // columns per tile
 constexpr int kCtPitch = kCtTile + 8;                     // LDS row pitch of a transposed tile (bf16 elements)
-static int g_ct_max_groups = 32;                          // column groups (bounds the P2 partials); see hyc_set_tuning
+static Knob g_ct_max_groups{32};                          // column groups (bounds the P2 partials); see hyc_set_tuning
 
 struct ContractArgs {
     const uint16_t* x;                   // dense X [T, N]
@@ -385,7 +385,7 @@ static void contract_launch_nb(ContractArgs a, dim3 grid, int nb, hipStream_t st
 static int64_t contract_geometry(int64_t T, int64_t N, int64_t R, int* tiles_per_group, int* groups, int64_t* strips,
                                  int* nb) {
     const int64_t tiles = cdiv(N, kCtTile);
-    *tiles_per_group = (int)cdiv(tiles, g_ct_max_groups);
+    *tiles_per_group = (int)cdiv(tiles, g_ct_max_groups.get());
     *groups = (int)cdiv(tiles, *tiles_per_group);
     *strips = cdiv(T, kCtStrip);
     *nb = (int)cdiv(R, 16);
@@ -395,7 +395,7 @@ static int64_t contract_geometry(int64_t T, int64_t N, int64_t R, int* tiles_per
 int tune_contract(const char* key, int value) {
     if (strcmp(key, "contract_max_groups") == 0) {
         if (value < 1 || value > 65536) return HYC_ERR_ARG;
-        g_ct_max_groups = value;
+        g_ct_max_groups.set(value);
         return HYC_OK;
     }
     return 1;

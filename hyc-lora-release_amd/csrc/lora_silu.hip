@@ -49,10 +49,10 @@ template <int QBIT> constexpr bool kStreamCodes = QBIT == 8;
 // workgroup is four strips of ONE column tile, and short strips do better: measured on [4096, 11008] and
 // [4096, 14336], forward 32 rows (69.9 / 64.4 % of peak against 70.7 / 60.0 % at 96), backward 16 rows
 // (65.1 / 67.0 % against 66.9 / 63.1 % at 32).
-static int g_fuse_rows_per_wave[2] = {0, 0};
+static Knob g_fuse_rows_per_wave[2]{0, 0};
 
 static int fuse_rows_per_wave(bool fwd, int q_bit, int64_t T, int64_t N) {
-    const int set = g_fuse_rows_per_wave[fwd ? 1 : 0];
+    const int set = g_fuse_rows_per_wave[fwd ? 1 : 0].get();
     if (set) return set;
     if (!fwd) return q_bit == 8 ? 16 : 32;
     if (q_bit == 8) return 32;
@@ -453,8 +453,8 @@ int tune_fuse(const char* key, int value) {
     const bool bwd = both || strcmp(key, "fuse_bwd_rows_per_wave") == 0;
     if (fwd || bwd) {
         if (value < 0 || value > 65536 || value % kTileRows != 0) return HYC_ERR_ARG;     // 0: by size
-        if (bwd) g_fuse_rows_per_wave[0] = value;
-        if (fwd) g_fuse_rows_per_wave[1] = value;
+        if (bwd) g_fuse_rows_per_wave[0].set(value);
+        if (fwd) g_fuse_rows_per_wave[1].set(value);
         return HYC_OK;
     }
     return 1;

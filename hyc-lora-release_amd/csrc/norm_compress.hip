@@ -177,8 +177,8 @@ void rmsnorm_fwd_compress_kernel(const NormCompressArgs a) {
 // and all codes are the same bits as from the kernel above.  The partial sums are double-buffered:
 // a wave can be at most one step ahead of the slowest one.
 constexpr int kSlabRows = 2;                        // rows per step; row counts must be a multiple of it
-static int g_slab_rows_per_group = 0;               // strip height per workgroup; 0 = from the row count
-static int g_slab_enabled = 1;
+static Knob g_slab_rows_per_group{0};               // strip height per workgroup; 0 = from the row count
+static Knob g_slab_enabled{1};
 
 // Compute units of the current device (asked once; 256 if the query fails).
 static int compute_units() {
@@ -624,11 +624,11 @@ static void launch_slab(K kernel, dim3 grid, dim3 block, size_t lds, hipStream_t
 
 template <int QBIT, bool W32>
 static int launch_nc(const NormCompressArgs& a, const XaArgs& xa, hipStream_t st) {
-    if ((g_slab_enabled || xa.nb > 0) && slab_shape(a.rows, a.N)) {
+    if ((g_slab_enabled.get() || xa.nb > 0) && slab_shape(a.rows, a.N)) {
         const int waves = a.N / (kWave * 8);
         // Strip height: all workgroups resident at once (16 waves per compute unit), each walking as
         // long a strip as that allows - the per-column constants are set up once per strip.
-        int rows_per_group = g_slab_rows_per_group;
+        int rows_per_group = g_slab_rows_per_group.get();
         if (rows_per_group == 0) {
             const int64_t resident = (int64_t)compute_units() * (16 / (waves <= 8 ? waves : 16));
             rows_per_group = (int)(cdiv(cdiv(a.rows, resident), (int64_t)kSlabRows) * kSlabRows);
@@ -669,12 +669,12 @@ static int launch_nc(const NormCompressArgs& a, const XaArgs& xa, hipStream_t st
 int tune_norm_compress(const char* key, int value) {
     if (strcmp(key, "norm_compress_slab") == 0) {
         if (value != 0 && value != 1) return HYC_ERR_ARG;
-        g_slab_enabled = value;
+        g_slab_enabled.set(value);
         return HYC_OK;
     }
     if (strcmp(key, "norm_compress_rows_per_group") == 0) {
         if (value < 0 || value > 65536 || value % kSlabRows != 0) return HYC_ERR_ARG;   // 0: choose from the row count
-        g_slab_rows_per_group = value;
+        g_slab_rows_per_group.set(value);
         return HYC_OK;
     }
     return 1;
@@ -766,7 +766,7 @@ extern "C" int hyc_rmsnorm_fwd_compress_lora(const void* x, const void* weight, 
 static int launch_bwd_slab(const NormBwdCodesArgs& a, int q_bit, int weight_is_fp32, hipStream_t st) {
     const int64_t rows = a.rows;
     const int waves = a.N / (kWave * 8);
-    int rows_per_group = g_slab_rows_per_group;
+    int rows_per_group = g_slab_rows_per_group.get();
     if (rows_per_group == 0) {
         const int64_t resident = (int64_t)compute_units() * (16 / (waves <= 8 ? waves : 16));
         rows_per_group = (int)(cdiv(cdiv(rows, resident), (int64_t)kSlabRows) * kSlabRows);
@@ -799,7 +799,7 @@ namespace hyc {
 // 4096 channels here.  Returns 1 when the shape does not fit the slabs (the caller keeps its own kernel).
 int rmsnorm_bwd_dense_slab(const void* dy, const void* x, const void* weight, int weight_is_fp32, const float* rstd,
                            const void* residual, void* dx, int64_t rows, int64_t N, void* stream) {
-    if (!g_slab_enabled || !slab_shape(rows, N)) return 1;       // "norm_compress_slab" 0: the row-per-wave kernel
+    if (!g_slab_enabled.get() || !slab_shape(rows, N)) return 1;       // "norm_compress_slab" 0: the row-per-wave kernel
     NormBwdCodesArgs a{};
     a.x = (const uint16_t*)x; a.dy = (const uint16_t*)dy; a.w = weight; a.rstd = rstd;
     a.res = (const uint16_t*)residual; a.dx = (uint16_t*)dx; a.rows = rows; a.N = (int)N; a.k = 0;

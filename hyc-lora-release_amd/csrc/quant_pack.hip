@@ -47,10 +47,10 @@ constexpr int kQuantThreads = kQuantWaves * kWave;
 constexpr int kRowUnroll = HYC_Q_UNROLL;       // quantiser: independent 128-bit loads in flight per lane
 constexpr int kDeqUnroll = HYC_D_UNROLL;       // dequantiser: rows per group
 
-static int g_quant_rows_per_wave = 8;     // strip heights; see hyc_set_tuning
-static int g_dequant_rows_per_wave = 2;
-static int g_quant_outlier_rows_per_wave = 8;     // the same two with an outlier list
-static int g_dequant_outlier_rows_per_wave = 8;
+static Knob g_quant_rows_per_wave{8};     // strip heights; see hyc_set_tuning
+static Knob g_dequant_rows_per_wave{2};
+static Knob g_quant_outlier_rows_per_wave{8};     // the same two with an outlier list
+static Knob g_dequant_outlier_rows_per_wave{8};
 
 struct QuantArgs {
     uint16_t* x;            // bf16 activations (input of quantise / output of dequantise)
@@ -529,7 +529,7 @@ extern "C" int hyc_quant_pack(const void* x, const void* scale, const void* zero
     if (zero_point && !aligned16(zero_point)) return HYC_ERR_ALIGN;
     const void* zp = zero_point;
     QuantArgs a = make_args(x, scale, zp, q, outlier_idx, k, x_outlier, zero_input, B, M, N, stride_b, stride_m,
-                            head_dim, stride_h, (outlier_idx && k) ? g_quant_outlier_rows_per_wave : g_quant_rows_per_wave);
+                            head_dim, stride_h, (outlier_idx && k) ? g_quant_outlier_rows_per_wave.get() : g_quant_rows_per_wave.get());
     const int64_t row_tiles = cdiv(a.T, (int64_t)kQuantWaves * a.rows_per_wave);
     if (row_tiles * a.col_tiles > INT32_MAX) return HYC_ERR_SHAPE;
     const dim3 grid((unsigned)(row_tiles * a.col_tiles)), block(kQuantThreads);
@@ -549,7 +549,7 @@ extern "C" int hyc_unpack_dequant(const void* q, const void* scale, const void* 
     if (!((reinterpret_cast<uintptr_t>(q) & 7u) == 0)) return HYC_ERR_ALIGN;
     const void* zp = zero_point;
     QuantArgs a = make_args(x, scale, zp, q, outlier_idx, k, x_outlier, 0, B, M, N, stride_b, stride_m, head_dim,
-                            stride_h, (outlier_idx && k) ? g_dequant_outlier_rows_per_wave : g_dequant_rows_per_wave);
+                            stride_h, (outlier_idx && k) ? g_dequant_outlier_rows_per_wave.get() : g_dequant_rows_per_wave.get());
     const int64_t row_tiles = cdiv(a.T, (int64_t)kQuantWaves * a.rows_per_wave);
     if (row_tiles * a.col_tiles > INT32_MAX) return HYC_ERR_SHAPE;
     const dim3 grid((unsigned)(row_tiles * a.col_tiles)), block(kQuantThreads);
@@ -559,14 +559,14 @@ extern "C" int hyc_unpack_dequant(const void* q, const void* scale, const void* 
 }
 
 int hyc::tune_quant(const char* key, int value) {
-    int* const knobs[4] = {&g_quant_rows_per_wave, &g_dequant_rows_per_wave, &g_quant_outlier_rows_per_wave,
+    Knob* const knobs[4] = {&g_quant_rows_per_wave, &g_dequant_rows_per_wave, &g_quant_outlier_rows_per_wave,
                            &g_dequant_outlier_rows_per_wave};
     const char* const names[4] = {"quant_rows_per_wave", "dequant_rows_per_wave", "quant_outlier_rows_per_wave",
                                   "dequant_outlier_rows_per_wave"};
     for (int i = 0; i < 4; ++i) {
         if (strcmp(key, names[i]) != 0) continue;
         if (value < 1 || value > 4096) return HYC_ERR_ARG;
-        *knobs[i] = value;
+        knobs[i]->set(value);
         return HYC_OK;
     }
     return 1;  // not one of this file's keys

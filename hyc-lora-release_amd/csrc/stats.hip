@@ -29,11 +29,11 @@ constexpr int kSelReplicas = 32;            // copies of each histogram bin, one
 
 // Waves the statistics launch aims for (hyc_set_tuning "stats_waves"): enough to keep every CU's memory
 // pipeline full, few enough that the per-strip partial rows stay a small fraction of the input.
-static int g_stat_waves = 4096;
+static Knob g_stat_waves{4096};
 
 static int stat_strips(int64_t M, int64_t N) {
     const int64_t col_tiles = cdiv(N, kStatTileCols);
-    int64_t strips = g_stat_waves / (kStatWaves * col_tiles);
+    int64_t strips = g_stat_waves.get() / (kStatWaves * col_tiles);
     const int64_t most = cdiv(M, (int64_t)kStatWaves * 4);          // at least four rows per wave
     if (strips > most) strips = most;
     if (strips > kStatMaxStrips) strips = kStatMaxStrips;
@@ -327,7 +327,7 @@ __global__ __launch_bounds__(kSelThreads) void channel_pick_rounds_kernel(const 
 int tune_stats(const char* key, int value) {
     if (strcmp(key, "stats_waves") != 0) return 1;
     if (value < 4 || value > (1 << 20)) return HYC_ERR_ARG;
-    g_stat_waves = value;
+    g_stat_waves.set(value);
     return HYC_OK;
 }
 

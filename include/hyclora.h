@@ -41,8 +41,11 @@ const char *hyc_error_string(int code);
 /* ABI revision; bumped when a signature changes or an entry point is added. */
 int hyc_abi_version(void);
 
-/* Launch-shape knobs for benchmarking (process-wide, not thread-safe against concurrent
- * launches).  Keys: "quant_rows_per_wave" (rows each wave walks in hyc_quant_pack,
+/* Launch-shape knobs, FOR BENCHMARKING ONLY: process-wide state in a library whose entry points are otherwise
+ * stateless.  Results never depend on them except where said ("stats_waves": the last bits of the sums of
+ * squares).  Each knob is an atomic integer that an entry point reads once per launch, so a launch on another
+ * thread runs with the old or the new value of each knob, never a torn one; a pair of calls that must agree
+ * (hyc_channel_stats_strips, then hyc_channel_stats) must not straddle a change.  Keys: "quant_rows_per_wave" (rows each wave walks in hyc_quant_pack,
  * default 8), "dequant_rows_per_wave" (same for hyc_unpack_dequant, default 2),
  * "quant_outlier_rows_per_wave" / "dequant_outlier_rows_per_wave" (the same two when called with
  * an outlier list; default 8 each: a wave first has to find its outlier columns in the list),
