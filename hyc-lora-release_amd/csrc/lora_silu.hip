@@ -41,6 +41,13 @@ constexpr int kFuseWaves = kFuseThreads / kWave;
 // meet in L2.  At 8 bits a wave writes and reads whole lines that nobody else touches: streaming accesses
 // (forward 95.0 -> 91.2 us, backward 117.7 -> 116.4 us on [4096, 14336]).
 template <int QBIT> constexpr bool kStreamCodes = QBIT == 8;
+// At 2 bits a tile's codes are 32 bytes a row, a quarter of a line, and the four pieces of a line come from the
+// four waves of a workgroup at four moments: 29 MB of 2-bit codes cost the forward kernel more time than 59 MB
+// of 4-bit codes.  There the waves hand their pieces over through LDS and each line goes to memory whole, from
+// one wave (forward 75.9 -> 71.9 us on [4096, 14336]).  At 4 bits (half lines) the same exchange gains 2 us on
+// [4096, 14336] and loses 1.4 us on [4096, 11008] - a barrier per tile couples waves that otherwise run
+// independently - and is left out.
+template <int QBIT> constexpr bool kMergeCodeLines = QBIT == 2;
 
 // Strip heights (backward, forward; see hyc_set_tuning).  0 = by code width and size: a wave sets up its
 // LoRA-B operands and per-column constants once per strip, which in the [N, R] layout of LoRA-B is 16
@@ -135,12 +142,24 @@ __device__ __forceinline__ void fuse_fwd_rows(const FuseArgs& a, int64_t row_beg
 // then for data requested a whole tile earlier, and the stores of the rows in between stay in
 // flight (loads and stores retire through one in-order counter).  The first tile is peeled so
 // that the loop is entered in the state its back edge carries; the last one requests nothing.
-template <int QBIT, int KSTEPS>
+template <int QBIT, int KSTEPS, bool MERGE = false>
 __device__ __forceinline__ void fuse_fwd_rows_full(const FuseArgs& a, int64_t row_begin, int64_t row_end, int lane,
                                                    int chunk, const QuantCols<QBIT>& c1, const QuantCols<QBIT>& c2,
-                                                   const BOperand<KSTEPS>& B1, const BOperand<KSTEPS>& B2) {
+                                                   const BOperand<KSTEPS>& B1, const BOperand<KSTEPS>& B2,
+                                                   int wave = 0, uint8_t* stage = nullptr) {
     const int g = lane >> 4, i = lane & 15;
     const int row_bytes = a.N * QBIT / 8;
+    // MERGE: the waves of a workgroup that share the 128-byte lines of a row's codes (CT neighbouring column
+    // tiles) hand their pieces over through LDS, and every line is written to memory whole, by one wave
+    constexpr int CT = kColTilesPerGroup<QBIT>, RS = kFuseWaves / CT;
+    constexpr int kUnit = kTileRows * 128;                    // a unit's 16 rows x one line, per tensor
+    constexpr int kBuf = 2 * RS * kUnit;                      // both tensors of all units
+    constexpr int BPL = 32 / CT;                              // bytes a lane writes out: 16 rows x 128 B over CT waves
+    const int unit = wave / CT, wiu = wave % CT;
+    const int loc = packed_store_offset<QBIT>(chunk) & 127;
+    const int out_row = (kTileRows / CT) * wiu + (lane * BPL) / 128, out_col = (lane * BPL) % 128;
+    const int64_t line0 = (int64_t)((chunk >> 4) / CT) * 128;  // the unit's line inside a packed row
+    int buf = 0;
     const float zero8[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     u32x4 xv1[4], xv2[4];
     u32x2 A1[KSTEPS], A2[KSTEPS];
@@ -171,10 +190,20 @@ __device__ __forceinline__ void fuse_fwd_rows_full(const FuseArgs& a, int64_t ro
             unpack8(xv2[v], f2);
             if constexpr (AHEAD) request_row(row0 + kTileRows, v);
             uint32_t lo, hi;
-            codes_to_words<QBIT, false, true>(f1, c1, zero8, lo, hi);
-            store_packed<QBIT, kStreamCodes<QBIT>>(a.q1 + r * row_bytes, chunk, true, lo, hi);
-            codes_to_words<QBIT, false, true>(f2, c2, zero8, lo, hi);
-            store_packed<QBIT, kStreamCodes<QBIT>>(a.q2 + r * row_bytes, chunk, true, lo, hi);
+            if constexpr (MERGE) {
+                uint8_t* s1 = stage + buf * kBuf + unit * kUnit + (4 * g + v) * 128 + loc;
+                codes_to_words<QBIT, false, true>(f1, c1, zero8, lo, hi);
+                merge_packed<QBIT>(chunk, lo, hi);
+                if (packed_store_lane<QBIT>(chunk)) *reinterpret_cast<uint32_t*>(s1) = lo;
+                codes_to_words<QBIT, false, true>(f2, c2, zero8, lo, hi);
+                merge_packed<QBIT>(chunk, lo, hi);
+                if (packed_store_lane<QBIT>(chunk)) *reinterpret_cast<uint32_t*>(s1 + RS * kUnit) = lo;
+            } else {
+                codes_to_words<QBIT, false, true>(f1, c1, zero8, lo, hi);
+                store_packed<QBIT, kStreamCodes<QBIT>>(a.q1 + r * row_bytes, chunk, true, lo, hi);
+                codes_to_words<QBIT, false, true>(f2, c2, zero8, lo, hi);
+                store_packed<QBIT, kStreamCodes<QBIT>>(a.q2 + r * row_bytes, chunk, true, lo, hi);
+            }
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
                 float y1 = rbf(f1[j] + lora_elem(L1[v], j));
@@ -184,6 +213,24 @@ __device__ __forceinline__ void fuse_fwd_rows_full(const FuseArgs& a, int64_t ro
             }
             st16_nt(a.o + r * a.N + chunk * 8, pack8(of));
             __builtin_amdgcn_sched_barrier(0);
+        }
+        if constexpr (MERGE) {
+            // LDS-only barrier: the rows just requested and the stores above stay in flight
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+            __builtin_amdgcn_s_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+            const uint8_t* s1 = stage + buf * kBuf + unit * kUnit + out_row * 128 + out_col;
+            const int64_t at = (row0 + out_row) * row_bytes + line0 + out_col;
+            if constexpr (BPL == 8) {
+                const u32x2 w1 = *reinterpret_cast<const u32x2*>(s1), w2 = *reinterpret_cast<const u32x2*>(s1 + RS * kUnit);
+                st8(a.q1 + at, w1);
+                st8(a.q2 + at, w2);
+            } else {
+                const u32x4 w1 = *reinterpret_cast<const u32x4*>(s1), w2 = *reinterpret_cast<const u32x4*>(s1 + RS * kUnit);
+                st16(a.q1 + at, w1);
+                st16(a.q2 + at, w2);
+            }
+            buf ^= 1;
         }
     };
     request_a(row_begin);
@@ -223,9 +270,27 @@ HYC_FUSE_KERNEL(HYC_FWD_DEEP) void lora_silu_fwd_kernel(const FuseArgs a) {
     const int64_t row_begin = (row_tile * RS + wave / CT) * (int64_t)a.rows_per_wave;
     int64_t row_end = row_begin + a.rows_per_wave;
     if (row_end > a.T) row_end = a.T;
+    constexpr bool kRoll = KSTEPS == 1 || (HYC_ROLL_DEEP && KSTEPS >= HYC_FWD_DEEP);
+    constexpr bool kCanMerge = kRoll && kMergeCodeLines<QBIT>;
+    __shared__ __align__(16) uint8_t stage[kCanMerge ? 2 * 2 * RS * kTileRows * 128 : 16];
+    const bool slow = __ballot(!(c1.fast && c2.fast)) != 0ull;
+    bool merged = false;
+    if constexpr (kCanMerge) {
+        // every wave of the workgroup votes before any of them leaves: the merged walk has a barrier per tile,
+        // so all of them must take it, with strips of the same whole number of tiles
+        const bool mine = !slow && (col_tile + 1) * (kTileCols / 8) <= a.C && row_end - row_begin == a.rows_per_wave &&
+                          a.rows_per_wave % kTileRows == 0;
+        merged = __syncthreads_and(mine) != 0;
+    }
     if (row_begin >= row_end) return;
     const bool full = (col_tile + 1) * (kTileCols / 8) <= a.C && (row_end - row_begin) % kTileRows == 0;   // uniform
-    if (__ballot(!(c1.fast && c2.fast)) != 0ull)
+    if constexpr (kCanMerge) {
+        if (merged) {
+            fuse_fwd_rows_full<QBIT, KSTEPS, true>(a, row_begin, row_end, lane, chunk, c1, c2, B1, B2, wave, stage);
+            return;
+        }
+    }
+    if (slow)
         fuse_fwd_rows<QBIT, KSTEPS, false>(a, row_begin, row_end, lane, chunk, active, c1, c2, B1, B2);
     else if ((KSTEPS == 1 || (HYC_ROLL_DEEP && KSTEPS >= HYC_FWD_DEEP)) && full)                  // deeper ranks have no registers to spare for it
         fuse_fwd_rows_full<QBIT, KSTEPS>(a, row_begin, row_end, lane, chunk, c1, c2, B1, B2);

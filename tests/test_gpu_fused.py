@@ -119,6 +119,34 @@ def test_fused_results_do_not_depend_on_the_strip_height(fz, dev, q_bit, R):
     assert_close_bf16(outs[0][5], gu_ref, what="grad_up vs oracle")
 
 
+@pytest.mark.parametrize("R", [16, 32])
+def test_two_bit_code_lines_written_whole(fz, dev, R):
+    """At 2 bits the four waves of a workgroup hand the 32-byte pieces of a row's code line over through LDS
+    and one wave writes the line, wherever the whole workgroup is on interior strips; workgroups at the
+    ragged edges (a last group of column tiles that is not complete, a last strip that is cut off, a column
+    whose step needs the division branch) store their pieces directly.  One launch with all of these side by
+    side must give the oracle's codes, at every strip height."""
+    from hyclora_amd import _lib
+    B, M, H, I = 1, 272, 64, 1536 + 128              # three whole groups of 512 columns and a quarter of one
+    t = mlp_inputs(11 + R, B, M, H, I, R)
+    xa1, b1, x1 = t["gate"]
+    xa2, b2, x2 = t["up"]
+    x1[:, :, 700] = 0                                # a constant column: step 0, the division branch, in group 1
+    s1 = O.scale_only_quant(x1, 2)
+    s2 = O.scale_only_quant(x2, 2)
+    assert s1.reshape(-1)[700].item() == 0
+    d = lambda *ts: [v.to(dev) for v in ts]
+    q1_ref, q2_ref, o_ref = O.fused_fwd(xa1, b1, x1, s1, xa2, b2, x2, s2, 2)
+    try:
+        for rows in (0, 16, 32, 96, 272 - 16):
+            _lib.set_tuning("fuse_rows_per_wave", rows)
+            q1, q2, o = fz.fwd(*d(xa1, b1, x1, s1, xa2, b2, x2, s2), 2)
+            assert torch.equal(q1.cpu(), q1_ref) and torch.equal(q2.cpu(), q2_ref), f"codes at strip height {rows}"
+            assert_close_bf16(o, o_ref, what=f"fused forward o vs oracle at strip height {rows}")
+    finally:
+        _lib.set_tuning("fuse_rows_per_wave", 0)
+
+
 def test_fused_lora_term_is_applied_per_row_and_column(fz, dev):
     # x1 = x2 = 0 and a one-hot xa isolates the MFMA operand mapping: y = b[r, :] for row r
     R, N, M = 16, 256, 32
