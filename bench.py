@@ -647,6 +647,27 @@ def main():
                "fwd_GBps": bytes_ff / ms_ff / 1e6, "bwd_GBps": bytes_fb / ms_fb / 1e6,
                "fwd_frac_of_hbm_peak": bytes_ff / ms_ff / 1e6 / HBM_PEAK_GBS,
                "bwd_frac_of_hbm_peak": bytes_fb / ms_fb / 1e6 / HBM_PEAK_GBS}
+        # what the memory system gives a kernel that only loads and stores the same bf16 tensors with the same
+        # access shape (a wave = 128 columns x 4 rows per instruction, 16-row tiles) and no arithmetic: forward-like
+        # = read two tensors, write one (the codes, q/8 bytes an element each, are on top of that in the real
+        # kernel); backward-like = read one, write three
+        import ctypes
+        ptrs = lambda ts: (ctypes.c_void_p * len(ts))(*[t.data_ptr() for t in ts])
+
+        def probe(n_reads, n_writes, rows):
+            def f(i, st=None):
+                d = sets[i % NF]
+                rd = ptrs([d["x1"], d["x2"]][:n_reads]) if n_reads == 2 else ptrs([d["g"]])
+                wr = ptrs([d["ob"], d["gg"], d["gu"]][:n_writes])
+                rc = L.hyc_stream_probe(rd, n_reads, wr, n_writes, Tf, Nf, 0, rows, st or stream)
+                assert rc == 0, _lib.error_string(rc)
+            f(0)
+            ms = timed_graph(f, Kf, Wf)[0]
+            nb = (n_reads + n_writes) * Ef * 2
+            return {"ms": ms, "GBps": nb / ms / 1e6, "frac_of_hbm_peak": nb / ms / 1e6 / HBM_PEAK_GBS, "rows_per_wave": rows}
+        res["memory_only_probe"] = {"read2_write1": probe(2, 1, 32), "read1_write3": probe(1, 3, 16),
+                                    "note": "hyc_stream_probe: loads and stores only, the fused kernels' access shape"}
+        # the probe overwrote the backward's outputs of set 0..2; nothing reads them afterwards
         if not with_torch:
             return res
         res["eager_fwd_ms"], _ = timed(f_fwd, Kf, Wf)

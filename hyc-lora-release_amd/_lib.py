@@ -26,7 +26,7 @@ class HycError(RuntimeError):
 
 
 # name -> (restype, argtypes)
-ABI_VERSION = 8          # hyc_abi_version() of the library these signatures describe
+ABI_VERSION = 9          # hyc_abi_version() of the library these signatures describe
 _P, _I, _L = c_void_p, c_int, c_int64
 
 
@@ -46,6 +46,7 @@ _SIGNATURES = {
     "hyc_channel_stats_strips": (_L, [_L, _L]),
     "hyc_channel_stats": (_I, [_P, _L, _L, _L, _L, _L, _P, _L, _P]),
     "hyc_channel_select": (_I, [_P, _L, _L, _L, _I, _I, _P, _P, _P, _P]),
+    "hyc_stream_probe": (_I, [_P, _I, _P, _I, _L, _L, _I, _I, _P]),
     "hyc_hist16": (_I, [_P, _L, _P, _P]),
     "hyc_hist_select": (_I, [_P, _L, _P, _P]),
     "hyc_sparse_num_segments": (_L, [_L]),

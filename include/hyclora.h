@@ -603,6 +603,20 @@ int hyc_lora_contract(const void *x, const void *q, const void *scale, const voi
                       void *workspace, int64_t workspace_bytes, int64_t T, int64_t N, int64_t R,
                       void *stream);
 
+/* ---------------------------------------------------------------------------------------
+ * Memory-only probe, FOR BENCHMARKING: loads n_reads and stores n_writes bf16 [T, N] tensors (1..3 each,
+ * arrays of device pointers in host memory, 16-byte aligned, N % 8 == 0) with the access shape of the
+ * kernels of this library and no arithmetic of the path, so that the rate the memory system gives a
+ * read / write mix can be put beside the kernel that has that mix (bench.py does, for the fused LoRA-SiLU
+ * kernels).  What is stored is the xor of what was loaded.  No counterpart in the reference.
+ *   shape 0: a wave owns 128 columns and four rows per instruction and walks rows_per_wave rows (multiple
+ *            of 16) in 16-row tiles, as the fused LoRA-SiLU / LoRA-add kernels do;
+ *   shape 1: a wave owns 512 columns (1 KiB) of one row per instruction, rows_per_wave a multiple of 4,
+ *            as the quantiser does.
+ */
+int hyc_stream_probe(const void *const *reads, int n_reads, void *const *writes, int n_writes, int64_t T,
+                     int64_t N, int shape, int rows_per_wave, void *stream);
+
 #ifdef __cplusplus
 }
 #endif
