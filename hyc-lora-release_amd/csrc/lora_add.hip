@@ -25,6 +25,7 @@ namespace hyc {
 
 constexpr int kAddThreads = 256;
 constexpr int kAddWaves = kAddThreads / kWave;
+constexpr int kAddPlainColTiles = 4;        // column tiles side by side in a workgroup of the plain add
 static Knob g_add_rows_per_wave[3]{32, 48, 48};   // plain, quantise, restore; see hyc_set_tuning
 
 enum { kAddPlain = 0, kAddQuant = 1, kAddRestore = 2 };
@@ -154,7 +155,9 @@ __device__ __forceinline__ void lora_add_rows(const LoraAddArgs& a, int64_t row_
 
 template <int QBIT, int KSTEPS, int MODE, bool ZP>
 __device__ __forceinline__ void lora_add_block(const LoraAddArgs& a, int block) {
-    constexpr int CT = MODE == kAddPlain ? 1 : kColTilesPerGroup<QBIT>, RS = kAddWaves / CT;
+    // the plain form shares no code lines, but four column tiles side by side (a workgroup touches 1 KiB of a row at
+    // a time) are worth 4 % at N = 4096 and 10 % at N = 14336 (47.5 -> 42.8 us), nothing at N = 11008
+    constexpr int CT = MODE == kAddPlain ? kAddPlainColTiles : kColTilesPerGroup<QBIT>, RS = kAddWaves / CT;
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int col_tile = (block % a.col_tiles) * CT + wave % CT;     // a.col_tiles counts groups of CT tiles
@@ -288,7 +291,7 @@ static int add_prepare(LoraAddArgs& a, int64_t T, int64_t N, int64_t R, int q_bi
     a.C = (int)(N / 8);
     a.R = (int)R;
     a.rows_per_wave = g_add_rows_per_wave[MODE].get();
-    const int ct = MODE == kAddPlain ? 1 : 8 / q_bit;
+    const int ct = MODE == kAddPlain ? kAddPlainColTiles : 8 / q_bit;
     a.col_tiles = (int)cdiv(cdiv(N, kTileCols), ct);
     const int64_t row_tiles = cdiv(T, (int64_t)(kAddWaves / ct) * a.rows_per_wave);
     if (row_tiles * a.col_tiles > INT32_MAX) return HYC_ERR_SHAPE;

@@ -48,22 +48,31 @@ template <int QBIT> constexpr bool kStreamCodes = QBIT == 8;
 // [4096, 14336] and loses 1.4 us on [4096, 11008] - a barrier per tile couples waves that otherwise run
 // independently - and is left out.
 template <int QBIT> constexpr bool kMergeCodeLines = QBIT == 2;
+// Column tiles side by side in a workgroup (its four waves are CT tiles x 4/CT row strips).  The tiles that share
+// a line of codes must be together (kColTilesPerGroup: 4 / 2 / 1 at 2 / 4 / 8 bits).  At 8 bits four tiles side
+// by side - a workgroup then touches 1 KiB of a row at a time instead of four rows' 256 bytes - are worth
+// 8 us forward and 3.6 us backward on [4096, 14336] (91.1 -> 83.0, 110.5 -> 106.9 us) and 2 / 1 us on
+// [4096, 11008]; at 4 bits four instead of two change nothing forward and lose 1.8 us backward on [4096, 11008].
+template <int QBIT> constexpr int kFuseColTiles = QBIT == 4 ? 2 : 4;
+static_assert(kFuseColTiles<2> % kColTilesPerGroup<2> == 0 && kFuseColTiles<4> % kColTilesPerGroup<4> == 0 &&
+              kFuseColTiles<8> % kColTilesPerGroup<8> == 0, "tiles that share a code line stay in one workgroup");
 
 // Strip heights (backward, forward; see hyc_set_tuning).  0 = by code width and size: a wave sets up its
 // LoRA-B operands and per-column constants once per strip, which in the [N, R] layout of LoRA-B is 16
 // scattered 8-byte loads per lane; 96-row strips spread that over six tiles once the tensor is
-// large enough to fill the machine with such strips (forward 70 -> 66 us on [4096, 11008]).  At 8 bits a
-// workgroup is four strips of ONE column tile, and short strips do better: measured on [4096, 11008] and
-// [4096, 14336], forward 32 rows (69.9 / 64.4 % of peak against 70.7 / 60.0 % at 96), backward 16 rows
-// (65.1 / 67.0 % against 66.9 / 63.1 % at 32).
+// large enough to fill the machine with such strips (forward 70 -> 66 us on [4096, 11008]).  At 8 bits
+// short strips do better, 32 rows in both directions (forward 68.3 / 70.8 % of the peak on [4096, 11008] /
+// [4096, 14336] against 66.6 / 66.9 % at 96 rows, backward 67.1 / 68.7 % against 66.1 / 68.3 % at 16 and 64.0 /
+// 64.8 % at 96), and 16 rows on tensors too small to fill the machine ([512, 4096]: 5.7 against 7.3 us).
 static Knob g_fuse_rows_per_wave[2]{0, 0};
 
 static int fuse_rows_per_wave(bool fwd, int q_bit, int64_t T, int64_t N) {
     const int set = g_fuse_rows_per_wave[fwd ? 1 : 0].get();
     if (set) return set;
-    if (!fwd) return q_bit == 8 ? 16 : 32;
-    if (q_bit == 8) return 32;
-    return T * N >= ((int64_t)1 << 24) ? 96 : 32;
+    const bool large = T * N >= ((int64_t)1 << 24);
+    if (q_bit == 8) return large ? 32 : 16;
+    if (!fwd) return 32;
+    return large ? 96 : 32;
 }
 
 struct FuseArgs {
@@ -151,7 +160,7 @@ __device__ __forceinline__ void fuse_fwd_rows_full(const FuseArgs& a, int64_t ro
     const int row_bytes = a.N * QBIT / 8;
     // MERGE: the waves of a workgroup that share the 128-byte lines of a row's codes (CT neighbouring column
     // tiles) hand their pieces over through LDS, and every line is written to memory whole, by one wave
-    constexpr int CT = kColTilesPerGroup<QBIT>, RS = kFuseWaves / CT;
+    constexpr int CT = kFuseColTiles<QBIT>, RS = kFuseWaves / CT;
     constexpr int kUnit = kTileRows * 128;                    // a unit's 16 rows x one line, per tensor
     constexpr int kBuf = 2 * RS * kUnit;                      // both tensors of all units
     constexpr int BPL = 32 / CT;                              // bytes a lane writes out: 16 rows x 128 B over CT waves
@@ -246,7 +255,7 @@ __device__ __forceinline__ void fuse_fwd_rows_full(const FuseArgs& a, int64_t ro
 
 template <int QBIT, int KSTEPS>
 HYC_FUSE_KERNEL(HYC_FWD_DEEP) void lora_silu_fwd_kernel(const FuseArgs a) {
-    constexpr int CT = kColTilesPerGroup<QBIT>, RS = kFuseWaves / CT;
+    constexpr int CT = kFuseColTiles<QBIT>, RS = kFuseWaves / CT;
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int col_tile = (blockIdx.x % a.col_tiles) * CT + wave % CT;     // a.col_tiles counts groups of CT tiles
@@ -301,7 +310,7 @@ HYC_FUSE_KERNEL(HYC_FWD_DEEP) void lora_silu_fwd_kernel(const FuseArgs a) {
 // ------------------------------------------------------------------------------------
 template <int QBIT, int KSTEPS>
 HYC_FUSE_KERNEL(HYC_BWD_DEEP) void lora_silu_bwd_kernel(const FuseArgs a) {
-    constexpr int CT = kColTilesPerGroup<QBIT>, RS = kFuseWaves / CT;
+    constexpr int CT = kFuseColTiles<QBIT>, RS = kFuseWaves / CT;
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int col_tile = (blockIdx.x % a.col_tiles) * CT + wave % CT;
@@ -500,7 +509,7 @@ static int fuse_launch(FuseArgs& a, int64_t T, int64_t N, int64_t R, int q_bit, 
     a.C = (int)(N / 8);
     a.R = (int)R;
     a.rows_per_wave = fuse_rows_per_wave(fwd, q_bit, T, N);
-    const int ct = 8 / q_bit;                                  // kColTilesPerGroup
+    const int ct = q_bit == 4 ? kFuseColTiles<4> : kFuseColTiles<8>;      // = kFuseColTiles<2>
     a.col_tiles = (int)cdiv(cdiv(N, kTileCols), ct);           // workgroups along the columns
     const int64_t row_tiles = cdiv(T, (int64_t)(kFuseWaves / ct) * a.rows_per_wave);
     if (row_tiles * a.col_tiles > INT32_MAX) return HYC_ERR_SHAPE;

@@ -54,8 +54,8 @@ int hyc_abi_version(void);
  * and "norm_compress_rows_per_group" (rows a workgroup of that kernel walks, even; 0 = chosen from the
  * row count, the default),
  * "fuse_rows_per_wave" (same for both fused LoRA-SiLU kernels, multiple of 16; default 0 = by code width
- * and size: backward 32, 16 at 8 bits; forward 96 for tensors of 2^24 elements and more, else 32, and 32
- * at 8 bits; "fuse_fwd_rows_per_wave" / "fuse_bwd_rows_per_wave" set one of them),
+ * and size: backward 32; forward 96 for tensors of 2^24 elements and more, else 32; at 8 bits 32 in both
+ * directions for tensors of 2^24 elements and more, else 16; "fuse_fwd_rows_per_wave" / "fuse_bwd_rows_per_wave" set one of them),
  * "contract_max_groups" (column groups hyc_lora_contract cuts a row strip into, default 32; changes the
  * workspace hyc_lora_contract_workspace asks for), "stats_waves" (waves hyc_channel_stats aims to launch,
  * default 4096; sets the number of row strips hyc_channel_stats_strips returns and so the order in which the
