@@ -47,7 +47,7 @@ def oracle_backward_from_saved_state(t, out, layer_type, q_bit, attention, exact
 TALLY = {"compared": 0, "direct": 0, "by the exact evaluation": 0}
 
 
-def compare(grads, expect, what, exact=None, rel_tol=1e-2, cos_tol=0.9999, library_noise=()):
+def compare(grads, expect, what, exact=None, rel_tol=1e-2, cos_tol=0.9999, library_noise=(), names=None):
     """Every gradient against the oracle's backward from the same saved state (`expect`, bf16 arithmetic as the
     reference's) at the operator tolerance: max rel err <= 1e-2, cosine >= 0.9999.
 
@@ -63,7 +63,7 @@ def compare(grads, expect, what, exact=None, rel_tol=1e-2, cos_tol=0.9999, libra
     this repository's (torch's flash-attention backward, which rounds its probabilities to bf16 where the
     restatement keeps fp32 matrices); at a few hundred rows those may be 2e-2 from the exact evaluation."""
     report, bad, noise = [], [], []
-    for i, (name, got, want) in enumerate(zip(NAMES, grads, expect)):
+    for i, (name, got, want) in enumerate(zip(names or NAMES, grads, expect)):
         if got is None:
             assert name.startswith("norm_w"), name
             continue

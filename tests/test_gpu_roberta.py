@@ -101,7 +101,9 @@ def test_roberta_layer_matches_oracle_layer(dev, layer_type, q_bit, padding):
     names = ["x"] + [f"{n}.lora_{ab}" for n in NAMES for ab in "AB"]
     for name, got, want in zip(names, grads, expect):
         rel, cos = rel_err_and_cos(got, want)
-        rel_tol = 0.2 if q_bit == 2 else 2e-2            # one flipped 2-bit code is a quarter of the range
+        # end-to-end sanity bound (forward redone by the oracle: a code may flip, a quarter of the range at 2 bits);
+        # the parity bar, 1e-2 / 0.9999 at every width from identical saved state, is tests/test_gpu_roberta_saved_state.py
+        rel_tol = 0.2 if q_bit == 2 else 2e-2
         assert rel <= rel_tol and cos >= 0.999, f"{layer_type} q{q_bit} grad {name}: rel {rel:.2e} cos {cos:.5f}"
 
 
