@@ -344,3 +344,50 @@ def test_saved_set_is_the_references_save_list(mode, attention, q_bit):
         idx, val = saved["a_o_indices"], saved["a_o_values"]
         assert idx.dtype == torch.int64 and val.dtype == BF16 and idx.shape == val.shape and idx.dim() == 1
         assert bool((idx[1:] > idx[:-1]).all()) and idx.numel() <= int(B * heads * S * S * 0.05) + 1
+
+
+@pytest.mark.parametrize("mode", ["intra", "intra_inter"])
+@pytest.mark.parametrize("q_bit", [4, 2, 8])
+def test_encoder_saved_set_is_the_references_save_list(mode, q_bit):
+    """The activation entries of the encoder layers' ctx.save_for_backward, read off
+    models/roberta/fused_roberta_layer_intra_inter.py:203-225 and fused_roberta_layer_intra.py:215-238 (a_o there is
+    the sparse COO tensor: its indices and values here), plus what backward reads from ctx attributes: the two
+    channel lists (:277-278) and the map's shape (:145).  mean / rstd are the fp32 [B*S] rows layernorm_forward
+    returns (operators/layernorm_kernels.py:131-132)."""
+    B, S, H, I, R, heads = 2, 24, 64, 128, 4, 4
+    gen = torch.Generator().manual_seed(5)
+    rn = lambda *s, sc=1.0: (torch.randn(*s, generator=gen) * sc).to(BF16)
+    dims = dict(q=(H, H), k=(H, H), v=(H, H), o=(H, H), up=(I, H), down=(H, I))
+    weights = {n: (rn(o, i, sc=1 / math.sqrt(i)), rn(o, sc=0.1), rn(R, i, sc=1 / math.sqrt(i)), rn(o, R, sc=0.3)) for n, (o, i) in dims.items()}
+    ln = [((1 + 0.1 * torch.randn(H, generator=gen)).to(BF16), (0.1 * torch.randn(H, generator=gen)).to(BF16)) for _ in range(2)]
+    _, saved = LO.roberta_layer_forward(rn(B, S, H), weights, ln[0], ln[1], None, heads, mode=mode, q_bit=q_bit,
+                                        softmax_ratio=0.05, layernorm_ratio=0.05)
+    u8, f32, i64 = torch.uint8, torch.float32, torch.int64
+    epp, k_out = 8 // q_bit, int(H * 0.05)
+    codes = lambda n: ((B, S, n // epp), u8)
+    step = lambda n: ((1, n), BF16)
+    xa = ((B, S, R), BF16)
+    want = {"x_q": codes(H), "x_scale": step(H), "q_lora_a": xa, "k_lora_a": xa, "v_lora_a": xa,
+            "a_o_indices": None, "a_o_values": None, "a_threshold": ((), f32), "a_shape": (B, heads, S, S),
+            "o_q": codes(H), "o_scale": step(H), "o_final_lora_a": xa,
+            "o_final_o": ((B, S, k_out), BF16), "o_final_q": codes(H), "o_final_scale": step(H), "o_final_channel_idx": ((k_out,), i64),
+            "mean_1": ((B * S,), f32), "rstd_1": ((B * S,), f32),
+            "x_medium_q": codes(H), "x_medium_scale": step(H), "up_lora_a": xa, "down_lora_a": xa,
+            "down_o": ((B, S, k_out), BF16), "down_q": codes(H), "down_scale": step(H), "down_channel_idx": ((k_out,), i64),
+            "mean_2": ((B * S,), f32), "rstd_2": ((B * S,), f32)}
+    if mode == "intra":
+        for n in ("q", "k", "v"):
+            want.update({n + "_q": codes(H), n + "_scale": step(H)})
+        want.update({"up_q": codes(I), "up_scale": step(I), "fn_q": codes(I), "fn_scale": step(I)})
+    else:
+        for n in ("q_main", "k_main", "v_main"):
+            want.update({n + "_q": codes(H), n + "_scale": step(H)})
+        want.update({"up_main_q": codes(I), "up_main_scale": step(I)})
+    assert set(saved) == set(want), f"only in the oracle: {sorted(set(saved) - set(want))}; only in the reference: {sorted(set(want) - set(saved))}"
+    for name, spec in want.items():
+        got = saved[name]
+        if name == "a_shape":
+            assert tuple(got) == spec
+        elif spec is not None:
+            shape, dtype = spec
+            assert tuple(got.shape) == shape and got.dtype == dtype, f"{name}: {tuple(got.shape)} {got.dtype}, reference {shape} {dtype}"
