@@ -1033,6 +1033,10 @@ def main():
         ms, _ = timed(lambda i: cf.compress_attention_map(a, thr), 5, 2)
         kernels["softmax_compress"] = {"ms": ms, "GBps": (2 * Ea + 10 * nnz) / ms / 1e6, "nnz": nnz,
                                        "note": "includes the host read-back of nnz"}
+        cap_a = nnz + nnz // 16 + 64
+        ms, _ = timed(lambda i: cf.compress_attention_map(a, thr, seg_a, capacity=cap_a), 10, 2)
+        kernels["sparse_write"] = {"ms": ms, "GBps": (2 * Ea + 10 * nnz) / ms / 1e6, "nnz": nnz,
+                                   "note": "the write pass alone: segment offsets given, lists sized from a capacity, no read-back"}
         ms, _ = timed(lambda i: cf.restore_attention_map(idx_a, val_a, seg_a, a.shape), 10, 2)
         kernels["softmax_restore"] = {"ms": ms, "GBps": (2 * Ea + 10 * nnz) / ms / 1e6}
         ms, _ = timed(lambda i: softmax_kernels.softmax_backward(a, g_a), 10, 2)
