@@ -847,6 +847,24 @@ def main():
                 assert L.hyc_lora_contract(None, q_l[j].data_ptr(), s_l.data_ptr(), None, QB, xa.data_ptr(), None, 0,
                                            p1s[i % 2].data_ptr(), None, wss[i % 2].data_ptr(), ws_bytes, T, Nw, R, st) == 0
 
+            # the input gradients of projections that share their input, added up: three LoRA adds chained through
+            # a running sum against the one-pass sum of the same three terms
+            xa3 = [randn(B, M, R) for _ in range(3)]
+            wb3 = [randn(Nw, R, scale=0.05) for _ in range(3)]
+
+            def c_sum_chain(i, st):
+                j = i % NBl
+                assert L.hyc_lora_add(xa3[0].data_ptr(), wb3[0].data_ptr(), 1, x_l[j].data_ptr(), None, y_l[j].data_ptr(), T, Nw, R, st) == 0
+                for c in (1, 2):
+                    assert L.hyc_lora_add(xa3[c].data_ptr(), wb3[c].data_ptr(), 1, x_l[(j + c) % NBl].data_ptr(), y_l[j].data_ptr(),
+                                          y_l[j].data_ptr(), T, Nw, R, st) == 0
+
+            def c_sum(i, st):
+                j = i % NBl
+                arr = (_lib.LoraSumMember * 3)(*[_lib.LoraSumMember(xa3[c].data_ptr(), wb3[c].data_ptr(), 1, x_l[(j + c) % NBl].data_ptr())
+                                                 for c in range(3)])
+                assert L.hyc_lora_add_sum(arr, 3, y_l[j].data_ptr(), T, Nw, R, st) == 0
+
             def on(st, fn):
                 with torch.cuda.stream(torch.cuda.ExternalStream(st)):
                     fn()
@@ -883,6 +901,12 @@ def main():
                 fn(0, stream)
                 torch.cuda.synchronize()
                 e[key] = {"ms": timed_graph(fn, Kl, 200)[0]}
+            c_sum_chain(0, stream)
+            want3 = y_l[0].clone()
+            c_sum(0, stream)
+            assert torch.equal(y_l[0], want3), "one-pass sum of three LoRA adds differs from the chain"
+            ms_c, ms_1 = timed_graph(c_sum_chain, Kl, 200)[0], timed_graph(c_sum, Kl, 200)[0]
+            e["sum_of_three_lora_adds"] = {"ms": ms_1, "GBps": 8 * El / ms_1 / 1e6, "chain_of_three_calls_ms": ms_c}
             lora[wname] = e
             del x_l, y_l, q_l, wss
 

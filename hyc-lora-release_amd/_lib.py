@@ -26,7 +26,7 @@ class HycError(RuntimeError):
 
 
 # name -> (restype, argtypes)
-ABI_VERSION = 9          # hyc_abi_version() of the library these signatures describe
+ABI_VERSION = 10          # hyc_abi_version() of the library these signatures describe
 _P, _I, _L = c_void_p, c_int, c_int64
 
 
@@ -35,6 +35,11 @@ class LoraAddMember(ctypes.Structure):
     _fields_ = [("xa", _P), ("b", _P), ("x", _P), ("scale", _P), ("zero_point", _P), ("q", _P), ("y", _P),
                 ("cos_t", _P), ("sin_t", _P), ("seq_len", _L), ("stride_cos", _L), ("stride_sin", _L), ("N", _L),
                 ("b_transposed", _I), ("table_is_fp32", _I)]
+
+
+class LoraSumMember(ctypes.Structure):
+    """hyc_lora_sum_member of include/hyclora.h: one term of hyc_lora_add_sum."""
+    _fields_ = [("xa", _P), ("b", _P), ("b_transposed", _I), ("x", _P)]
 
 
 _SIGNATURES = {
@@ -87,6 +92,7 @@ _SIGNATURES = {
     "hyc_lora_add_restore": (_I, [_P, _P, _I] + [_P] * 4 + [_L, _L, _L, _I, _P]),
     "hyc_lora_add_quant_rope": (_I, [_P, _P, _I] + [_P] * 7 + [_I, _L, _L, _L, _L, _L, _L, _I, _P]),
     "hyc_lora_add_restore_rope": (_I, [_P, _P, _I] + [_P] * 6 + [_I, _L, _L, _L, _L, _L, _L, _I, _P]),
+    "hyc_lora_add_sum": (_I, [_P, _I, _P, _L, _L, _L, _P]),
     "hyc_lora_add_quant_group": (_I, [_P, _I, _L, _L, _I, _P]),
     "hyc_lora_add_restore_group": (_I, [_P, _I, _L, _L, _I, _P]),
 }

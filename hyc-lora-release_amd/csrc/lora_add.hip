@@ -365,6 +365,77 @@ static int add_group_launch(const hyc_lora_add_member* members, int count, int64
     return check_launch();
 }
 
+// ------------------------------------------------------------------------------------
+// Sum of two or three LoRA adds in one pass: y = t_0 (+) t_1 (+) t_2 with t_i = bf16(x_i + bf16(xa_i . b_i)) and
+// every (+) a bf16 addition - the bits of the chain hyc_lora_add(x_0), hyc_lora_add(x_1, residual = y),
+// hyc_lora_add(x_2, residual = y), which is how the input gradients of projections that share an input (q, k, v;
+// gate, up) are accumulated (`grad_x += grad_x_temp`), without writing and re-reading the running sum.  Rank <= 16.
+constexpr int kAddSumMax = 3;
+struct LoraSumArgs {
+    const uint16_t* xa[kAddSumMax]; const uint16_t* b[kAddSumMax]; const uint16_t* x[kAddSumMax];
+    int b_transposed[kAddSumMax];
+    uint16_t* y;
+    int64_t T;
+    int N, C, R;
+    int rows_per_wave, col_tiles;
+};
+
+template <int NSRC>
+__global__ __launch_bounds__(kAddThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void lora_add_sum_kernel(const LoraSumArgs a) {
+    constexpr int CT = kAddPlainColTiles, RS = kAddWaves / CT;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int col_tile = ((int)blockIdx.x % a.col_tiles) * CT + wave % CT;
+    const int64_t row_tile = (int)blockIdx.x / a.col_tiles;
+    const int chunk = col_tile * (kTileCols / 8) + (lane & 15);
+    const bool active = chunk < a.C;
+    const int col0 = chunk * 8;
+    const int g = lane >> 4;
+    BOperand<1> B[NSRC];
+#pragma unroll
+    for (int i = 0; i < NSRC; ++i) B[i].load(a.b[i], a.N, a.R, col0, active, g, a.b_transposed[i] != 0);
+    const int64_t row_begin = (row_tile * RS + wave / CT) * (int64_t)a.rows_per_wave;
+    int64_t row_end = row_begin + a.rows_per_wave;
+    if (row_end > a.T) row_end = a.T;
+    for (int64_t row0 = row_begin; row0 < row_end; row0 += kTileRows) {
+        u32x4 xv[NSRC][4];
+#pragma unroll
+        for (int i = 0; i < NSRC; ++i)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int64_t t = row0 + 4 * g + v;
+                xv[i][v] = u32x4{0, 0, 0, 0};
+                if (active && t < row_end) xv[i][v] = ld16_nt(a.x[i] + t * a.N + col0);
+            }
+        // the running sum is a bf16 value after every step, so it is carried packed (4 registers a row); the
+        // terms are kept apart in the instruction schedule, or their temporaries add up to a wave per SIMD less
+        u32x4 acc[4];
+#pragma unroll
+        for (int i = 0; i < NSRC; ++i) {
+            uint32_t L[4][4];
+            lora_tile_bf16<1>(a.xa[i], a.R, row0, row_end, lane, B[i], L);
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                float f[8], s[8], y[8];
+                unpack8(xv[i][v], f);
+                if (i != 0) unpack8(acc[v], s);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const float t = f[j] + lora_elem(L[v], j);
+                    y[j] = i == 0 ? t : s[j] + rbf(t);
+                }
+                acc[v] = pack8(y);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int64_t t = row0 + 4 * g + v;
+            if (active && t < row_end) st16_nt(a.y + t * a.N + col0, acc[v]);
+        }
+    }
+}
+
 int tune_add(const char* key, int value) {
     static const char* keys[3] = {"add_rows_per_wave", "add_quant_rows_per_wave", "add_restore_rows_per_wave"};
     for (int m = 0; m < 3; ++m) {
@@ -449,4 +520,38 @@ extern "C" int hyc_lora_add_quant_group(const hyc_lora_add_member* members, int 
 extern "C" int hyc_lora_add_restore_group(const hyc_lora_add_member* members, int count, int64_t T, int64_t R,
                                           int q_bit, void* stream) {
     return add_group_launch<kAddRestore>(members, count, T, R, q_bit, stream);
+}
+
+extern "C" int hyc_lora_add_sum(const hyc_lora_sum_member* members, int count, void* y, int64_t T, int64_t N, int64_t R,
+                                void* stream) {
+    if (!members) return HYC_ERR_NULL;
+    if (count < 2 || count > kAddSumMax) return HYC_ERR_ARG;
+    if (T < 0 || N < 0 || N % 32 != 0 || N > (1 << 28) || T > ((int64_t)1 << 40)) return HYC_ERR_SHAPE;
+    if (R < 4 || R > 16 || R % 4 != 0) return HYC_ERR_RANK;
+    if (T * N == 0) return HYC_OK;
+    if (!y) return HYC_ERR_NULL;
+    if (!aligned16(y)) return HYC_ERR_ALIGN;
+    LoraSumArgs a{};
+    for (int i = 0; i < count; ++i) {
+        const hyc_lora_sum_member& m = members[i];
+        if (!m.xa || !m.b || !m.x) return HYC_ERR_NULL;
+        if (!aligned16(m.x) || (reinterpret_cast<uintptr_t>(m.xa) & 7u) ||
+            !(m.b_transposed ? (reinterpret_cast<uintptr_t>(m.b) & 7u) == 0 : aligned16(m.b)))
+            return HYC_ERR_ALIGN;
+        a.xa[i] = (const uint16_t*)m.xa; a.b[i] = (const uint16_t*)m.b; a.x[i] = (const uint16_t*)m.x;
+        a.b_transposed[i] = m.b_transposed;
+    }
+    a.y = (uint16_t*)y;
+    a.T = T;
+    a.N = (int)N;
+    a.C = (int)(N / 8);
+    a.R = (int)R;
+    a.rows_per_wave = g_add_rows_per_wave[kAddPlain].get();
+    a.col_tiles = (int)cdiv(cdiv(N, kTileCols), kAddPlainColTiles);
+    const int64_t row_tiles = cdiv(T, (int64_t)(kAddWaves / kAddPlainColTiles) * a.rows_per_wave);
+    if (row_tiles * a.col_tiles > INT32_MAX) return HYC_ERR_SHAPE;
+    const dim3 grid((unsigned)(row_tiles * a.col_tiles)), block(kAddThreads);
+    if (count == 2) hipLaunchKernelGGL((lora_add_sum_kernel<2>), grid, block, 0, (hipStream_t)stream, a);
+    else hipLaunchKernelGGL((lora_add_sum_kernel<3>), grid, block, 0, (hipStream_t)stream, a);
+    return check_launch();
 }

@@ -78,7 +78,8 @@ def lora_parts(w, w_quant_state, w_lora_a, b, x, x_lora_a=None):
     return x_main, x_lora_a.to(wt.dtype)
 
 
-def lora_backward(w, w_quant_state, w_lora_a, w_lora_b, x, x_lora_a, grad_y, x_codes=None, accumulate=None):
+def lora_backward(w, w_quant_state, w_lora_a, w_lora_b, x, x_lora_a, grad_y, x_codes=None, accumulate=None,
+                  defer_input=False):
     """-> (grad lora_A, grad lora_B, grad x).  Reference :28-36.
 
     With bf16 operands the rank-R products stream their wide operand once on the matrix cores:
@@ -88,7 +89,9 @@ def lora_backward(w, w_quant_state, w_lora_a, w_lora_b, x, x_lora_a, grad_y, x_c
     fp32 and have the parameters' shapes; the torch expressions below return one gradient per batch
     element, as the reference does, and leave the sum to autograd.  `accumulate`, a running sum of
     input gradients, is added to grad x in the pass that adds its LoRA part (`grad_x += grad_x_temp`
-    in the layers) and may be overwritten."""
+    in the layers) and may be overwritten.  With `defer_input` the third result is not grad x but its
+    two terms and the operand that joins them, `(grad_y @ W, grad_y @ B^T, A^T)`, for lora_input_sum, which
+    adds up the input gradients of projections that share their input in one pass."""
     wd = dense_weight(w, w_quant_state)          # [out, in]
     dt = wd.dtype
     grad_y = grad_y.to(dt)
@@ -114,6 +117,8 @@ def lora_backward(w, w_quant_state, w_lora_a, w_lora_b, x, x_lora_a, grad_y, x_c
         else:
             grad_a = x.to(dt).mT @ grad_mid
     grad_x = grad_y @ wd
+    if defer_input:
+        return grad_a, grad_b, (grad_x, grad_mid, w_lora_a.mT)
     if lora_kernels.supported(grad_x, grad_mid, w_lora_a.mT) and (accumulate is None or accumulate.dtype == dt):
         grad_x = lora_kernels.lora_add(grad_x, grad_mid, w_lora_a.mT, inplace=True, residual=accumulate)
     else:
@@ -121,6 +126,24 @@ def lora_backward(w, w_quant_state, w_lora_a, w_lora_b, x, x_lora_a, grad_y, x_c
         if accumulate is not None:
             grad_x = accumulate + grad_x
     return grad_a, grad_b, grad_x
+
+
+def lora_input_sum(parts):
+    """Sum of the input gradients of projections that share their input, from the deferred terms lora_backward
+    returns: acc = t_0; acc += t_1; ... with t_i = (grad_y @ W)_i + (grad_y @ B^T)_i @ A_i^T, every operation
+    rounded as the chain of lora_backward(..., accumulate=acc) calls rounds it (the reference's
+    `grad_x += grad_x_temp`).  Two or three bf16 terms of rank <= 16 take one pass over their operands."""
+    terms = list(parts)
+    if lora_kernels.supported_sum(terms):
+        return lora_kernels.lora_add_sum(terms)
+    acc = None
+    for grad_x, grad_mid, a_t in terms:
+        if lora_kernels.supported(grad_x, grad_mid, a_t) and (acc is None or acc.dtype == grad_x.dtype):
+            acc = lora_kernels.lora_add(grad_x, grad_mid, a_t, inplace=True, residual=acc)
+        else:
+            grad_x += grad_mid @ a_t
+            acc = grad_x if acc is None else acc + grad_x
+    return acc
 
 
 def repeat_kv(h: torch.Tensor, n_rep: int):

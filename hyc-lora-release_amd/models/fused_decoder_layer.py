@@ -59,7 +59,7 @@ from ..operators.softmax_kernels import softmax_backward, softmax_backward_from_
 from ..operators.triton_fuse_lora_silu_hadamard_backward_kernels import triton_fuse_silu_backward
 from ..operators.triton_fuse_lora_silu_hadamard_forward_kernels import triton_fuse_silu_forward
 from ..operators import lora_kernels
-from .compute_utils import (head_to_hidden_shape, heads_matmul, hidden_to_head_shape, lora_backward, lora_forward, lora_parts,
+from .compute_utils import (head_to_hidden_shape, heads_matmul, hidden_to_head_shape, lora_backward, lora_forward, lora_input_sum, lora_parts,
                             repeat_kv, repeat_kv_backward, rope_backward, rope_forward)
 
 MODES = ("baseline", "intra", "intra_inter", "intra_inter_full_fuse")
@@ -429,9 +429,10 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
                                                                     q_bit, **kw)
             return decompression_dequantization(S[name + "_q"], S[name + "_s"], q_bit, **kw)
 
-        def back(name, inp, inp_lora_a, grad_y, accumulate=None):
+        def back(name, inp, inp_lora_a, grad_y, accumulate=None, defer_input=False):
             """Backward of projection `name`.  `inp` is its input, or the name under which the layer
-            saved that input: a compressed one is then read from its codes, not dequantised."""
+            saved that input: a compressed one is then read from its codes, not dequantised.  With
+            `defer_input` the input gradient comes back as its terms, for lora_input_sum."""
             w, _, qs, la, lb = W[name]
             codes = None
             if isinstance(inp, str):
@@ -439,7 +440,8 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
                     inp = S[inp + "_raw"]
                 else:
                     codes, inp = (S[inp + "_q"], S[inp + "_s"], S.get(inp + "_z"), q_bit), None
-            ga, gb, gx = lora_backward(w, qs, la, lb, inp, inp_lora_a, grad_y, x_codes=codes, accumulate=accumulate)
+            ga, gb, gx = lora_backward(w, qs, la, lb, inp, inp_lora_a, grad_y, x_codes=codes, accumulate=accumulate,
+                                       defer_input=defer_input)
             G[name] = (ga, gb)
             return gx
 
@@ -543,8 +545,9 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
                 grad_fn = silu_backward(gate, grad_h1)
                 del grad_h1
             del grad_down, up, fn, gate
-        grad_x2 = back("gate", "x_norm_2", S["gate_lora_a"], grad_fn)
-        grad_x2 = back("up", "x_norm_2", S["up_lora_a"], grad_h2, accumulate=grad_x2)
+        # gate and up share their input: their input gradients are added up in one pass (`grad_x += grad_x_temp`)
+        grad_x2 = lora_input_sum([back("gate", "x_norm_2", S["gate_lora_a"], grad_fn, defer_input=True),
+                                  back("up", "x_norm_2", S["up_lora_a"], grad_h2, defer_input=True)])
         del grad_fn, grad_h2
         grad_medium, grad_nw2 = norm_backward(grad_x2, "x_medium", norm_weight_2, S["rstd_2"], ctx.norm_grads[1], grad_output)
         del grad_x2
@@ -607,9 +610,9 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
         grad_k = rope_backward(grad_k.transpose(1, 2), cos, sin).transpose(1, 2)
         grad_q, grad_k, grad_v = (head_to_hidden_shape(t) for t in (grad_q, grad_k, grad_v))
 
-        grad_x = back("q", "x_norm_1", S["q_lora_a"], grad_q)
-        grad_x = back("k", "x_norm_1", S["k_lora_a"], grad_k, accumulate=grad_x)
-        grad_x = back("v", "x_norm_1", S["v_lora_a"], grad_v, accumulate=grad_x)
+        grad_x = lora_input_sum([back("q", "x_norm_1", S["q_lora_a"], grad_q, defer_input=True),
+                                 back("k", "x_norm_1", S["k_lora_a"], grad_k, defer_input=True),
+                                 back("v", "x_norm_1", S["v_lora_a"], grad_v, defer_input=True)])
         del grad_q, grad_k, grad_v
         as_reference = spec.reference_outlier_list and spec.mode in ("intra_inter", "intra_inter_full_fuse")
         grad_input, grad_nw1 = norm_backward(grad_x, "x", norm_weight_1, S["rstd_1"], ctx.norm_grads[0], grad_medium,

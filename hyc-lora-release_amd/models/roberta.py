@@ -23,7 +23,7 @@ from ..operators.gelu_kernels import gelu_backward
 from ..operators.layernorm_kernels import layernorm_backward, layernorm_forward
 from ..operators.softmax_kernels import softmax_backward, softmax_backward_from_compressed, softmax_forward
 from ..operators import lora_kernels
-from .compute_utils import (head_to_hidden_shape, heads_matmul, hidden_to_head_shape, lora_backward, lora_forward,
+from .compute_utils import (head_to_hidden_shape, heads_matmul, hidden_to_head_shape, lora_backward, lora_forward, lora_input_sum,
                             lora_parts)
 
 MODES = ("baseline", "intra", "intra_inter")
@@ -211,7 +211,7 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
             return outlier_addition_fuse_decompression_dequantization(S[name + "_q"], S[name + "_s"], S[name + "_o"],
                                                                       S[name + "_idx"], q_bit)
 
-        def back(name, inp, inp_lora_a, grad_y, accumulate=None):
+        def back(name, inp, inp_lora_a, grad_y, accumulate=None, defer_input=False):
             """Backward of projection `name`; `inp` is its input or the name the layer saved it under
             (a compressed input is then read from its codes, not dequantised)."""
             w, qs, la, lb = W[name]
@@ -222,7 +222,7 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
                 else:
                     codes, inp = (S[inp + "_q"], S[inp + "_s"], None, q_bit), None
             G[name + "_a"], G[name + "_b"], gx = lora_backward(w, qs, la, lb, inp, inp_lora_a, grad_y, x_codes=codes,
-                                                                 accumulate=accumulate)
+                                                                 accumulate=accumulate, defer_input=defer_input)
             return gx
 
         def rebuilt(name):
@@ -280,9 +280,10 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
         del grad_s, q, k
         grad_q, grad_k, grad_v = (head_to_hidden_shape(t) for t in (grad_q, grad_k, grad_v))
 
-        grad_x = back("q", "x", S["q_lora_a"], grad_q)
-        grad_x = back("k", "x", S["k_lora_a"], grad_k, accumulate=grad_x)
-        grad_x = back("v", "x", S["v_lora_a"], grad_v, accumulate=grad_x)
+        # q, k and v share their input: their input gradients are added up in one pass
+        grad_x = lora_input_sum([back("q", "x", S["q_lora_a"], grad_q, defer_input=True),
+                                 back("k", "x", S["k_lora_a"], grad_k, defer_input=True),
+                                 back("v", "x", S["v_lora_a"], grad_v, defer_input=True)])
         grad_input = grad_x + grad_ln1
 
         def five(n):

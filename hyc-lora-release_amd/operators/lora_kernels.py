@@ -83,6 +83,49 @@ def lora_add(x_main, xa, b, inplace=False, residual=None):
     return y
 
 
+SUM_MAX_RANK = 16          # hyc_lora_add_sum holds the LoRA-B operands of all its terms in registers
+
+
+def supported_sum(terms):
+    """Whether lora_add_sum takes these (x_main, xa, b) terms: two or three, one shape, rank <= SUM_MAX_RANK."""
+    if not 2 <= len(terms) <= 3:
+        return False
+    shape = terms[0][0].shape
+    return all(x.shape == shape and x.dtype == BF16 and supported(x, xa, b) and b.shape[0] <= SUM_MAX_RANK and
+               b.shape[0] == terms[0][2].shape[0] for x, xa, b in terms)
+
+
+def lora_add_sum(terms):
+    """t_0 (+) t_1 [(+) t_2] with t_i = bf16(x_i + bf16(xa_i @ b_i)) and (+) the bf16 addition, in that order: the
+    bits of lora_add(x_0, ...), lora_add(x_1, ..., residual=that), lora_add(x_2, ..., residual=that), in one
+    pass.  terms: (x_main, xa, b) triples of one shape; the result overwrites the first x_main when that is a
+    contiguous bf16 tensor, and is returned."""
+    if not 2 <= len(terms) <= 3:
+        raise ValueError(f"lora_add_sum takes two or three terms, got {len(terms)}")
+    shape = terms[0][0].shape
+    n = shape[-1]
+    rows = terms[0][0].numel() // max(n, 1)
+    members, keep, rank = [], [], None
+    for x_main, xa, b in terms:
+        if x_main.shape != shape:
+            raise ValueError(f"every term must have the shape {tuple(shape)}, got {tuple(x_main.shape)}")
+        r = _check(xa, b, n, rows)
+        if rank not in (None, r):
+            raise ValueError("the terms share one LoRA rank")
+        rank = r
+        _lib.require_gpu(x_main, xa, b)
+        x = x_main if (x_main.dtype == BF16 and x_main.is_contiguous() and x_main.data_ptr() % 16 == 0) else _prep(x_main, "x_main")
+        xa, (b, bt) = _prep(xa, "xa"), _lora_b(b)
+        members.append(_lib.LoraSumMember(xa.data_ptr(), b.data_ptr(), bt, x.data_ptr()))
+        keep.append((x, xa, b))
+    if rank > SUM_MAX_RANK:
+        raise ValueError(f"lora_add_sum takes ranks up to {SUM_MAX_RANK}, got {rank}")
+    y = keep[0][0]
+    arr = (_lib.LoraSumMember * len(members))(*members)
+    _lib.call("hyc_lora_add_sum", arr, len(members), y.data_ptr(), rows, n, rank, _lib.stream_of(y))
+    return y
+
+
 def _vec_ok(t, n, name):
     if t is not None and t.numel() != n:
         raise ValueError(f"{name} must have {n} elements (one per channel), got {t.numel()}")

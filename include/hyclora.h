@@ -604,6 +604,30 @@ int hyc_lora_contract(const void *x, const void *q, const void *scale, const voi
                       void *stream);
 
 /* ---------------------------------------------------------------------------------------
+ * Sum of two or three LoRA adds in one pass:  y = t_0 (+) t_1 [(+) t_2],  t_i = bf16(x_i + bf16(xa_i . b_i)),
+ * every (+) a bf16 addition in that order - the bits of hyc_lora_add(x_0), then hyc_lora_add(x_1, residual = y),
+ * then hyc_lora_add(x_2, residual = y).
+ *
+ * Replaces the accumulation of the input gradients of projections that share an input in the layers'
+ * backward - `grad_x = ...; grad_x += grad_x_temp` after each lora_backward of q, k, v and of gate, up
+ * (models/llama/fused_llama_layer_intra_inter_full_fuse.py:403-462 with models/utils/compute_utils.py:28-36) -
+ * without writing and re-reading the running sum.
+ *
+ *   members  count (2 or 3) operand sets in host memory (copied at the call): xa bf16 [T, R], b the LoRA
+ *            operand [R, N] (or [N, R] with b_transposed), x bf16 [T, N] (for the backward: grad_y @ W);
+ *   y        bf16 [T, N]; may be one of the x_i.
+ *   R a multiple of 4 up to 16 (HYC_ERR_RANK beyond: call hyc_lora_add in a chain); N % 32 == 0.
+ */
+typedef struct {
+    const void *xa;
+    const void *b;
+    int b_transposed;
+    const void *x;
+} hyc_lora_sum_member;
+int hyc_lora_add_sum(const hyc_lora_sum_member *members, int count, void *y, int64_t T, int64_t N, int64_t R,
+                     void *stream);
+
+/* ---------------------------------------------------------------------------------------
  * Memory-only probe, FOR BENCHMARKING: loads n_reads and stores n_writes bf16 [T, N] tensors (1..3 each,
  * arrays of device pointers in host memory, 16-byte aligned, N % 8 == 0) with the access shape of the
  * kernels of this library and no arithmetic of the path, so that the rate the memory system gives a

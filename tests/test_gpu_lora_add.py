@@ -268,3 +268,50 @@ def test_grouped_launch_rejects_mixed_zero_points(K, dev):
                                            dict(x_main=main, xa=xa, b=b, scale=s)], 4)
     with pytest.raises(ValueError):
         lora_kernels.lora_add_quant_group([dict(x_main=main, xa=xa, b=b, scale=s)] * 5, 4)
+
+
+@pytest.mark.parametrize("count", [2, 3])
+@pytest.mark.parametrize("T,N,R", [(64, 256, 16), (100, 1184, 8), (37, 96, 4), (272, 4096, 16), (4096, 1024, 12)])
+@pytest.mark.parametrize("transposed", [False, True])
+def test_sum_of_lora_adds_equals_the_chain(dev, count, T, N, R, transposed):
+    """hyc_lora_add_sum is the chain lora_add(x_0), lora_add(x_1, residual=.), lora_add(x_2, residual=.) bit for bit:
+    how the input gradients of projections that share an input are accumulated."""
+    import hyclora_amd  # noqa: F401
+    from hyclora_amd.operators import lora_kernels as lk
+    g = torch.Generator().manual_seed(T + N + R + count)
+    rn = lambda *s, sc=1.0: (torch.randn(*s, generator=g) * sc).to(BF16).to(dev)
+    terms = []
+    for _ in range(count):
+        b = rn(N, R, sc=0.2).t() if transposed else rn(R, N, sc=0.2)
+        terms.append((rn(1, T, N), rn(1, T, R), b))
+    assert lk.supported_sum(terms)
+    originals = [(x.cpu().clone(), xa.cpu(), b.cpu()) for x, xa, b in terms]
+    chain = None
+    for x, xa, b in terms:
+        chain = lk.lora_add(x.clone(), xa, b, inplace=True, residual=chain)
+    first = terms[0][0]
+    got = lk.lora_add_sum([(x.clone() if i else x, xa, b) for i, (x, xa, b) in enumerate(terms)])
+    assert got.data_ptr() == first.data_ptr(), "the sum overwrites the first term"
+    assert torch.equal(got, chain)
+    # and the oracle's statement of one add (compute_utils.py:21-24), composed with bf16 additions
+    want = None
+    for x, xa, b in originals:
+        t = O.lora_add(x, xa, b.contiguous())
+        want = t if want is None else (want.float() + t.float()).to(BF16)
+    assert_close_bf16(got, want, what="sum of LoRA adds vs the oracle's composition")
+
+
+def test_sum_of_lora_adds_rejects_what_it_cannot_run(dev):
+    import hyclora_amd  # noqa: F401
+    from hyclora_amd.operators import lora_kernels as lk
+    g = torch.Generator().manual_seed(3)
+    rn = lambda *s: torch.randn(*s, generator=g).to(BF16).to(dev)
+    ok = [(rn(1, 32, 128), rn(1, 32, 16), rn(16, 128)) for _ in range(2)]
+    assert lk.supported_sum(ok)
+    assert not lk.supported_sum(ok[:1]) and not lk.supported_sum(ok * 2)
+    wide = [(rn(1, 32, 128), rn(1, 32, 32), rn(32, 128)) for _ in range(2)]
+    assert not lk.supported_sum(wide)
+    with pytest.raises(ValueError):
+        lk.lora_add_sum(wide)
+    with pytest.raises(ValueError):
+        lk.lora_add_sum([ok[0], (rn(1, 32, 256), rn(1, 32, 16), rn(16, 256))])
