@@ -213,10 +213,12 @@ def bench_layers(torch, dev, only_case="", arm="both", seq=0, dims_override=None
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
+        h0 = time.perf_counter()
         for _ in range(steps):
             clear()
             fn().backward(t.grad)
         e1.record()
+        measure.host_ms = (time.perf_counter() - h0) * 1e3 / steps      # the host's share: enqueueing one step
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / steps, saved, result
 
@@ -258,12 +260,12 @@ def bench_layers(torch, dev, only_case="", arm="both", seq=0, dims_override=None
         entry, saved_p, plain, res_b = {}, 0, None, None
         if arm != "compressed":
             ms_p, saved_p, plain = measure(lambda: run_plain(t, mask, sdpa), t)
-            entry["bf16_uncompressed"] = {"fwd_bwd_ms": ms_p, "saved_activation_MB": saved_p / 1e6}
+            entry["bf16_uncompressed"] = {"fwd_bwd_ms": ms_p, "host_enqueue_ms": measure.host_ms, "saved_activation_MB": saved_p / 1e6}
             # the reference's own comparison arm: its default layer type, hand-written backward, nothing compressed
             base = llama_flash_attn.FusedLlamaLayerBaseline() if maker is None else maker(cfg("baseline", 0))
             base.set_hyclora_config(cfg("baseline", 0))
             ms_b, saved_b, res_b = measure(lambda: run_fused(base, t, mask), t)
-            entry["baseline_layer"] = {"fwd_bwd_ms": ms_b, "saved_activation_MB": saved_b / 1e6,
+            entry["baseline_layer"] = {"fwd_bwd_ms": ms_b, "host_enqueue_ms": measure.host_ms, "saved_activation_MB": saved_b / 1e6,
                                        "check_against_uncompressed": agreement(res_b, plain)}
             del base
         for q in (qbits if arm != "plain" else []):
@@ -275,7 +277,7 @@ def bench_layers(torch, dev, only_case="", arm="both", seq=0, dims_override=None
             for _ in range(3):                       # run past calibration so the steady state is timed
                 run_fused(layer, t, mask).backward(t.grad)
             ms_f, saved_f, res_f = measure(lambda: run_fused(layer, t, mask), t)
-            entry[f"compressed_q{q}"] = {"fwd_bwd_ms": ms_f, "saved_activation_MB": saved_f / 1e6,
+            entry[f"compressed_q{q}"] = {"fwd_bwd_ms": ms_f, "host_enqueue_ms": measure.host_ms, "saved_activation_MB": saved_f / 1e6,
                                          "saved_vs_bf16": saved_p / max(saved_f, 1) if saved_p else None,
                                          "check_against_uncompressed": agreement(res_f, plain, q) if plain else None,
                                          "check_against_baseline_layer": agreement(res_f, res_b, q) if res_b else None}
@@ -412,13 +414,15 @@ def bench_stack(torch, dev, n_layers=4, steps=5):
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
+        h0 = time.perf_counter()
         for _ in range(steps):
             forward(arm).backward()
         e1.record()
+        host_ms = (time.perf_counter() - h0) * 1e3 / steps       # the host's share: enqueueing one step
         torch.cuda.synchronize()
         ms = e0.elapsed_time(e1) / steps
         out[arm] = {"static_MiB": static, "allocated_after_forward_minus_static_MiB": after,
-                    "fwd_bwd_ms": ms, "sequences_per_s": B / (ms * 1e-3)}
+                    "fwd_bwd_ms": ms, "host_enqueue_ms": host_ms, "sequences_per_s": B / (ms * 1e-3)}
     out["activation_memory_ratio"] = out["plain"]["allocated_after_forward_minus_static_MiB"][1] / \
         out["compressed"]["allocated_after_forward_minus_static_MiB"][1]
     return out

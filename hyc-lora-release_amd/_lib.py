@@ -140,8 +140,16 @@ def ptr(t):
     return None if t is None else t.data_ptr()
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def stream_of(t: torch.Tensor):
-    """The HIP stream torch is currently enqueuing on for t's device."""
+    """The HIP stream torch is currently enqueuing on for t's device.  Asked of torch's C layer
+    directly where it offers that: building a torch.cuda.Stream object per launch costs about as
+    much host time as the launch itself."""
+    if _raw_stream is not None:
+        index = t.device.index
+        return _raw_stream(torch.cuda.current_device() if index is None else index)
     return torch.cuda.current_stream(t.device).cuda_stream
 
 

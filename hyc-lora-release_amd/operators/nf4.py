@@ -18,6 +18,18 @@ NF4_TABLE = (-1.0, -0.6961928009986877, -0.5250730514526367, -0.3949174880981445
              0.7229568362236023, 1.0)
 
 
+_DEFAULT_TABLE = {}      # device -> the NF4 levels as a float32 tensor there
+
+
+def _default_table(dev):
+    """The NF4 levels on `dev`, uploaded once: a host tensor copied at every call would make each
+    dequantisation wait for the stream to drain (a pageable host-to-device copy is synchronous)."""
+    t = _DEFAULT_TABLE.get(dev)
+    if t is None:
+        t = _DEFAULT_TABLE[dev] = torch.tensor(NF4_TABLE, dtype=torch.float32).to(dev)
+    return t
+
+
 def make_quant_state(absmax, shape, blocksize=64, dtype=torch.bfloat16, code=None, offset=None, state2=None):
     """A plain stand-in for bitsandbytes.functional.QuantState with the fields dequantize_nf4 reads."""
     return SimpleNamespace(absmax=absmax, shape=torch.Size(shape), dtype=dtype, blocksize=blocksize, quant_type="nf4",
@@ -39,8 +51,8 @@ def dequantize_nf4(w, quant_state):
     packed = w.reshape(-1).contiguous()
     if packed.dtype != torch.uint8 or packed.numel() * 2 != n:
         raise ValueError(f"{packed.numel()} packed bytes do not hold {n} 4-bit codes")
-    table = qs.code if getattr(qs, "code", None) is not None else torch.tensor(NF4_TABLE)
-    table = table.to(device=dev, dtype=torch.float32).contiguous()
+    table = getattr(qs, "code", None)
+    table = _default_table(dev) if table is None else table.to(device=dev, dtype=torch.float32).contiguous()
     if table.numel() != 16:
         raise ValueError("the 4-bit code book must have 16 entries")
     out = torch.empty(n, device=dev, dtype=torch.bfloat16)
