@@ -87,3 +87,17 @@ def test_decoder_layer_on_nf4_weights(nf4, dev):
     assert torch.equal(outs[0][0], outs[1][0])
     for a, b in zip(outs[0][1], outs[1][1]):
         assert (a is None and b is None) or torch.equal(a, b)
+
+
+def test_default_code_book_is_uploaded_once(nf4, dev):
+    """Without a code book in the quant state the published table is used from a device tensor made once
+    per device: a host tensor copied at every call would stall the stream (a pageable copy waits for it)."""
+    table = nf4._default_table(torch.device(dev))
+    assert table.is_cuda and table.dtype == torch.float32
+    assert torch.equal(table.cpu(), torch.tensor(nf4.NF4_TABLE))
+    packed = torch.zeros(64, dtype=torch.uint8, device=dev)
+    qs = nf4.make_quant_state(torch.ones(2, device=dev), (128,), blocksize=64)
+    before = dict(nf4._DEFAULT_TABLE)
+    nf4.dequantize_nf4(packed, qs)
+    nf4.dequantize_nf4(packed, qs)
+    assert nf4._DEFAULT_TABLE == before and nf4._default_table(packed.device) is table

@@ -188,3 +188,23 @@ def test_full_size_properties_config2_shape(cf, dev, q_bit):
     # a 64-row sample against the oracle
     rows = x[:, 100:116, :].cpu()
     assert torch.equal(p[:, 100:116, :].cpu(), O.compress(rows, s.cpu(), q_bit))
+
+
+def test_wrappers_enqueue_on_torchs_current_stream(cf, dev):
+    """Inside `with torch.cuda.stream(side)` the kernels go to `side`: its handle is what the wrappers
+    hand to the library, and a result produced there is ordered after work queued on `side` before it."""
+    from hyclora_amd import _lib
+    side = torch.cuda.Stream(device=dev)
+    x = torch.randn(2, 64, 512, device=dev).to(BF16)
+    s = cf.get_statistics_only_quant(x, 4, 'per-channel')
+    want = cf.compression_quantization(x, s, 4)
+    assert _lib.stream_of(x) == torch.cuda.current_stream(dev).cuda_stream
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        assert _lib.stream_of(x) == side.cuda_stream != 0
+        y = torch.zeros_like(x)
+        torch.cuda._sleep(20_000_000)                  # keeps `side` busy while the next two calls are queued
+        y.copy_(x)                                     # on `side`, after the sleep
+        got = cf.compression_quantization(y, s, 4)     # must wait for that copy: same stream
+    side.synchronize()
+    assert torch.equal(got, want)
