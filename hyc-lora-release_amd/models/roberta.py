@@ -25,6 +25,7 @@ from ..operators.softmax_kernels import softmax_backward, softmax_backward_from_
 from ..operators import lora_kernels
 from .compute_utils import (head_to_hidden_shape, heads_matmul, hidden_to_head_shape, lora_backward, lora_forward, lora_input_sum,
                             lora_parts)
+from .fused_decoder_layer import _note_map_entries
 
 MODES = ("baseline", "intra", "intra_inter")
 _PROJ = ("q", "k", "v", "o", "up", "down")
@@ -58,7 +59,7 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
                 w_up, b_up, qs_up, a_up, bb_up, w_down, b_down, qs_down, a_down, bb_down,
                 norm_weight_2, norm_bias_2, attention_mask, num_heads, head_dim,
                 iteration, iteration_threshold, static_value, softmax_outlier_ratio, layernorm_outlier_ratio,
-                q_bit, mode):
+                q_bit, mode, host_state=None):
         if mode not in MODES:
             raise ValueError(f"layer_type must be one of {MODES}, got {mode!r}")
         W = dict(q=(w_q, b_q, qs_q, a_q, bb_q), k=(w_k, b_k, qs_k, a_k, bb_k), v=(w_v, b_v, qs_v, a_v, bb_v),
@@ -140,12 +141,23 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
             a = torch.softmax(s, dim=-1, dtype=v.dtype)
         del s
         o = heads_matmul(a, v, out_hidden=True)
+        map_pending = None
         if raw:
             saved["a_raw"] = a
         else:
             thr = get_statistics_softmax(a, softmax_outlier_ratio) if calib else sv['a']['outlier']
             stats[("a", "outlier")] = thr
-            saved["a_idx"], saved["a_val"], saved["a_seg"] = compress_attention_map(a, thr, seg)
+            capacity = None if (calib or host_state is None) else host_state.get("map_capacity")
+            if capacity is None:
+                # sizes the lists from nnz read back from the device, as to_sparse() does
+                saved["a_idx"], saved["a_val"], saved["a_seg"] = compress_attention_map(a, thr, seg)
+                if host_state is not None:
+                    _note_map_entries(host_state, saved["a_idx"].numel())
+            else:
+                # frozen threshold: lists with room for a little more than the recent steps needed, nothing read
+                # back here; whether they fitted is looked at once the o projection has been enqueued
+                saved["a_idx"], saved["a_val"], saved["a_seg"], count = compress_attention_map(a, thr, seg, capacity=capacity)
+                map_pending = (a, thr, count, capacity)
         del a
         if whole:
             quant("v", v)
@@ -154,6 +166,13 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
         o_final, _, saved["o_lora_a"] = proj("o", o, residual=x)        # o_proj(o) + x in the projection's add pass
         quant("o", o)
         del o
+        if map_pending is not None:
+            a, thr, count, capacity = map_pending
+            nnz = count.value()                   # waits for the compaction only, enqueued before the projection
+            if nnz > capacity:                    # did not fit: write the lists again at their exact size
+                saved["a_idx"], saved["a_val"], saved["a_seg"] = compress_attention_map(a, thr, saved["a_seg"])
+            _note_map_entries(host_state, nnz)
+            del a, map_pending
 
         # ---- first LayerNorm (post-norm: on the residual sum) ----------------------------------
         x_medium, saved["mean_1"], saved["rstd_1"], _, _ = layernorm_forward(o_final, norm_weight_1, norm_bias_1, _EPS)
@@ -289,7 +308,7 @@ class FusedRobertaLayerFunc(torch.autograd.Function):
         def five(n):
             return (None, None, None, G[n + "_a"], G[n + "_b"])
         return (grad_input, *five("q"), *five("k"), *five("v"), *five("o"), None, None,
-                *five("up"), *five("down"), None, None) + (None,) * 10
+                *five("up"), *five("down"), None, None) + (None,) * 11
 
 
 class _FusedRobertaLayerBase(torch.nn.Module):
@@ -302,6 +321,9 @@ class _FusedRobertaLayerBase(torch.nn.Module):
         super().__init__()
         self.iteration = 0
         self.static_value = self._empty()
+        # host-side bookkeeping outside the calibration state (not checkpointed): recent kept-entry counts of
+        # the attention map, from which the next step's lists are sized without reading the count back first
+        self.host_state = {}
         self.use_hyclora = False
 
     def _empty(self):
@@ -364,7 +386,7 @@ class _FusedRobertaLayerBase(torch.nn.Module):
             *five(up_proj_base, up_proj_lora_a, up_proj_lora_b), *five(down_proj_base, down_proj_lora_a, down_proj_lora_b),
             norm_weight_2, norm_bias_2, attention_mask, num_heads, head_dim,
             self.iteration, self.iteration_threshold, self.static_value,
-            self.softmax_outlier_ratio, self.layernorm_outlier_ratio, self.q_bit, self.layer_type)
+            self.softmax_outlier_ratio, self.layernorm_outlier_ratio, self.q_bit, self.layer_type, self.host_state)
         y, stat_values = outs[0], outs[1:]
         if self.iteration < self.iteration_threshold:
             fresh = {}

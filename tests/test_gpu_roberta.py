@@ -163,3 +163,39 @@ def test_roberta_calibration_freezes_and_paths_agree(dev, tmp_path):
     assert torch.equal(y2, y1)
     with pytest.raises(ValueError):
         roberta.make_fused_roberta_layer(config("intra_inter_full_fuse", 4))
+
+
+@pytest.mark.parametrize("layer_type", ["intra", "intra_inter"])
+def test_roberta_map_lists_sized_without_a_read_back(dev, layer_type):
+    """With a frozen threshold the encoder layers size the attention map's lists from the kept-entry counts
+    of recent steps and look at the current step's count only after the o projection has been enqueued: the
+    results equal the exact-size path's bit for bit, when the lists fit and when they do not."""
+    import hyclora_amd  # noqa: F401
+    from hyclora_amd.models import roberta
+
+    def steps(tamper):
+        t = make_inputs(dev, seed=77, B=2, S=256, hidden=256, heads=4, inter=512)
+        layer = roberta.make_fused_roberta_layer(config(layer_type, 4, sm_ratio=0.05, thr=1))
+        outs = []
+        for it in range(3):
+            if it >= 1:
+                tamper(layer)
+            y = run_fused(layer, t)
+            y.backward(t.grad)
+            outs.append((y.detach().clone(), t.x.grad.clone(), [m.weight.grad.clone() for n in NAMES for m in t.P[n][1:]]))
+            t.x.grad = None
+            for n in NAMES:
+                for m in t.P[n][1:]:
+                    m.weight.grad = None
+        return layer, outs
+
+    ref_layer, ref = steps(lambda layer: layer.host_state.pop("map_capacity", None))    # nnz read back every step
+    layer, got = steps(lambda layer: None)
+    nnz = ref_layer.host_state["map_history"][-1]
+    assert nnz > 0 and layer.host_state["map_history"] == [nnz] * 3
+    assert nnz < layer.host_state["map_capacity"] <= nnz * 1.07 + 64
+    small_layer, small = steps(lambda layer: layer.host_state.__setitem__("map_capacity", 5))
+    assert small_layer.host_state["map_history"] == [nnz] * 3
+    for a, b, c in zip(ref, got, small):
+        for u, v, w in zip((a[0], a[1], *a[2]), (b[0], b[1], *b[2]), (c[0], c[1], *c[2])):
+            assert torch.equal(u, v) and torch.equal(u, w)
