@@ -38,6 +38,7 @@ Deliberate differences from the reference:
 from __future__ import annotations
 
 import math
+import weakref
 from dataclasses import dataclass
 
 import torch
@@ -113,6 +114,40 @@ class LayerSpec:
 
 
 _PROJ = ("q", "k", "v", "o", "gate", "up", "down")
+
+_ALL_KEPT = {}      # id(mask tensor) -> (weak reference to it, its version, whether every position is kept)
+
+
+def _nothing_padded(mask2d):
+    """Whether a [B, S] key-padding mask keeps every position.  The answer needs one read-back from the
+    device; it is kept with the mask tensor (weakly, and only while the tensor is not modified in place),
+    because every layer of a model is handed the same mask object in a step."""
+    key = id(mask2d)
+    hit = _ALL_KEPT.get(key)
+    if hit is not None and hit[0]() is mask2d and hit[1] == mask2d._version:
+        return hit[2]
+    full = bool((mask2d != 0).all().item())
+    _ALL_KEPT[key] = (weakref.ref(mask2d, lambda _r, k=key: _ALL_KEPT.pop(k, None)), mask2d._version, full)
+    return full
+
+
+def key_padding_attention_mask(mask2d, dtype):
+    """The map-free layers of the reference take a key-padding mask [B, S] (non-zero = a real token) and run
+    the varlen flash kernel, causal, on the unpadded tokens; the attention output of padded positions is zero
+    (llama_flash_attn/fused_llama_layer_intra_inter.py:160-178).  -> (None, None) when nothing is padded -
+    the plain causal kernel is that computation - else (additive mask [B, 1, S, S]: 0 where query i may look
+    at key j <= i of a real token or at itself, -inf elsewhere; keep [B, 1, S, 1] in `dtype`, by which the
+    attention output is multiplied)."""
+    if mask2d.dim() != 2:
+        raise ValueError(f"a key-padding mask is [batch, seq], got shape {tuple(mask2d.shape)}")
+    if _nothing_padded(mask2d):
+        return None, None
+    keep = mask2d != 0
+    s = keep.shape[1]
+    causal = torch.ones(s, s, dtype=torch.bool, device=keep.device).tril()
+    allowed = (causal[None] & keep[:, None, :]) | torch.eye(s, dtype=torch.bool, device=keep.device)[None]
+    additive = torch.zeros(allowed.shape, dtype=dtype, device=keep.device).masked_fill_(~allowed, float("-inf"))
+    return additive[:, None], keep[:, None, :, None].to(dtype)
 
 
 class FusedDecoderLayerFunc(torch.autograd.Function):
@@ -315,6 +350,12 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             # forward (the reference keeps flash-attn's softmax_lse the same way,
             # llama_flash_attn/fused_llama_layer_intra_inter.py:169-180, :459-468)
             ctx.flash = None
+            query_keep = ctx.key_padding = None
+            if attention_mask is not None and attention_mask.dim() == 2:      # the reference's key-padding mask
+                key_padding = attention_mask
+                attention_mask, query_keep = key_padding_attention_mask(key_padding, q.dtype)
+                if query_keep is not None:
+                    ctx.key_padding = key_padding      # backward builds the [B, 1, S, S] mask again instead of keeping it
             if KEEP_ATTENTION_LSE and attention_mask is None and q.is_cuda:
                 try:
                     res = torch.ops.aten._scaled_dot_product_flash_attention(q, k, v, 0.0, True, False)
@@ -325,6 +366,8 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
                     ctx.flash = None
             if ctx.flash is None:
                 o = F.scaled_dot_product_attention(q, k, v, attn_mask=attention_mask, is_causal=attention_mask is None)
+                if query_keep is not None:
+                    o = o * query_keep
             del q, k, v
         o = head_to_hidden_shape(o)
         x_medium, _, saved["o_lora_a"] = proj("o", o, residual=x)       # x + o_proj(o) in the projection's add pass
@@ -398,7 +441,7 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
         ctx.spec, ctx.q_bit = spec, q_bit
         ctx.num_heads, ctx.num_key_value_heads, ctx.head_dim = num_heads, num_key_value_heads, head_dim
         ctx.has_mask = attention_mask is not None
-        ctx.attention_mask = attention_mask
+        ctx.attention_mask = None if spec.attention == "sdpa" and ctx.key_padding is not None else attention_mask
         ctx.norm_grads = (norm_weight_1.requires_grad, norm_weight_2.requires_grad)
         out_stats = tuple(stats[slot] for slot in spec.stat_slots())
         ctx.mark_non_differentiable(*[t for t in out_stats if torch.is_tensor(t)])
@@ -600,8 +643,12 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
         else:
             with torch.enable_grad():
                 q_, k_, v_ = (t.detach().requires_grad_() for t in (q, k, v))
-                o_ = F.scaled_dot_product_attention(q_, k_, v_, attn_mask=ctx.attention_mask,
-                                                    is_causal=not ctx.has_mask)
+                mask, query_keep = ctx.attention_mask, None
+                if ctx.key_padding is not None:
+                    mask, query_keep = key_padding_attention_mask(ctx.key_padding, q.dtype)
+                o_ = F.scaled_dot_product_attention(q_, k_, v_, attn_mask=mask, is_causal=not ctx.has_mask)
+                if query_keep is not None:
+                    o_ = o_ * query_keep
                 grad_q, grad_k, grad_v = torch.autograd.grad(o_, (q_, k_, v_), grad_o)
             del q, k, v, q_, k_, v_, o_, grad_o
         grad_v = repeat_kv_backward(grad_v, n_rep)
@@ -716,7 +763,12 @@ class FusedDecoderLayer(torch.nn.Module):
                 norm_weight_2, norm_bias_2,
                 gate_proj_base, gate_proj_lora_a, gate_proj_lora_b, up_proj_base, up_proj_lora_a, up_proj_lora_b,
                 down_proj_base, down_proj_lora_a, down_proj_lora_b,
-                attention_mask, num_heads, head_dim, num_key_value_heads):
+                attention_mask, num_heads, head_dim, num_key_value_heads=None):
+        # the reference's map-free modules are called without num_key_value_heads
+        # (llama_flash_attn/modeling_llama.py:620-653): as many key / value heads as query heads
+        if num_key_value_heads is None:
+            num_key_value_heads = num_heads
+
         def five(base, la, lb):
             w = base.weight
             return (w, getattr(base, "bias", None), getattr(w, "quant_state", None),

@@ -1,6 +1,6 @@
 """Llama decoder layers with compressed saved activations; class names as in the reference
 (models/llama/fused_llama_layer_{baseline,intra,intra_inter,intra_inter_full_fuse}.py)."""
-from .fused_decoder_layer import FusedDecoderLayer
+from ..fused_decoder_layer import FusedDecoderLayer
 
 
 class FusedLlamaLayerBaseline(FusedDecoderLayer):
@@ -36,3 +36,15 @@ def make_fused_llama_layer(hyclora_config):
         raise ValueError(f"Unknown layer type: {hyclora_config.layer_type}") from None
     layer.set_hyclora_config(hyclora_config)
     return layer
+
+
+def set_fused_llama_layer(model, hyclora_config):
+    """LlamaForCausalLM.set_fused_llama_layer of the reference as a function of the model
+    (models/llama/modeling_llama.py:1151-1180): every decoder layer in `model.model.layers` gets a configured
+    fused layer of the configured type as its `fused_llama_layer`, which the decoder layer's forward calls
+    while training (:745-786).  The configuration is kept on the model as `hyclora_config`."""
+    if hyclora_config.layer_type not in LAYER_TYPES:
+        raise ValueError(f"Unknown layer type: {hyclora_config.layer_type} (available: {sorted(LAYER_TYPES)})")
+    model.hyclora_config = hyclora_config
+    for layer in model.model.layers:
+        layer.fused_llama_layer = make_fused_llama_layer(hyclora_config)

@@ -2,7 +2,7 @@
 the reference (models/mistral/fused_mistral_layer_*.py).  The computation is the generic layer: the
 reference's Mistral files differ from the Llama ones only in always calling repeat_kv and in a dtype
 cast of lora_B (fused_mistral_layer_intra_inter_full_fuse.py:226-227), both covered there."""
-from .fused_decoder_layer import FusedDecoderLayer
+from ..fused_decoder_layer import FusedDecoderLayer
 
 
 class FusedMistralLayerBaseline(FusedDecoderLayer):
@@ -36,3 +36,14 @@ def make_fused_mistral_layer(hyclora_config):
         raise ValueError(f"Unknown layer type: {hyclora_config.layer_type}") from None
     layer.set_hyclora_config(hyclora_config)
     return layer
+
+
+def set_fused_mistral_layer(model, hyclora_config):
+    """MistralForCausalLM.set_fused_mistral_layer of the reference as a function of the model
+    (models/mistral/modeling_mistral.py:998-1027): a configured fused layer per decoder layer, as
+    `fused_mistral_layer`."""
+    if hyclora_config.layer_type not in LAYER_TYPES:
+        raise ValueError(f"Unknown layer type: {hyclora_config.layer_type} (available: {sorted(LAYER_TYPES)})")
+    model.hyclora_config = hyclora_config
+    for layer in model.model.layers:
+        layer.fused_mistral_layer = make_fused_mistral_layer(hyclora_config)

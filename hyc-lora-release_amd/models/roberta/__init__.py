@@ -14,18 +14,18 @@ import math
 
 import torch
 
-from ..operators.compress_function import (compress_attention_map, compression_pack_channel_base,
+from ...operators.compress_function import (compress_attention_map, compression_pack_channel_base,
                                            compression_pack_quant_base, decompression_dequantization,
                                            get_statistics_only_quant, get_statistics_softmax,
                                            outlier_addition_fuse_decompression_dequantization, update_dict,
                                            validate_channel_list)
-from ..operators.gelu_kernels import gelu_backward
-from ..operators.layernorm_kernels import layernorm_backward, layernorm_forward
-from ..operators.softmax_kernels import softmax_backward, softmax_backward_from_compressed, softmax_forward
-from ..operators import lora_kernels
-from .compute_utils import (head_to_hidden_shape, heads_matmul, hidden_to_head_shape, lora_backward, lora_forward, lora_input_sum,
+from ...operators.gelu_kernels import gelu_backward
+from ...operators.layernorm_kernels import layernorm_backward, layernorm_forward
+from ...operators.softmax_kernels import softmax_backward, softmax_backward_from_compressed, softmax_forward
+from ...operators import lora_kernels
+from ..compute_utils import (head_to_hidden_shape, heads_matmul, hidden_to_head_shape, lora_backward, lora_forward, lora_input_sum,
                             lora_parts)
-from .fused_decoder_layer import _note_map_entries
+from ..fused_decoder_layer import _note_map_entries
 
 MODES = ("baseline", "intra", "intra_inter")
 _PROJ = ("q", "k", "v", "o", "up", "down")
@@ -427,3 +427,14 @@ def make_fused_roberta_layer(hyclora_config):
         raise ValueError(f"Unknown layer type: {hyclora_config.layer_type}") from None
     layer.set_hyclora_config(hyclora_config)
     return layer
+
+
+def set_fused_roberta_layer(model, hyclora_config):
+    """RobertaForSequenceClassification.set_fused_roberta_layer of the reference as a function of the model
+    (models/roberta/modeling_roberta.py:982-1009): a configured fused layer per encoder layer in
+    `model.roberta.encoder.layer`, as `fused_roberta_layer`."""
+    if hyclora_config.layer_type not in LAYER_TYPES:
+        raise ValueError(f"Unknown layer type: {hyclora_config.layer_type} (available: {sorted(LAYER_TYPES)})")
+    model.hyclora_config = hyclora_config
+    for layer in model.roberta.encoder.layer:
+        layer.fused_roberta_layer = make_fused_roberta_layer(hyclora_config)

@@ -61,7 +61,7 @@ class RefRMSNorm(torch.autograd.Function):
         return O.rmsnorm_bwd(dy, x, w, rstd)
 
 
-def reference_layer(t, sdpa=False):
+def reference_layer(t, sdpa=False, key_padding=None):
     from hyclora_amd.models.compute_utils import hidden_to_head_shape, head_to_hidden_shape, repeat_kv
     rope_forward = O.rope                      # differentiable torch ops; the HIP operator works in place
     P = t.P
@@ -77,7 +77,18 @@ def reference_layer(t, sdpa=False):
     q = rope_forward(q.transpose(1, 2), t.cos, t.sin).transpose(1, 2)
     k = rope_forward(k.transpose(1, 2), t.cos, t.sin).transpose(1, 2)
     k, v = repeat_kv(k, t.heads // t.kv_heads), repeat_kv(v, t.heads // t.kv_heads)
-    if sdpa:                    # causal attention without a materialised map (long sequences)
+    if key_padding is not None:
+        # the reference's map-free layers on a padded batch: causal attention among the real tokens, zero output
+        # at padded positions (llama_flash_attn/fused_llama_layer_intra_inter.py:160-178), written densely
+        keep = key_padding != 0
+        S = keep.shape[1]
+        allowed = (torch.ones(S, S, dtype=torch.bool, device=keep.device).tril()[None] & keep[:, None, :]) | \
+            torch.eye(S, dtype=torch.bool, device=keep.device)[None]
+        s = (q @ k.transpose(-2, -1)).float() / math.sqrt(t.hd)
+        s = s.masked_fill(~allowed[:, None], float("-inf"))
+        a = torch.softmax(s, dim=-1).to(BF16)
+        o = head_to_hidden_shape((a @ v) * keep[:, None, :, None].to(BF16))
+    elif sdpa:                    # causal attention without a materialised map (long sequences)
         o = head_to_hidden_shape(F.scaled_dot_product_attention(q, k, v, is_causal=True))
     else:
         s = q @ k.transpose(-2, -1) / math.sqrt(t.hd) + t.mask
@@ -525,3 +536,83 @@ def test_saved_activation_footprint(dev):
     T = B * S
     baseline = 8 * T * Hd * 2 + 4 * T * I * 2 + 7 * T * R * 2          # the bf16 save list of the uncompressed layer
     assert fused_bytes < 0.4 * baseline, (fused_bytes, baseline)
+
+
+def _run_map_free(layer, t, mask, with_kv_heads=True):
+    P = t.P
+    args = [t.x, t.nw1, None, t.cos, t.sin]
+    for n in ("q", "k", "v", "o"):
+        args += list(P[n])
+    args += [t.nw2, None]
+    for n in ("gate", "up", "down"):
+        args += list(P[n])
+    args += [mask, t.heads, t.hd] + ([t.kv_heads] if with_kv_heads else [])
+    return layer(*args)
+
+
+def test_map_free_layer_takes_the_references_call_and_key_padding_mask(dev):
+    """The reference calls its map-free modules without num_key_value_heads and with a key-padding mask
+    [B, S] (llama_flash_attn/modeling_llama.py:620-653, fused_llama_layer_intra_inter.py:160-163).  A mask that
+    pads nothing must give the bits of the causal kernel; it is looked at on the host once per mask object."""
+    import hyclora_amd  # noqa: F401
+    from hyclora_amd.models import fused_decoder_layer as fdl
+    from hyclora_amd.models import llama_flash_attn as lf
+    t = make_layer_inputs(dev, seed=5, S=128)
+    results = []
+    for mask, with_kv in ((None, True), (torch.ones(2, 128, dtype=torch.int64, device=dev), False),
+                          (torch.ones(2, 128, dtype=torch.bool, device=dev), True)):
+        layer = lf.FusedLlamaLayerIntraInter()
+        layer.set_hyclora_config(config("intra_inter", 4, thr=1))
+        outs = []
+        for _ in range(2):                                # a calibrating and a frozen step
+            out = _run_map_free(layer, t, mask, with_kv)
+            outs.append((out.detach().clone(), grads_of(t, out)))
+        results.append(outs)
+        if mask is not None:
+            assert fdl._ALL_KEPT[id(mask)][2] is True
+    for other in results[1:]:
+        for (o_a, g_a), (o_b, g_b) in zip(results[0], other):
+            assert torch.equal(o_a, o_b)
+            for a, b in zip(g_a, g_b):
+                assert torch.equal(a, b)
+    # a mask changed in place is looked at again
+    mask = torch.ones(2, 128, dtype=torch.int64, device=dev)
+    assert fdl._nothing_padded(mask) is True
+    mask[1, 100:] = 0
+    assert fdl._nothing_padded(mask) is False
+
+
+@pytest.mark.parametrize("side", ["right", "left"])
+def test_map_free_layer_on_a_padded_batch(dev, side):
+    """Key-padding mask with padded positions: causal attention among the real tokens and a zero attention
+    output at padded positions, against a dense torch-autograd statement of the same layer - the uncompressed
+    layer type to bf16 rounding, the compressed one at 8 bits to the sanity bound of the other layer tests."""
+    import hyclora_amd  # noqa: F401
+    from hyclora_amd.models import llama_flash_attn as lf
+    t = make_layer_inputs(dev, seed=8, S=96)
+    mask = torch.ones(2, 96, dtype=torch.int64, device=dev)
+    if side == "right":
+        mask[1, 70:] = 0
+    else:
+        mask[1, :26] = 0
+    real = mask.bool()[:, :, None]
+    t.grad = t.grad * real                               # a loss that ignores padded positions
+    ref_out = reference_layer(t, key_padding=mask)
+    ref_grads = grads_of(t, ref_out)
+    names = ["x", "norm_w1", "norm_w2"] + [f"{n}.lora_{ab}" for n in ("q", "k", "v", "o", "gate", "up", "down") for ab in "AB"]
+    base = lf.FusedLlamaLayerBaseline()
+    base.set_hyclora_config(SimpleNamespace(use_hyclora=True, layer_type="baseline"))
+    out = _run_map_free(base, t, mask, with_kv_heads=False)
+    rel, cos = rel_err_and_cos(out, ref_out)
+    assert rel <= 1e-2 and cos >= 0.9999, f"forward: rel {rel:.2e} cos {cos:.6f}"
+    for name, g, gr in zip(names, grads_of(t, out), ref_grads):
+        rel, cos = rel_err_and_cos(g, gr)
+        assert rel <= 2e-2 and cos >= 0.9999, f"baseline, {side} padding, grad {name}: rel {rel:.2e} cos {cos:.6f}"
+    layer = lf.FusedLlamaLayerIntraInter()
+    layer.set_hyclora_config(config("intra_inter", 8))
+    out = _run_map_free(layer, t, mask)
+    rel, cos = rel_err_and_cos(out, ref_out)
+    assert rel <= 1e-2 and cos >= 0.9999
+    for name, g, gr in zip(names, grads_of(t, out), ref_grads):
+        rel, cos = rel_err_and_cos(g, gr)
+        assert cos >= COS_FLOOR[8], f"intra_inter q8, {side} padding, grad {name}: rel {rel:.2e} cos {cos:.5f}"

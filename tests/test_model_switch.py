@@ -1,0 +1,129 @@
+"""The host layers under the reference's module and class names, its model-level switch
+(`set_fused_*_layer`) as functions of a model, and the call forms of its model files (CPU: nothing is run)."""
+import importlib
+import inspect
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+import hyclora_amd  # noqa: F401
+
+CFG = SimpleNamespace(use_hyclora=True, layer_type="intra_inter", iteration_threshold=5, softmax_outlier_ratio=0.05,
+                      layernorm_outlier_ratio=0.005, q_bit=2)
+
+# module -> class, as the reference's model files import them (models/llama/modeling_llama.py:52-55,
+# models/mistral/modeling_mistral.py, models/llama_flash_attn/modeling_llama.py, models/roberta/modeling_roberta.py)
+REFERENCE_IMPORTS = {
+    "llama.fused_llama_layer_baseline": "FusedLlamaLayerBaseline",
+    "llama.fused_llama_layer_intra": "FusedLlamaLayerIntra",
+    "llama.fused_llama_layer_intra_inter": "FusedLlamaLayerIntraInter",
+    "llama.fused_llama_layer_intra_inter_full_fuse": "FusedLlamaLayerIntraInterFullFuse",
+    "mistral.fused_mistral_layer_baseline": "FusedMistralLayerBaseline",
+    "mistral.fused_mistral_layer_intra": "FusedMistralLayerIntra",
+    "mistral.fused_mistral_layer_intra_inter": "FusedMistralLayerIntraInter",
+    "mistral.fused_mistral_layer_intra_inter_full_fuse": "FusedMistralLayerIntraInterFullFuse",
+    "llama_flash_attn.fused_llama_layer_baseline": "FusedLlamaLayerBaseline",
+    "llama_flash_attn.fused_llama_layer_intra": "FusedLlamaLayerIntra",
+    "llama_flash_attn.fused_llama_layer_intra_inter": "FusedLlamaLayerIntraInter",
+    "roberta.fused_roberta_layer_baseline": "FusedRobertaLayer",
+    "roberta.fused_roberta_layer_intra": "FusedRobertaLayerIntra",
+    "roberta.fused_roberta_layer_intra_inter": "FusedRobertaLayerIntraInter",
+}
+
+
+@pytest.mark.parametrize("module, name", sorted(REFERENCE_IMPORTS.items()))
+def test_reference_module_names_export_the_classes(module, name):
+    mod = importlib.import_module("hyclora_amd.models." + module)
+    cls = getattr(mod, name)
+    family, kind = module.split(".")
+    layer = cls()
+    layer.set_hyclora_config(CFG)
+    assert layer.use_hyclora and layer.q_bit == 2 and layer.iteration == 0
+    want = "baseline" if kind.endswith("baseline") else kind.split("_layer_")[1]
+    assert layer.layer_type == want
+    if family == "llama_flash_attn":
+        assert layer.spec.attention == "sdpa"
+    elif family != "roberta":
+        assert layer.spec.attention == "map"
+
+
+def _dummy(n_layers, path):
+    layers = [SimpleNamespace() for _ in range(n_layers)]
+    root = SimpleNamespace()
+    node = root
+    for part in path[:-1]:
+        setattr(node, part, SimpleNamespace())
+        node = getattr(node, part)
+    setattr(node, path[-1], layers)
+    return root, layers
+
+
+@pytest.mark.parametrize("family, attr, path", [("llama", "fused_llama_layer", ("model", "layers")),
+                                                ("mistral", "fused_mistral_layer", ("model", "layers")),
+                                                ("llama_flash_attn", "fused_llama_layer", ("model", "layers")),
+                                                ("roberta", "fused_roberta_layer", ("roberta", "encoder", "layer"))])
+def test_model_level_switch(family, attr, path):
+    pkg = importlib.import_module("hyclora_amd.models." + family)
+    switch = getattr(pkg, "set_" + attr)
+    model, layers = _dummy(3, path)
+    switch(model, CFG)
+    assert model.hyclora_config is CFG
+    fused = [getattr(layer, attr) for layer in layers]
+    assert len({id(f) for f in fused}) == 3                       # one module, one calibration state per layer
+    for f in fused:
+        assert type(f) is pkg.LAYER_TYPES["intra_inter"] and f.use_hyclora and f.iteration_threshold == 5
+    with pytest.raises(ValueError):
+        switch(model, SimpleNamespace(use_hyclora=True, layer_type="no_such_type"))
+
+
+def test_switch_on_stock_transformers_models():
+    """The attribute paths the switch walks are those of the stock model classes."""
+    transformers = pytest.importorskip("transformers")
+    from hyclora_amd.models import llama, roberta
+    cfg = transformers.LlamaConfig(vocab_size=64, hidden_size=64, intermediate_size=128, num_hidden_layers=2,
+                                   num_attention_heads=2, num_key_value_heads=2, max_position_embeddings=64)
+    model = transformers.LlamaForCausalLM(cfg)
+    llama.set_fused_llama_layer(model, CFG)
+    assert all(isinstance(layer.fused_llama_layer, llama.FusedLlamaLayerIntraInter) for layer in model.model.layers)
+    # registered as submodules: the calibration state travels with the model's state_dict
+    assert any(k.endswith("fused_llama_layer._extra_state") for k in model.state_dict())
+    rcfg = transformers.RobertaConfig(vocab_size=64, hidden_size=64, intermediate_size=128, num_hidden_layers=2,
+                                      num_attention_heads=2, max_position_embeddings=66)
+    rmodel = transformers.RobertaForSequenceClassification(rcfg)
+    roberta.set_fused_roberta_layer(rmodel, CFG)
+    assert all(isinstance(layer.fused_roberta_layer, roberta.FusedRobertaLayerIntraInter)
+               for layer in rmodel.roberta.encoder.layer)
+
+
+def test_forward_signatures_take_the_references_calls():
+    """Positional argument counts of the calls in the reference's model files: 32 for the Llama / Mistral map
+    layers (…, attention_mask, num_heads, head_dim, num_key_value_heads; modeling_llama.py:753-786), 31 for the
+    map-free ones (no num_key_value_heads; llama_flash_attn/modeling_llama.py:620-653), 26 for the encoder
+    layers (modeling_roberta.py:429-456)."""
+    from hyclora_amd.models import llama, llama_flash_attn, roberta
+    dec = inspect.signature(llama.FusedLlamaLayerIntraInter.forward).parameters
+    names = list(dec)[1:]
+    assert len(names) == 32 and names[-4:] == ["attention_mask", "num_heads", "head_dim", "num_key_value_heads"]
+    assert dec["num_key_value_heads"].default is None            # may be left out, as the map-free call does
+    assert llama_flash_attn.FusedLlamaLayerIntraInter.forward is llama.FusedLlamaLayerIntraInter.forward
+    enc = list(inspect.signature(roberta.FusedRobertaLayerIntraInter.forward).parameters)[1:]
+    assert len(enc) == 26 and enc[-3:] == ["attention_mask", "num_heads", "head_dim"]
+
+
+def test_key_padding_mask_helper_on_cpu():
+    """[B, S] key-padding mask -> additive causal mask among the real tokens + the rows to keep; a mask that
+    pads nothing -> (None, None)."""
+    from hyclora_amd.models.fused_decoder_layer import key_padding_attention_mask
+    full = torch.ones(2, 5, dtype=torch.int64)
+    assert key_padding_attention_mask(full, torch.float32) == (None, None)
+    mask = torch.tensor([[1, 1, 1, 1], [0, 1, 1, 0]])
+    add, keep = key_padding_attention_mask(mask, torch.float32)
+    assert add.shape == (2, 1, 4, 4) and keep.shape == (2, 1, 4, 1)
+    ninf = float("-inf")
+    assert add[0, 0].tolist() == [[0, ninf, ninf, ninf], [0, 0, ninf, ninf], [0, 0, 0, ninf], [0, 0, 0, 0]]
+    # batch 1: positions 0 and 3 are padding; a padded query sees itself only where nothing else is allowed
+    assert add[1, 0].tolist() == [[0, ninf, ninf, ninf], [ninf, 0, ninf, ninf], [ninf, 0, 0, ninf], [ninf, 0, 0, 0]]
+    assert keep[:, 0, :, 0].tolist() == [[1, 1, 1, 1], [0, 1, 1, 0]]
+    with pytest.raises(ValueError):
+        key_padding_attention_mask(torch.ones(2, 1, 4, 4), torch.float32)
