@@ -146,17 +146,39 @@ def lora_input_sum(parts):
     return acc
 
 
-def repeat_kv(h: torch.Tensor, n_rep: int):
+def repeat_kv(hidden_states: torch.Tensor, n_rep: int):
+    """[B, KV, S, D] -> [B, KV * n_rep, S, D], every key / value head n_rep times in a row.  Reference :38-43."""
     if n_rep == 1:
-        return h
-    b, kv, s, d = h.shape
-    return h[:, :, None, :, :].expand(b, kv, n_rep, s, d).reshape(b, kv * n_rep, s, d)
+        return hidden_states
+    b, kv, s, d = hidden_states.shape
+    return hidden_states[:, :, None, :, :].expand(b, kv, n_rep, s, d).reshape(b, kv * n_rep, s, d)
 
 
-def repeat_kv_backward(g: torch.Tensor, n_rep: int):
+def repeat_kv_backward(grad_output: torch.Tensor, n_rep: int):
+    """Gradient of repeat_kv: the n_rep copies of a head summed.  Reference :46-50."""
     if n_rep == 1:
-        return g
-    return g.unflatten(1, (g.shape[1] // n_rep, n_rep)).sum(dim=2)
+        return grad_output
+    return grad_output.unflatten(1, (grad_output.shape[1] // n_rep, n_rep)).sum(dim=2)
+
+
+def unpad_input(hidden_states, attention_mask):
+    """[B, S, ...] and a key-padding mask [B, S] (non-zero = a real token) -> (the real tokens' rows
+    [nnz, ...], their positions in the flattened [B * S] axis, cumulative sequence lengths int32 [B + 1], the
+    longest sequence as an int).  Reference :69-97 (flash-attn's padding helper; its map-free layers call it,
+    the ones in this package mask instead).  Reads the longest length back from the device, as there."""
+    lengths = attention_mask.sum(dim=-1, dtype=torch.int32)
+    indices = torch.nonzero(attention_mask.flatten(), as_tuple=False).flatten()
+    cu_seqlens = torch.nn.functional.pad(torch.cumsum(lengths, dim=0, dtype=torch.int32), (1, 0))
+    rows = hidden_states.reshape(-1, *hidden_states.shape[2:])
+    return rows[indices], indices, cu_seqlens, int(lengths.max().item())
+
+
+def pad_input(hidden_states, indices, batch, seqlen):
+    """Inverse of unpad_input: rows [nnz, ...] back at `indices` of a zero-filled [batch, seqlen, ...].
+    Reference :53-66."""
+    out = hidden_states.new_zeros((batch * seqlen,) + tuple(hidden_states.shape[1:]))
+    out[indices] = hidden_states
+    return out.reshape(batch, seqlen, *hidden_states.shape[1:])
 
 
 from ..operators.rope_kernels import rope_backward, rope_forward  # noqa: E402,F401  (in place, HIP)

@@ -127,3 +127,21 @@ def test_key_padding_mask_helper_on_cpu():
     assert keep[:, 0, :, 0].tolist() == [[1, 1, 1, 1], [0, 1, 1, 0]]
     with pytest.raises(ValueError):
         key_padding_attention_mask(torch.ones(2, 1, 4, 4), torch.float32)
+
+
+def test_padding_helpers_round_trip():
+    """unpad_input / pad_input of the reference's compute_utils (models/utils/compute_utils.py:53-97)."""
+    from hyclora_amd.models.compute_utils import pad_input, repeat_kv, repeat_kv_backward, unpad_input
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(3, 5, 2, 4, generator=g)
+    mask = torch.tensor([[1, 1, 1, 0, 0], [1, 1, 1, 1, 1], [0, 0, 1, 1, 0]])
+    rows, indices, cu, longest = unpad_input(x, mask)
+    assert rows.shape == (10, 2, 4) and longest == 5 and cu.dtype == torch.int32 and cu.tolist() == [0, 3, 8, 10]
+    assert indices.tolist() == [0, 1, 2, 5, 6, 7, 8, 9, 12, 13]
+    back = pad_input(rows, indices, 3, 5)
+    assert torch.equal(back, x * mask[:, :, None, None])
+    # keyword names of the reference's signatures
+    h = torch.randn(2, 2, 3, 4, generator=g)
+    r = repeat_kv(hidden_states=h, n_rep=3)
+    assert r.shape == (2, 6, 3, 4) and torch.equal(r[:, 3:6], h[:, 1:2].expand(2, 3, 3, 4))
+    assert torch.allclose(repeat_kv_backward(grad_output=r, n_rep=3), 3 * h)
