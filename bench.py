@@ -843,13 +843,13 @@ def main():
             def c_both(i, st):
                 j = i % NBl
                 assert L.hyc_lora_contract(x_l[j].data_ptr(), None, None, None, 0, xa.data_ptr(), w_b.data_ptr(), 1,
-                                           p1s[i % 2].data_ptr(), p2s[i % 2].data_ptr(), wss[i % 2].data_ptr(), ws_bytes,
+                                           p1s[i % 2].data_ptr(), 0, p2s[i % 2].data_ptr(), wss[i % 2].data_ptr(), ws_bytes,
                                            T, Nw, R, st) == 0
 
             def c_codes(i, st):
                 j = i % NBl
                 assert L.hyc_lora_contract(None, q_l[j].data_ptr(), s_l.data_ptr(), None, QB, xa.data_ptr(), None, 0,
-                                           p1s[i % 2].data_ptr(), None, wss[i % 2].data_ptr(), ws_bytes, T, Nw, R, st) == 0
+                                           p1s[i % 2].data_ptr(), 0, None, wss[i % 2].data_ptr(), ws_bytes, T, Nw, R, st) == 0
 
             # the input gradients of projections that share their input, added up: three LoRA adds chained through
             # a running sum against the one-pass sum of the same three terms

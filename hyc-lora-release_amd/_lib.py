@@ -26,7 +26,7 @@ class HycError(RuntimeError):
 
 
 # name -> (restype, argtypes)
-ABI_VERSION = 10          # hyc_abi_version() of the library these signatures describe
+ABI_VERSION = 11          # hyc_abi_version() of the library these signatures describe
 _P, _I, _L = c_void_p, c_int, c_int64
 
 
@@ -86,7 +86,7 @@ _SIGNATURES = {
     "hyc_lora_silu_mul_fwd": (_I, [_P] * 11 + [_L, _L, _L, _I, _I, _P]),
     "hyc_lora_silu_mul_bwd": (_I, [_P] * 12 + [_L, _L, _L, _I, _I, _P]),
     "hyc_lora_contract_workspace": (_L, [_L, _L, _L, _I, _I]),
-    "hyc_lora_contract": (_I, [_P, _P, _P, _P, _I, _P, _P, _I, _P, _P, _P, _L, _L, _L, _L, _P]),
+    "hyc_lora_contract": (_I, [_P, _P, _P, _P, _I, _P, _P, _I, _P, _I, _P, _P, _L, _L, _L, _L, _P]),
     "hyc_lora_add": (_I, [_P, _P, _I, _P, _P, _P, _L, _L, _L, _P]),
     "hyc_lora_add_quant": (_I, [_P, _P, _I] + [_P] * 5 + [_L, _L, _L, _I, _P]),
     "hyc_lora_add_restore": (_I, [_P, _P, _I] + [_P] * 4 + [_L, _L, _L, _I, _P]),

@@ -16,7 +16,7 @@ extern "C" const char* hyc_error_string(int code) {
     }
 }
 
-extern "C" int hyc_abi_version(void) { return 10; }
+extern "C" int hyc_abi_version(void) { return 11; }
 
 extern "C" int hyc_set_tuning(const char* key, int value) {
     if (!key) return HYC_ERR_NULL;

@@ -330,7 +330,48 @@ struct ReduceJob {
     int64_t rows_out, rows_part;
     int cols_out, cols_part, planes;
     int64_t blocks;
+    int transposed;          // out is [cols_out][rows_out]: rows_out <= 64 and even, cols_out % 4 == 0
 };
+constexpr int kReduceTCols = 64;     // columns a block of the transposed form owns (all rows of them)
+
+// out[c][i] = bf16( sum_k part[k][i][c] ): the sums of kReduceTCols columns x all rows meet in LDS and leave as
+// one contiguous run of the transposed output.  Planes are added in index order, as in the plain form, so
+// the values are the plain form's.
+__device__ __forceinline__ void reduce_transposed(const ReduceJob& jb, int64_t blk) {
+    __shared__ uint16_t tile[kReduceTCols * 64];
+    const int c4 = threadIdx.x & 15, r0 = threadIdx.x >> 4;
+    const int64_t c0 = blk * kReduceTCols;
+    const int64_t c = c0 + 4 * c4;
+    const int rows = (int)jb.rows_out;
+    const int64_t plane = jb.rows_part * (int64_t)jb.cols_part;
+    if (c < jb.cols_out) {
+        for (int r = r0; r < rows; r += 16) {
+            const float* p = jb.part + (int64_t)r * jb.cols_part + c;
+            f32x4 sum = {0.0f, 0.0f, 0.0f, 0.0f};
+            int k = 0;
+            for (; k + 4 <= jb.planes; k += 4) {
+                f32x4 v[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) v[u] = *reinterpret_cast<const f32x4*>(p + (k + u) * plane);
+#pragma unroll
+                for (int u = 0; u < 4; ++u) sum += v[u];
+            }
+            for (; k < jb.planes; ++k) sum += *reinterpret_cast<const f32x4*>(p + k * plane);
+            const uint32_t lo = pk_bf16(sum.x, sum.y), hi = pk_bf16(sum.z, sum.w);
+            tile[(4 * c4 + 0) * rows + r] = (uint16_t)lo;
+            tile[(4 * c4 + 1) * rows + r] = (uint16_t)(lo >> 16);
+            tile[(4 * c4 + 2) * rows + r] = (uint16_t)hi;
+            tile[(4 * c4 + 3) * rows + r] = (uint16_t)(hi >> 16);
+        }
+    }
+    __syncthreads();
+    const int64_t cols_here = jb.cols_out - c0 < kReduceTCols ? jb.cols_out - c0 : kReduceTCols;
+    const int n_pairs = (int)(cols_here * rows / 2);
+    uint32_t* out = reinterpret_cast<uint32_t*>(jb.out + c0 * rows);
+    const uint32_t* src = reinterpret_cast<const uint32_t*>(tile);
+    for (int i = threadIdx.x; i < n_pairs; i += 256) out[i] = src[i];
+}
+
 // A thread owns W neighbouring outputs of one row (cols_out % W == 0) and reads one W-wide vector
 // per plane; planes are added in index order.
 template <int W>
@@ -339,6 +380,10 @@ __global__ __launch_bounds__(256) void contract_reduce_kernel(const ReduceJob j0
     const bool second = (int64_t)blockIdx.x >= j0.blocks;
     const ReduceJob& jb = second ? j1 : j0;
     const int64_t blk = second ? blockIdx.x - j0.blocks : blockIdx.x;
+    if (jb.transposed) {                  // the same for every thread of the block
+        reduce_transposed(jb, blk);
+        return;
+    }
     const int64_t n_out = jb.rows_out * jb.cols_out;
     const int64_t idx = (blk * 256 + threadIdx.x) * W;
     if (idx >= n_out) return;
@@ -417,7 +462,7 @@ extern "C" int64_t hyc_lora_contract_workspace(int64_t T, int64_t N, int64_t R, 
 }
 
 extern "C" int hyc_lora_contract(const void* x, const void* q, const void* scale, const void* zero_point, int q_bit,
-                                 const void* u, const void* v, int v_transposed, void* p1, void* p2,
+                                 const void* u, const void* v, int v_transposed, void* p1, int p1_transposed, void* p2,
                                  void* workspace, int64_t workspace_bytes, int64_t T, int64_t N, int64_t R,
                                  void* stream) {
     const bool codes = q != nullptr;
@@ -477,6 +522,10 @@ extern "C" int hyc_lora_contract(const void* x, const void* q, const void* scale
         j1.part = a.part1; j1.out = (uint16_t*)p1; j1.rows_out = R; j1.rows_part = 16 * nb;
         j1.cols_out = (int)N; j1.cols_part = (int)N; j1.planes = (int)strips;
         j1.blocks = cdiv(R * N, 256 * w);
+        if (p1_transposed) {
+            j1.transposed = 1;
+            j1.blocks = cdiv(N, kReduceTCols);
+        }
     }
     if (want2) {
         j2.part = a.part2; j2.out = (uint16_t*)p2; j2.rows_out = T; j2.rows_part = T;

@@ -98,7 +98,10 @@ def lora_backward(w, w_quant_state, w_lora_a, w_lora_b, x, x_lora_a, grad_y, x_c
     w_lora_a, w_lora_b = w_lora_a.to(dt), w_lora_b.to(dt)
     r = w_lora_b.shape[0]
     if lora_kernels.contract_supported(grad_y, grad_y.shape[-1], r) and x_lora_a.dtype == dt:
-        grad_b, grad_mid = lora_kernels.lora_products(grad_y, u=x_lora_a, v=w_lora_b)
+        # xa^T @ grad_y written as [N, R], the layout of the lora_B weight this gradient ends up in: what is
+        # returned is its [R, N] view, and autograd's transpose back is then contiguous and stored without a copy
+        grad_b, grad_mid = lora_kernels.lora_products(grad_y, u=x_lora_a, v=w_lora_b, p1_transposed=True)
+        grad_b = grad_b.t()
     else:
         grad_mid = grad_y @ w_lora_b.mT
         grad_b = x_lora_a.to(dt).mT @ grad_y

@@ -546,7 +546,8 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             r = lb.shape[0]
             fast = lora_kernels.contract_supported(g, g.shape[-1], r) and S["down_lora_a"].dtype == g.dtype
             if fast:                      # both rank-R products of grad_output from one pass over it
-                grad_b_down, grad_mid = lora_kernels.lora_products(g, u=S["down_lora_a"], v=lb)
+                grad_b_down, grad_mid = lora_kernels.lora_products(g, u=S["down_lora_a"], v=lb, p1_transposed=True)
+                grad_b_down = grad_b_down.t()         # [R, N] view of the [N, R] result, as in lora_backward
             else:
                 grad_b_down = S["down_lora_a"].to(wd.dtype).mT @ g
                 grad_mid = g @ lb.mT

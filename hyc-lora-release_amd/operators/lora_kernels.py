@@ -316,7 +316,7 @@ def contract_supported(x, n, r):
     return x.is_cuda and x.dtype == BF16 and n % 32 == 0 and 2 <= r <= 64 and r % 2 == 0 and x.numel() > 0
 
 
-def _contract(x, codes, u, v, T, n, r, dev):
+def _contract(x, codes, u, v, T, n, r, dev, p1_transposed=False):
     want1, want2 = u is not None, v is not None
     vt = 0
     if want1:
@@ -329,18 +329,19 @@ def _contract(x, codes, u, v, T, n, r, dev):
         v, vt = _lora_b(v)
     nbytes = _lib.lib().hyc_lora_contract_workspace(T, n, r, int(want1), int(want2))
     ws = torch.empty(max(nbytes, 16), device=dev, dtype=torch.uint8)
-    p1 = torch.empty((r, n), device=dev, dtype=BF16) if want1 else None
+    p1 = torch.empty((n, r) if p1_transposed else (r, n), device=dev, dtype=BF16) if want1 else None
     p2 = torch.empty((T, r), device=dev, dtype=BF16) if want2 else None
     q, s, z, bits = codes if codes is not None else (None, None, None, 0)
     _lib.call("hyc_lora_contract", _lib.ptr(x), _lib.ptr(q), _lib.ptr(s), _lib.ptr(z), bits, _lib.ptr(u), _lib.ptr(v), vt,
-              _lib.ptr(p1), _lib.ptr(p2), ws.data_ptr(), ws.numel(), T, n, r, _lib.stream_of(ws))
+              _lib.ptr(p1), int(p1_transposed), _lib.ptr(p2), ws.data_ptr(), ws.numel(), T, n, r, _lib.stream_of(ws))
     return p1, p2
 
 
-def lora_products(x, u=None, v=None):
+def lora_products(x, u=None, v=None, p1_transposed=False):
     """x [..., N] bf16 read once -> (u^T x as [R, N] or None, x v^T as [..., R] or None), u [..., R], v [R, N]
     (a `weight.T` view of an [N, R] weight is read in place).  fp32 accumulation over the whole
-    contraction, one bf16 rounding."""
+    contraction, one bf16 rounding.  p1_transposed: the first result comes as x^T u, [N, R] contiguous - the
+    layout of a lora_B weight, so that its gradient needs no copy on the way into `.grad`."""
     if u is None and v is None:
         raise ValueError("nothing to compute: pass u, v or both")
     n = x.shape[-1]
@@ -355,7 +356,7 @@ def lora_products(x, u=None, v=None):
     lead = tuple(x.shape[:-1])
     x = _prep(x, "x")
     T = x.numel() // n
-    p1, p2 = _contract(x, None, u, v, T, n, r, x.device)
+    p1, p2 = _contract(x, None, u, v, T, n, r, x.device, p1_transposed)
     return p1, (p2.reshape(*lead, r) if p2 is not None else None)
 
 

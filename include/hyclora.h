@@ -583,7 +583,8 @@ int hyc_lora_add_restore_group(const hyc_lora_add_member *members, int count, in
  *     p2 = bf16( X . V^T )   [T, R]      V bf16 [R, N] (v_transposed 0) or [N, R] (v_transposed 1)
  * X is dense bf16 [T, N] (x), or - p1 only - the packed codes of hyc_quant_pack (q, scale,
  * optional zero_point, q_bit; x NULL), dequantised in registers to the value hyc_unpack_dequant
- * gives.  Pass p1 or p2 as NULL to skip that product.
+ * gives.  Pass p1 or p2 as NULL to skip that product.  With p1_transposed, p1 is written as [N, R] - the
+ * memory layout of a lora_B weight, whose gradient xa^T @ grad_y is (the same values, transposed).
  *
  * Replaces the rank-R GEMMs of lora_forward / lora_backward (models/utils/compute_utils.py:22,
  * :30-33): x @ A (p2, V = lora_A.weight), grad_y @ B^T with xa^T @ grad_y (p2 and p1 of X = grad_y),
@@ -599,7 +600,7 @@ int hyc_lora_add_restore_group(const hyc_lora_add_member *members, int count, in
  */
 int64_t hyc_lora_contract_workspace(int64_t T, int64_t N, int64_t R, int want_p1, int want_p2);
 int hyc_lora_contract(const void *x, const void *q, const void *scale, const void *zero_point, int q_bit,
-                      const void *u, const void *v, int v_transposed, void *p1, void *p2,
+                      const void *u, const void *v, int v_transposed, void *p1, int p1_transposed, void *p2,
                       void *workspace, int64_t workspace_bytes, int64_t T, int64_t N, int64_t R,
                       void *stream);
 

@@ -61,6 +61,12 @@ def test_both_products_from_one_pass(K, dev, lead, N, R):
     vt = d(v).t().contiguous().t()
     b1, b2 = K.products(d(x), d(u), vt)
     assert np.array_equal(bits(b1), bits(p1)) and np.array_equal(bits(b2), bits(p2))
+    # the first product in the layout of a lora_B weight, [N, R]: the same values transposed
+    t1, t2 = K.products(d(x), d(u), d(v), p1_transposed=True)
+    assert t1.shape == (N, R) and t1.is_contiguous()
+    assert torch.equal(t1.t(), p1) and np.array_equal(bits(t2), bits(p2))
+    t1_alone, _ = K.products(d(x), u=d(u), p1_transposed=True)
+    assert torch.equal(t1_alone, t1)
 
 
 @pytest.mark.parametrize("q_bit", [2, 4, 8])
@@ -105,3 +111,23 @@ def test_argument_checks(K, dev):
         K.products(d(x), None, d(v)[:, :32])
     with pytest.raises(RuntimeError):
         K.products(x, u, v)
+
+
+def test_lora_b_gradient_arrives_in_the_weights_layout(dev):
+    """lora_backward returns grad lora_B as the [R, N] view of an [N, R] tensor: autograd's transpose on the way to
+    the `weight.T` leaf is then contiguous and `.grad` takes it without the copy a strided gradient costs."""
+    import hyclora_amd  # noqa: F401
+    from hyclora_amd.models.compute_utils import lora_backward
+    g = torch.Generator().manual_seed(3)
+    T, n_in, n_out, r = 64, 256, 384, 16
+    w = torch.randn(n_out, n_in, generator=g).to(BF16).to(dev)
+    la = torch.randn(r, n_in, generator=g).to(BF16).to(dev)
+    lb = torch.randn(n_out, r, generator=g).to(BF16).to(dev)
+    x = torch.randn(1, T, n_in, generator=g).to(BF16).to(dev)
+    gy = torch.randn(1, T, n_out, generator=g).to(BF16).to(dev)
+    xa = x @ la.t()
+    grad_a, grad_b, grad_x = lora_backward(w, None, la.t(), lb.t(), x, xa, gy)
+    assert grad_b.shape == (r, n_out) and grad_b.t().is_contiguous()
+    assert grad_a.shape == (n_in, r) and grad_a.t().is_contiguous()
+    want_b = (xa.float().reshape(T, r).t() @ gy.float().reshape(T, n_out))
+    assert_close_bf16(grad_b.cpu(), want_b.to(BF16).cpu(), what="grad lora_B")
