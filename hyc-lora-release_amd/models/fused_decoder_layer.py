@@ -352,7 +352,7 @@ class FusedDecoderLayerFunc(torch.autograd.Function):
             ctx.flash = None
             query_keep = ctx.key_padding = None
             if attention_mask is not None and attention_mask.dim() == 2:      # the reference's key-padding mask
-                key_padding = attention_mask
+                key_padding = attention_mask if attention_mask.device == q.device else attention_mask.to(q.device)
                 attention_mask, query_keep = key_padding_attention_mask(key_padding, q.dtype)
                 if query_keep is not None:
                     ctx.key_padding = key_padding      # backward builds the [B, 1, S, S] mask again instead of keeping it
