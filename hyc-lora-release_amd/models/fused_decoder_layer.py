@@ -794,3 +794,25 @@ class FusedDecoderLayer(torch.nn.Module):
                 self.static_value[key] = update_dict(self.static_value[key], fields, self.iteration)
         self.iteration += 1
         return y
+
+
+def call_from_decoder_layer(fused_layer, decoder_layer, hidden_states, attention_mask, cos, sin, num_key_value_heads=None):
+    """The call the reference's decoder layers make while training (models/llama/modeling_llama.py:745-786,
+    models/mistral/modeling_mistral.py:611-646): hands the fused layer the norm weights and, for each of the seven
+    projections, the frozen `base_layer` and the `lora_A` / `lora_B` containers of a PEFT-wrapped linear, taken
+    from a decoder layer with the stock attribute names (`input_layernorm`, `self_attn.{q,k,v,o}_proj`,
+    `post_attention_layernorm`, `mlp.{gate,up,down}_proj`).  Head counts come from the layer's attention config."""
+    attn, mlp = decoder_layer.self_attn, decoder_layer.mlp
+    cfg = getattr(attn, "config", None)
+    num_heads = getattr(attn, "num_heads", None) or getattr(attn, "num_attention_heads", None) or cfg.num_attention_heads
+    head_dim = getattr(attn, "head_dim", None) or cfg.hidden_size // num_heads
+    if num_key_value_heads is None:
+        num_key_value_heads = getattr(attn, "num_key_value_heads", None) or getattr(cfg, "num_key_value_heads", num_heads)
+
+    def parts(linear):
+        return linear.base_layer, linear.lora_A, linear.lora_B
+    return fused_layer(hidden_states, decoder_layer.input_layernorm.weight, None, cos, sin,
+                       *parts(attn.q_proj), *parts(attn.k_proj), *parts(attn.v_proj), *parts(attn.o_proj),
+                       decoder_layer.post_attention_layernorm.weight, None,
+                       *parts(mlp.gate_proj), *parts(mlp.up_proj), *parts(mlp.down_proj),
+                       attention_mask, num_heads, head_dim, num_key_value_heads)

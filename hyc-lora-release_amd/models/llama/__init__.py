@@ -1,6 +1,6 @@
 """Llama decoder layers with compressed saved activations; class names as in the reference
 (models/llama/fused_llama_layer_{baseline,intra,intra_inter,intra_inter_full_fuse}.py)."""
-from ..fused_decoder_layer import FusedDecoderLayer
+from ..fused_decoder_layer import FusedDecoderLayer, call_from_decoder_layer
 
 
 class FusedLlamaLayerBaseline(FusedDecoderLayer):
@@ -48,3 +48,10 @@ def set_fused_llama_layer(model, hyclora_config):
     model.hyclora_config = hyclora_config
     for layer in model.model.layers:
         layer.fused_llama_layer = make_fused_llama_layer(hyclora_config)
+
+
+def decoder_layer_forward(decoder_layer, hidden_states, attention_mask, cos, sin):
+    """What the reference's decoder layer does in training mode (models/llama/modeling_llama.py:745-786): one call of the layer's
+    `fused_llama_layer` with the layer's own weights.  `decoder_layer` is a decoder layer with the stock attribute names
+    whose linears are PEFT-style LoRA wrappers (`base_layer`, `lora_A`, `lora_B`)."""
+    return call_from_decoder_layer(decoder_layer.fused_llama_layer, decoder_layer, hidden_states, attention_mask, cos, sin)

@@ -4,7 +4,7 @@ with a zero point, norm weights receive gradients
 of the reference are replaced by the flash kernels behind torch's scaled_dot_product_attention, called
 through their aten entry points: forward returns the log-sum-exps, backward takes them and the
 dequantised attention output, as the reference's call does (…intra_inter.py:450-468)."""
-from ..fused_decoder_layer import FusedDecoderLayer
+from ..fused_decoder_layer import FusedDecoderLayer, call_from_decoder_layer
 
 
 class FusedLlamaLayerBaseline(FusedDecoderLayer):
@@ -54,3 +54,10 @@ def set_fused_llama_layer(model, hyclora_config):
     model.hyclora_config = hyclora_config
     for layer in model.model.layers:
         layer.fused_llama_layer = make_fused_llama_layer(hyclora_config)
+
+
+def decoder_layer_forward(decoder_layer, hidden_states, attention_mask, cos, sin):
+    """What the reference's decoder layer does in training mode (models/llama_flash_attn/modeling_llama.py:610-654): one call of the layer's
+    `fused_llama_layer` with the layer's own weights.  `decoder_layer` is a decoder layer with the stock attribute names
+    whose linears are PEFT-style LoRA wrappers (`base_layer`, `lora_A`, `lora_B`)."""
+    return call_from_decoder_layer(decoder_layer.fused_llama_layer, decoder_layer, hidden_states, attention_mask, cos, sin)

@@ -2,7 +2,7 @@
 the reference (models/mistral/fused_mistral_layer_*.py).  The computation is the generic layer: the
 reference's Mistral files differ from the Llama ones only in always calling repeat_kv and in a dtype
 cast of lora_B (fused_mistral_layer_intra_inter_full_fuse.py:226-227), both covered there."""
-from ..fused_decoder_layer import FusedDecoderLayer
+from ..fused_decoder_layer import FusedDecoderLayer, call_from_decoder_layer
 
 
 class FusedMistralLayerBaseline(FusedDecoderLayer):
@@ -47,3 +47,10 @@ def set_fused_mistral_layer(model, hyclora_config):
     model.hyclora_config = hyclora_config
     for layer in model.model.layers:
         layer.fused_mistral_layer = make_fused_mistral_layer(hyclora_config)
+
+
+def decoder_layer_forward(decoder_layer, hidden_states, attention_mask, cos, sin):
+    """What the reference's decoder layer does in training mode (models/mistral/modeling_mistral.py:611-646): one call of the layer's
+    `fused_mistral_layer` with the layer's own weights.  `decoder_layer` is a decoder layer with the stock attribute names
+    whose linears are PEFT-style LoRA wrappers (`base_layer`, `lora_A`, `lora_B`)."""
+    return call_from_decoder_layer(decoder_layer.fused_mistral_layer, decoder_layer, hidden_states, attention_mask, cos, sin)

@@ -1,0 +1,116 @@
+"""The fused layers inside stock transformers models: every decoder layer of a small random LlamaForCausalLM /
+MistralForCausalLM (eager attention, PEFT-style LoRA wrappers around its seven linears) runs through
+`decoder_layer_forward` - the call the reference's model files make (models/llama/modeling_llama.py:745-786) -
+and logits, loss and adapter gradients are compared with the stock model's own forward and autograd.  That is an
+independent statement of the layer (transformers' RMSNorm, rotary embedding, grouped-query attention and MLP), not
+this repository's."""
+import types
+
+import pytest
+import torch
+
+from helpers import BF16, rel_err_and_cos
+from test_gpu_layers import RefRMSNorm, config
+
+pytestmark = pytest.mark.gpu
+transformers = pytest.importorskip("transformers")
+
+WIRING_FLOOR = {8: 0.9, 4: 0.8}      # cosine of a compressed layer's adapter gradients against uncompressed autograd
+
+
+class LoraLinear(torch.nn.Module):
+    """A linear wrapped the way PEFT wraps it: `base_layer`, `lora_A` / `lora_B` as ModuleDicts keyed by adapter name."""
+
+    def __init__(self, base, rank, gen):
+        super().__init__()
+        self.base_layer = base
+        base.weight.requires_grad_(False)
+        dev = base.weight.device
+        a = torch.nn.Linear(base.in_features, rank, bias=False, device=dev, dtype=BF16)
+        b = torch.nn.Linear(rank, base.out_features, bias=False, device=dev, dtype=BF16)
+        with torch.no_grad():
+            a.weight.copy_(torch.randn(a.weight.shape, generator=gen, device=dev) / base.in_features ** 0.5)
+            b.weight.copy_(torch.randn(b.weight.shape, generator=gen, device=dev) * 0.05)
+        self.lora_A = torch.nn.ModuleDict({"default": a})
+        self.lora_B = torch.nn.ModuleDict({"default": b})
+
+    def forward(self, x):
+        return self.base_layer(x) + self.lora_B["default"](self.lora_A["default"](x))
+
+
+def build(dev, family, head_dim):
+    heads, kv = 4, (4 if family == "llama" else 2)
+    common = dict(vocab_size=128, hidden_size=heads * head_dim, intermediate_size=768, num_hidden_layers=2,
+                  num_attention_heads=heads, num_key_value_heads=kv, max_position_embeddings=256, rms_norm_eps=1e-5,
+                  attn_implementation="eager")
+    torch.manual_seed(5)
+    if family == "llama":
+        model = transformers.LlamaForCausalLM(transformers.LlamaConfig(**common))
+    else:
+        model = transformers.MistralForCausalLM(transformers.MistralConfig(sliding_window=None, **common))
+    model = model.to(device=dev, dtype=BF16)
+    gen = torch.Generator(device=dev).manual_seed(9)
+    for p in model.parameters():
+        p.requires_grad_(False)
+    for layer in model.model.layers:
+        for parent, names in ((layer.self_attn, ("q_proj", "k_proj", "v_proj", "o_proj")),
+                              (layer.mlp, ("gate_proj", "up_proj", "down_proj"))):
+            for n in names:
+                setattr(parent, n, LoraLinear(getattr(parent, n), 16, gen))
+    model.train()
+    return model
+
+
+def loss_and_grads(model, ids):
+    for p in model.parameters():
+        p.grad = None
+    out = model(input_ids=ids, labels=ids, use_cache=False)
+    out.loss.backward()
+    grads = {n: p.grad.clone() for n, p in model.named_parameters() if p.requires_grad}
+    return out.logits.detach().clone(), out.loss.item(), grads
+
+
+@pytest.mark.parametrize("family, head_dim", [("llama", 64), ("llama", 128), ("mistral", 128)])
+@pytest.mark.parametrize("layer_type, q_bit", [("baseline", 0), ("intra_inter_full_fuse", 8), ("intra_inter", 4)])
+def test_stock_model_through_the_fused_layers(dev, family, head_dim, layer_type, q_bit):
+    import hyclora_amd  # noqa: F401
+    from hyclora_amd.models import llama, mistral
+    pkg = llama if family == "llama" else mistral
+    model = build(dev, family, head_dim)
+    ids = torch.randint(0, 128, (2, 256), generator=torch.Generator().manual_seed(1)).to(dev)
+    # The stock layers and autograd - with one exception: the decoder layers' two norms take the reference's
+    # RMSNorm backward (rmsnorm_kernels.py:92-100, whose mean term is not part of a true RMSNorm's derivative and
+    # which the fused layers reproduce), so that the comparison is about everything else.
+    for layer in model.model.layers:
+        for norm in (layer.input_layernorm, layer.post_attention_layernorm):
+            norm.forward = types.MethodType(lambda self, x: RefRMSNorm.apply(x, self.weight), norm)
+    ref_logits, ref_loss, ref_grads = loss_and_grads(model, ids)
+
+    switch = llama.set_fused_llama_layer if family == "llama" else mistral.set_fused_mistral_layer
+    switch(model, config(layer_type, q_bit, sm_ratio=0.999, thr=5) if q_bit else
+           types.SimpleNamespace(use_hyclora=True, layer_type="baseline"))
+
+    def forward(self, hidden_states, attention_mask=None, position_embeddings=None, **_):
+        cos, sin = position_embeddings
+        return pkg.decoder_layer_forward(self, hidden_states, attention_mask, cos, sin)
+    for layer in model.model.layers:
+        layer.forward = types.MethodType(forward, layer)
+    logits, loss, grads = loss_and_grads(model, ids)
+
+    rel, cos = rel_err_and_cos(logits, ref_logits)
+    assert rel <= 2e-2 and cos >= 0.9999, f"logits: rel {rel:.2e} cos {cos:.6f}"       # two layers of bf16 rounding
+    assert abs(loss - ref_loss) <= 1e-2 * abs(ref_loss)
+    assert set(grads) == set(ref_grads) and len(grads) == 2 * 7 * 2
+    worst = (0.0, 1.0, "")
+    for name in sorted(grads):
+        rel, cos = rel_err_and_cos(grads[name], ref_grads[name])
+        if cos < worst[1]:
+            worst = (rel, cos, name)
+        if layer_type == "baseline":
+            assert rel <= 3e-2 and cos >= 0.999, f"{family} d{head_dim} baseline {name}: rel {rel:.2e} cos {cos:.6f}"
+        else:
+            # the scheme's own quantisation error on a 512-token batch whose steps come from batch element 0 of this
+            # very step; a mis-wired projection would give a cosine near zero
+            assert cos >= WIRING_FLOOR[q_bit], f"{family} d{head_dim} {layer_type} q{q_bit} {name}: rel {rel:.2e} cos {cos:.5f}"
+    print(f"{family} d{head_dim} {layer_type} q{q_bit}: logits rel {rel_err_and_cos(logits, ref_logits)[0]:.2e}, "
+          f"worst gradient {worst[2]}: rel {worst[0]:.2e} cos {worst[1]:.5f}")
