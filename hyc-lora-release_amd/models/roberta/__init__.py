@@ -438,3 +438,21 @@ def set_fused_roberta_layer(model, hyclora_config):
     model.hyclora_config = hyclora_config
     for layer in model.roberta.encoder.layer:
         layer.fused_roberta_layer = make_fused_roberta_layer(hyclora_config)
+
+
+def encoder_layer_forward(encoder_layer, hidden_states, attention_mask):
+    """What the reference's encoder layer does in training mode (models/roberta/modeling_roberta.py:428-457): one call
+    of the layer's `fused_roberta_layer` with the layer's own weights.  `encoder_layer` is an encoder layer with the
+    stock attribute names (`attention.self.{query,key,value}`, `attention.output.{dense,LayerNorm}`,
+    `intermediate.dense`, `output.{dense,LayerNorm}`) whose linears are PEFT-style LoRA wrappers
+    (`base_layer`, `lora_A`, `lora_B`)."""
+    att, out = encoder_layer.attention, encoder_layer.output
+    heads = att.self.num_attention_heads
+
+    def parts(linear):
+        return linear.base_layer, linear.lora_A, linear.lora_B
+    return encoder_layer.fused_roberta_layer(
+        hidden_states, *parts(att.self.query), *parts(att.self.key), *parts(att.self.value), *parts(att.output.dense),
+        att.output.LayerNorm.weight, att.output.LayerNorm.bias,
+        *parts(encoder_layer.intermediate.dense), *parts(out.dense), out.LayerNorm.weight, out.LayerNorm.bias,
+        attention_mask, heads, hidden_states.shape[-1] // heads)

@@ -114,3 +114,71 @@ def test_stock_model_through_the_fused_layers(dev, family, head_dim, layer_type,
             assert cos >= WIRING_FLOOR[q_bit], f"{family} d{head_dim} {layer_type} q{q_bit} {name}: rel {rel:.2e} cos {cos:.5f}"
     print(f"{family} d{head_dim} {layer_type} q{q_bit}: logits rel {rel_err_and_cos(logits, ref_logits)[0]:.2e}, "
           f"worst gradient {worst[2]}: rel {worst[0]:.2e} cos {worst[1]:.5f}")
+
+
+@pytest.mark.parametrize("layer_type, q_bit", [("baseline", 0), ("intra_inter", 8), ("intra", 4)])
+@pytest.mark.parametrize("padding", [False, True])
+def test_stock_roberta_through_the_fused_layers(dev, layer_type, q_bit, padding):
+    """The encoder layers the same way: a two-layer random RobertaForSequenceClassification (no dropout) whose
+    layers call `encoder_layer_forward` (models/roberta/modeling_roberta.py:428-457) against the stock forward
+    and autograd - transformers' attention, exact GELU and LayerNorm (the fused layer's GELU backward is the
+    reference's tanh form, gelu_kernels.py:49-56)."""
+    import hyclora_amd  # noqa: F401
+    from hyclora_amd.models import roberta
+    torch.manual_seed(6)
+    cfg = transformers.RobertaConfig(vocab_size=128, hidden_size=256, intermediate_size=768, num_hidden_layers=2,
+                                     num_attention_heads=4, max_position_embeddings=260, attn_implementation="eager",
+                                     hidden_dropout_prob=0.0, attention_probs_dropout_prob=0.0, num_labels=3)
+    model = transformers.RobertaForSequenceClassification(cfg).to(device=dev, dtype=BF16)
+    gen = torch.Generator(device=dev).manual_seed(4)
+    for p in model.parameters():
+        p.requires_grad_(False)
+    for layer in model.roberta.encoder.layer:
+        for parent, names in ((layer.attention.self, ("query", "key", "value")), (layer.attention.output, ("dense",)),
+                              (layer.intermediate, ("dense",)), (layer.output, ("dense",))):
+            for n in names:
+                setattr(parent, n, LoraLinear(getattr(parent, n), 16, gen))
+    model.train()
+    ids = torch.randint(3, 128, (4, 256), generator=torch.Generator().manual_seed(2)).to(dev)
+    mask = torch.ones(4, 256, dtype=torch.long, device=dev)
+    if padding:
+        mask[1, 200:] = 0
+        mask[3, 97:] = 0
+    labels = torch.tensor([0, 2, 1, 1], device=dev)
+
+    def run():
+        for p in model.parameters():
+            p.grad = None
+        out = model(input_ids=ids, attention_mask=mask, labels=labels)
+        out.loss.backward()
+        return out.logits.detach().clone(), out.loss.item(), {n: p.grad.clone() for n, p in model.named_parameters() if p.requires_grad}
+    ref_logits, ref_loss, ref_grads = run()
+    roberta.set_fused_roberta_layer(model, config(layer_type, q_bit, sm_ratio=0.999, thr=5) if q_bit else
+                                    types.SimpleNamespace(use_hyclora=True, layer_type="baseline"))
+
+    def forward(self, hidden_states, attention_mask=None, *args, **kwargs):
+        return roberta.encoder_layer_forward(self, hidden_states, attention_mask)
+    for layer in model.roberta.encoder.layer:
+        layer.forward = types.MethodType(forward, layer)
+    logits, loss, grads = run()
+    rel, cos = rel_err_and_cos(logits, ref_logits)
+    assert rel <= 2e-2 and cos >= 0.9999, f"logits: rel {rel:.2e} cos {cos:.6f}"
+    assert abs(loss - ref_loss) <= 1e-2 * abs(ref_loss)
+    assert set(grads) == set(ref_grads) and len(grads) == 2 * 6 * 2
+    worst = (0.0, 1.0, "")
+    for name in sorted(grads):
+        rel, cos = rel_err_and_cos(grads[name], ref_grads[name])
+        if cos < worst[1]:
+            worst = (rel, cos, name)
+        if layer_type == "baseline":
+            assert rel <= 3e-2 and cos >= 0.999, f"roberta baseline {name}: rel {rel:.2e} cos {cos:.6f}"
+        elif ".attention.output.dense.lora_A" in name:
+            # formed from the restored attention output.  Without a causal mask a randomly initialised model's
+            # attention is nearly uniform, every token's output is close to the mean of v, and the reference's
+            # symmetric codes (step = (max - min) / 255, no zero point) clip a channel whose mean is far outside
+            # its own range: the scheme's error, the same at 8 and at 4 bits.
+            assert cos >= 0.5, f"roberta {layer_type} q{q_bit} {name}: rel {rel:.2e} cos {cos:.5f}"
+        else:
+            assert cos >= WIRING_FLOOR[q_bit], f"roberta {layer_type} q{q_bit} {name}: rel {rel:.2e} cos {cos:.5f}"
+    print(f"roberta {layer_type} q{q_bit} padding={padding}: logits rel {rel_err_and_cos(logits, ref_logits)[0]:.2e}, "
+          f"worst gradient {worst[2]}: rel {worst[0]:.2e} cos {worst[1]:.5f}")
