@@ -796,6 +796,17 @@ class FusedDecoderLayer(torch.nn.Module):
         return y
 
 
+def lora_linear_parts(linear):
+    """(base_layer, lora_A, lora_B) of a PEFT-style LoRA linear.  The layers compute `x @ W^T + (x @ A^T) @ B^T`
+    without a scaling factor, like the reference, whose scripts refuse lora_alpha != rank (run_gsm8k.py:373-374):
+    a wrapper that carries another scaling is refused here."""
+    scaling = getattr(linear, "scaling", None)
+    values = list(scaling.values()) if isinstance(scaling, dict) else ([] if scaling is None else [scaling])
+    if any(float(v) != 1.0 for v in values):
+        raise ValueError(f"LoRA scaling {values} is not supported: the fused layers apply none (lora_alpha must equal the rank)")
+    return linear.base_layer, linear.lora_A, linear.lora_B
+
+
 def call_from_decoder_layer(fused_layer, decoder_layer, hidden_states, attention_mask, cos, sin, num_key_value_heads=None):
     """The call the reference's decoder layers make while training (models/llama/modeling_llama.py:745-786,
     models/mistral/modeling_mistral.py:611-646): hands the fused layer the norm weights and, for each of the seven
@@ -810,7 +821,7 @@ def call_from_decoder_layer(fused_layer, decoder_layer, hidden_states, attention
         num_key_value_heads = getattr(attn, "num_key_value_heads", None) or getattr(cfg, "num_key_value_heads", num_heads)
 
     def parts(linear):
-        return linear.base_layer, linear.lora_A, linear.lora_B
+        return lora_linear_parts(linear)
     return fused_layer(hidden_states, decoder_layer.input_layernorm.weight, None, cos, sin,
                        *parts(attn.q_proj), *parts(attn.k_proj), *parts(attn.v_proj), *parts(attn.o_proj),
                        decoder_layer.post_attention_layernorm.weight, None,

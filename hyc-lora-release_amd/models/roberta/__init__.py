@@ -25,7 +25,7 @@ from ...operators.softmax_kernels import softmax_backward, softmax_backward_from
 from ...operators import lora_kernels
 from ..compute_utils import (head_to_hidden_shape, heads_matmul, hidden_to_head_shape, lora_backward, lora_forward, lora_input_sum,
                             lora_parts)
-from ..fused_decoder_layer import _note_map_entries
+from ..fused_decoder_layer import _note_map_entries, lora_linear_parts
 
 MODES = ("baseline", "intra", "intra_inter")
 _PROJ = ("q", "k", "v", "o", "up", "down")
@@ -450,7 +450,7 @@ def encoder_layer_forward(encoder_layer, hidden_states, attention_mask):
     heads = att.self.num_attention_heads
 
     def parts(linear):
-        return linear.base_layer, linear.lora_A, linear.lora_B
+        return lora_linear_parts(linear)
     return encoder_layer.fused_roberta_layer(
         hidden_states, *parts(att.self.query), *parts(att.self.key), *parts(att.self.value), *parts(att.output.dense),
         att.output.LayerNorm.weight, att.output.LayerNorm.bias,

@@ -145,3 +145,15 @@ def test_padding_helpers_round_trip():
     r = repeat_kv(hidden_states=h, n_rep=3)
     assert r.shape == (2, 6, 3, 4) and torch.equal(r[:, 3:6], h[:, 1:2].expand(2, 3, 3, 4))
     assert torch.allclose(repeat_kv_backward(grad_output=r, n_rep=3), 3 * h)
+
+
+def test_lora_scaling_other_than_one_is_refused():
+    """The fused layers apply no LoRA scaling, like the reference (run_gsm8k.py:373-374 refuses lora_alpha != rank)."""
+    from hyclora_amd.models.fused_decoder_layer import lora_linear_parts
+    lin = SimpleNamespace(base_layer=1, lora_A=2, lora_B=3)
+    assert lora_linear_parts(lin) == (1, 2, 3)
+    lin.scaling = {"default": 1.0}
+    assert lora_linear_parts(lin) == (1, 2, 3)
+    lin.scaling = {"default": 2.0}
+    with pytest.raises(ValueError):
+        lora_linear_parts(lin)
