@@ -193,3 +193,67 @@ def test_stock_roberta_through_the_fused_layers(dev, layer_type, q_bit, padding)
             assert cos >= WIRING_FLOOR[q_bit], f"roberta {layer_type} q{q_bit} {name}: rel {rel:.2e} cos {cos:.5f}"
     print(f"roberta {layer_type} q{q_bit} padding={padding}: logits rel {rel_err_and_cos(logits, ref_logits)[0]:.2e}, "
           f"worst gradient {worst[2]}: rel {worst[0]:.2e} cos {worst[1]:.5f}")
+
+
+@pytest.mark.parametrize("family", ["llama", "mistral", "roberta"])
+def test_install_routes_training_steps_through_the_fused_layers(dev, family):
+    """`hyclora_amd.models.hf.install` on a stock model: training-mode steps run the fused layers (the calibration
+    counter of every layer advances, gradients agree with the stock model's), evaluation runs the stock layers
+    (bit-identical outputs), as the reference's model files do (modeling_llama.py:745, :788-790)."""
+    import hyclora_amd  # noqa: F401
+    from hyclora_amd.models import hf
+    if family == "roberta":
+        torch.manual_seed(6)
+        cfg = transformers.RobertaConfig(vocab_size=128, hidden_size=256, intermediate_size=768, num_hidden_layers=2,
+                                         num_attention_heads=4, max_position_embeddings=260, attn_implementation="eager",
+                                         hidden_dropout_prob=0.0, attention_probs_dropout_prob=0.0, num_labels=3)
+        model = transformers.RobertaForSequenceClassification(cfg).to(device=dev, dtype=BF16)
+        gen = torch.Generator(device=dev).manual_seed(4)
+        for p in model.parameters():
+            p.requires_grad_(False)
+        layers = model.roberta.encoder.layer
+        for layer in layers:
+            for parent, names in ((layer.attention.self, ("query", "key", "value")), (layer.attention.output, ("dense",)),
+                                  (layer.intermediate, ("dense",)), (layer.output, ("dense",))):
+                for n in names:
+                    setattr(parent, n, LoraLinear(getattr(parent, n), 16, gen))
+        ids = torch.randint(3, 128, (2, 128), generator=torch.Generator().manual_seed(2)).to(dev)
+        call = lambda: model(input_ids=ids, labels=torch.tensor([0, 2], device=dev))
+        attr = "fused_roberta_layer"
+    else:
+        model = build(dev, family, 128)
+        layers = model.model.layers
+        ids = torch.randint(0, 128, (2, 128), generator=torch.Generator().manual_seed(1)).to(dev)
+        call = lambda: model(input_ids=ids, labels=ids, use_cache=False)
+        attr = "fused_llama_layer" if family == "llama" else "fused_mistral_layer"
+        for layer in layers:                     # the reference's norm backward in the stock run, as in the tests above
+            for norm in (layer.input_layernorm, layer.post_attention_layernorm):
+                norm.forward = types.MethodType(lambda self, x: RefRMSNorm.apply(x, self.weight), norm)
+
+    def step():
+        for p in model.parameters():
+            p.grad = None
+        out = call()
+        out.loss.backward()
+        return out.logits.detach().clone(), {n: p.grad.clone() for n, p in model.named_parameters() if p.requires_grad}
+    model.train()
+    ref_logits, ref_grads = step()
+    model.eval()
+    with torch.no_grad():
+        eval_before = call().logits.clone()
+    assert hf.install(model, types.SimpleNamespace(use_hyclora=True, layer_type="baseline")) is model
+    model.train()
+    logits, grads = step()
+    assert all(getattr(layer, attr).iteration == 1 for layer in layers)          # the fused layers ran
+    rel, cos = rel_err_and_cos(logits, ref_logits)
+    assert rel <= 2e-2 and cos >= 0.9999
+    for name in grads:
+        rel, cos = rel_err_and_cos(grads[name], ref_grads[name])
+        assert rel <= 3e-2 and cos >= 0.999, f"{family} {name}: rel {rel:.2e} cos {cos:.6f}"
+    model.eval()
+    with torch.no_grad():
+        eval_after = call().logits
+    assert torch.equal(eval_after, eval_before)                                  # evaluation takes the stock layers
+    assert all(getattr(layer, attr).iteration == 1 for layer in layers)
+    with pytest.raises(ValueError):
+        hf.install(types.SimpleNamespace(config=types.SimpleNamespace(model_type="gpt2")), None)

@@ -157,3 +157,28 @@ def test_lora_scaling_other_than_one_is_refused():
     lin.scaling = {"default": 2.0}
     with pytest.raises(ValueError):
         lora_linear_parts(lin)
+
+
+def test_install_on_a_stock_model_routes_by_training_mode():
+    """hyclora_amd.models.hf.install on the CPU: evaluation keeps the stock layers (same bits as before); a
+    training-mode step reaches the fused layers, which refuse CPU tensors (there is no fallback path)."""
+    transformers = pytest.importorskip("transformers")
+    from hyclora_amd.models import hf, llama
+    cfg = transformers.LlamaConfig(vocab_size=64, hidden_size=64, intermediate_size=128, num_hidden_layers=2,
+                                   num_attention_heads=2, num_key_value_heads=2, max_position_embeddings=64,
+                                   attn_implementation="eager")
+    torch.manual_seed(0)
+    model = transformers.LlamaForCausalLM(cfg).eval()
+    ids = torch.randint(0, 64, (2, 8))
+    with torch.no_grad():
+        before = model(input_ids=ids).logits
+        hf.install(model, CFG)
+        assert all(isinstance(layer.fused_llama_layer, llama.FusedLlamaLayerIntraInter) for layer in model.model.layers)
+        assert torch.equal(model(input_ids=ids).logits, before)
+    model.train()
+    with pytest.raises((RuntimeError, AttributeError)):          # no LoRA wrappers / no GPU: the fused path is taken and fails loudly
+        model(input_ids=ids, use_cache=False)
+    with pytest.raises(ValueError):
+        hf.install(SimpleNamespace(config=SimpleNamespace(model_type="gpt2")), CFG)
+    with pytest.raises(ValueError):
+        hf.install(SimpleNamespace(config=SimpleNamespace(model_type="mistral")), CFG, map_free=True)
