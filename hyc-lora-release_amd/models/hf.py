@@ -26,6 +26,14 @@ def _causal_mask(seq_len, device, dtype):
     return mask
 
 
+def _additive(mask, dtype):
+    """A boolean attention mask (True = may attend; what transformers hands its layers with the sdpa back end) as the
+    additive mask the fused layers take, with the most negative finite value where its eager back end puts it."""
+    if mask is None or mask.dtype != torch.bool:
+        return mask
+    return torch.zeros(mask.shape, dtype=dtype, device=mask.device).masked_fill_(~mask, torch.finfo(dtype).min)
+
+
 def install(model, hyclora_config, map_free=False):
     """Attach fused layers to `model` (a stock Llama, Mistral or RoBERTa model of transformers, chosen by
     `model.config.model_type`) and route its layers through them in training mode.  `map_free=True` takes the
@@ -66,7 +74,7 @@ def _route_decoder_layer(layer, pkg, attr, map_free):
         elif attention_mask is None:              # attention back ends that build the causal mask themselves
             mask = _causal_mask(hidden_states.shape[1], hidden_states.device, hidden_states.dtype)
         else:
-            mask = attention_mask
+            mask = _additive(attention_mask, hidden_states.dtype)
         return pkg.decoder_layer_forward(self, hidden_states, mask, cos, sin)
     layer.forward = types.MethodType(forward, layer)
 
@@ -78,5 +86,5 @@ def _route_encoder_layer(layer):
         fused = self.fused_roberta_layer
         if not (self.training and fused.use_hyclora):
             return stock_forward(hidden_states, attention_mask, *args, **kwargs)
-        return roberta.encoder_layer_forward(self, hidden_states, attention_mask)
+        return roberta.encoder_layer_forward(self, hidden_states, _additive(attention_mask, hidden_states.dtype))
     layer.forward = types.MethodType(forward, layer)

@@ -195,6 +195,50 @@ def test_stock_roberta_through_the_fused_layers(dev, layer_type, q_bit, padding)
           f"worst gradient {worst[2]}: rel {worst[0]:.2e} cos {worst[1]:.5f}")
 
 
+@pytest.mark.parametrize("padding", [False, True])
+def test_install_under_the_sdpa_back_end(dev, padding):
+    """With transformers' default attention back end the layers are handed no mask (causal, nothing padded) or a
+    boolean one: `install` turns either into the additive mask of the fused layers.  Against the same model under
+    the eager back end and autograd."""
+    import hyclora_amd  # noqa: F401
+    from hyclora_amd.models import hf
+    ids = torch.randint(0, 128, (2, 128), generator=torch.Generator().manual_seed(1)).to(dev)
+    mask = torch.ones(2, 128, dtype=torch.long, device=dev)
+    if padding:
+        mask[1, 100:] = 0
+    labels = ids.masked_fill(mask == 0, -100)
+    results = []
+    for impl, fused in (("eager", False), ("sdpa", True)):
+        model = build(dev, "llama", 128)
+        model.config._attn_implementation = impl
+        for layer in model.model.layers:
+            for norm in (layer.input_layernorm, layer.post_attention_layernorm):
+                norm.forward = types.MethodType(lambda self, x: RefRMSNorm.apply(x, self.weight), norm)
+        seen = []
+        if fused:
+            hf.install(model, types.SimpleNamespace(use_hyclora=True, layer_type="baseline"))
+            model.model.layers[0].register_forward_pre_hook(
+                lambda mod, args, kwargs: seen.append(kwargs.get("attention_mask", args[1] if len(args) > 1 else None)),
+                with_kwargs=True)
+        for p in model.parameters():
+            p.grad = None
+        out = model(input_ids=ids, attention_mask=mask if padding else None, labels=labels, use_cache=False)
+        out.loss.backward()
+        if fused:
+            assert all(layer.fused_llama_layer.iteration == 1 for layer in model.model.layers)
+            # what this back end hands a layer: nothing, or a boolean mask
+            assert len(seen) == 1 and (seen[0].dtype == torch.bool if padding else seen[0] is None), seen
+        results.append((out.logits.detach()[mask.bool()].clone(), out.loss.item(),
+                        {n: p.grad.clone() for n, p in model.named_parameters() if p.requires_grad}))
+    (ref_logits, ref_loss, ref_grads), (logits, loss, grads) = results
+    rel, cos = rel_err_and_cos(logits, ref_logits)                 # logits of the real tokens
+    assert rel <= 2e-2 and cos >= 0.9999, f"logits: rel {rel:.2e} cos {cos:.6f}"
+    assert abs(loss - ref_loss) <= 1e-2 * abs(ref_loss)
+    for name in grads:
+        rel, cos = rel_err_and_cos(grads[name], ref_grads[name])
+        assert rel <= 3e-2 and cos >= 0.999, f"{name}: rel {rel:.2e} cos {cos:.6f}"
+
+
 @pytest.mark.parametrize("family", ["llama", "mistral", "roberta"])
 def test_install_routes_training_steps_through_the_fused_layers(dev, family):
     """`hyclora_amd.models.hf.install` on a stock model: training-mode steps run the fused layers (the calibration
