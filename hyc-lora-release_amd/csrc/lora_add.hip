@@ -26,7 +26,7 @@ namespace hyc {
 constexpr int kAddThreads = 256;
 constexpr int kAddWaves = kAddThreads / kWave;
 constexpr int kAddPlainColTiles = 4;        // column tiles side by side in a workgroup of the plain add
-static Knob g_add_rows_per_wave[3]{32, 48, 48};   // plain, quantise, restore; see hyc_set_tuning
+static Knob g_add_rows_per_wave[3]{0, 48, 48};   // plain (0 = chosen per shape), quantise, restore; see hyc_set_tuning
 
 enum { kAddPlain = 0, kAddQuant = 1, kAddRestore = 2 };
 
@@ -263,6 +263,27 @@ static void add_launch_k(const LoraAddArgs& a, dim3 grid, int ksteps, hipStream_
 
 // Checks one operand set and fills in its launch shape: 1 = launch `blocks` workgroups, HYC_OK = nothing to do,
 // negative = error.
+// Strip height of the plain add.  The kernel keeps three waves per SIMD resident (3072 on the 256 compute units):
+// a launch of 4096 waves runs as one full generation and a third of one.  Of 32, 48 and 64 rows a wave the height
+// whose wave count fills its generations best is taken, 32 unless another is better by a twentieth (measured on
+// [4096, N]: N = 4096 14.5 us at 48 rows against 16.1 at 32; N = 5120, 11008, 14336 fastest at 32).
+static int plain_rows_per_wave(int64_t T, int col_tiles) {
+    constexpr double kResident = 3.0 * 4 * 256;
+    int best = 32;
+    double best_fill = 0.0;
+    for (int rows = 32; rows <= 64; rows += 16) {
+        const double waves = (double)kAddWaves * col_tiles * (double)cdiv(T, (int64_t)rows);
+        if (rows == 32 && waves <= kResident) return 32;            // everything is resident at once anyway
+        const double generations = (double)cdiv((int64_t)waves, (int64_t)kResident);
+        const double fill = waves / (generations * kResident);
+        if (fill > best_fill * (rows == 32 ? 1.0 : 1.05)) {
+            best_fill = fill;
+            best = rows;
+        }
+    }
+    return best;
+}
+
 template <int MODE>
 static int add_prepare(LoraAddArgs& a, int64_t T, int64_t N, int64_t R, int q_bit, int64_t& blocks) {
     blocks = 0;
@@ -290,9 +311,10 @@ static int add_prepare(LoraAddArgs& a, int64_t T, int64_t N, int64_t R, int q_bi
     a.N = (int)N;
     a.C = (int)(N / 8);
     a.R = (int)R;
-    a.rows_per_wave = g_add_rows_per_wave[MODE].get();
     const int ct = MODE == kAddPlain ? kAddPlainColTiles : 8 / q_bit;
     a.col_tiles = (int)cdiv(cdiv(N, kTileCols), ct);
+    a.rows_per_wave = g_add_rows_per_wave[MODE].get();
+    if (a.rows_per_wave == 0) a.rows_per_wave = plain_rows_per_wave(T, a.col_tiles);
     const int64_t row_tiles = cdiv(T, (int64_t)(kAddWaves / ct) * a.rows_per_wave);
     if (row_tiles * a.col_tiles > INT32_MAX) return HYC_ERR_SHAPE;
     blocks = row_tiles * a.col_tiles;
@@ -440,6 +462,10 @@ int tune_add(const char* key, int value) {
     static const char* keys[3] = {"add_rows_per_wave", "add_quant_rows_per_wave", "add_restore_rows_per_wave"};
     for (int m = 0; m < 3; ++m) {
         if (strcmp(key, keys[m]) == 0) {
+            if (value == 0 && m == kAddPlain) {              // back to the per-shape choice
+                g_add_rows_per_wave[m].set(0);
+                return HYC_OK;
+            }
             if (value < kTileRows || value > 65536 || value % kTileRows != 0) return HYC_ERR_ARG;
             g_add_rows_per_wave[m].set(value);
             return HYC_OK;
@@ -547,6 +573,7 @@ extern "C" int hyc_lora_add_sum(const hyc_lora_sum_member* members, int count, v
     a.C = (int)(N / 8);
     a.R = (int)R;
     a.rows_per_wave = g_add_rows_per_wave[kAddPlain].get();
+    if (a.rows_per_wave == 0) a.rows_per_wave = 32;
     a.col_tiles = (int)cdiv(cdiv(N, kTileCols), kAddPlainColTiles);
     const int64_t row_tiles = cdiv(T, (int64_t)(kAddWaves / kAddPlainColTiles) * a.rows_per_wave);
     if (row_tiles * a.col_tiles > INT32_MAX) return HYC_ERR_SHAPE;

@@ -521,7 +521,7 @@ int hyc_lora_silu_mul_bwd(const void *xa1, const void *b1, const void *q1, const
  *   scale, zero_point bf16 [N] (zero_point NULL: symmetric codes);  q uint8 [T, N*q_bit/8].
  *   R: multiple of 4, 4..64; N % 32 == 0; any T.
  * Tuning keys "add_rows_per_wave", "add_quant_rows_per_wave", "add_restore_rows_per_wave" (multiples of
- * 16; defaults 32, 48, 48).
+ * 16; defaults 0 = 32, 48 or 64 chosen per shape so that the waves fill their generations, 48, 48).
  */
 int hyc_lora_add(const void *xa, const void *b, int b_transposed, const void *x, const void *residual,
                  void *y, int64_t T, int64_t N, int64_t R, void *stream);

@@ -315,3 +315,28 @@ def test_sum_of_lora_adds_rejects_what_it_cannot_run(dev):
         lk.lora_add_sum(wide)
     with pytest.raises(ValueError):
         lk.lora_add_sum([ok[0], (rn(1, 32, 256), rn(1, 32, 16), rn(16, 256))])
+
+
+@pytest.mark.parametrize("dims", [(1, 300, 640, 16), (4, 1024, 4096, 16), (2, 1000, 1536, 8)])
+def test_plain_add_does_not_depend_on_the_strip_height(K, dev, dims):
+    """The plain add picks its strip height per shape (32, 48 or 64 rows a wave, whichever fills the resident
+    waves' generations best; [4096, 4096] takes 48): every height gives the same bits, with and without a
+    residual, and 0 restores the per-shape choice."""
+    from hyclora_amd import _lib
+    B, M, N, R = dims
+    main, xa, b = inputs(7 + N, B, M, N, R)
+    res = torch.randn(B, M, N, generator=torch.Generator().manual_seed(3)).to(BF16)
+    d = lambda t: t.to(dev)
+    want = K.add(d(main), d(xa), d(b))
+    want_res = K.add(d(main), d(xa), d(b), residual=d(res))
+    mostly_same_bits(want, O.lora_add(main, xa, b), "auto height")
+    try:
+        for rows in (16, 32, 48, 64, 112):
+            _lib.set_tuning("add_rows_per_wave", rows)
+            assert torch.equal(K.add(d(main), d(xa), d(b)), want), rows
+            assert torch.equal(K.add(d(main), d(xa), d(b), residual=d(res)), want_res), rows
+    finally:
+        _lib.set_tuning("add_rows_per_wave", 0)
+    assert torch.equal(K.add(d(main), d(xa), d(b)), want)
+    with pytest.raises(Exception):
+        _lib.set_tuning("add_quant_rows_per_wave", 0)          # only the plain add has a per-shape choice
