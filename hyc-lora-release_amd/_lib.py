@@ -6,6 +6,7 @@ code, an exception is raised — there is no CPU or torch fallback.
 from __future__ import annotations
 
 import ctypes
+import weakref
 from ctypes import c_char_p, c_int, c_int64, c_void_p
 from pathlib import Path
 
@@ -161,3 +162,22 @@ def require_gpu(*tensors) -> None:
 
 def set_tuning(key: str, value: int) -> None:
     call("hyc_set_tuning", key.encode(), int(value))
+
+
+_BF16_VECTORS = {}       # id(tensor) -> (weak reference to it, its version, its bfloat16 copy)
+
+
+def bf16_vector(t: torch.Tensor) -> torch.Tensor:
+    """`t.to(bfloat16).reshape(-1)` for a per-channel vector that is not bfloat16 (a frozen zero point is kept as the
+    running mean of int8 values, a float tensor), converted once per tensor object: the frozen statistics are the
+    same objects step after step, and a conversion kernel per use costs a launch each.  The copy is kept with the
+    tensor (weakly) and made again when the tensor has been modified in place."""
+    if t.dtype == torch.bfloat16:
+        return t.reshape(-1)
+    key = id(t)
+    hit = _BF16_VECTORS.get(key)
+    if hit is not None and hit[0]() is t and hit[1] == t._version:
+        return hit[2]
+    conv = t.to(torch.bfloat16).reshape(-1).contiguous()
+    _BF16_VECTORS[key] = (weakref.ref(t, lambda _r, k=key: _BF16_VECTORS.pop(k, None)), t._version, conv)
+    return conv

@@ -76,7 +76,7 @@ class _Addr:
 
 def _vec(t: torch.Tensor, n: int, name: str) -> torch.Tensor:
     """A per-channel vector ([1, N], [N], ...) as contiguous, aligned bf16 [N]."""
-    t = t.to(BF16).reshape(-1)
+    t = _lib.bf16_vector(t)
     if t.numel() != n:
         raise ValueError(f"{name} must have {n} elements (one per channel), got {t.numel()}")
     if not t.is_contiguous() or t.data_ptr() % 16:

@@ -133,7 +133,7 @@ def _vec_ok(t, n, name):
 
 def _vec(t, n, name):
     _vec_ok(t, n, name)
-    return _prep(t.to(BF16).reshape(-1), name)
+    return _prep(_lib.bf16_vector(t), name)
 
 
 ROPE_HEAD_DIM = 128          # the fused rotation needs heads as wide as a column tile

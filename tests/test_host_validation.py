@@ -116,3 +116,24 @@ def test_compressed_map_lists_must_belong_to_the_map():
             sk.softmax_backward_from_compressed(*bad, g)
         with pytest.raises(ValueError, match="compressed map|seg_offsets"):
             cf.restore_attention_map(*bad, g.shape)
+
+
+def test_bf16_vector_is_converted_once_per_tensor_and_again_after_a_change():
+    """Frozen per-channel statistics that are not bfloat16 (a zero point kept as a running mean) are converted once
+    per tensor object, not at every call; an in-place change of the tensor invalidates the copy."""
+    import torch
+    from hyclora_amd import _lib
+    z = torch.tensor([[1.0, -3.0, 7.5, 0.25]])
+    a = _lib.bf16_vector(z)
+    assert a.dtype == torch.bfloat16 and a.shape == (4,) and a.tolist() == [1.0, -3.0, 7.5, 0.25]
+    assert _lib.bf16_vector(z) is a
+    z[0, 1] = 2.0
+    b = _lib.bf16_vector(z)
+    assert b is not a and b.tolist() == [1.0, 2.0, 7.5, 0.25]
+    s = torch.ones(1, 4, dtype=torch.bfloat16)
+    assert _lib.bf16_vector(s).data_ptr() == s.data_ptr()          # already bfloat16: a view, nothing kept
+    n = len(_lib._BF16_VECTORS)
+    del z, a, b
+    import gc
+    gc.collect()
+    assert len(_lib._BF16_VECTORS) == n - 1
